@@ -1,0 +1,249 @@
+/*
+ * blaze_hip.h -- C ABI of the MI355X (gfx950) kernel layer behind Blaze's sparse
+ * CTR inference hot path: Embedding gather/pool, fused FC, batched matmul,
+ * standalone activations.
+ *
+ * Conventions
+ *   - every pointer named *_dev / documented "device" is HIP device memory on the
+ *     current device; the library never allocates, frees or synchronises;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work
+ *     is stream ordered;
+ *   - return 0 on success, a negative BZ_E* code otherwise; bz_last_error() gives
+ *     the message for the calling thread; nothing throws across this boundary.
+ *
+ * The reference has no C layer at this level: its operators are C++ templates that
+ * call cuBLAS / CUDA kernels directly.  Each entry point below names the reference
+ * code it stands in for (paths relative to the reference's blaze/ directory).
+ */
+#ifndef BLAZE_HIP_H_
+#define BLAZE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BZ_API __attribute__((visibility("default")))
+
+typedef void* bz_stream_t;
+
+enum bz_status {
+  BZ_OK = 0,
+  BZ_EINVAL = -22,  /* bad argument (shape, alignment, enum) */
+  BZ_ENOTSUP = -95, /* valid request this build has no kernel for */
+  BZ_EHIP = -5      /* a HIP runtime call failed */
+};
+
+/* element types; values of the first five follow blaze/proto/blaze.proto:6-19 (DataType) */
+enum bz_dtype {
+  BZ_F32 = 1,
+  BZ_I32 = 2,
+  BZ_I8 = 7,
+  BZ_I64 = 10,
+  BZ_F16 = 12,
+  BZ_BF16 = 100 /* not a Blaze DataType; used by the bf16 dense tower */
+};
+
+/* pooling kinds, blaze/proto/embedding.proto:20-25 and blaze/store/store.h:21-25 */
+enum bz_udf { BZ_SUM = 0, BZ_AVG = 1, BZ_ASSIGN = 2 };
+/* blaze/proto/embedding.proto:14-17, blaze/store/sparse_puller.h:35-38 */
+enum bz_trunc { BZ_ORDER = 0, BZ_REVERSE = 1 };
+
+/* message of the last failing call on this thread (never NULL); mirrors the
+ * thread-local error buffer of blaze/api/c_api/c_api_error.cc:12-28 */
+BZ_API const char* bz_last_error(void);
+
+/* library / device probe: fills name (<= cap bytes) with the gcnArchName of the
+ * current device, returns BZ_ENOTSUP when it is not gfx950 */
+BZ_API int bz_device_check(char* name, size_t cap);
+
+/* ------------------------------------------------------------------------- */
+/* Embedding                                                                  */
+/* ------------------------------------------------------------------------- */
+
+/*
+ * One (feature group -> block item) unit of work.  An array of these lives in
+ * DEVICE memory and is owned by the caller (the Embedding operator), which
+ * rewrites it when an input blob moves.  It carries what the reference passes as
+ * SparsePullerInput + SparsePullerInput::Param + SparsePullerOutput::OutItem
+ * (blaze/store/sparse_puller.h:40-75) plus the resolved table.
+ *
+ * Table layout (repacked at load time from the QED blob, whose rows start at
+ * byte offset 1 and are unaligned, blaze/store/quick_embedding/weight_blob.h:20,42-52):
+ * row r starts at table + r*pitch, pitch is a multiple of 16 bytes, the base is
+ * 16-byte aligned, bytes between dim*sizeof(elem) and pitch are zero.
+ *
+ * ids are row numbers (id outside [0, rows) = not in table) unless hash_buckets is
+ * set; then ids are 64-bit keys resolved exactly as HashTable::Lookup does
+ * (blaze/store/quick_embedding/hashtable.cc:45-64): bucket = (uint32)key %
+ * hash_bucket_size, linear scan of the bucket's (u64 key, u64 row) pairs.
+ */
+typedef struct bz_embed_slot {
+  const void* table;          /* device; NULL = unknown table: the item's columns are zero-filled */
+  const float* row_scale;     /* device [rows]; BZ_I8 tables only */
+  const uint64_t* hash_buckets; /* device [hash_bucket_size] records {offset:40 (bytes into pairs), size:24}; or NULL */
+  const uint64_t* hash_pairs;   /* device (key,row) pairs */
+  const int64_t* ids;         /* device [nnz]   "<fg>.ids"      */
+  const float* values;        /* device [nnz]   "<fg>.values"   */
+  const int32_t* segments;    /* device [batch] "<fg>.segments": ids per sample (counts, not offsets) */
+  int64_t* offsets;           /* device [batch+1] scratch: exclusive scan of segments (written by
+                                 bz_segments_to_offsets_slots, read by bz_embed_pool) */
+  void* out;                  /* device: block base + this item's column offset */
+  int64_t rows;
+  int64_t out_stride;         /* elements between consecutive samples of the block */
+  uint32_t hash_bucket_size;
+  int32_t pitch;              /* bytes between table rows */
+  int32_t dim;
+  int32_t table_dtype;        /* BZ_F32 | BZ_F16 | BZ_I8 */
+  int32_t out_dtype;          /* BZ_F32 | BZ_F16 */
+  int32_t udf;                /* bz_udf */
+  int32_t trunc_dir;          /* bz_trunc, BZ_ASSIGN only */
+  int32_t trunc_num;          /* BZ_ASSIGN only */
+  int32_t batch;
+  int32_t wg_begin;           /* filled by bz_embed_plan: first workgroup of this slot */
+  int32_t wg_count;           /* filled by bz_embed_plan */
+  int32_t reserved_;
+} bz_embed_slot;
+
+/*
+ * Host-side planning: validates the slots (host copy) and fills wg_begin/wg_count.
+ * Returns the total number of workgroups in *total_wg.  The caller then copies the
+ * array to the device.  No reference counterpart (launch geometry).
+ */
+BZ_API int bz_embed_plan(bz_embed_slot* slots_host, int n_slots, int* total_wg);
+
+/*
+ * segments -> offsets for one array: off[i] = sum(segments[0..i)), off[n] = nnz.
+ * Stands in for the pointer walk `key += num; value += num` of
+ * QuickEmbeddingDict::Get (blaze/store/quick_embedding/quick_embedding_dict.cc:111-140).
+ * n <= 2^24.
+ */
+BZ_API int bz_segments_to_offsets(const int32_t* segments_dev, int64_t* offsets_dev, int64_t n, bz_stream_t stream);
+
+/* the same scan for every slot of a descriptor array in ONE launch (slot.segments -> slot.offsets) */
+BZ_API int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_slots, bz_stream_t stream);
+
+/*
+ * Gather + pool every slot in ONE launch.  Stands in for SparsePuller::Get as the
+ * Embedding operator calls it (blaze/operator/sparse_op/embedding/embedding_op.h:243)
+ * = QuickEmbeddingDict::Get (quick_embedding_dict.cc:76-148) over the
+ * K{Sum,Avg,Assign}Processors (udf_processor.h:43-133), including the per-item
+ * zero fill (InitProcess).  fp32 accumulate, multiply then add (not fused), ids in
+ * order: the fp32 output is bit-identical to the reference's loop.
+ * slots_dev must already hold offsets (bz_segments_to_offsets_slots).
+ */
+BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, int n_slots, int total_wg, bz_stream_t stream);
+
+/* name of the pooling kernel as profilers report it (for tooling) */
+BZ_API const char* bz_embed_pool_kernel_name(void);
+
+/* ------------------------------------------------------------------------- */
+/* Dense                                                                      */
+/* ------------------------------------------------------------------------- */
+
+enum bz_act {
+  BZ_ACT_NONE = 0,
+  BZ_ACT_PRELU = 1,      /* blaze/operator/op/prelu_op.cc:11-30: y = x*((x>0)+(x<0)*w[n % act_size]) */
+  BZ_ACT_DICE = 2,       /* blaze/operator/op/dice_op.cc:15-34 */
+  BZ_ACT_LEAKY_RELU = 3, /* blaze/operator/op/leaky_relu_op.cc:15-21: x>=0 ? x : act_alpha*x */
+  BZ_ACT_SIGMOID = 4,    /* blaze/operator/op/sigmoid_op.cc:15-21: e^x/(1+e^x) */
+  BZ_ACT_SOFTMAX = 5     /* blaze/operator/op/softmax_op.cc:21-78 over the N axis; N <= 64 only */
+};
+
+/*
+ * Y[M,N] = act( alpha * A[M,K] * W + beta * bias )
+ * = Gemm op (blaze/operator/op/gemm_op.h:33-107: Y <- broadcast(C); Y = alpha*op(A)op(B) + beta*Y)
+ * followed by the separate PRelu / Dice / LeakyRelu / Sigmoid / Softmax op the
+ * importer emits after it (blaze/model_importer/ulf_importer.cc:661-782).
+ *
+ * A is row major with leading dimension lda (elements).  W is the weight in the
+ * PACKED layout [N, ldw] = K contiguous per output column (the reference's
+ * transB=true form); bz_fc_pack_weight produces it from either form.  A 3-D
+ * Gemm with a shared weight (gemm_op.h:52-58,77-91) is the same call with
+ * M = batch*M.
+ */
+typedef struct bz_fc_desc {
+  const void* a;       /* device [M, lda] */
+  const void* w;       /* device [N, ldw] packed */
+  const void* bias;    /* device [N] (bias_rows==1) or [M, N] (bias_rows==M) or NULL; same dtype as out_acc_dtype F32 */
+  void* y;             /* device [M, ldy] */
+  const float* act_p0; /* PRELU: slope [act_size]; DICE: gamma [N] */
+  const float* act_p1; /* DICE: mean [N] */
+  const float* act_p2; /* DICE: var [N] */
+  int64_t lda, ldw, ldy;
+  int32_t m, n, k;
+  int32_t in_dtype;    /* BZ_F16 | BZ_BF16 | BZ_F32: type of a and w */
+  int32_t out_dtype;   /* BZ_F16 | BZ_BF16 | BZ_F32 */
+  int32_t bias_rows;   /* 0 none, 1 = [N] broadcast over rows, m = full [M,N] */
+  int32_t act;         /* bz_act */
+  int32_t act_size;    /* PRELU slope count (1 or N) */
+  int32_t dice_nosqrt; /* DICE: divide by var instead of sqrt(var+1e-8) */
+  float alpha, beta;
+  float act_alpha;     /* LEAKY_RELU slope */
+  int32_t reserved_;
+} bz_fc_desc;
+
+BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);
+
+/*
+ * Repack a Blaze weight blob for bz_fc_fused: src is [K,N] (trans_b=0) or [N,K]
+ * (trans_b=1) row major in src_dtype (F32 or F16); dst is [N, ldw] in dst_dtype
+ * with zero fill between K and ldw.  fp32 -> fp16 narrows with round-to-nearest-
+ * even like the reference's ConstantFill (blaze/common/proto_helper.cc:174,
+ * blaze/common/types.h:78-80).  ldw must be a multiple of 8 elements.
+ */
+BZ_API int bz_fc_pack_weight(const void* src_dev, int src_dtype, int trans_b, int k, int n, void* dst_dev, int dst_dtype,
+                             int64_t ldw, bz_stream_t stream);
+
+/*
+ * Strided-batched C[i] = alpha*op(A[i])*op(B[i]) + beta*C[i], row major, element
+ * strides (0 = operand shared by the whole batch).  Stands in for
+ * GemmStridedBatched (blaze/math/gemm.cc:82-139 / gemm.cu:251-336) as reached from
+ * MatMul (blaze/operator/op/matmul_op.h:77-89 via BroadcastGemm_NxN,
+ * blaze/math/broadcast.h:157-222), FusedParallelGemm
+ * (blaze/operator/fused_op/fused_parallel_gemm_op.h:96-129) and
+ * FusedParallelMatMul (fused_parallel_matmul_op.h:36-93).  The DIN attention
+ * weighted sum is the case M=1, K=T, N=D.
+ */
+typedef struct bz_bgemm_desc {
+  const void* a;
+  const void* b;
+  void* c;
+  int64_t stride_a, stride_b, stride_c;
+  int32_t trans_a, trans_b;
+  int32_t m, n, k;
+  int32_t batch;
+  int32_t dtype;     /* BZ_F32 | BZ_F16 for a, b, c alike (fp32 accumulate) */
+  float alpha, beta;
+} bz_bgemm_desc;
+
+BZ_API int bz_gemm_strided_batched(const bz_bgemm_desc* desc, bz_stream_t stream);
+
+/*
+ * Standalone activation ops over a [rows, cols] fp32 or fp16 tensor (in place
+ * allowed), for graphs where the producer is not a Gemm.  Same formulas and
+ * reference citations as bz_act above.
+ */
+typedef struct bz_act_desc {
+  const void* x;
+  void* y;
+  const float* p0;
+  const float* p1;
+  const float* p2;
+  int64_t rows, cols;
+  int32_t dtype;
+  int32_t act;
+  int32_t act_size;
+  int32_t dice_nosqrt;
+  float act_alpha;
+  int32_t reserved_;
+} bz_act_desc;
+
+BZ_API int bz_activation(const bz_act_desc* desc, bz_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLAZE_HIP_H_ */

@@ -1,0 +1,284 @@
+"""GPU parity of the dense path (bz_fc_fused, bz_fc_pack_weight, bz_gemm_strided_batched, bz_activation).
+
+The oracle is the reference's composition Activation(Gemm(x, W, b)) in fp32 (oracle/blaze_oracle.c) plus an
+fp64 product used to scale tolerances: MKL's / MFMA's summation orders differ, so the error bound is taken
+relative to sum_k |a||b| (the condition of the dot product), not to the possibly cancelled result.
+  fp32 path:       |got - want| <= 1e-5 * (sum|a||b| + |bias|)        (contract: rel 1e-5)
+  fp16/bf16 path:  |got - want| <= 2e-3 * (sum|a||b| + |bias|) (+ out rounding)   (contract: 2e-3)
+where want is computed from the same fp16/bf16-rounded inputs the kernel reads.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ACT = {"none": 0, "prelu": 1, "dice": 2, "relu": 3, "sigmoid": 4, "softmax": 5}
+
+
+@pytest.fixture(scope="module")
+def bz():
+    import torch
+    import blaze_hip
+    assert torch.cuda.is_available(), "no GPU visible"
+    blaze_hip.device_check()
+    return blaze_hip
+
+
+def _dev(x, dtype=None):
+    import torch
+    t = torch.from_numpy(np.ascontiguousarray(x)).cuda()
+    return t if dtype is None else t.to(dtype)
+
+
+def _tdtype(name):
+    import torch
+    return {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[name]
+
+
+def _round_to(x, name):
+    """numpy fp32 array rounded to the kernel's input precision (returned as fp32)."""
+    import torch
+    if name == "f32":
+        return x.astype(np.float32)
+    return torch.from_numpy(x.astype(np.float32)).to(_tdtype(name)).to(torch.float32).numpy()
+
+
+def _fc_case(bz, oracle, M, N, K, in_name, out_name, act, seed, trans_b=False, lda_pad=0, full_bias=False, alpha=1.0,
+             beta=1.0, bias=True):
+    import torch
+    rng = np.random.default_rng(seed)
+    A = _round_to(rng.standard_normal((M, K)), in_name)
+    Wkn = _round_to(rng.standard_normal((K, N)) / np.sqrt(K), in_name)
+    b = None
+    if bias:
+        b = (rng.standard_normal((M, N) if full_bias else N) * 0.1).astype(np.float32)
+    params_np, act_kwargs = (), {}
+    if act == "prelu":
+        params_np = (rng.uniform(0.1, 0.4, N).astype(np.float32),)
+    elif act == "dice":
+        params_np = ((rng.standard_normal(N) * 0.1).astype(np.float32), (rng.standard_normal(N) * 0.1).astype(np.float32),
+                     rng.uniform(0.5, 1.5, N).astype(np.float32))
+    # device inputs
+    a_dev = torch.zeros((M, K + lda_pad), dtype=_tdtype(in_name), device="cuda")
+    a_dev[:, :K] = _dev(A, _tdtype(in_name))
+    a_view = a_dev[:, :K]
+    w_src = _dev(Wkn.T.copy() if trans_b else Wkn, _tdtype(in_name) if in_name != "f32" else None)
+    wp = bz.pack_weight(w_src, trans_b, {"f32": bz.F32, "f16": bz.F16, "bf16": bz.BF16}[in_name])
+    out = bz.fc_fused(a_view, wp, K, bias=None if b is None else _dev(b), act=ACT[act],
+                      act_params=tuple(_dev(p) for p in params_np),
+                      out_dtype={"f32": bz.F32, "f16": bz.F16, "bf16": bz.BF16}[out_name], alpha=alpha, beta=beta,
+                      act_alpha=0.0)
+    torch.cuda.synchronize()
+    got = out.to(torch.float32).cpu().numpy()
+    # oracle: pre-activation in fp64 (tolerance scale) and the reference composition in fp32
+    pre64 = alpha * (A.astype(np.float64) @ Wkn.astype(np.float64))
+    scale = abs(alpha) * (np.abs(A).astype(np.float64) @ np.abs(Wkn).astype(np.float64))
+    if b is not None:
+        pre64 = pre64 + beta * b
+        scale = scale + np.abs(beta * b)
+    pre32 = pre64.astype(np.float32)
+    if act == "none":
+        want = pre32
+    elif act == "prelu":
+        want = oracle.prelu(pre32, params_np[0])
+    elif act == "dice":
+        want = oracle.dice(pre32, *params_np)
+    elif act == "relu":
+        want = oracle.leaky_relu(pre32, 0.0)
+    elif act == "sigmoid":
+        want = oracle.sigmoid(pre32)
+    else:
+        want = oracle.softmax(pre32, 1)
+    tol = 1e-5 if in_name == "f32" else 2e-3
+    out_eps = {"f32": 0.0, "f16": 2.0**-11, "bf16": 2.0**-8}[out_name]
+    # activations on this path are 1-Lipschitz up to the Dice gate (|d/dx| <= 1 + |gamma-1|*0.25*|x|/den): bound by 2
+    bound = 2.0 * tol * scale + out_eps * np.abs(want) + 1e-7
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert np.all(err <= bound), "M=%d N=%d K=%d %s->%s act=%s: err %.3e > bound %.3e at %s (got %r want %r)" % (
+        M, N, K, in_name, out_name, act, err[worst], bound[worst], worst, got[worst], want[worst])
+    return got, want
+
+
+def test_reference_gemm_kat_on_gpu(bz, kats):
+    import torch
+    from test_oracle_pins import _tensor
+    c = kats["gemm_net_v1_cpu"]
+    A, B, bias = (_tensor(c["tensors"][n]) for n in ("A_output", "B_output", "Bias_output"))
+    wp = bz.pack_weight(_dev(B), False, bz.F32)
+    out = bz.fc_fused(_dev(A), wp, 3, bias=_dev(bias))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(out.cpu().numpy(), np.array(c["expected"]["output"]["values"], np.float32).reshape(2, 2),
+                               rtol=0, atol=1e-6)
+
+
+def test_pack_weight_layout_and_rounding(bz):
+    import torch
+    rng = np.random.default_rng(0)
+    W = rng.standard_normal((37, 21)).astype(np.float32)  # [K, N]
+    for trans_b in (False, True):
+        src = _dev(W.T.copy() if trans_b else W)
+        for dt, tdt in ((bz.F32, torch.float32), (bz.F16, torch.float16), (bz.BF16, torch.bfloat16)):
+            p = bz.pack_weight(src, trans_b, dt)
+            torch.cuda.synchronize()
+            assert p.shape == (21, 40)
+            want = torch.from_numpy(W.T.copy()).to(tdt)
+            assert torch.equal(p[:, :37].cpu(), want)
+            assert not p[:, 37:].cpu().to(torch.float32).numpy().any()
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 200, 192), (128, 80, 200), (1, 80, 200), (33, 70, 20), (257, 129, 162)])
+@pytest.mark.parametrize("act", ["none", "prelu", "dice", "relu", "sigmoid"])
+def test_fc_fp32(bz, oracle, M, N, K, act):
+    print("case fp32 M=%d N=%d K=%d act=%s" % (M, N, K, act), flush=True)
+    _fc_case(bz, oracle, M, N, K, "f32", "f32", act, seed=M * 7 + N + K)
+
+
+@pytest.mark.parametrize("in_name,out_name", [("f16", "f16"), ("f16", "f32"), ("bf16", "bf16"), ("bf16", "f32")])
+@pytest.mark.parametrize("M,N,K,act", [(2048, 512, 896, "prelu"), (2048, 256, 512, "prelu"), (300, 80, 216, "dice"),
+                                       (300, 40, 80, "dice"), (64, 200, 168, "dice"), (4096, 2048, 256, "relu"),
+                                       (100, 100, 104, "none")])
+def test_fc_half(bz, oracle, in_name, out_name, M, N, K, act):
+    print("case %s->%s M=%d N=%d K=%d act=%s" % (in_name, out_name, M, N, K, act), flush=True)
+    _fc_case(bz, oracle, M, N, K, in_name, out_name, act, seed=M + N * 3 + K)
+
+
+@pytest.mark.parametrize("in_name", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,act", [(2048, 2, 256, "softmax"), (128, 2, 80, "softmax"), (5000, 1, 40, "none"),
+                                       (8192, 1, 256, "sigmoid"), (7, 8, 1000, "prelu"), (3, 3, 12, "dice")])
+def test_fc_skinny(bz, oracle, in_name, M, N, K, act):
+    print("case skinny %s M=%d N=%d K=%d act=%s" % (in_name, M, N, K, act), flush=True)
+    _fc_case(bz, oracle, M, N, K, in_name, "f32", act, seed=M + N + K)
+
+
+def test_fc_variants(bz, oracle):
+    """transB weights, padded lda, unaligned K with element-wise loads, full [M,N] bias, alpha/beta, no bias."""
+    _fc_case(bz, oracle, 70, 90, 64, "f16", "f16", "prelu", seed=1, trans_b=True)
+    _fc_case(bz, oracle, 70, 90, 162, "f16", "f32", "dice", seed=2, lda_pad=6)     # lda=168: vector loads + K tail
+    _fc_case(bz, oracle, 70, 90, 162, "f16", "f32", "dice", seed=3, lda_pad=0)     # lda=162: element-wise loads
+    _fc_case(bz, oracle, 70, 90, 50, "f32", "f32", "none", seed=4, lda_pad=1)      # fp32 unaligned
+    _fc_case(bz, oracle, 40, 48, 32, "f32", "f32", "none", seed=5, full_bias=True, alpha=0.5, beta=-2.0)
+    _fc_case(bz, oracle, 40, 48, 32, "f16", "f32", "relu", seed=6, bias=False)
+    _fc_case(bz, oracle, 40, 5, 32, "f16", "f32", "none", seed=7, full_bias=True, alpha=0.5, beta=-2.0)
+
+
+def test_fc_argument_errors(bz):
+    import torch
+    a = torch.zeros((4, 8), dtype=torch.float16, device="cuda")
+    w = torch.zeros((16, 8), dtype=torch.float16, device="cuda")
+    with pytest.raises(bz.BlazeHipError, match="softmax"):
+        bz.fc_fused(a, w, 8, act=ACT["softmax"])
+    with pytest.raises(bz.BlazeHipError, match="PRelu"):
+        bz.fc_fused(a, w, 8, act=ACT["prelu"], act_params=(torch.zeros(3, device="cuda"),))
+    with pytest.raises(bz.BlazeHipError, match="unknown activation"):
+        bz.fc_fused(a, w, 8, act=99)
+
+
+# ------------------------------------------------------------------------------ strided batched / matmul family
+def _bgemm(bz, A, B, M, N, K, batch, sa, sb, ta, tb, dtype, C0=None, alpha=1.0, beta=0.0):
+    import torch
+    a, b = _dev(A, dtype), _dev(B, dtype)
+    c = torch.zeros((batch, M, N), dtype=dtype, device="cuda") if C0 is None else _dev(C0, dtype)
+    bz.gemm_strided_batched(a, b, c, M, N, K, batch, sa, sb, M * N, ta, tb, alpha, beta)
+    torch.cuda.synchronize()
+    return c.to(torch.float32).cpu().numpy()
+
+
+@pytest.mark.parametrize("name", ["matmul_net_v1_cpu", "fused_parallel_matmul_net_v1_cpu", "fused_parallel_matmul_net_v2_cpu",
+                                  "fused_parallel_matmul_net_v3_cpu"])
+def test_reference_matmul_kats_on_gpu(bz, kats, name):
+    import torch
+    from test_oracle_pins import _tensor
+    c = kats[name]
+    op = c["ops"][0]
+    A, B = (_tensor(c["tensors"][n]) for n in op["inputs"])
+    ta, tb = bool(op["args"].get("transA", 0)), bool(op["args"].get("transB", 0))
+    P = op["args"].get("parallel_num", 1)
+    M, K = A.shape[-2:]
+    if ta:
+        M, K = K, M
+    N = B.shape[-2] if tb else B.shape[-1]
+    exp = c["expected"]["output"]
+    want = np.array(exp["values"], np.float32).reshape(exp["shape"])
+    ab, bb = A.shape[0] // P, B.shape[0] // P
+    cb = max(ab, bb)
+    got = np.zeros((P * cb, M, N), np.float32)
+    for p in range(P):  # BatchedBroadcastGemm: one strided-batched call per parallel slice (broadcast.h:340-378)
+        Ap, Bp = A[p * ab:(p + 1) * ab], B[p * bb:(p + 1) * bb]
+        got[p * cb:(p + 1) * cb] = _bgemm(bz, Ap, Bp, M, N, K, cb, 0 if ab == 1 else M * K, 0 if bb == 1 else K * N, ta, tb,
+                                          torch.float32)
+    np.testing.assert_allclose(got.reshape(want.shape), want, rtol=0, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["fused_parallel_gemm_net_v%d_cpu" % i for i in range(1, 6)])
+def test_reference_fused_parallel_gemm_kats_on_gpu(bz, kats, name):
+    """FusedParallelGemm = P FCs sharing the input: strided batched with stride_a = 0 (fused_parallel_gemm_op.h:115-129)
+    after the batched bias broadcast-assign."""
+    import torch
+    from test_oracle_pins import _tensor
+    c = kats[name]
+    op = c["ops"][0]
+    ins = [_tensor(c["tensors"][n]) for n in op["inputs"]]
+    A, B = ins[0], ins[1]
+    ta, tb = bool(op["args"].get("transA", 0)), bool(op["args"].get("transB", 0))
+    P = op["args"]["parallel_num"]
+    M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+    N = B.shape[0] // P if tb else B.shape[1]
+    C0 = np.zeros((P, M, N), np.float32)
+    beta = 0.0
+    if len(ins) > 2:
+        C0[:] = ins[2].reshape(P, 1, N)
+        beta = 1.0
+    got = _bgemm(bz, A, B, M, N, K, P, 0, K * N, ta, tb, torch.float32, C0=C0, alpha=1.0, beta=beta)
+    exp = c["expected"]["output"]
+    np.testing.assert_allclose(got.reshape(exp["shape"]), np.array(exp["values"], np.float32).reshape(exp["shape"]), rtol=0,
+                               atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype_name", ["f32", "f16"])
+def test_attention_weighted_sum(bz, oracle, dtype_name):
+    """DIN batchdot: scores [B,T,1] (transA) x history [B,T,D] -> [B,1,D]; config 3 shape B=1024, T=50, D=54."""
+    import torch
+    rng = np.random.default_rng(3)
+    Bn, T, D = 1024, 50, 54
+    w = _round_to(rng.standard_normal((Bn, T, 1)), dtype_name)
+    H = _round_to(rng.standard_normal((Bn, T, D)) * 0.1, dtype_name)
+    got = _bgemm(bz, w, H, 1, D, T, Bn, T, T * D, True, False, _tdtype(dtype_name))
+    want = oracle.matmul_op(w, H, transa=True, transb=False)
+    scale = np.einsum("btk,btd->bkd", np.abs(w), np.abs(H))
+    tol = 1e-5 if dtype_name == "f32" else 2e-3
+    assert np.all(np.abs(got - want) <= tol * scale + 1e-7)
+
+
+# ------------------------------------------------------------------------------ standalone activations
+@pytest.mark.parametrize("name,act", [("prelu_net_v1_cpu", 1), ("dice_net_v1_cpu", 2), ("leaky_relu_net_v1_cpu", 3),
+                                      ("sigmoid_net_v1_cpu", 4), ("softmax_net_v1_cpu", 5)])
+def test_reference_activation_kats_on_gpu(bz, kats, name, act):
+    import torch
+    from test_oracle_pins import _tensor
+    c = kats[name]
+    op = c["ops"][0]
+    ins = [_tensor(c["tensors"][n]) for n in op["inputs"]]
+    out = bz.activation(_dev(ins[0]), act, params=tuple(_dev(p) for p in ins[1:]), act_alpha=op["args"].get("alpha", 0.0))
+    torch.cuda.synchronize()
+    exp = c["expected"]["output"]
+    np.testing.assert_allclose(out.cpu().numpy(), np.array(exp["values"], np.float32).reshape(exp["shape"]), rtol=0,
+                               atol=1e-6)
+
+
+def test_activation_random_vs_oracle(bz, oracle):
+    import torch
+    rng = np.random.default_rng(11)
+    X = (rng.standard_normal((513, 77)) * 3).astype(np.float32)
+    g, mu, var = ((rng.standard_normal(77) * 0.1).astype(np.float32), (rng.standard_normal(77) * 0.1).astype(np.float32),
+                  rng.uniform(0.5, 1.5, 77).astype(np.float32))
+    slope = rng.uniform(0, 1, 77).astype(np.float32)
+    xd = _dev(X)
+    cases = [(1, (slope,), oracle.prelu(X, slope), {}), (2, (g, mu, var), oracle.dice(X, g, mu, var), {}),
+             (2, (g, mu, var), oracle.dice(X, g, mu, var, True), {"dice_nosqrt": True}),
+             (3, (), oracle.leaky_relu(X, 0.1), {"act_alpha": 0.1}), (4, (), oracle.sigmoid(X), {}),
+             (5, (), oracle.softmax(X, 1), {})]
+    for act, params, want, kw in cases:
+        got = bz.activation(xd, act, params=tuple(_dev(p) for p in params), **kw)
+        torch.cuda.synchronize()
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-6)

@@ -1,0 +1,245 @@
+"""GPU parity of the Embedding path (bz_segments_to_offsets*, bz_embed_pool) against the CPU oracle.
+
+Bars: offsets bit-exact (int64); pooled fp32 output bit-exact (the kernel sums in the
+reference's order with unfused multiply/add; the contract in the benchmark spec is rel 1e-5);
+fp16 output equal to the oracle's fp32 result rounded to nearest even (contract: 2e-3).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def bz():
+    import torch
+    import blaze_hip
+    assert torch.cuda.is_available(), "no GPU visible"
+    blaze_hip.device_check()
+    return blaze_hip
+
+
+def _dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def _bits(a):
+    a = np.ascontiguousarray(a)
+    return a.view(np.uint32) if a.dtype == np.float32 else a.view(np.uint16)
+
+
+@pytest.mark.parametrize("n", [1, 2, 63, 64, 65, 2047, 2048, 2049, 8192, 100003])
+def test_segments_to_offsets_bit_exact(bz, oracle, n):
+    import torch
+    rng = np.random.default_rng(n)
+    seg = rng.integers(0, 70, size=n).astype(np.int32)
+    print("case n=%d" % n, flush=True)
+    off = bz.segments_to_offsets(_dev(seg))
+    torch.cuda.synchronize()
+    assert np.array_equal(off.cpu().numpy(), oracle.segments_to_offsets(seg))
+
+
+def test_segments_to_offsets_no_32bit_wrap(bz, oracle):
+    import torch
+    seg = np.full(5, 2**31 - 1, np.int32)
+    off = bz.segments_to_offsets(_dev(seg))
+    torch.cuda.synchronize()
+    assert np.array_equal(off.cpu().numpy(), oracle.segments_to_offsets(seg))
+
+
+def _run_gpu(bz, tables_np, specs, inputs, batch, out_np_dtype, strides_cols):
+    """specs: list of (table index|None, udf, tdir, tnum, dim); one block, items packed at given cols."""
+    import torch
+    stride, cols = strides_cols
+    out = torch.full((batch, stride), float("nan"), dtype=torch.float32 if out_np_dtype == np.float32 else torch.float16,
+                     device="cuda")
+    dts = [None if t is None else bz.DeviceTable(t["data"], scale=t.get("scale"), keys=t.get("keys")) for t in tables_np]
+    items = []
+    for (ti, udf, tdir, tnum, dim), col, (ids, vals, seg) in zip(specs, cols, inputs):
+        items.append(dict(table=None if ti is None else dts[ti], ids=_dev(ids), values=_dev(vals), segments=_dev(seg),
+                          out=out, col=col, udf=udf, trunc_dir=tdir, trunc_num=tnum, dim=dim))
+    plan = bz.EmbeddingPlan(items)
+    plan.run()
+    torch.cuda.synchronize()
+    offs = [o.cpu().numpy() for o in plan.offsets]
+    return out.cpu().numpy(), offs
+
+
+def _run_oracle(oracle, tables_np, specs, inputs, batch, strides_cols):
+    stride, cols = strides_cols
+    out = np.full((batch, stride), np.nan, np.float32)
+    for (ti, udf, tdir, tnum, dim), col, (ids, vals, seg) in zip(specs, cols, inputs):
+        width = dim * tnum if udf == 2 else dim
+        if ti is None:
+            out[:, col:col + width] = 0  # Setup memsets the block; an unknown table writes nothing
+            continue
+        t = tables_np[ti]
+        table = oracle.Table(t["data"], scale=t.get("scale"), keys=t.get("keys"))
+        oracle.embed_get(table, ids, vals, seg, [(udf, tdir, tnum, out, col)])
+    return out
+
+
+def test_reference_qed_kat_on_gpu(bz, oracle):
+    """The reference's QuickEmbeddingDict.Get known answers through the device hash path."""
+    from test_oracle_pins import CASE1, CASE2, CASE3, CASE4, QED_KEYS, _qed_expected, _qed_inputs
+    import torch
+    ins = _qed_inputs()
+    b1 = torch.full((2, 12), float("nan"), device="cuda")
+    b2 = torch.full((2, 24), float("nan"), device="cuda")
+    t1 = bz.DeviceTable(np.array([CASE1], np.float32), keys=np.array(QED_KEYS["101"]))
+    t2 = bz.DeviceTable(np.array([CASE2], np.float32), keys=np.array(QED_KEYS["102"]))
+    t3 = bz.DeviceTable(np.array([CASE3, CASE4], np.float32), keys=np.array(QED_KEYS["104_7"]))
+    items = []
+    for (fg, t, out, col, udf, tn) in (("101", t1, b1, 0, 0, 0), ("102", t2, b1, 4, 0, 0), ("104_7", t3, b2, 0, 2, 4)):
+        ids, vals, seg = ins[fg]
+        items.append(dict(table=t, ids=_dev(ids), values=_dev(vals), segments=_dev(seg), out=out, col=col, udf=udf,
+                          trunc_dir=0, trunc_num=tn))
+    bz.EmbeddingPlan(items).run()
+    torch.cuda.synchronize()
+    e1, e2 = _qed_expected()
+    np.testing.assert_allclose(b1.cpu().numpy(), e1, rtol=5e-7, atol=0)
+    np.testing.assert_allclose(b2.cpu().numpy(), e2, rtol=5e-7, atol=0)
+
+
+def test_reference_embedding_op_kat_on_gpu(bz, kats):
+    """embedding_v1.conf (mock puller: every key resolves to a row of ones)."""
+    import torch
+    from test_oracle_pins import _tensor
+    case = kats["embedding_v1"]
+    t = case["tensors"]
+    b1 = torch.full((2, 12), float("nan"), device="cuda")
+    b2 = torch.full((2, 24), float("nan"), device="cuda")
+    items = []
+    for fg, dim, out, col, udf, tn in (("101", 4, b1, 0, 0, 0), ("102", 8, b1, 4, 0, 0), ("104_7", 6, b2, 0, 2, 4)):
+        ids = _tensor(t[fg + ".ids"])
+        keys = np.unique(ids)
+        table = bz.DeviceTable(np.ones((keys.size, dim), np.float32), keys=keys)
+        items.append(dict(table=table, ids=_dev(ids), values=_dev(_tensor(t[fg + ".values"])),
+                          segments=_dev(_tensor(t[fg + ".segments"])), out=out, col=col, udf=udf, trunc_dir=0,
+                          trunc_num=tn))
+    bz.EmbeddingPlan(items).run()
+    torch.cuda.synchronize()
+    for got, name in ((b1, "block1_values"), (b2, "block2_values")):
+        exp = case["expected"][name]
+        np.testing.assert_allclose(got.cpu().numpy(), np.array(exp["values"], np.float32).reshape(exp["shape"]), rtol=0,
+                                   atol=1e-6)
+
+
+def _make_table(rng, kind, rows, dim, with_keys):
+    t = {}
+    if kind == "f32":
+        t["data"] = (rng.standard_normal((rows, dim)) * 0.1).astype(np.float32)
+    elif kind == "f16":
+        t["data"] = (rng.standard_normal((rows, dim)) * 0.1).astype(np.float16)
+    else:
+        t["data"] = rng.integers(-127, 128, (rows, dim)).astype(np.int8)
+        t["scale"] = rng.uniform(1e-3, 1e-2, rows).astype(np.float32)
+    if with_keys:
+        t["keys"] = np.unique(rng.integers(-2**62, 2**62, size=rows * 2, dtype=np.int64))[:rows]
+        assert t["keys"].size == rows
+    return t
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "i8"])
+@pytest.mark.parametrize("out_dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("with_keys", [False, True])
+def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys):
+    """Ragged segments (incl. empty), absent ids, random values, odd dims and unaligned columns."""
+    seed = sum(map(ord, kind)) * 7 + (13 if out_dtype == np.float16 else 0) + (101 if with_keys else 0)
+    rng = np.random.default_rng(seed)
+    batch = 333
+    dims = [1, 4, 16, 18, 32, 33, 64, 100, 300]
+    tables, specs, inputs, cols = [], [], [], []
+    col = 1  # odd start column -> unaligned stores
+    for i, dim in enumerate(dims):
+        rows = int(rng.integers(5, 400))
+        tables.append(_make_table(rng, kind, rows, dim, with_keys))
+        udf, tdir, tnum = [(0, 0, 0), (1, 0, 0), (2, 0, 3), (2, 1, 4)][i % 4]
+        seg = rng.integers(0, 12, batch).astype(np.int32)
+        seg[rng.integers(0, batch, 20)] = 0
+        nnz = int(seg.sum())
+        if with_keys:
+            pool = np.concatenate([tables[-1]["keys"], rng.integers(-2**62, 2**62, size=rows // 4 + 1, dtype=np.int64)])
+            ids = rng.choice(pool, nnz)
+        else:
+            ids = rng.integers(-3, rows + 3, nnz)
+        vals = rng.standard_normal(nnz).astype(np.float32)
+        specs.append((i, udf, tdir, tnum, dim))
+        inputs.append((ids.astype(np.int64), vals, seg))
+        cols.append(col)
+        col += dim * tnum if udf == 2 else dim
+    stride = col + 3
+    print("case kind=%s out=%s keys=%s seed=%d" % (kind, out_dtype.__name__, with_keys, seed), flush=True)
+    got, offs = _run_gpu(bz, tables, specs, inputs, batch, out_dtype, (stride, cols))
+    want = _run_oracle(oracle, tables, specs, inputs, batch, (stride, cols))
+    for off, (_, _, seg) in zip(offs, inputs):
+        assert np.array_equal(off, oracle.segments_to_offsets(seg))
+    written = ~np.isnan(want)
+    assert np.array_equal(np.isnan(got.astype(np.float32)), ~written), "kernel wrote outside its items' columns"
+    if out_dtype == np.float32:
+        assert np.array_equal(_bits(got)[written], _bits(want)[written])
+    else:
+        with np.errstate(invalid="ignore"):
+            want16 = want.astype(np.float16)
+        assert np.array_equal(_bits(got)[written], _bits(want16)[written])
+
+
+def test_unknown_table_and_empty_batch(bz, oracle):
+    rng = np.random.default_rng(9)
+    batch = 70
+    t = _make_table(rng, "f32", 10, 8, False)
+    seg = rng.integers(0, 4, batch).astype(np.int32)
+    nnz = int(seg.sum())
+    ins = (rng.integers(0, 10, nnz).astype(np.int64), np.ones(nnz, np.float32), seg)
+    specs = [(None, 0, 0, 0, 8), (0, 0, 0, 0, 8), (None, 2, 0, 3, 8)]
+    cols = [0, 8, 16]
+    got, _ = _run_gpu(bz, [t], specs, [ins] * 3, batch, np.float32, (40, cols))
+    want = _run_oracle(oracle, [t], specs, [ins] * 3, batch, (40, cols))
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+def _config2_inputs(rng, batch, slots, rows):
+    """Config-2 shaped ids: length Poisson(8) clipped to [1,64], Zipf(1.1) ranks scattered over the rows."""
+    out = []
+    for _ in range(slots):
+        seg = np.clip(rng.poisson(8, batch), 1, 64).astype(np.int32)
+        nnz = int(seg.sum())
+        ranks = rng.zipf(1.1, nnz * 2)
+        ranks = ranks[ranks <= rows][:nnz]
+        while ranks.size < nnz:
+            more = rng.zipf(1.1, nnz)
+            ranks = np.concatenate([ranks, more[more <= rows]])[:nnz]
+        ids = ((ranks.astype(np.int64) - 1) * 2654435761) % rows
+        out.append((ids, np.ones(nnz, np.float32), seg))
+    return out
+
+
+def test_config2_full_size(bz, oracle):
+    """26 slots x [1M,32] fp16, batch 2048, ksum into a [2048, 896] fp16 block at column 64 (dense features first)."""
+    import torch
+    rng = np.random.default_rng(20240613)
+    batch, slots, rows, dim = 2048, 26, 1_000_000, 32
+    inputs = _config2_inputs(rng, batch, slots, rows)
+    out = torch.zeros((batch, 896), dtype=torch.float16, device="cuda")
+    items, tables = [], []
+    g = torch.Generator(device="cuda").manual_seed(7)
+    for s in range(slots):
+        data = (torch.randn((rows, dim), generator=g, device="cuda") * 0.01).to(torch.float16)
+        tables.append(data)
+        ids, vals, seg = inputs[s]
+        items.append(dict(table=bz.DeviceTable(data), ids=_dev(ids), values=_dev(vals), segments=_dev(seg), out=out,
+                          col=64 + s * dim, udf=0))
+    plan = bz.EmbeddingPlan(items)
+    plan.run()
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert not got[:, :64].any(), "dense-feature columns must be left alone"
+    for s in (0, 7, 25):  # three slots checked in full against the oracle (touched rows only are copied to the host)
+        ids, vals, seg = inputs[s]
+        uniq, inv = np.unique(ids, return_inverse=True)
+        sub = tables[s][torch.from_numpy(uniq).cuda()].cpu().numpy()
+        want = np.zeros((batch, dim), np.float32)
+        oracle.embed_get(oracle.Table(sub), inv, vals, seg, [(0, 0, 0, want, 0)])
+        assert np.array_equal(_bits(got[:, 64 + s * dim:64 + (s + 1) * dim]), _bits(want.astype(np.float16)))
+        assert np.array_equal(plan.offsets[s].cpu().numpy(), oracle.segments_to_offsets(seg))

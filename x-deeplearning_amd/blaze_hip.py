@@ -1,0 +1,325 @@
+"""ctypes binding of lib/libblaze_hip.so (the C ABI of include/blaze_hip.h) for tests and the benchmark.
+
+PyTorch is used here only to own device memory and streams.  There is no CPU or
+PyTorch fallback: if the library is missing or the device is not gfx950 this
+module raises.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libblaze_hip.so")
+
+# enum bz_dtype / bz_udf / bz_trunc / bz_act
+F32, I32, I8, I64, F16, BF16 = 1, 2, 7, 10, 12, 100
+SUM, AVG, ASSIGN = 0, 1, 2
+ORDER, REVERSE = 0, 1
+ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 2, 3, 4, 5
+
+EXPORTS = [
+    "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
+    "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
+    "bz_activation"
+]
+
+
+class EmbedSlot(C.Structure):
+    _fields_ = [("table", C.c_void_p), ("row_scale", C.c_void_p), ("hash_buckets", C.c_void_p),
+                ("hash_pairs", C.c_void_p), ("ids", C.c_void_p), ("values", C.c_void_p), ("segments", C.c_void_p),
+                ("offsets", C.c_void_p), ("out", C.c_void_p), ("rows", C.c_int64), ("out_stride", C.c_int64),
+                ("hash_bucket_size", C.c_uint32), ("pitch", C.c_int32), ("dim", C.c_int32), ("table_dtype", C.c_int32),
+                ("out_dtype", C.c_int32), ("udf", C.c_int32), ("trunc_dir", C.c_int32), ("trunc_num", C.c_int32),
+                ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("reserved_", C.c_int32)]
+
+
+class FcDesc(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("act_p0", C.c_void_p),
+                ("act_p1", C.c_void_p), ("act_p2", C.c_void_p), ("lda", C.c_int64), ("ldw", C.c_int64),
+                ("ldy", C.c_int64), ("m", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("in_dtype", C.c_int32),
+                ("out_dtype", C.c_int32), ("bias_rows", C.c_int32), ("act", C.c_int32), ("act_size", C.c_int32),
+                ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
+                ("reserved_", C.c_int32)]
+
+
+class BgemmDesc(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p), ("stride_a", C.c_int64),
+                ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("trans_a", C.c_int32), ("trans_b", C.c_int32),
+                ("m", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("batch", C.c_int32), ("dtype", C.c_int32),
+                ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class ActDesc(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("p0", C.c_void_p), ("p1", C.c_void_p), ("p2", C.c_void_p),
+                ("rows", C.c_int64), ("cols", C.c_int64), ("dtype", C.c_int32), ("act", C.c_int32),
+                ("act_size", C.c_int32), ("dice_nosqrt", C.c_int32), ("act_alpha", C.c_float), ("reserved_", C.c_int32)]
+
+
+class BlazeHipError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    """Load the library (never builds it: build with __graft_entry__.build() or csrc/Makefile)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise BlazeHipError("%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                                "(there is no CPU fallback)" % LIB_PATH)
+        l = C.CDLL(LIB_PATH)
+        vp, i32, i64 = C.c_void_p, C.c_int32, C.c_int64
+        missing = [name for name in EXPORTS if not hasattr(l, name)]
+        if missing:
+            raise BlazeHipError("%s does not export %s (stale build?)" % (LIB_PATH, ", ".join(missing)))
+        l.bz_last_error.restype = C.c_char_p
+        l.bz_device_check.argtypes = [C.c_char_p, C.c_size_t]
+        l.bz_embed_plan.argtypes = [C.POINTER(EmbedSlot), C.c_int, C.POINTER(C.c_int)]
+        l.bz_segments_to_offsets.argtypes = [vp, vp, i64, vp]
+        l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
+        l.bz_embed_pool.argtypes = [vp, C.c_int, C.c_int, vp]
+        l.bz_embed_pool_kernel_name.restype = C.c_char_p
+        l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
+        l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
+        l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
+        l.bz_activation.argtypes = [C.POINTER(ActDesc), vp]
+        _lib = l
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise BlazeHipError("rc=%d: %s" % (rc, lib().bz_last_error().decode()))
+
+
+def device_check():
+    buf = C.create_string_buffer(64)
+    check(lib().bz_device_check(buf, 64))
+    return buf.value.decode()
+
+
+def _stream_ptr(stream=None):
+    import torch
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def torch_dtype(dt):
+    import torch
+    return {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16, I8: torch.int8, I32: torch.int32,
+            I64: torch.int64}[dt]
+
+
+def bz_dtype(t):
+    import torch
+    return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8, torch.int32: I32,
+            torch.int64: I64}[t]
+
+
+# ----------------------------------------------------------------------------------- tables
+class DeviceTable:
+    """An embedding table repacked for the kernels: row pitch padded to 16 bytes, zero padding.
+
+    rows: torch tensor [rows, dim] on cuda (float32 | float16 | int8) or a numpy array (uploaded).
+    keys: optional int64/uint64 numpy array -> device hash index with the reference's bucket rule.
+    """
+
+    def __init__(self, rows, scale=None, keys=None, device="cuda"):
+        import torch
+        if isinstance(rows, np.ndarray):
+            if rows.dtype == np.uint16:
+                rows = rows.view(np.float16)
+            rows = torch.from_numpy(np.ascontiguousarray(rows)).to(device)
+        self.dtype = bz_dtype(rows.dtype)
+        assert self.dtype in (F32, F16, I8)
+        self.rows, self.dim = rows.shape
+        esz = rows.element_size()
+        row_bytes = self.dim * esz
+        self.pitch = (row_bytes + 15) // 16 * 16
+        if self.pitch == row_bytes:
+            self.data = rows.contiguous()
+        else:
+            pad = torch.zeros((self.rows, self.pitch // esz), dtype=rows.dtype, device=device)
+            pad[:, :self.dim] = rows
+            self.data = pad
+        assert self.data.data_ptr() % 16 == 0
+        self.scale = None
+        if scale is not None:
+            if isinstance(scale, np.ndarray):
+                scale = torch.from_numpy(np.ascontiguousarray(scale, dtype=np.float32))
+            self.scale = scale.to(device=device, dtype=torch.float32).contiguous()
+        self.hash_buckets = self.hash_pairs = None
+        self.hash_bucket_size = 0
+        if keys is not None:
+            self._build_hash(np.ascontiguousarray(keys).astype(np.uint64), device)
+
+    def _build_hash(self, keys, device):
+        """Device image of BulkLoadHashTable (hashtable.cc:137-187): prime bucket count, pairs sorted by
+        (bucket, key), bucket record = offset:40 | size:24 -- with the row number as the value."""
+        import torch
+        steps = [53, 97, 193, 389, 769, 1543, 3079, 6151, 12289, 24593, 49157, 98317, 196613, 393241, 786433, 1572869,
+                 3145739, 6291469, 12582917, 25165843, 50331653, 100663319, 201326611, 402653189, 805306457]
+        n = keys.size
+        nb = next((s for s in steps if s > n), steps[-1])
+        bucket = (keys & np.uint64(0xFFFFFFFF)) % np.uint64(nb)
+        order = np.lexsort((keys, bucket))
+        sk, sb = keys[order], bucket[order].astype(np.int64)
+        pairs = np.empty(2 * n, np.uint64)
+        pairs[0::2] = sk
+        pairs[1::2] = order.astype(np.uint64)
+        counts = np.bincount(sb, minlength=nb).astype(np.uint64)
+        first = np.zeros(nb, np.uint64)
+        uniq, idx = np.unique(sb, return_index=True)
+        first[uniq] = idx.astype(np.uint64) * np.uint64(16)
+        rec = (first & np.uint64(0xFFFFFFFFFF)) | (counts << np.uint64(40))
+        self.hash_bucket_size = nb
+        self.hash_buckets = torch.from_numpy(rec.view(np.int64)).to(device)
+        self.hash_pairs = torch.from_numpy(pairs.view(np.int64)).to(device)
+
+
+# ----------------------------------------------------------------------------------- embedding
+class EmbeddingPlan:
+    """Device-resident slot descriptors of one Embedding operator invocation.
+
+    items: list of dicts {table: DeviceTable|None, ids, values, segments (cuda tensors), out (cuda tensor
+    [B, stride]), col (element offset inside the block), udf, trunc_dir, trunc_num, dim}.
+    """
+
+    def __init__(self, items):
+        import torch
+        self.items = items
+        n = len(items)
+        arr = (EmbedSlot * n)()
+        self.offsets = []
+        for i, it in enumerate(items):
+            t = it["table"]
+            seg, out = it["segments"], it["out"]
+            assert seg.dtype == torch.int32 and it["ids"].dtype == torch.int64 and it["values"].dtype == torch.float32
+            assert out.dim() == 2 and out.stride(1) == 1
+            batch = seg.numel()
+            off = torch.empty(batch + 1, dtype=torch.int64, device=out.device)
+            self.offsets.append(off)
+            s = arr[i]
+            if t is not None:
+                s.table = t.data.data_ptr()
+                s.row_scale = t.scale.data_ptr() if t.scale is not None else None
+                s.hash_buckets = t.hash_buckets.data_ptr() if t.hash_buckets is not None else None
+                s.hash_pairs = t.hash_pairs.data_ptr() if t.hash_pairs is not None else None
+                s.hash_bucket_size = t.hash_bucket_size
+                s.rows, s.pitch, s.table_dtype = t.rows, t.pitch, t.dtype
+                s.dim = t.dim
+            else:
+                s.table = None
+                s.rows, s.pitch, s.table_dtype = 0, 0, F32
+                s.dim = it["dim"]
+            s.ids = it["ids"].data_ptr()
+            s.values = it["values"].data_ptr()
+            s.segments = seg.data_ptr()
+            s.offsets = off.data_ptr()
+            s.out = out.data_ptr() + it.get("col", 0) * out.element_size()
+            s.out_stride = out.stride(0)
+            s.out_dtype = bz_dtype(out.dtype)
+            s.udf = it.get("udf", SUM)
+            s.trunc_dir = it.get("trunc_dir", REVERSE)
+            s.trunc_num = it.get("trunc_num", 0)
+            s.batch = batch
+        total = C.c_int(0)
+        check(lib().bz_embed_plan(arr, n, C.byref(total)))
+        self.n, self.total_wg = n, total.value
+        self.host = arr
+        raw = np.frombuffer(bytes(arr), dtype=np.uint8).copy()
+        self.slots_dev = torch.from_numpy(raw).to(items[0]["out"].device)
+
+    def scan(self, stream=None):
+        check(lib().bz_segments_to_offsets_slots(self.slots_dev.data_ptr(), self.n, _stream_ptr(stream)))
+
+    def pool(self, stream=None):
+        check(lib().bz_embed_pool(self.slots_dev.data_ptr(), self.n, self.total_wg, _stream_ptr(stream)))
+
+    def run(self, stream=None):
+        self.scan(stream)
+        self.pool(stream)
+
+
+def segments_to_offsets(segments, stream=None):
+    import torch
+    assert segments.dtype == torch.int32 and segments.is_cuda
+    off = torch.empty(segments.numel() + 1, dtype=torch.int64, device=segments.device)
+    check(lib().bz_segments_to_offsets(segments.data_ptr(), off.data_ptr(), segments.numel(), _stream_ptr(stream)))
+    return off
+
+
+# ----------------------------------------------------------------------------------- dense
+def pack_weight(w, trans_b, dst_dtype, stream=None):
+    """Blaze weight [K,N] (trans_b False) or [N,K] (True) -> packed [N, ldw] for fc_fused."""
+    import torch
+    k, n = (w.shape[1], w.shape[0]) if trans_b else (w.shape[0], w.shape[1])
+    ldw = (k + 7) // 8 * 8
+    dst = torch.empty((n, ldw), dtype=torch_dtype(dst_dtype), device=w.device)
+    check(lib().bz_fc_pack_weight(w.data_ptr(), bz_dtype(w.dtype), int(trans_b), k, n, dst.data_ptr(), dst_dtype, ldw,
+                                  _stream_ptr(stream)))
+    return dst
+
+
+def fc_fused(a, w_packed, k, bias=None, act=ACT_NONE, act_params=(), out=None, out_dtype=None, alpha=1.0, beta=1.0,
+             act_alpha=0.0, dice_nosqrt=False, stream=None):
+    import torch
+    m = a.shape[0]
+    n = w_packed.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch_dtype(out_dtype or bz_dtype(a.dtype)), device=a.device)
+    d = FcDesc()
+    d.a, d.w, d.y = a.data_ptr(), w_packed.data_ptr(), out.data_ptr()
+    d.lda, d.ldw, d.ldy = a.stride(0), w_packed.stride(0), out.stride(0)
+    d.m, d.n, d.k = m, n, k
+    d.in_dtype, d.out_dtype = bz_dtype(a.dtype), bz_dtype(out.dtype)
+    assert w_packed.dtype == a.dtype
+    if bias is not None:
+        assert bias.dtype == torch.float32
+        d.bias = bias.data_ptr()
+        d.bias_rows = 1 if bias.numel() == n else m
+    d.act = act
+    ps = list(act_params) + [None] * 3
+    for name, p in zip(("act_p0", "act_p1", "act_p2"), ps):
+        if p is not None:
+            assert p.dtype == torch.float32
+            setattr(d, name, p.data_ptr())
+    d.act_size = ps[0].numel() if ps[0] is not None else 0
+    d.dice_nosqrt = int(dice_nosqrt)
+    d.alpha, d.beta, d.act_alpha = alpha, beta, act_alpha
+    check(lib().bz_fc_fused(C.byref(d), _stream_ptr(stream)))
+    return out
+
+
+def gemm_strided_batched(a, b, c, m, n, k, batch, stride_a, stride_b, stride_c, trans_a=False, trans_b=False, alpha=1.0,
+                         beta=0.0, stream=None):
+    d = BgemmDesc()
+    d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    d.stride_a, d.stride_b, d.stride_c = stride_a, stride_b, stride_c
+    d.trans_a, d.trans_b = int(trans_a), int(trans_b)
+    d.m, d.n, d.k, d.batch = m, n, k, batch
+    d.dtype = bz_dtype(a.dtype)
+    d.alpha, d.beta = alpha, beta
+    check(lib().bz_gemm_strided_batched(C.byref(d), _stream_ptr(stream)))
+    return c
+
+
+def activation(x, act, params=(), out=None, act_alpha=0.0, dice_nosqrt=False, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    d = ActDesc()
+    d.x, d.y = x.data_ptr(), out.data_ptr()
+    d.cols = x.shape[-1]
+    d.rows = x.numel() // x.shape[-1]
+    d.dtype, d.act = bz_dtype(x.dtype), act
+    ps = list(params) + [None] * 3
+    for name, p in zip(("p0", "p1", "p2"), ps):
+        if p is not None:
+            setattr(d, name, p.data_ptr())
+    d.act_size = ps[0].numel() if ps[0] is not None else 0
+    d.dice_nosqrt, d.act_alpha = int(dice_nosqrt), act_alpha
+    check(lib().bz_activation(C.byref(d), _stream_ptr(stream)))
+    return out

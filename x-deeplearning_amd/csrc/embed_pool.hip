@@ -1,0 +1,424 @@
+// embed_pool.hip -- Embedding gather + segmented pooling for gfx950 (MI355X).
+//
+// Replaces, for device-resident tables, the CPU loop of
+// blaze/store/quick_embedding/quick_embedding_dict.cc:89-148 (QuickEmbeddingDict::Get)
+// with its pooling processors blaze/store/quick_embedding/udf_processor.h:43-133 and
+// the key lookup blaze/store/quick_embedding/hashtable.cc:45-64.
+//
+// Work decomposition.  The workload is memory bound: per id one random table row
+// (36..256 bytes) plus 12 bytes of id/value.  A row is cut into 16-byte chunks
+// (one 128-bit load); a *lane group* of `lpr` = pow2(chunks per row) lanes owns one
+// (sample, slot) segment and walks its ids in order, so every output element is
+// summed in exactly the reference's order (bit-identical fp32).  A 256-thread
+// workgroup holds 256/lpr segments of consecutive samples of one slot; their
+// offsets are staged through LDS with one coalesced read.  The id loop is
+// unrolled by kUnroll with all row loads issued before the first add, which is
+// where the memory-level parallelism comes from.  One launch covers every slot
+// of the operator; the linear workgroup id is remapped so that each of the 8 XCDs
+// (each with its own L2) serves a contiguous range of slots and therefore caches
+// the hot rows of only those tables.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include "bz_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 8;
+
+// ---------------------------------------------------------------------------------------------
+// segments -> offsets (exclusive scan), one workgroup per array
+// ---------------------------------------------------------------------------------------------
+constexpr int kScanItems = 8;  // int32 per thread per tile -> 2048 per workgroup tile
+
+__device__ __forceinline__ int64_t wave_incl_scan(int64_t v, int lane) {
+#pragma unroll
+  for (int d = 1; d < bz::kWave; d <<= 1) {
+    int64_t t = __shfl_up(v, d, bz::kWave);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+__device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restrict__ off, int64_t n) {
+  __shared__ int64_t wave_tot[kThreads / bz::kWave];
+  __shared__ int64_t carry_s;
+  const int tid = threadIdx.x;
+  const int lane = tid & (bz::kWave - 1);
+  const int wave = tid / bz::kWave;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t base = 0; base < n; base += (int64_t)kThreads * kScanItems) {
+    int64_t i0 = base + (int64_t)tid * kScanItems;
+    int32_t v[kScanItems];
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) v[k] = (i0 + k < n) ? seg[i0 + k] : 0;
+    int64_t local = 0;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) local += v[k];
+    int64_t incl = wave_incl_scan(local, lane);
+    if (lane == bz::kWave - 1) wave_tot[wave] = incl;
+    __syncthreads();
+    int64_t before = carry_s;
+    for (int w = 0; w < wave; ++w) before += wave_tot[w];
+    int64_t run = before + incl - local;
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      if (i0 + k < n) off[i0 + k] = run;
+      run += v[k];
+    }
+    __syncthreads();
+    if (tid == kThreads - 1) carry_s = run;  // last thread's running total = total so far
+    __syncthreads();
+  }
+  if (tid == 0) off[n] = carry_s;
+}
+
+__global__ __launch_bounds__(kThreads) void bz_scan_segments_kernel(const int32_t* __restrict__ seg,
+                                                                    int64_t* __restrict__ off, int64_t n) {
+  scan_segments(seg, off, n);
+}
+
+__global__ __launch_bounds__(kThreads) void bz_scan_segments_slots_kernel(const bz_embed_slot* __restrict__ slots) {
+  const bz_embed_slot* s = &slots[blockIdx.x];
+  scan_segments(s->segments, s->offsets, s->batch);
+}
+
+// ---------------------------------------------------------------------------------------------
+// pooling
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+struct RowTraits;
+template <>
+struct RowTraits<BZ_F32> {
+  static constexpr int kElems = 4;  // per 16-byte chunk
+};
+template <>
+struct RowTraits<BZ_F16> {
+  static constexpr int kElems = 8;
+};
+template <>
+struct RowTraits<BZ_I8> {
+  static constexpr int kElems = 16;
+};
+
+// widen one 16-byte chunk to fp32 weights.  int8: w = scale * (float)q, one rounding.
+template <int DT>
+__device__ __forceinline__ void widen(const uint4& raw, float scale, float (&w)[RowTraits<DT>::kElems]) {
+  const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+  if constexpr (DT == BZ_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = __uint_as_float(r[i]);
+  } else if constexpr (DT == BZ_F16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      w[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xffffu)));
+      w[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int q = (int)(int8_t)((r[i] >> (8 * b)) & 0xffu);
+        w[4 * i + b] = __fmul_rn(scale, (float)q);
+      }
+    }
+  }
+}
+
+// key / id -> table row, or -1 when absent.  Hash path = HashTable::Lookup
+// (hashtable.cc:45-64): bucket record {offset:40, size:24}, (key,row) pairs.
+__device__ __forceinline__ int64_t resolve_row(const bz_embed_slot& s, int64_t id) {
+  if (s.hash_buckets != nullptr) {
+    const uint64_t key = (uint64_t)id;
+    const uint32_t h = (uint32_t)key;
+    const uint64_t rec = s.hash_buckets[h % s.hash_bucket_size];
+    const uint32_t cnt = (uint32_t)(rec >> 40);
+    const uint64_t* p = s.hash_pairs + ((rec & 0xffffffffffull) >> 3);
+    for (uint32_t i = 0; i < cnt; ++i) {
+      if (p[2 * i] == key) {
+        const uint64_t row = p[2 * i + 1];
+        return row < (uint64_t)s.rows ? (int64_t)row : -1;
+      }
+    }
+    return -1;
+  }
+  return (id >= 0 && id < s.rows) ? id : -1;
+}
+
+// Store `nvalid` fp32 results as the slot's output dtype at element pointer `dst`
+// using the widest store the address allows.
+template <int N>
+__device__ __forceinline__ void store_elems(void* dst_base, int64_t elem_off, const float (&v)[N], int nvalid,
+                                            int out_dtype) {
+  if (out_dtype == BZ_F32) {
+    float* dst = (float*)dst_base + elem_off;
+    if (nvalid == N && (((uintptr_t)dst) & 15) == 0) {
+#pragma unroll
+      for (int i = 0; i < N; i += 4) *(float4*)(dst + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i)
+        if (i < nvalid) dst[i] = v[i];
+    }
+  } else {  // BZ_F16, round to nearest even
+    __half* dst = (__half*)dst_base + elem_off;
+    uint32_t pk[N / 2];
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) {
+      uint32_t lo = __half_as_ushort(__float2half_rn(v[2 * i]));
+      uint32_t hi = __half_as_ushort(__float2half_rn(v[2 * i + 1]));
+      pk[i] = lo | (hi << 16);
+    }
+    const uintptr_t a = (uintptr_t)dst;
+    if (nvalid == N && (a & 15) == 0 && N >= 8) {
+#pragma unroll
+      for (int i = 0; i + 4 <= N / 2; i += 4) *(uint4*)((uint32_t*)dst + i) = make_uint4(pk[i], pk[i + 1], pk[i + 2], pk[i + 3]);
+    } else if (nvalid == N && (a & 7) == 0) {
+#pragma unroll
+      for (int i = 0; i < N / 2; i += 2) *(uint2*)((uint32_t*)dst + i) = make_uint2(pk[i], pk[i + 1]);
+    } else if ((a & 3) == 0) {
+#pragma unroll
+      for (int i = 0; i < N / 2; ++i) {
+        if (2 * i + 1 < nvalid)
+          ((uint32_t*)dst)[i] = pk[i];
+        else if (2 * i < nvalid)
+          dst[2 * i] = __ushort_as_half((unsigned short)(pk[i] & 0xffffu));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < N; ++i)
+        if (i < nvalid) dst[i] = __ushort_as_half((unsigned short)((pk[i / 2] >> (16 * (i & 1))) & 0xffffu));
+    }
+  }
+}
+
+// ksum / kavg for one lane: chunk `c` of the segment [start, end) of sample b.
+template <int DT>
+__device__ __forceinline__ void pool_sum(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b) {
+  constexpr int CE = RowTraits<DT>::kElems;
+  float acc[CE];
+#pragma unroll
+  for (int i = 0; i < CE; ++i) acc[i] = 0.f;
+  const char* table = (const char*)s.table + (int64_t)c * 16;
+  for (int64_t j = start; j < end; j += kUnroll) {
+    const int n = (int)((end - j) < kUnroll ? (end - j) : kUnroll);
+    int64_t row[kUnroll];
+    float val[kUnroll];
+    uint4 raw[kUnroll];
+    float sc[kUnroll];
+    // clamp instead of branching: the tail repeats the last id (cache hit), results ignored
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t jj = (u < n) ? j + u : end - 1;
+      row[u] = resolve_row(s, s.ids[jj]);
+      val[u] = s.values[jj];
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t r = row[u] < 0 ? 0 : row[u];
+      raw[u] = *(const uint4*)(table + r * (int64_t)s.pitch);
+      sc[u] = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      if (u < n && row[u] >= 0) {
+        float w[CE];
+        widen<DT>(raw[u], sc[u], w);
+        // out = out + value * w: two roundings, never an FMA (udf_processor.h:66)
+#pragma unroll
+        for (int i = 0; i < CE; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(val[u], w[i]));
+      }
+    }
+  }
+  if (s.udf == BZ_AVG) {
+    const int64_t num = end - start;
+    if (num != 0) {
+      const float inv = (float)(1.0 / (double)num);  // ValueType(1.0 / size), udf_processor.h:88
+#pragma unroll
+      for (int i = 0; i < CE; ++i) acc[i] = __fmul_rn(acc[i], inv);
+    }
+  }
+  const int e0 = c * CE;
+  const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
+  store_elems<CE>(s.out, b * s.out_stride + e0, acc, nvalid, s.out_dtype);
+}
+
+// kassign: position p of the output holds id j = p (in order) or num - trunc + p (reverse);
+// positions without an id, and ids absent from the table, are zero (udf_processor.h:103-131).
+template <int DT>
+__device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b) {
+  constexpr int CE = RowTraits<DT>::kElems;
+  const int64_t num = end - start;
+  const int e0 = c * CE;
+  const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
+  const char* table = (const char*)s.table + (int64_t)c * 16;
+  const int64_t shift = (s.trunc_dir == BZ_ORDER) ? 0 : num - (int64_t)s.trunc_num;
+  for (int p = 0; p < s.trunc_num; ++p) {
+    const int64_t j = shift + p;
+    float out[CE];
+#pragma unroll
+    for (int i = 0; i < CE; ++i) out[i] = 0.f;
+    if (j >= 0 && j < num) {
+      const int64_t r = resolve_row(s, s.ids[start + j]);
+      if (r >= 0) {
+        const float val = s.values[start + j];
+        const uint4 raw = *(const uint4*)(table + r * (int64_t)s.pitch);
+        const float sc = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
+        float w[CE];
+        widen<DT>(raw, sc, w);
+#pragma unroll
+        for (int i = 0; i < CE; ++i) out[i] = __fmul_rn(val, w[i]);
+      }
+    }
+    store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * s.dim + e0, out, nvalid, s.out_dtype);
+  }
+}
+
+// zero fill of one item's columns (unknown table name: quick_embedding_dict.cc:95 leaves the
+// memset block untouched)
+__device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int l, int lpr) {
+  const int width = (s.udf == BZ_ASSIGN) ? s.dim * s.trunc_num : s.dim;
+  for (int e = l; e < width; e += lpr) {
+    if (s.out_dtype == BZ_F32)
+      ((float*)s.out)[b * s.out_stride + e] = 0.f;
+    else
+      ((__half*)s.out)[b * s.out_stride + e] = __ushort_as_half(0);
+  }
+}
+
+__device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (dt == BZ_F16 ? 8 : 16); }
+
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
+                                                                 int total_wg, int wg_per_xcd) {
+  __shared__ int64_t s_off[kThreads + 1];
+  // XCD-aware order: hardware deals consecutive workgroup ids round robin over the 8 XCDs; give
+  // each XCD a contiguous range of the logical workgroup space (= a contiguous range of slots).
+  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
+  if (v >= total_wg) return;
+  int lo = 0, hi = n_slots - 1;  // last slot with wg_begin <= v (empty slots share a begin: take the last)
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (slots[mid].wg_begin <= v)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  // slots with wg_count == 0 sharing this begin come before the one that owns the workgroup
+  const bz_embed_slot s = slots[lo];
+  const int ce = chunk_elems(s.table_dtype);
+  const int nchunks = (s.dim + ce - 1) / ce;
+  int lpr = 1;
+  while (lpr < nchunks && lpr < bz::kWave) lpr <<= 1;
+  const int groups = kThreads / lpr;
+  const int tid = threadIdx.x;
+  const int g = tid / lpr;
+  const int l = tid - g * lpr;
+  const int64_t b0 = (int64_t)(v - s.wg_begin) * groups;
+  // stage this workgroup's offsets through LDS (one coalesced read instead of 2 per lane)
+  for (int t = tid; t <= groups; t += kThreads)
+    if (b0 + t <= s.batch) s_off[t] = s.offsets[b0 + t];
+  __syncthreads();
+  const int64_t b = b0 + g;
+  if (b >= s.batch) return;
+  if (s.table == nullptr) {
+    pool_zero(s, b, l, lpr);
+    return;
+  }
+  const int64_t start = s_off[g], end = s_off[g + 1];
+  for (int c = l; c < nchunks; c += lpr) {
+    if (s.udf == BZ_ASSIGN) {
+      switch (s.table_dtype) {
+        case BZ_F32: pool_assign<BZ_F32>(s, start, end, c, b); break;
+        case BZ_F16: pool_assign<BZ_F16>(s, start, end, c, b); break;
+        default: pool_assign<BZ_I8>(s, start, end, c, b); break;
+      }
+    } else {
+      switch (s.table_dtype) {
+        case BZ_F32: pool_sum<BZ_F32>(s, start, end, c, b); break;
+        case BZ_F16: pool_sum<BZ_F16>(s, start, end, c, b); break;
+        default: pool_sum<BZ_I8>(s, start, end, c, b); break;
+      }
+    }
+  }
+}
+
+int groups_per_wg(const bz_embed_slot& s) {
+  const int ce = s.table_dtype == BZ_F32 ? 4 : (s.table_dtype == BZ_F16 ? 8 : 16);
+  const int nchunks = (s.dim + ce - 1) / ce;
+  int lpr = 1;
+  while (lpr < nchunks && lpr < bz::kWave) lpr <<= 1;
+  return kThreads / lpr;
+}
+
+}  // namespace
+
+extern "C" {
+
+int bz_embed_plan(bz_embed_slot* slots, int n_slots, int* total_wg) {
+  BZ_REQUIRE(slots != nullptr && total_wg != nullptr && n_slots > 0, "bz_embed_plan: null argument or n_slots=%d", n_slots);
+  int64_t total = 0;
+  for (int i = 0; i < n_slots; ++i) {
+    bz_embed_slot& s = slots[i];
+    BZ_REQUIRE(s.table_dtype == BZ_F32 || s.table_dtype == BZ_F16 || s.table_dtype == BZ_I8,
+               "slot %d: unsupported table dtype %d", i, s.table_dtype);
+    BZ_REQUIRE(s.out_dtype == BZ_F32 || s.out_dtype == BZ_F16, "slot %d: unsupported out dtype %d", i, s.out_dtype);
+    BZ_REQUIRE(s.udf == BZ_SUM || s.udf == BZ_AVG || s.udf == BZ_ASSIGN, "slot %d: Unsupported udf type: %d", i, s.udf);
+    BZ_REQUIRE(s.dim > 0 && s.batch >= 0, "slot %d: dim=%d batch=%d", i, s.dim, s.batch);
+    if (s.udf == BZ_ASSIGN)
+      BZ_REQUIRE(s.trunc_num > 0 && (s.trunc_dir == BZ_ORDER || s.trunc_dir == BZ_REVERSE),
+                 "slot %d: kAssign needs trunc_num > 0 and a trunc direction (trunc_num=%d dir=%d)", i, s.trunc_num,
+                 s.trunc_dir);
+    BZ_REQUIRE(s.out != nullptr && s.offsets != nullptr && (s.batch == 0 || s.segments != nullptr),
+               "slot %d: null out/offsets/segments", i);
+    if (s.table != nullptr) {
+      const int esz = bz::dtype_size(s.table_dtype);
+      BZ_REQUIRE(s.pitch % 16 == 0 && s.pitch >= ((s.dim * esz + 15) / 16) * 16,
+                 "slot %d: row pitch %d must be a multiple of 16 covering dim*elem=%d", i, s.pitch, s.dim * esz);
+      BZ_REQUIRE(((uintptr_t)s.table & 15) == 0, "slot %d: table base not 16-byte aligned", i);
+      BZ_REQUIRE(s.table_dtype != BZ_I8 || s.row_scale != nullptr, "slot %d: int8 table without row_scale", i);
+      BZ_REQUIRE(s.rows > 0, "slot %d: rows=%lld", i, (long long)s.rows);
+      if (s.hash_buckets != nullptr)
+        BZ_REQUIRE(s.hash_pairs != nullptr && s.hash_bucket_size > 0, "slot %d: incomplete hash index", i);
+    }
+    const int g = groups_per_wg(s);
+    s.wg_begin = (int32_t)total;
+    s.wg_count = (int32_t)((s.batch + g - 1) / g);
+    total += s.wg_count;
+    BZ_REQUIRE(total < (1ll << 30), "too many workgroups");
+  }
+  *total_wg = (int)total;
+  return BZ_OK;
+}
+
+int bz_segments_to_offsets(const int32_t* segments, int64_t* offsets, int64_t n, bz_stream_t stream) {
+  BZ_REQUIRE(offsets != nullptr && n >= 0 && (n == 0 || segments != nullptr), "bz_segments_to_offsets: null argument");
+  BZ_REQUIRE(n <= (1ll << 24), "bz_segments_to_offsets: n=%lld exceeds 2^24", (long long)n);
+  hipLaunchKernelGGL(bz_scan_segments_kernel, dim3(1), dim3(kThreads), 0, bz::as_stream(stream), segments, offsets, n);
+  BZ_LAUNCH_OK("bz_scan_segments_kernel");
+  return BZ_OK;
+}
+
+int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_slots, bz_stream_t stream) {
+  BZ_REQUIRE(slots_dev != nullptr && n_slots > 0, "bz_segments_to_offsets_slots: null argument or n_slots=%d", n_slots);
+  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(n_slots), dim3(kThreads), 0, bz::as_stream(stream), slots_dev);
+  BZ_LAUNCH_OK("bz_scan_segments_slots_kernel");
+  return BZ_OK;
+}
+
+int bz_embed_pool(const bz_embed_slot* slots_dev, int n_slots, int total_wg, bz_stream_t stream) {
+  BZ_REQUIRE(slots_dev != nullptr && n_slots > 0 && total_wg >= 0, "bz_embed_pool: null argument, n_slots=%d total_wg=%d",
+             n_slots, total_wg);
+  if (total_wg == 0) return BZ_OK;
+  const int per_xcd = (total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
+  hipLaunchKernelGGL(bz_embed_pool_kernel, dim3(per_xcd * bz::kNumXcd), dim3(kThreads), 0, bz::as_stream(stream), slots_dev,
+                     n_slots, total_wg, per_xcd);
+  BZ_LAUNCH_OK("bz_embed_pool_kernel");
+  return BZ_OK;
+}
+
+const char* bz_embed_pool_kernel_name(void) { return "bz_embed_pool_kernel"; }
+
+}  // extern "C"

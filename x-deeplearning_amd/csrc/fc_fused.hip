@@ -1,0 +1,529 @@
+// fc_fused.hip -- FC layer = GEMM + bias + activation in one kernel, for gfx950 MFMA.
+//
+// Stands in for the reference's pair  Gemm op (blaze/operator/op/gemm_op.h:33-107:
+// Y <- broadcast(bias); Y = alpha*A*B + beta*Y via cblas/cuBLAS, blaze/math/gemm.cc:13-27,
+// gemm.cu:35-104)  +  the separate PRelu / Dice / LeakyRelu / Sigmoid / Softmax op that
+// follows it (prelu_op.cc:11-30, dice_op.cc:15-34, leaky_relu_op.cc:15-21,
+// sigmoid_op.cc:15-21, softmax_op.cc:21-78).  The result equals the composition
+// Activation(Gemm(x, W, b)) evaluated in fp32.
+//
+// Main kernel: C tile BM x BN per workgroup, K stepped by BK through double-buffered LDS
+// (global -> registers -> LDS, one barrier per step, next tile's global loads in flight
+// during the MFMAs).  Operands are both "K contiguous" (A row major, W packed [N,K]) so
+// a lane's MFMA fragment is one 16-byte LDS read; rows are padded by 16 bytes, which
+// spreads the 16 lanes of a ds_read_b128 phase over all 64 banks.  fp16/bf16 use
+// v_mfma_f32_32x32x16 (K=16 per instruction, fp32 accumulate); fp32 uses
+// v_mfma_f32_32x32x2 with a K permutation inside each 8-wide step so its fragments are
+// 16-byte reads as well.  In the accumulator a lane owns one output column and 16
+// rows, so per-column epilogue parameters (bias, PReLU slope, Dice gamma/mean/var) are
+// lane constants.
+//
+// Skinny kernel (N <= 8: the 256->2 softmax head, the 40->1 attention score, the 256->1
+// sigmoid head): bandwidth bound on A; a lane group of pow2(K/8) lanes owns a row, the
+// weight fragments live in registers, the N dot products are reduced by shuffles.
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "bz_common.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr float kDiceEps = 1e-8f;  // blaze/operator/common_helper.h:90
+
+struct Epilogue {
+  const float* bias;
+  const float* p0;
+  const float* p1;
+  const float* p2;
+  int bias_rows;
+  int act;
+  int act_size;
+  int dice_nosqrt;
+  float alpha, beta, act_alpha;
+};
+
+__device__ __forceinline__ float apply_act(float v, int n, const Epilogue& e) {
+  switch (e.act) {
+    case BZ_ACT_PRELU: {
+      const float w = e.p0[e.act_size == 1 ? 0 : n];
+      return v * ((float)(v > 0.f) + (float)(v < 0.f) * w);  // math/activation.h:37-42
+    }
+    case BZ_ACT_DICE: {
+      const float var = e.p2[n];
+      const float den = e.dice_nosqrt ? var : sqrtf(var + kDiceEps);
+      const float t = expf(-1.f * (v - e.p1[n]) / den);
+      const float p = 1.f / (1.f + t);
+      return (1.f - p) * e.p0[n] * v + p * v;
+    }
+    case BZ_ACT_LEAKY_RELU:
+      return v >= 0.f ? v : e.act_alpha * v;
+    case BZ_ACT_SIGMOID: {
+      const float t = expf(v);
+      return t / (1.f + t);
+    }
+    default:
+      return v;
+  }
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store_out(OutT* p, float v);
+template <>
+__device__ __forceinline__ void store_out<float>(float* p, float v) {
+  *p = v;
+}
+template <>
+__device__ __forceinline__ void store_out<__half>(__half* p, float v) {
+  *p = __float2half_rn(v);
+}
+template <>
+__device__ __forceinline__ void store_out<__hip_bfloat16>(__hip_bfloat16* p, float v) {
+  *p = __float2bfloat16(v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// element traits
+// ---------------------------------------------------------------------------------------------
+template <int DT>
+struct In;
+template <>
+struct In<BZ_F16> {
+  static constexpr int kSize = 2;
+  static constexpr int kChunk = 8;   // elements per 16 bytes
+  static constexpr int kStepK = 16;  // K consumed per fragment pair (both lane halves)
+  static __device__ __forceinline__ void mma(const uint4& a, const uint4& b, floatx16& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(*(const half8*)&a, *(const half8*)&b, acc, 0, 0, 0);
+  }
+};
+template <>
+struct In<BZ_BF16> {
+  static constexpr int kSize = 2;
+  static constexpr int kChunk = 8;
+  static constexpr int kStepK = 16;
+  static __device__ __forceinline__ void mma(const uint4& a, const uint4& b, floatx16& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)&a, *(const bf16x8*)&b, acc, 0, 0, 0);
+  }
+};
+template <>
+struct In<BZ_F32> {
+  static constexpr int kSize = 4;
+  static constexpr int kChunk = 4;
+  static constexpr int kStepK = 8;
+  // lane half h holds k = 4h..4h+3 of the 8-wide step; instruction i multiplies element i of both
+  // halves, i.e. k in {i, 4+i}: a permutation of k applied equally to A and W.
+  static __device__ __forceinline__ void mma(const uint4& a, const uint4& b, floatx16& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), acc, 0, 0, 0);
+  }
+};
+
+// one 16-byte chunk of a K-contiguous operand row; zero beyond K; element-wise when unaligned
+template <int DT>
+__device__ __forceinline__ uint4 load_chunk(const char* base, int64_t row, int64_t ld, int k, int K, bool vec_ok) {
+  constexpr int ES = In<DT>::kSize;
+  constexpr int CH = In<DT>::kChunk;
+  uint4 out = make_uint4(0, 0, 0, 0);
+  if (k >= K) return out;
+  const char* p = base + (row * ld + k) * ES;
+  if (vec_ok && k + CH <= K) return *(const uint4*)p;
+  if constexpr (ES == 2) {
+    unsigned short e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) e[i] = (k + i < K) ? *(const unsigned short*)(p + 2 * i) : (unsigned short)0;
+    out.x = e[0] | ((uint32_t)e[1] << 16);
+    out.y = e[2] | ((uint32_t)e[3] << 16);
+    out.z = e[4] | ((uint32_t)e[5] << 16);
+    out.w = e[6] | ((uint32_t)e[7] << 16);
+  } else {
+    uint32_t e[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = (k + i < K) ? *(const uint32_t*)(p + 4 * i) : 0u;
+    out = make_uint4(e[0], e[1], e[2], e[3]);
+  }
+  return out;
+}
+
+// ---------------------------------------------------------------------------------------------
+// tiled MFMA kernel
+// ---------------------------------------------------------------------------------------------
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __restrict__ A, const char* __restrict__ W,
+                                                                  OutT* __restrict__ Y, int M, int N, int K, int64_t lda,
+                                                                  int64_t ldw, int64_t ldy, bool vec_a, bool vec_w,
+                                                                  int tiles_m, Epilogue ep) {
+  using T = In<DT>;
+  constexpr int NT = WM * WN * 64;
+  constexpr int ES = T::kSize;
+  constexpr int ROWB = BK * ES;        // bytes of one tile row
+  constexpr int PITCH = ROWB + 16;     // padded LDS pitch
+  constexpr int CPR = ROWB / 16;       // 16-byte chunks per row
+  constexpr int A_CHUNKS = BM * CPR, W_CHUNKS = BN * CPR;
+  constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, W_PER = (W_CHUNKS + NT - 1) / NT;
+  constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
+  constexpr int TM = WTM / 32, TN = WTN / 32;  // 32x32 blocks per wave
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % T::kStepK == 0, "tile shape");
+
+  __shared__ __attribute__((aligned(16))) char lds[2][(BM + BN) * PITCH];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  // consecutive workgroups walk down M within one N panel: the W panel stays hot in L2
+  const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  uint4 ra[A_PER], rw[W_PER];
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int q = tid + i * NT;
+      if (A_CHUNKS % NT == 0 || q < A_CHUNKS) {
+        const int r = q / CPR, ch = q % CPR;
+        int m = m0 + r;
+        m = m < M ? m : M - 1;
+        ra[i] = load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int q = tid + i * NT;
+      if (W_CHUNKS % NT == 0 || q < W_CHUNKS) {
+        const int r = q / CPR, ch = q % CPR;
+        int n = n0 + r;
+        n = n < N ? n : N - 1;
+        rw[i] = load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w);
+      }
+    }
+  };
+  auto lstore = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int q = tid + i * NT;
+      if (A_CHUNKS % NT == 0 || q < A_CHUNKS) *(uint4*)&lds[buf][(q / CPR) * PITCH + (q % CPR) * 16] = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+      const int q = tid + i * NT;
+      if (W_CHUNKS % NT == 0 || q < W_CHUNKS) *(uint4*)&lds[buf][(BM + q / CPR) * PITCH + (q % CPR) * 16] = rw[i];
+    }
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int KT = (K + BK - 1) / BK;
+  gload(0);
+  lstore(0);
+  __syncthreads();
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) gload((kt + 1) * BK);
+    const char* la = &lds[buf][(wm * WTM + frag_row) * PITCH + frag_half * 16];
+    const char* lw = &lds[buf][(BM + wn * WTN + frag_row) * PITCH + frag_half * 16];
+#pragma unroll
+    for (int ks = 0; ks < BK / T::kStepK; ++ks) {
+      uint4 fa[TM], fw[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(la + i * 32 * PITCH + ks * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fw[j] = *(const uint4*)(lw + j * 32 * PITCH + ks * 32);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) T::mma(fa[i], fw[j], acc[i][j]);
+    }
+    if (kt + 1 < KT) lstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: lane owns column n, rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+    if (n >= N) continue;
+    const float bcol = (ep.bias_rows == 1) ? ep.beta * ep.bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < M) {
+          float v = ep.alpha * acc[i][j][r];
+          if (ep.bias_rows == 1)
+            v += bcol;
+          else if (ep.bias_rows > 1)
+            v += ep.beta * ep.bias[(int64_t)m * N + n];
+          store_out<OutT>(Y + (int64_t)m * ldy + n, apply_act(v, n, ep));
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// skinny kernel: N <= 8
+// ---------------------------------------------------------------------------------------------
+constexpr int kSkinnyMaxN = 8;
+
+template <int DT>
+__device__ __forceinline__ void chunk_to_float(const uint4& c, float (&f)[In<DT>::kChunk]) {
+  const uint32_t r[4] = {c.x, c.y, c.z, c.w};
+  if constexpr (DT == BZ_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r[i]);
+  } else if constexpr (DT == BZ_F16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xffffu)));
+      f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
+    }
+  } else {  // bf16: the upper 16 bits of the fp32 pattern
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(r[i] << 16);
+      f[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+}
+
+template <int DT, typename OutT>
+__global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restrict__ A, const char* __restrict__ W,
+                                                           OutT* __restrict__ Y, int M, int N, int K, int64_t lda,
+                                                           int64_t ldw, int64_t ldy, bool vec_a, bool vec_w, int lpr,
+                                                           Epilogue ep) {
+  constexpr int CH = In<DT>::kChunk;
+  const int tid = threadIdx.x;
+  const int g = tid / lpr, l = tid - g * lpr;
+  const int rows_per_wg = 256 / lpr;
+  const int nchunks = (K + CH - 1) / CH;
+  for (int64_t m = (int64_t)blockIdx.x * rows_per_wg + g; m < M; m += (int64_t)gridDim.x * rows_per_wg) {
+    float acc[kSkinnyMaxN];
+#pragma unroll
+    for (int n = 0; n < kSkinnyMaxN; ++n) acc[n] = 0.f;
+    for (int c = l; c < nchunks; c += lpr) {
+      float a[CH];
+      chunk_to_float<DT>(load_chunk<DT>(A, m, lda, c * CH, K, vec_a), a);
+#pragma unroll
+      for (int n = 0; n < kSkinnyMaxN; ++n) {
+        if (n < N) {
+          float w[CH];
+          chunk_to_float<DT>(load_chunk<DT>(W, n, ldw, c * CH, K, vec_w), w);
+#pragma unroll
+          for (int i = 0; i < CH; ++i) acc[n] = fmaf(a[i], w[i], acc[n]);
+        }
+      }
+    }
+    // reduce over the lane group (lpr is a power of two <= 64, groups are lane aligned)
+    for (int d = lpr >> 1; d > 0; d >>= 1) {
+#pragma unroll
+      for (int n = 0; n < kSkinnyMaxN; ++n) acc[n] += __shfl_xor(acc[n], d, 64);
+    }
+    if (l == 0) {
+      float v[kSkinnyMaxN];
+#pragma unroll
+      for (int n = 0; n < kSkinnyMaxN; ++n) {
+        v[n] = 0.f;
+        if (n < N) {
+          float x = ep.alpha * acc[n];
+          if (ep.bias_rows == 1)
+            x += ep.beta * ep.bias[n];
+          else if (ep.bias_rows > 1)
+            x += ep.beta * ep.bias[m * N + n];
+          v[n] = x;
+        }
+      }
+      if (ep.act == BZ_ACT_SOFTMAX) {  // softmax_op.cc:21-78: subtract max, exp, sum in order, divide
+        float mx = v[0];
+#pragma unroll
+        for (int n = 1; n < kSkinnyMaxN; ++n)
+          if (n < N) mx = v[n] > mx ? v[n] : mx;
+        float sum = 0.f;
+#pragma unroll
+        for (int n = 0; n < kSkinnyMaxN; ++n)
+          if (n < N) {
+            v[n] = expf(v[n] - mx);
+            sum += v[n];
+          }
+#pragma unroll
+        for (int n = 0; n < kSkinnyMaxN; ++n)
+          if (n < N) v[n] = v[n] / sum;
+      } else {
+#pragma unroll
+        for (int n = 0; n < kSkinnyMaxN; ++n)
+          if (n < N) v[n] = apply_act(v[n], n, ep);
+      }
+#pragma unroll
+      for (int n = 0; n < kSkinnyMaxN; ++n)
+        if (n < N) store_out<OutT>(Y + m * ldy + n, v[n]);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// weight packing
+// ---------------------------------------------------------------------------------------------
+template <typename SrcT, typename DstT>
+__global__ void bz_pack_weight_kernel(const SrcT* __restrict__ src, DstT* __restrict__ dst, int K, int N, int64_t ldw,
+                                      int trans_b) {
+  const int64_t total = (int64_t)N * ldw;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t n = i / ldw, k = i % ldw;
+    float v = 0.f;
+    if (k < K) v = (float)src[trans_b ? n * K + k : k * (int64_t)N + n];
+    dst[i] = (DstT)v;
+  }
+}
+
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN>
+int launch_mfma(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
+  const int tiles_m = (d.m + BM - 1) / BM, tiles_n = (d.n + BN - 1) / BN;
+  hipLaunchKernelGGL((bz_fc_mfma_kernel<DT, OutT, BM, BN, BK, WM, WN>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), 0, st,
+                     (const char*)d.a, (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, vec_a, vec_w,
+                     tiles_m, ep);
+  BZ_LAUNCH_OK("bz_fc_mfma_kernel");
+  return BZ_OK;
+}
+
+template <int DT, typename OutT>
+int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
+  constexpr int BK = In<DT>::kSize == 2 ? 64 : 32;
+  const int64_t wg128 = (int64_t)((d.m + 127) / 128) * ((d.n + 127) / 128);
+  const int64_t wg64 = (int64_t)((d.m + 63) / 64) * ((d.n + 63) / 64);
+  if (wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2>(d, ep, vec_a, vec_w, st);
+  if (wg64 >= 256) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2>(d, ep, vec_a, vec_w, st);
+  return launch_mfma<DT, OutT, 32, 64, BK, 1, 2>(d, ep, vec_a, vec_w, st);
+}
+
+template <int DT, typename OutT>
+int dispatch_skinny(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
+  const int nchunks = (d.k + In<DT>::kChunk - 1) / In<DT>::kChunk;
+  int lpr = 1;
+  while (lpr < nchunks && lpr < 64) lpr <<= 1;
+  const int rows_per_wg = 256 / lpr;
+  int64_t grid = ((int64_t)d.m + rows_per_wg - 1) / rows_per_wg;
+  if (grid > 256 * 32) grid = 256 * 32;
+  hipLaunchKernelGGL((bz_fc_skinny_kernel<DT, OutT>), dim3((int)grid), dim3(256), 0, st, (const char*)d.a,
+                     (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, vec_a, vec_w, lpr, ep);
+  BZ_LAUNCH_OK("bz_fc_skinny_kernel");
+  return BZ_OK;
+}
+
+template <int DT>
+int dispatch_out(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
+  const bool skinny = d.n <= kSkinnyMaxN;
+  switch (d.out_dtype) {
+    case BZ_F32:
+      return skinny ? dispatch_skinny<DT, float>(d, ep, vec_a, vec_w, st) : dispatch_tiles<DT, float>(d, ep, vec_a, vec_w, st);
+    case BZ_F16:
+      return skinny ? dispatch_skinny<DT, __half>(d, ep, vec_a, vec_w, st)
+                    : dispatch_tiles<DT, __half>(d, ep, vec_a, vec_w, st);
+    case BZ_BF16:
+      return skinny ? dispatch_skinny<DT, __hip_bfloat16>(d, ep, vec_a, vec_w, st)
+                    : dispatch_tiles<DT, __hip_bfloat16>(d, ep, vec_a, vec_w, st);
+    default:
+      return bz::fail(BZ_EINVAL, "bz_fc_fused: unsupported out dtype %d", d.out_dtype);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_fc_fused: null descriptor");
+  const bz_fc_desc& d = *desc;
+  BZ_REQUIRE(d.a && d.w && d.y, "bz_fc_fused: null a/w/y");
+  BZ_REQUIRE(d.m >= 0 && d.n > 0 && d.k > 0, "bz_fc_fused: bad shape m=%d n=%d k=%d", d.m, d.n, d.k);
+  BZ_REQUIRE(d.lda >= d.k && d.ldw >= d.k && d.ldy >= d.n, "bz_fc_fused: leading dimension smaller than row (lda=%lld ldw=%lld ldy=%lld)",
+             (long long)d.lda, (long long)d.ldw, (long long)d.ldy);
+  BZ_REQUIRE(d.in_dtype == BZ_F16 || d.in_dtype == BZ_BF16 || d.in_dtype == BZ_F32, "bz_fc_fused: unsupported in dtype %d",
+             d.in_dtype);
+  BZ_REQUIRE(d.bias_rows == 0 || d.bias != nullptr, "bz_fc_fused: bias_rows=%d without bias", d.bias_rows);
+  BZ_REQUIRE(d.bias_rows == 0 || d.bias_rows == 1 || d.bias_rows == d.m, "bz_fc_fused: bias_rows=%d must be 0, 1 or m=%d",
+             d.bias_rows, d.m);
+  switch (d.act) {
+    case BZ_ACT_NONE:
+    case BZ_ACT_LEAKY_RELU:
+    case BZ_ACT_SIGMOID:
+      break;
+    case BZ_ACT_PRELU:
+      BZ_REQUIRE(d.act_p0 && (d.act_size == 1 || d.act_size == d.n), "bz_fc_fused: PRelu slope size %d must be 1 or n=%d",
+                 d.act_size, d.n);
+      break;
+    case BZ_ACT_DICE:
+      BZ_REQUIRE(d.act_p0 && d.act_p1 && d.act_p2, "bz_fc_fused: Dice needs gamma, mean and var");
+      break;
+    case BZ_ACT_SOFTMAX:
+      if (d.n > kSkinnyMaxN) return bz::fail(BZ_ENOTSUP, "bz_fc_fused: fused softmax needs n <= %d (n=%d)", kSkinnyMaxN, d.n);
+      break;
+    default:
+      return bz::fail(BZ_EINVAL, "bz_fc_fused: unknown activation %d", d.act);
+  }
+  if (d.m == 0) return BZ_OK;
+  Epilogue ep;
+  ep.bias = (const float*)d.bias;
+  ep.p0 = d.act_p0;
+  ep.p1 = d.act_p1;
+  ep.p2 = d.act_p2;
+  ep.bias_rows = d.bias_rows;
+  ep.act = d.act;
+  ep.act_size = d.act_size;
+  ep.dice_nosqrt = d.dice_nosqrt;
+  ep.alpha = d.alpha;
+  ep.beta = d.beta;
+  ep.act_alpha = d.act_alpha;
+  const int es = bz::dtype_size(d.in_dtype);
+  const bool vec_a = ((uintptr_t)d.a % 16 == 0) && ((d.lda * es) % 16 == 0);
+  const bool vec_w = ((uintptr_t)d.w % 16 == 0) && ((d.ldw * es) % 16 == 0);
+  hipStream_t st = bz::as_stream(stream);
+  switch (d.in_dtype) {
+    case BZ_F16: return dispatch_out<BZ_F16>(d, ep, vec_a, vec_w, st);
+    case BZ_BF16: return dispatch_out<BZ_BF16>(d, ep, vec_a, vec_w, st);
+    default: return dispatch_out<BZ_F32>(d, ep, vec_a, vec_w, st);
+  }
+}
+
+int bz_fc_pack_weight(const void* src, int src_dtype, int trans_b, int k, int n, void* dst, int dst_dtype, int64_t ldw,
+                      bz_stream_t stream) {
+  BZ_REQUIRE(src && dst && k > 0 && n > 0, "bz_fc_pack_weight: null pointer or bad shape k=%d n=%d", k, n);
+  BZ_REQUIRE(ldw >= k && ldw % 8 == 0, "bz_fc_pack_weight: ldw=%lld must be >= k=%d and a multiple of 8", (long long)ldw, k);
+  const int64_t total = (int64_t)n * ldw;
+  const int grid = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+  hipStream_t st = bz::as_stream(stream);
+#define BZ_PACK(S, D)                                                                                        \
+  hipLaunchKernelGGL((bz_pack_weight_kernel<S, D>), dim3(grid), dim3(256), 0, st, (const S*)src, (D*)dst, k, n, ldw, \
+                     trans_b)
+  if (src_dtype == BZ_F32 && dst_dtype == BZ_F32)
+    BZ_PACK(float, float);
+  else if (src_dtype == BZ_F32 && dst_dtype == BZ_F16)
+    BZ_PACK(float, _Float16);
+  else if (src_dtype == BZ_F32 && dst_dtype == BZ_BF16)
+    BZ_PACK(float, __bf16);
+  else if (src_dtype == BZ_F16 && dst_dtype == BZ_F16)
+    BZ_PACK(_Float16, _Float16);
+  else if (src_dtype == BZ_F16 && dst_dtype == BZ_F32)
+    BZ_PACK(_Float16, float);
+  else if (src_dtype == BZ_BF16 && dst_dtype == BZ_BF16)
+    BZ_PACK(__bf16, __bf16);
+  else
+    return bz::fail(BZ_ENOTSUP, "bz_fc_pack_weight: no conversion %d -> %d", src_dtype, dst_dtype);
+#undef BZ_PACK
+  BZ_LAUNCH_OK("bz_pack_weight_kernel");
+  return BZ_OK;
+}
+
+}  // extern "C"
