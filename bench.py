@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Benchmark of the Blaze sparse CTR inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward pass (Embedding gather/pool -> FC 896-512-256-2 with PReLU -> softmax) over one
+synthetic batch of 2048 samples (config 2), inputs already resident in HBM.  A pool of pre-generated
+batches is cycled so the id stream is not one cached batch.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "x-deeplearning_amd"))
+sys.path.insert(1, os.path.join(ROOT, "oracle"))
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, vendor figure
+MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--pool", type=int, default=32, help="number of distinct pre-generated batches")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of replaying HIP graphs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (one process, no collectives); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import blaze_hip as bz
+    from pipeline import CtrForward
+    from synth import Config2
+
+    assert torch.cuda.is_available(), "no GPU visible"
+    arch = bz.device_check()
+    cfg = Config2()
+    tables = cfg.tables()
+    mlp = cfg.mlp()
+    sparse, dense = cfg.batches(args.pool)
+    fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16")
+    torch.cuda.synchronize()
+    K, W = args.steps, args.warmup
+
+    # one HIP graph per pooled batch: the five launches of a step replay as one submission
+    graphs = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fwd.step(0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graphs = []
+        for i in range(fwd.n_batches):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                fwd.step(i)
+            graphs.append(g)
+
+    def run_step(i):
+        if graphs is not None:
+            graphs[i % fwd.n_batches].replay()
+        else:
+            fwd.step(i)
+
+    # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations
+    for i in range(W):
+        run_step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        run_step(W + i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K
+    samples_per_s = cfg.batch * K / (t1 - t0)
+
+    # ---- latency: each step submitted and waited for on its own
+    lat = []
+    for i in range(min(K, 2000)):
+        a = time.perf_counter()
+        run_step(i)
+        torch.cuda.synchronize()
+        lat.append((time.perf_counter() - a) * 1e3)
+    lat = np.sort(np.array(lat))
+    p50, p99 = float(lat[len(lat) // 2]), float(lat[int(len(lat) * 0.99)])
+
+    # ---- per-kernel durations: HIP events on the launch stream around R back-to-back launches
+    def timed(fn, reps):
+        for i in range(20):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps  # us
+
+    R = max(200, min(K, 1000))
+    kern_us = {"bz_embed_pool_kernel": timed(fwd.pool, R)}
+    for li in range(len(fwd.weights)):
+        kern_us["bz_fc[%d]" % li] = timed(lambda i, li=li: fwd.fc(i, li), R)
+    emb_bytes = float(np.mean([fwd.embedding_bytes(i) for i in range(fwd.n_batches)]))
+    flops = fwd.fc_flops()
+    pool_us = kern_us["bz_embed_pool_kernel"]
+    pool_gbs = emb_bytes / pool_us / 1e3
+    fc_us = sum(kern_us["bz_fc[%d]" % li] for li in range(len(flops)))
+    fc_tflops = sum(flops) / fc_us / 1e6
+    dominant = max(kern_us, key=kern_us.get)
+    if dominant.startswith("bz_fc"):
+        li = int(dominant[6:-1])
+        ach = flops[li] / kern_us[dominant] / 1e6
+        roofline = {"kernel": "bz_fc_mfma_kernel layer %d" % li, "bound": "mfma", "achieved": round(ach, 2),
+                    "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK_TFLOPS, 5), "traffic": None}
+    else:
+        roofline = {"kernel": "bz_embed_pool_kernel", "bound": "hbm", "achieved": round(pool_gbs, 1), "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": round(pool_gbs / HBM_PEAK_GBS, 5), "traffic": None,
+                    "algorithmic_bytes_per_launch": int(emb_bytes), "avg_launch_us": round(pool_us, 2)}
+
+    # ---- CPU baseline: the oracle (a scalar port of the reference's CPU path), one predictor per thread
+    cpu = None
+    if not args.no_cpu_baseline:
+        import blaze_oracle as orc
+        from pipeline import oracle_forward
+        orc.build()
+        tabs = [orc.Table(t.cpu().numpy()) for t in tables]
+        mlp_np = [(w.cpu().numpy(), b.cpu().numpy(), s.cpu().numpy()) for (w, b, s) in mlp]
+        threads = max(1, min(16, len(os.sched_getaffinity(0))))
+        per_thread = 1
+        def worker(t):
+            for j in range(per_thread):
+                b = (t * per_thread + j) % len(sparse)
+                oracle_forward(orc, cfg, tabs, mlp_np, sparse[b], dense[b])
+        oracle_forward(orc, cfg, tabs, mlp_np, sparse[0], dense[0])  # warm the page cache of the tables
+        c0 = time.perf_counter()
+        ths = [threading.Thread(target=worker, args=(t, )) for t in range(threads)]
+        for t in ths:
+            t.start()
+        for t in ths:
+            t.join()
+        c1 = time.perf_counter()
+        cpu = {"value": round(cfg.batch * threads * per_thread / (c1 - c0), 1), "unit": "samples/s", "cores": threads,
+               "kind": "port",
+               "sample": "%d batches of %d (one per thread, one single-threaded predictor per core), fp32 oracle: "
+                         "hash-free row lookup, ksum, textbook sgemm + separate PReLU pass, softmax" % (
+                             threads * per_thread, cfg.batch)}
+
+    out = {
+        "metric": "samples/sec @batch 2048 fp16 (sparse CTR forward: embedding pool + FC stack)",
+        "value": round(samples_per_s, 1),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 5),
+        "p50_ms": round(p50, 4),
+        "p99_ms": round(p99, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic (seeded; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
+        "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
+                   "batch_pool": fwd.n_batches, "submission": "per-kernel launches" if graphs is None else "hip graph per step",
+                   "device": arch},
+        "roofline": roofline,
+        "embedding_pool": {"GB/s": round(pool_gbs, 1), "frac_of_hbm_peak": round(pool_gbs / HBM_PEAK_GBS, 5),
+                           "algorithmic_bytes": int(emb_bytes), "us": round(pool_us, 2)},
+        "fc_stack": {"TFLOP/s": round(fc_tflops, 2), "frac_of_mfma_peak": round(fc_tflops / MFMA_PEAK_TFLOPS, 5),
+                     "flops": int(sum(flops)), "us": round(fc_us, 2)},
+        "kernel_us": {k: round(v, 2) for k, v in kern_us.items()},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

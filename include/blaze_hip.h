@@ -89,7 +89,7 @@ typedef struct bz_embed_slot {
   const float* values;        /* device [nnz]   "<fg>.values"   */
   const int32_t* segments;    /* device [batch] "<fg>.segments": ids per sample (counts, not offsets) */
   int64_t* offsets;           /* device [batch+1] scratch: exclusive scan of segments (written by
-                                 bz_segments_to_offsets_slots, read by bz_embed_pool) */
+                                 bz_segments_to_offsets_slots, read by bz_embed_pool); NULL = fused scan */
   void* out;                  /* device: block base + this item's column offset */
   int64_t rows;
   int64_t out_stride;         /* elements between consecutive samples of the block */
@@ -108,11 +108,27 @@ typedef struct bz_embed_slot {
 } bz_embed_slot;
 
 /*
- * Host-side planning: validates the slots (host copy) and fills wg_begin/wg_count.
- * Returns the total number of workgroups in *total_wg.  The caller then copies the
- * array to the device.  No reference counterpart (launch geometry).
+ * Launch geometry of one Embedding invocation, produced on the host by bz_embed_plan
+ * and handed back to bz_embed_pool.  No reference counterpart.
  */
-BZ_API int bz_embed_plan(bz_embed_slot* slots_host, int n_slots, int* total_wg);
+typedef struct bz_embed_launch {
+  int32_t n_slots;
+  int32_t total_wg;     /* workgroups over all slots */
+  int32_t wg_per_slot;  /* > 0 when every slot takes the same number of workgroups, else 0 */
+  int32_t variant;      /* 0 = generic kernel; else (table_dtype << 8) | lanes_per_row: the specialised
+                           ksum/kavg kernel (all slots share dtype, row width class and are sum/avg) */
+  int32_t fused_scan;   /* 1: no slot carries offsets; the pooling kernel scans the segments itself */
+  int32_t reserved_;
+} bz_embed_launch;
+
+/*
+ * Host-side planning: validates the slots (host copy), fills wg_begin/wg_count and
+ * the launch record.  The caller then copies the slot array to the device.
+ * A slot with offsets == NULL asks for the fused scan (the pooling kernel derives
+ * each workgroup's offsets from the segments itself; sensible up to a few
+ * thousand samples); either all slots carry offsets or none does.
+ */
+BZ_API int bz_embed_plan(bz_embed_slot* slots_host, int n_slots, bz_embed_launch* launch);
 
 /*
  * segments -> offsets for one array: off[i] = sum(segments[0..i)), off[n] = nnz.
@@ -132,9 +148,10 @@ BZ_API int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_sl
  * K{Sum,Avg,Assign}Processors (udf_processor.h:43-133), including the per-item
  * zero fill (InitProcess).  fp32 accumulate, multiply then add (not fused), ids in
  * order: the fp32 output is bit-identical to the reference's loop.
- * slots_dev must already hold offsets (bz_segments_to_offsets_slots).
+ * Unless launch->fused_scan, slots_dev must already hold offsets
+ * (bz_segments_to_offsets_slots on the same stream).
  */
-BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, int n_slots, int total_wg, bz_stream_t stream);
+BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream);
 
 /* name of the pooling kernel as profilers report it (for tooling) */
 BZ_API const char* bz_embed_pool_kernel_name(void);

@@ -48,7 +48,7 @@ def test_segments_to_offsets_no_32bit_wrap(bz, oracle):
     assert np.array_equal(off.cpu().numpy(), oracle.segments_to_offsets(seg))
 
 
-def _run_gpu(bz, tables_np, specs, inputs, batch, out_np_dtype, strides_cols):
+def _run_gpu(bz, tables_np, specs, inputs, batch, out_np_dtype, strides_cols, fused_scan=True):
     """specs: list of (table index|None, udf, tdir, tnum, dim); one block, items packed at given cols."""
     import torch
     stride, cols = strides_cols
@@ -59,11 +59,11 @@ def _run_gpu(bz, tables_np, specs, inputs, batch, out_np_dtype, strides_cols):
     for (ti, udf, tdir, tnum, dim), col, (ids, vals, seg) in zip(specs, cols, inputs):
         items.append(dict(table=None if ti is None else dts[ti], ids=_dev(ids), values=_dev(vals), segments=_dev(seg),
                           out=out, col=col, udf=udf, trunc_dir=tdir, trunc_num=tnum, dim=dim))
-    plan = bz.EmbeddingPlan(items)
+    plan = bz.EmbeddingPlan(items, fused_scan=fused_scan)
     plan.run()
     torch.cuda.synchronize()
     offs = [o.cpu().numpy() for o in plan.offsets]
-    return out.cpu().numpy(), offs
+    return out.cpu().numpy(), offs, plan.launch.variant
 
 
 def _run_oracle(oracle, tables_np, specs, inputs, batch, strides_cols):
@@ -144,8 +144,10 @@ def _make_table(rng, kind, rows, dim, with_keys):
 @pytest.mark.parametrize("kind", ["f32", "f16", "i8"])
 @pytest.mark.parametrize("out_dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("with_keys", [False, True])
-def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys):
-    """Ragged segments (incl. empty), absent ids, random values, odd dims and unaligned columns."""
+@pytest.mark.parametrize("fused_scan", [True, False])
+def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys, fused_scan):
+    """Ragged segments (incl. empty), absent ids, random values, odd dims and unaligned columns; slots of mixed
+    shape and pooling kind go through the generic kernel, with the fused and with the separate scan."""
     seed = sum(map(ord, kind)) * 7 + (13 if out_dtype == np.float16 else 0) + (101 if with_keys else 0)
     rng = np.random.default_rng(seed)
     batch = 333
@@ -171,8 +173,10 @@ def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys):
         col += dim * tnum if udf == 2 else dim
     stride = col + 3
     print("case kind=%s out=%s keys=%s seed=%d" % (kind, out_dtype.__name__, with_keys, seed), flush=True)
-    got, offs = _run_gpu(bz, tables, specs, inputs, batch, out_dtype, (stride, cols))
+    got, offs, variant = _run_gpu(bz, tables, specs, inputs, batch, out_dtype, (stride, cols), fused_scan)
+    assert variant == 0
     want = _run_oracle(oracle, tables, specs, inputs, batch, (stride, cols))
+    assert len(offs) == (0 if fused_scan else len(inputs))
     for off, (_, _, seg) in zip(offs, inputs):
         assert np.array_equal(off, oracle.segments_to_offsets(seg))
     written = ~np.isnan(want)
@@ -185,6 +189,47 @@ def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys):
         assert np.array_equal(_bits(got)[written], _bits(want16)[written])
 
 
+SPECIALISED = [("f32", 4, 1), ("f32", 16, 4), ("f32", 30, 8), ("f32", 64, 16), ("f32", 128, 32), ("f32", 250, 64),
+               ("f16", 8, 1), ("f16", 16, 2), ("f16", 18, 4), ("f16", 32, 4), ("f16", 64, 8), ("f16", 100, 16),
+               ("f16", 200, 32), ("f16", 512, 64), ("i8", 16, 1), ("i8", 64, 4), ("i8", 100, 8), ("i8", 1000, 64)]
+
+
+@pytest.mark.parametrize("kind,dim,lpr", SPECIALISED)
+@pytest.mark.parametrize("with_keys", [False, True])
+def test_pooling_specialised_kernels_bit_exact(bz, oracle, kind, dim, lpr, with_keys):
+    """Slots of one shape, ksum/kavg only: every (table dtype, lanes-per-row) instance of the specialised kernel,
+    segments longer than one 16-id step, empty segments, absent ids, fp32 and fp16 outputs."""
+    rng = np.random.default_rng(dim * 31 + lpr + (7 if with_keys else 0))
+    batch = 300
+    for out_dtype in (np.float32, np.float16):
+        tables, specs, inputs, cols = [], [], [], []
+        col = 0
+        for i in range(3):
+            rows = int(rng.integers(20, 300))
+            tables.append(_make_table(rng, kind, rows, dim, with_keys))
+            seg = rng.integers(0, 40, batch).astype(np.int32)
+            seg[rng.integers(0, batch, 30)] = 0
+            nnz = int(seg.sum())
+            if with_keys:
+                pool = np.concatenate([tables[-1]["keys"], rng.integers(-2**62, 2**62, size=rows // 4 + 1, dtype=np.int64)])
+                ids = rng.choice(pool, nnz)
+            else:
+                ids = rng.integers(-3, rows + 3, nnz)
+            specs.append((i, i % 2, 0, 0, dim))
+            inputs.append((ids.astype(np.int64), rng.standard_normal(nnz).astype(np.float32), seg))
+            cols.append(col)
+            col += dim
+        print("case kind=%s dim=%d lpr=%d keys=%s out=%s" % (kind, dim, lpr, with_keys, out_dtype.__name__), flush=True)
+        for fused in (True, False):
+            got, offs, variant = _run_gpu(bz, tables, specs, inputs, batch, out_dtype, (col, cols), fused)
+            code = {"f32": bz.F32, "f16": bz.F16, "i8": bz.I8}[kind]
+            assert variant == (code << 8 | lpr), "expected the specialised kernel, got variant %#x" % variant
+            want = _run_oracle(oracle, tables, specs, inputs, batch, (col, cols))
+            if out_dtype == np.float16:
+                want = want.astype(np.float16)
+            assert np.array_equal(_bits(got), _bits(want))
+
+
 def test_unknown_table_and_empty_batch(bz, oracle):
     rng = np.random.default_rng(9)
     batch = 70
@@ -194,7 +239,7 @@ def test_unknown_table_and_empty_batch(bz, oracle):
     ins = (rng.integers(0, 10, nnz).astype(np.int64), np.ones(nnz, np.float32), seg)
     specs = [(None, 0, 0, 0, 8), (0, 0, 0, 0, 8), (None, 2, 0, 3, 8)]
     cols = [0, 8, 16]
-    got, _ = _run_gpu(bz, [t], specs, [ins] * 3, batch, np.float32, (40, cols))
+    got, _, _ = _run_gpu(bz, [t], specs, [ins] * 3, batch, np.float32, (40, cols))
     want = _run_oracle(oracle, [t], specs, [ins] * 3, batch, (40, cols))
     assert np.array_equal(_bits(got), _bits(want))
 
@@ -231,6 +276,7 @@ def test_config2_full_size(bz, oracle):
         items.append(dict(table=bz.DeviceTable(data), ids=_dev(ids), values=_dev(vals), segments=_dev(seg), out=out,
                           col=64 + s * dim, udf=0))
     plan = bz.EmbeddingPlan(items)
+    assert plan.launch.variant == (bz.F16 << 8 | 4) and plan.launch.fused_scan == 1
     plan.run()
     torch.cuda.synchronize()
     got = out.cpu().numpy()
@@ -242,4 +288,10 @@ def test_config2_full_size(bz, oracle):
         want = np.zeros((batch, dim), np.float32)
         oracle.embed_get(oracle.Table(sub), inv, vals, seg, [(0, 0, 0, want, 0)])
         assert np.array_equal(_bits(got[:, 64 + s * dim:64 + (s + 1) * dim]), _bits(want.astype(np.float16)))
-        assert np.array_equal(plan.offsets[s].cpu().numpy(), oracle.segments_to_offsets(seg))
+    plan2 = bz.EmbeddingPlan(items, fused_scan=False)  # separate scan launch: offsets are observable and bit-exact
+    out.zero_()
+    plan2.run()
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), got)
+    for s in range(slots):
+        assert np.array_equal(plan2.offsets[s].cpu().numpy(), oracle.segments_to_offsets(inputs[s][2]))

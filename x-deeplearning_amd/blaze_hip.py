@@ -34,6 +34,11 @@ class EmbedSlot(C.Structure):
                 ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("reserved_", C.c_int32)]
 
 
+class EmbedLaunch(C.Structure):
+    _fields_ = [("n_slots", C.c_int32), ("total_wg", C.c_int32), ("wg_per_slot", C.c_int32), ("variant", C.c_int32),
+                ("fused_scan", C.c_int32), ("reserved_", C.c_int32)]
+
+
 class FcDesc(C.Structure):
     _fields_ = [("a", C.c_void_p), ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("act_p0", C.c_void_p),
                 ("act_p1", C.c_void_p), ("act_p2", C.c_void_p), ("lda", C.c_int64), ("ldw", C.c_int64),
@@ -77,10 +82,10 @@ def lib():
             raise BlazeHipError("%s does not export %s (stale build?)" % (LIB_PATH, ", ".join(missing)))
         l.bz_last_error.restype = C.c_char_p
         l.bz_device_check.argtypes = [C.c_char_p, C.c_size_t]
-        l.bz_embed_plan.argtypes = [C.POINTER(EmbedSlot), C.c_int, C.POINTER(C.c_int)]
+        l.bz_embed_plan.argtypes = [C.POINTER(EmbedSlot), C.c_int, C.POINTER(EmbedLaunch)]
         l.bz_segments_to_offsets.argtypes = [vp, vp, i64, vp]
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
-        l.bz_embed_pool.argtypes = [vp, C.c_int, C.c_int, vp]
+        l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
@@ -188,9 +193,12 @@ class EmbeddingPlan:
     [B, stride]), col (element offset inside the block), udf, trunc_dir, trunc_num, dim}.
     """
 
-    def __init__(self, items):
+    def __init__(self, items, fused_scan=True):
+        """fused_scan: the pooling kernel derives offsets from the segments itself (one launch); otherwise
+        run() first scans every slot's segments into an offsets buffer (two launches)."""
         import torch
         self.items = items
+        self.fused_scan = fused_scan
         n = len(items)
         arr = (EmbedSlot * n)()
         self.offsets = []
@@ -200,8 +208,10 @@ class EmbeddingPlan:
             assert seg.dtype == torch.int32 and it["ids"].dtype == torch.int64 and it["values"].dtype == torch.float32
             assert out.dim() == 2 and out.stride(1) == 1
             batch = seg.numel()
-            off = torch.empty(batch + 1, dtype=torch.int64, device=out.device)
-            self.offsets.append(off)
+            off = None
+            if not fused_scan:
+                off = torch.empty(batch + 1, dtype=torch.int64, device=out.device)
+                self.offsets.append(off)
             s = arr[i]
             if t is not None:
                 s.table = t.data.data_ptr()
@@ -218,7 +228,7 @@ class EmbeddingPlan:
             s.ids = it["ids"].data_ptr()
             s.values = it["values"].data_ptr()
             s.segments = seg.data_ptr()
-            s.offsets = off.data_ptr()
+            s.offsets = off.data_ptr() if off is not None else None
             s.out = out.data_ptr() + it.get("col", 0) * out.element_size()
             s.out_stride = out.stride(0)
             s.out_dtype = bz_dtype(out.dtype)
@@ -226,9 +236,9 @@ class EmbeddingPlan:
             s.trunc_dir = it.get("trunc_dir", REVERSE)
             s.trunc_num = it.get("trunc_num", 0)
             s.batch = batch
-        total = C.c_int(0)
-        check(lib().bz_embed_plan(arr, n, C.byref(total)))
-        self.n, self.total_wg = n, total.value
+        self.launch = EmbedLaunch()
+        check(lib().bz_embed_plan(arr, n, C.byref(self.launch)))
+        self.n, self.total_wg = n, self.launch.total_wg
         self.host = arr
         raw = np.frombuffer(bytes(arr), dtype=np.uint8).copy()
         self.slots_dev = torch.from_numpy(raw).to(items[0]["out"].device)
@@ -237,10 +247,11 @@ class EmbeddingPlan:
         check(lib().bz_segments_to_offsets_slots(self.slots_dev.data_ptr(), self.n, _stream_ptr(stream)))
 
     def pool(self, stream=None):
-        check(lib().bz_embed_pool(self.slots_dev.data_ptr(), self.n, self.total_wg, _stream_ptr(stream)))
+        check(lib().bz_embed_pool(self.slots_dev.data_ptr(), C.byref(self.launch), _stream_ptr(stream)))
 
     def run(self, stream=None):
-        self.scan(stream)
+        if not self.fused_scan:
+            self.scan(stream)
         self.pool(stream)
 
 

@@ -10,13 +10,23 @@
 // (one 128-bit load); a *lane group* of `lpr` = pow2(chunks per row) lanes owns one
 // (sample, slot) segment and walks its ids in order, so every output element is
 // summed in exactly the reference's order (bit-identical fp32).  A 256-thread
-// workgroup holds 256/lpr segments of consecutive samples of one slot; their
-// offsets are staged through LDS with one coalesced read.  The id loop is
-// unrolled by kUnroll with all row loads issued before the first add, which is
-// where the memory-level parallelism comes from.  One launch covers every slot
-// of the operator; the linear workgroup id is remapped so that each of the 8 XCDs
-// (each with its own L2) serves a contiguous range of slots and therefore caches
-// the hot rows of only those tables.
+// workgroup holds 256/lpr segments of consecutive samples of one slot.  One launch
+// covers every slot of the operator; the linear workgroup id is remapped so that
+// each of the 8 XCDs (each with its own L2) serves a contiguous range of slots and
+// therefore caches the hot rows of only those tables.
+//
+// The kernel is latency bound before it is bandwidth bound (a batch-2048 launch moves
+// ~36 MB), so the dependent chain is kept at: slot record -> segments -> ids -> rows.
+//   * segments -> offsets is fused: a workgroup sums the counts before its first
+//     sample and scans its own 256/lpr counts in LDS (no separate scan launch, no
+//     offsets round trip);
+//   * with equal work per slot the slot index is a division, not a search;
+//   * the specialised ksum/kavg kernel walks a segment 16 ids at a time: the lanes of
+//     a group load disjoint ids/values (one coalesced read), resolve them to rows,
+//     pass rows and values around with ds_bpermute, then issue up to 16 row loads
+//     before the first add -- that is where the memory-level parallelism comes from.
+// A generic kernel covers kassign, mixed slot shapes, rows wider than 64 chunks and
+// precomputed offsets.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
@@ -289,11 +299,142 @@ __device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// offsets of one workgroup's samples, derived from the segment counts
+// ---------------------------------------------------------------------------------------------
+// s_off[0..groups] <- exclusive offsets of samples b0 .. b0+groups (clipped to batch).
+// All 256 threads call it; ends with a barrier.
+__device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0, int groups, int64_t* s_off,
+                                              int64_t* s_part) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (bz::kWave - 1), wave = tid / bz::kWave;
+  if (s.offsets != nullptr) {
+    for (int t = tid; t <= groups; t += kThreads)
+      if (b0 + t <= s.batch) s_off[t] = s.offsets[b0 + t];
+    __syncthreads();
+    return;
+  }
+  // base = sum of the counts before b0 (independent coalesced reads), local = this thread's sample
+  int64_t part = 0;
+  for (int64_t i = tid; i < b0; i += kThreads) part += s.segments[i];
+  const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)s.segments[b0 + tid] : 0;
+  int64_t base = part;
+#pragma unroll
+  for (int d = bz::kWave / 2; d > 0; d >>= 1) base += __shfl_xor(base, d, bz::kWave);
+  const int64_t incl = wave_incl_scan(mine, lane);
+  if (lane == bz::kWave - 1) {
+    s_part[wave] = base;
+    s_part[kThreads / bz::kWave + wave] = incl;
+  }
+  __syncthreads();
+  int64_t before = 0;
+#pragma unroll
+  for (int w = 0; w < kThreads / bz::kWave; ++w) {
+    before += s_part[w];
+    if (w < wave) before += s_part[kThreads / bz::kWave + w];
+  }
+  if (tid < groups) s_off[tid + 1] = before + incl;
+  if (tid == 0) s_off[0] = before;
+  __syncthreads();
+}
+
+// ---------------------------------------------------------------------------------------------
+// specialised ksum / kavg kernel: every slot has table dtype DT and LPR lanes per row
+// ---------------------------------------------------------------------------------------------
+constexpr int kBlockIds = 16;  // ids walked per step
+
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
+                                                                 int total_wg, int wg_per_xcd, int wg_per_slot) {
+  constexpr int CE = RowTraits<DT>::kElems;
+  constexpr int GROUPS = kThreads / LPR;
+  constexpr int SRC = LPR < kBlockIds ? LPR : kBlockIds;  // lanes of a group that fetch ids
+  constexpr int KPL = kBlockIds / SRC;                    // ids fetched per such lane
+  __shared__ int64_t s_off[GROUPS + 1];
+  __shared__ int64_t s_part[2 * kThreads / bz::kWave];
+  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
+  if (v >= total_wg) return;
+  const int si = v / wg_per_slot;
+  const bz_embed_slot s = slots[si];
+  const int tid = threadIdx.x;
+  const int g = tid / LPR, l = tid % LPR;
+  const int64_t b0 = (int64_t)(v - si * wg_per_slot) * GROUPS;
+  stage_offsets(s, b0, GROUPS, s_off, s_part);
+  const int64_t b = b0 + g;
+  if (b >= s.batch) return;
+  const int nchunks = (s.dim + CE - 1) / CE;
+  const bool has_chunk = l < nchunks;
+  const int64_t start = s_off[g], end = s_off[g + 1];
+  const int gbase = (tid & (bz::kWave - 1)) - l;  // first lane of this group within the wave
+  const char* table = (const char*)s.table + (int64_t)l * 16;
+  float acc[CE];
+#pragma unroll
+  for (int i = 0; i < CE; ++i) acc[i] = 0.f;
+  for (int64_t j = start; j < end; j += kBlockIds) {
+    const int cnt = (int)((end - j) < kBlockIds ? (end - j) : kBlockIds);
+    // each fetching lane takes ids j + k*SRC + l: one coalesced read per k for the whole group
+    int row_own[KPL];
+    float val_own[KPL];
+#pragma unroll
+    for (int k = 0; k < KPL; ++k) {
+      const int idx = k * SRC + l;
+      row_own[k] = -1;
+      val_own[k] = 0.f;
+      if (l < SRC && idx < cnt) {
+        row_own[k] = (int)resolve_row(s, s.ids[j + idx]);
+        val_own[k] = s.values[j + idx];
+      }
+    }
+    int row[kBlockIds];
+    float val[kBlockIds];
+    uint4 raw[kBlockIds];
+    float sc[kBlockIds];
+#pragma unroll
+    for (int u = 0; u < kBlockIds; ++u) {
+      row[u] = __shfl(row_own[u / SRC], gbase + (u % SRC), bz::kWave);
+      val[u] = __shfl(val_own[u / SRC], gbase + (u % SRC), bz::kWave);
+    }
+#pragma unroll
+    for (int u = 0; u < kBlockIds; ++u) {
+      raw[u] = make_uint4(0, 0, 0, 0);
+      sc[u] = 1.f;
+      if (has_chunk && row[u] >= 0) {  // row[u] is -1 beyond cnt
+        raw[u] = *(const uint4*)(table + (int64_t)row[u] * s.pitch);
+        if (DT == BZ_I8) sc[u] = s.row_scale[row[u]];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBlockIds; ++u) {
+      if (row[u] >= 0) {
+        float w[CE];
+        widen<DT>(raw[u], sc[u], w);
+        // out = out + value * w: two roundings, never an FMA (udf_processor.h:66)
+#pragma unroll
+        for (int i = 0; i < CE; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(val[u], w[i]));
+      }
+    }
+  }
+  if (s.udf == BZ_AVG) {
+    const int64_t num = end - start;
+    if (num != 0) {
+      const float inv = (float)(1.0 / (double)num);  // ValueType(1.0 / size), udf_processor.h:88
+#pragma unroll
+      for (int i = 0; i < CE; ++i) acc[i] = __fmul_rn(acc[i], inv);
+    }
+  }
+  if (has_chunk) {
+    const int e0 = l * CE;
+    const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
+    store_elems<CE>(s.out, b * s.out_stride + e0, acc, nvalid, s.out_dtype);
+  }
+}
+
 __device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (dt == BZ_F16 ? 8 : 16); }
 
-__global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
-                                                                 int total_wg, int wg_per_xcd) {
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const bz_embed_slot* __restrict__ slots,
+                                                                         int n_slots, int total_wg, int wg_per_xcd) {
   __shared__ int64_t s_off[kThreads + 1];
+  __shared__ int64_t s_part[2 * kThreads / bz::kWave];
   // XCD-aware order: hardware deals consecutive workgroup ids round robin over the 8 XCDs; give
   // each XCD a contiguous range of the logical workgroup space (= a contiguous range of slots).
   const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
@@ -317,10 +458,7 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
   const int g = tid / lpr;
   const int l = tid - g * lpr;
   const int64_t b0 = (int64_t)(v - s.wg_begin) * groups;
-  // stage this workgroup's offsets through LDS (one coalesced read instead of 2 per lane)
-  for (int t = tid; t <= groups; t += kThreads)
-    if (b0 + t <= s.batch) s_off[t] = s.offsets[b0 + t];
-  __syncthreads();
+  stage_offsets(s, b0, groups, s_off, s_part);
   const int64_t b = b0 + g;
   if (b >= s.batch) return;
   if (s.table == nullptr) {
@@ -357,9 +495,11 @@ int groups_per_wg(const bz_embed_slot& s) {
 
 extern "C" {
 
-int bz_embed_plan(bz_embed_slot* slots, int n_slots, int* total_wg) {
-  BZ_REQUIRE(slots != nullptr && total_wg != nullptr && n_slots > 0, "bz_embed_plan: null argument or n_slots=%d", n_slots);
+int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
+  BZ_REQUIRE(slots != nullptr && launch != nullptr && n_slots > 0, "bz_embed_plan: null argument or n_slots=%d", n_slots);
   int64_t total = 0;
+  bool uniform_wg = true, uniform_shape = true, any_offsets = false, all_offsets = true;
+  int lpr0 = 0;
   for (int i = 0; i < n_slots; ++i) {
     bz_embed_slot& s = slots[i];
     BZ_REQUIRE(s.table_dtype == BZ_F32 || s.table_dtype == BZ_F16 || s.table_dtype == BZ_I8,
@@ -371,25 +511,39 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, int* total_wg) {
       BZ_REQUIRE(s.trunc_num > 0 && (s.trunc_dir == BZ_ORDER || s.trunc_dir == BZ_REVERSE),
                  "slot %d: kAssign needs trunc_num > 0 and a trunc direction (trunc_num=%d dir=%d)", i, s.trunc_num,
                  s.trunc_dir);
-    BZ_REQUIRE(s.out != nullptr && s.offsets != nullptr && (s.batch == 0 || s.segments != nullptr),
-               "slot %d: null out/offsets/segments", i);
+    BZ_REQUIRE(s.out != nullptr && (s.batch == 0 || s.segments != nullptr), "slot %d: null out/segments", i);
     if (s.table != nullptr) {
       const int esz = bz::dtype_size(s.table_dtype);
       BZ_REQUIRE(s.pitch % 16 == 0 && s.pitch >= ((s.dim * esz + 15) / 16) * 16,
                  "slot %d: row pitch %d must be a multiple of 16 covering dim*elem=%d", i, s.pitch, s.dim * esz);
       BZ_REQUIRE(((uintptr_t)s.table & 15) == 0, "slot %d: table base not 16-byte aligned", i);
       BZ_REQUIRE(s.table_dtype != BZ_I8 || s.row_scale != nullptr, "slot %d: int8 table without row_scale", i);
-      BZ_REQUIRE(s.rows > 0, "slot %d: rows=%lld", i, (long long)s.rows);
+      BZ_REQUIRE(s.rows > 0 && s.rows < (1ll << 31), "slot %d: rows=%lld outside (0, 2^31)", i, (long long)s.rows);
+      BZ_REQUIRE(s.ids != nullptr && s.values != nullptr, "slot %d: null ids/values", i);
       if (s.hash_buckets != nullptr)
         BZ_REQUIRE(s.hash_pairs != nullptr && s.hash_bucket_size > 0, "slot %d: incomplete hash index", i);
     }
+    any_offsets |= s.offsets != nullptr;
+    all_offsets &= s.offsets != nullptr;
     const int g = groups_per_wg(s);
+    const int lpr = kThreads / g;
+    const int ce = s.table_dtype == BZ_F32 ? 4 : (s.table_dtype == BZ_F16 ? 8 : 16);
     s.wg_begin = (int32_t)total;
     s.wg_count = (int32_t)((s.batch + g - 1) / g);
     total += s.wg_count;
     BZ_REQUIRE(total < (1ll << 30), "too many workgroups");
+    if (i == 0) lpr0 = lpr;
+    uniform_wg &= s.wg_count == slots[0].wg_count;
+    uniform_shape &= s.table != nullptr && s.udf != BZ_ASSIGN && lpr == lpr0 && s.table_dtype == slots[0].table_dtype &&
+                     (s.dim + ce - 1) / ce <= lpr;
   }
-  *total_wg = (int)total;
+  BZ_REQUIRE(all_offsets || !any_offsets, "either every slot carries offsets or none does");
+  launch->n_slots = n_slots;
+  launch->total_wg = (int32_t)total;
+  launch->wg_per_slot = (uniform_wg && slots[0].wg_count > 0) ? slots[0].wg_count : 0;
+  launch->variant = (uniform_shape && launch->wg_per_slot > 0) ? ((slots[0].table_dtype << 8) | lpr0) : 0;
+  launch->fused_scan = any_offsets ? 0 : 1;
+  launch->reserved_ = 0;
   return BZ_OK;
 }
 
@@ -408,13 +562,45 @@ int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_slots, bz
   return BZ_OK;
 }
 
-int bz_embed_pool(const bz_embed_slot* slots_dev, int n_slots, int total_wg, bz_stream_t stream) {
-  BZ_REQUIRE(slots_dev != nullptr && n_slots > 0 && total_wg >= 0, "bz_embed_pool: null argument, n_slots=%d total_wg=%d",
-             n_slots, total_wg);
-  if (total_wg == 0) return BZ_OK;
-  const int per_xcd = (total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
-  hipLaunchKernelGGL(bz_embed_pool_kernel, dim3(per_xcd * bz::kNumXcd), dim3(kThreads), 0, bz::as_stream(stream), slots_dev,
-                     n_slots, total_wg, per_xcd);
+int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
+  BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool: null argument");
+  const bz_embed_launch& L = *launch;
+  BZ_REQUIRE(L.n_slots > 0 && L.total_wg >= 0 && L.wg_per_slot >= 0, "bz_embed_pool: bad launch record (n_slots=%d total_wg=%d)",
+             L.n_slots, L.total_wg);
+  if (L.total_wg == 0) return BZ_OK;
+  const int per_xcd = (L.total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
+  const dim3 grid(per_xcd * bz::kNumXcd), block(kThreads);
+  hipStream_t st = bz::as_stream(stream);
+  if (L.variant == 0) {
+    hipLaunchKernelGGL(bz_embed_pool_generic_kernel, grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd);
+    BZ_LAUNCH_OK("bz_embed_pool_generic_kernel");
+    return BZ_OK;
+  }
+  BZ_REQUIRE(L.wg_per_slot > 0 && (int64_t)L.wg_per_slot * L.n_slots == L.total_wg,
+             "bz_embed_pool: variant %#x needs equal work per slot", L.variant);
+  const int dt = L.variant >> 8, lpr = L.variant & 0xff;
+#define BZ_POOL(DT, LPR)                                                                                             \
+  hipLaunchKernelGGL((bz_embed_pool_kernel<DT, LPR>), grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd, \
+                     L.wg_per_slot)
+#define BZ_POOL_LPR(DT)                                                                      \
+  switch (lpr) {                                                                             \
+    case 1: BZ_POOL(DT, 1); break;                                                           \
+    case 2: BZ_POOL(DT, 2); break;                                                           \
+    case 4: BZ_POOL(DT, 4); break;                                                           \
+    case 8: BZ_POOL(DT, 8); break;                                                           \
+    case 16: BZ_POOL(DT, 16); break;                                                         \
+    case 32: BZ_POOL(DT, 32); break;                                                         \
+    case 64: BZ_POOL(DT, 64); break;                                                         \
+    default: return bz::fail(BZ_EINVAL, "bz_embed_pool: bad lanes-per-row %d in variant", lpr); \
+  }
+  switch (dt) {
+    case BZ_F32: BZ_POOL_LPR(BZ_F32); break;
+    case BZ_F16: BZ_POOL_LPR(BZ_F16); break;
+    case BZ_I8: BZ_POOL_LPR(BZ_I8); break;
+    default: return bz::fail(BZ_EINVAL, "bz_embed_pool: bad table dtype %d in variant", dt);
+  }
+#undef BZ_POOL_LPR
+#undef BZ_POOL
   BZ_LAUNCH_OK("bz_embed_pool_kernel");
   return BZ_OK;
 }

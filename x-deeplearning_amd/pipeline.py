@@ -1,0 +1,131 @@
+"""The CTR forward pass (Embedding -> FC stack -> softmax head) as prebuilt C-ABI calls.
+
+Harness for bench.py / smoke: every descriptor is built once, a step is four calls into
+libblaze_hip.so (pool with fused scan, FC, FC, FC+softmax) on the current stream.  The sequence mirrors what
+the reference's SimpleNet would run for this model: Embedding, Concat with the dense features (here
+the Embedding op writes its block straight into the FC input buffer at the dense features' column
+offset), then Gemm + PRelu per layer and Softmax (blaze/graph/simple_net.cc:35-46).
+"""
+import ctypes as C
+
+import numpy as np
+
+import blaze_hip as bz
+
+
+class CtrForward:
+    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True):
+        import torch
+        self.cfg = cfg
+        self.fused_scan = fused_scan
+        self.lib = bz.lib()
+        tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
+        bdt = {"f16": bz.F16, "bf16": bz.BF16, "f32": bz.F32}[dtype]
+        self.tables = [bz.DeviceTable(t) for t in tables]
+        self.weights = []
+        for (w, b, slope) in mlp:
+            self.weights.append((bz.pack_weight(w, False, bdt), b.float().contiguous(), slope.float().contiguous(),
+                                 w.shape[0]))
+        self.n_batches = len(sparse_batches)
+        self.steps = []
+        self.nnz = []
+        B = cfg.batch
+        for sp, dn in zip(sparse_batches, dense_batches):
+            x = torch.zeros((B, cfg.in_dim), dtype=tdt, device="cuda")
+            x[:, :cfg.dense] = torch.from_numpy(dn).cuda().to(tdt)  # the dense "Feed"
+            items = []
+            nnz = 0
+            keep = []
+            for s, (ids, vals, seg) in enumerate(sp):
+                d_ids, d_vals, d_seg = (torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(),
+                                        torch.from_numpy(seg).cuda())
+                keep.append((d_ids, d_vals, d_seg))
+                nnz += ids.size
+                items.append(dict(table=self.tables[s], ids=d_ids, values=d_vals, segments=d_seg, out=x,
+                                  col=cfg.dense + s * cfg.dim, udf=bz.SUM))
+            plan = bz.EmbeddingPlan(items, fused_scan=fused_scan)
+            acts = [x]
+            descs = []
+            nl = len(self.weights)
+            for li, (wp, b, slope, k) in enumerate(self.weights):
+                last = li == nl - 1
+                y = torch.empty((B, wp.shape[0]), dtype=torch.float32 if last else tdt, device="cuda")
+                d = bz.FcDesc()
+                a = acts[-1]
+                d.a, d.w, d.y, d.bias = a.data_ptr(), wp.data_ptr(), y.data_ptr(), b.data_ptr()
+                d.lda, d.ldw, d.ldy = a.stride(0), wp.stride(0), y.stride(0)
+                d.m, d.n, d.k = B, wp.shape[0], k
+                d.in_dtype, d.out_dtype = bdt, bz.bz_dtype(y.dtype)
+                d.bias_rows = 1
+                d.alpha = d.beta = 1.0
+                if last:
+                    d.act = bz.ACT_SOFTMAX
+                else:
+                    d.act, d.act_p0, d.act_size = bz.ACT_PRELU, slope.data_ptr(), slope.numel()
+                descs.append(d)
+                acts.append(y)
+            self.steps.append(dict(plan=plan, descs=descs, acts=acts, keep=keep, x=x))
+            self.nnz.append(nnz)
+
+    # --- launches (current stream) ---------------------------------------------------------------
+    def _stream(self):
+        import torch
+        return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def scan(self, i, st=None):
+        p = self.steps[i % self.n_batches]["plan"]
+        bz.check(self.lib.bz_segments_to_offsets_slots(p.slots_dev.data_ptr(), p.n, st or self._stream()))
+
+    def pool(self, i, st=None):
+        p = self.steps[i % self.n_batches]["plan"]
+        bz.check(self.lib.bz_embed_pool(p.slots_dev.data_ptr(), C.byref(p.launch), st or self._stream()))
+
+    def fc(self, i, layer, st=None):
+        d = self.steps[i % self.n_batches]["descs"][layer]
+        bz.check(self.lib.bz_fc_fused(C.byref(d), st or self._stream()))
+
+    def step(self, i):
+        st = self._stream()
+        if not self.fused_scan:
+            self.scan(i, st)
+        self.pool(i, st)
+        for layer in range(len(self.weights)):
+            self.fc(i, layer, st)
+
+    def output(self, i):
+        return self.steps[i % self.n_batches]["acts"][-1]
+
+    def pooled(self, i):
+        return self.steps[i % self.n_batches]["x"]
+
+    # --- accounting ------------------------------------------------------------------------------
+    def embedding_bytes(self, i):
+        from synth import embedding_bytes
+        cfg = self.cfg
+        return embedding_bytes(self.nnz[i % self.n_batches], cfg.batch, cfg.slots, cfg.dim * 2, 0, cfg.slots * cfg.dim, 2)
+
+    def fc_flops(self):
+        L = self.cfg.layers
+        return [2.0 * self.cfg.batch * L[i] * L[i + 1] for i in range(len(L) - 1)]
+
+
+def oracle_forward(oracle, cfg, tables_np, mlp_np, sparse, dense, in_round=None):
+    """The same forward on the CPU oracle (fp32 path fed the kernel's rounded inputs).  tables_np: list of
+    oracle.Table; mlp_np: [(W [K,N] fp32, b, slope)].  Returns (pooled [B, in_dim] fp32, probs [B, 2])."""
+    B = cfg.batch
+    x = np.zeros((B, cfg.in_dim), np.float32)
+    x[:, :cfg.dense] = dense if in_round is None else in_round(dense)
+    for s, (ids, vals, seg) in enumerate(sparse):
+        oracle.embed_get(tables_np[s], ids, vals, seg, [(0, 0, 0, x, cfg.dense + s * cfg.dim)])
+    h = x if in_round is None else in_round(x)
+    pooled = h.copy()
+    n = len(mlp_np)
+    for li, (w, b, slope) in enumerate(mlp_np):
+        wt = np.ascontiguousarray(w.T)  # [N,K] + transB: same k-ascending sums, contiguous inner loop
+        if li == n - 1:
+            h = oracle.fc(h, wt, b, act="softmax", transb=True)
+        else:
+            h = oracle.fc(h, wt, b, act="prelu", act_params=(slope, ), transb=True)
+            if in_round is not None:
+                h = in_round(h)
+    return pooled, h
