@@ -96,20 +96,28 @@ def main():
     lat = np.sort(np.array(lat))
     p50, p99 = float(lat[len(lat) // 2]), float(lat[int(len(lat) * 0.99)])
 
-    # ---- per-kernel durations: HIP events on the launch stream around R back-to-back launches
+    # ---- per-kernel durations: HIP events on the launch stream around a replayed HIP graph that holds
+    # R back-to-back launches of the one kernel (over the pooled batches), so host launch cost is not in it
     def timed(fn, reps):
-        for i in range(20):
+        for i in range(fwd.n_batches):
             fn(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(reps):
+                fn(i)
+        g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        rounds = 5
         e0.record()
-        for i in range(reps):
-            fn(i)
+        for _ in range(rounds):
+            g.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / reps  # us
+        return e0.elapsed_time(e1) * 1e3 / (reps * rounds)  # us
 
-    R = max(200, min(K, 1000))
+    R = 8 * fwd.n_batches
     kern_us = {"bz_embed_pool_kernel": timed(fwd.pool, R)}
     for li in range(len(fwd.weights)):
         kern_us["bz_fc[%d]" % li] = timed(lambda i, li=li: fwd.fc(i, li), R)

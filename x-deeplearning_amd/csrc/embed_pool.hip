@@ -315,8 +315,18 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
     return;
   }
   // base = sum of the counts before b0 (independent coalesced reads), local = this thread's sample
+  // (8 loads in flight per thread: a rolled loop would wait for each load before issuing the next)
   int64_t part = 0;
-  for (int64_t i = tid; i < b0; i += kThreads) part += s.segments[i];
+  for (int64_t i0 = 0; i0 < b0; i0 += 8 * kThreads) {
+    int32_t c[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t i = i0 + k * kThreads + tid;
+      c[k] = i < b0 ? s.segments[i] : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) part += c[k];
+  }
   const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)s.segments[b0 + tid] : 0;
   int64_t base = part;
 #pragma unroll
@@ -370,21 +380,34 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
   float acc[CE];
 #pragma unroll
   for (int i = 0; i < CE; ++i) acc[i] = 0.f;
+  // each fetching lane takes ids j + k*SRC + l: one coalesced read per k for the whole group.  The
+  // next step's ids are requested before this step's rows, so the two round trips overlap.
+  int64_t id_next[KPL];  // raw ids: resolved to rows only when consumed, so the wait lands after the row loads
+  float val_next[KPL];
+  auto fetch_ids = [&](int64_t j) {
+    const int cnt = (int)((end - j) < kBlockIds ? (end - j) : kBlockIds);
+#pragma unroll
+    for (int k = 0; k < KPL; ++k) {
+      const int idx = k * SRC + l;
+      id_next[k] = -1;  // resolves to "absent" on both the direct and (as a never-stored key) the hash path
+      val_next[k] = 0.f;
+      if (l < SRC && idx < cnt) {
+        id_next[k] = s.ids[j + idx];
+        val_next[k] = s.values[j + idx];
+      }
+    }
+  };
+  if (start < end) fetch_ids(start);
   for (int64_t j = start; j < end; j += kBlockIds) {
     const int cnt = (int)((end - j) < kBlockIds ? (end - j) : kBlockIds);
-    // each fetching lane takes ids j + k*SRC + l: one coalesced read per k for the whole group
     int row_own[KPL];
     float val_own[KPL];
 #pragma unroll
     for (int k = 0; k < KPL; ++k) {
-      const int idx = k * SRC + l;
-      row_own[k] = -1;
-      val_own[k] = 0.f;
-      if (l < SRC && idx < cnt) {
-        row_own[k] = (int)resolve_row(s, s.ids[j + idx]);
-        val_own[k] = s.values[j + idx];
-      }
+      row_own[k] = (l < SRC && k * SRC + l < cnt) ? (int)resolve_row(s, id_next[k]) : -1;
+      val_own[k] = val_next[k];
     }
+    if (j + kBlockIds < end) fetch_ids(j + kBlockIds);
     int row[kBlockIds];
     float val[kBlockIds];
     uint4 raw[kBlockIds];

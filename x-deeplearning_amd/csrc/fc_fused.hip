@@ -8,8 +8,8 @@
 // Activation(Gemm(x, W, b)) evaluated in fp32.
 //
 // Main kernel: C tile BM x BN per workgroup, K stepped by BK through double-buffered LDS
-// (global -> registers -> LDS, one barrier per step, next tile's global loads in flight
-// during the MFMAs).  Operands are both "K contiguous" (A row major, W packed [N,K]) so
+// (global -> registers -> LDS, one barrier per step) with the global loads of the next D
+// tiles in flight in D register sets while the current tile is multiplied.  Operands are both "K contiguous" (A row major, W packed [N,K]) so
 // a lane's MFMA fragment is one 16-byte LDS read; rows are padded by 16 bytes, which
 // spreads the 16 lanes of a ds_read_b128 phase over all 64 banks.  fp16/bf16 use
 // v_mfma_f32_32x32x16 (K=16 per instruction, fp32 accumulate); fp32 uses
@@ -59,6 +59,28 @@ __device__ __forceinline__ float apply_act(float v, int n, const Epilogue& e) {
       const float t = expf(-1.f * (v - e.p1[n]) / den);
       const float p = 1.f / (1.f + t);
       return (1.f - p) * e.p0[n] * v + p * v;
+    }
+    case BZ_ACT_LEAKY_RELU:
+      return v >= 0.f ? v : e.act_alpha * v;
+    case BZ_ACT_SIGMOID: {
+      const float t = expf(v);
+      return t / (1.f + t);
+    }
+    default:
+      return v;
+  }
+}
+
+// the same with the column's parameters already in registers (p0 = slope | gamma, p1 = mean, p2 = var)
+__device__ __forceinline__ float apply_act_regs(float v, const Epilogue& e, float p0, float p1, float p2) {
+  switch (e.act) {
+    case BZ_ACT_PRELU:
+      return v * ((float)(v > 0.f) + (float)(v < 0.f) * p0);
+    case BZ_ACT_DICE: {
+      const float den = e.dice_nosqrt ? p2 : sqrtf(p2 + kDiceEps);
+      const float t = expf(-1.f * (v - p1) / den);
+      const float p = 1.f / (1.f + t);
+      return (1.f - p) * p0 * v + p * v;
     }
     case BZ_ACT_LEAKY_RELU:
       return v >= 0.f ? v : e.act_alpha * v;
@@ -150,14 +172,24 @@ __device__ __forceinline__ uint4 load_chunk(const char* base, int64_t row, int64
   return out;
 }
 
+// the same for operands whose rows are 16-byte aligned and K a multiple of the chunk: no branches, so
+// the loads of several K tiles can stay in flight (a chunk is either wholly inside K or zero)
+template <int DT>
+__device__ __forceinline__ uint4 load_chunk_aligned(const char* base, int64_t row, int64_t ld, int k, int K) {
+  constexpr int ES = In<DT>::kSize;
+  constexpr int CH = In<DT>::kChunk;
+  const int kc = k < K ? k : K - CH;
+  return *(const uint4*)(base + (row * ld + kc) * ES);  // caller zeroes chunks with k >= K when it consumes them
+}
+
 // ---------------------------------------------------------------------------------------------
 // tiled MFMA kernel
 // ---------------------------------------------------------------------------------------------
-template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN>
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED>
 __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __restrict__ A, const char* __restrict__ W,
                                                                   OutT* __restrict__ Y, int M, int N, int K, int64_t lda,
                                                                   int64_t ldw, int64_t ldy, bool vec_a, bool vec_w,
-                                                                  int tiles_m, Epilogue ep) {
+                                                                  bool vec_y, int tiles_m, Epilogue ep) {
   using T = In<DT>;
   constexpr int NT = WM * WN * 64;
   constexpr int ES = T::kSize;
@@ -180,8 +212,11 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  uint4 ra[A_PER], rw[W_PER];
-  auto gload = [&](int k0) {
+  // D register sets: K tiles kt+1 .. kt+D are in flight from global memory while tile kt is multiplied out of
+  // LDS.  The kernel is latency bound at CTR sizes (a tile's MFMAs take ~0.1 us, a round trip ~1 us), so the
+  // number of exposed round trips, ceil(KT / D), is what sets its duration.
+  uint4 ra[D][A_PER], rw[D][W_PER];
+  auto gload = [&](int set, int k0) {
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int q = tid + i * NT;
@@ -189,7 +224,8 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         const int r = q / CPR, ch = q % CPR;
         int m = m0 + r;
         m = m < M ? m : M - 1;
-        ra[i] = load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a);
+        ra[set][i] = ALIGNED ? load_chunk_aligned<DT>(A, m, lda, k0 + ch * T::kChunk, K)
+                             : load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a);
       }
     }
 #pragma unroll
@@ -199,77 +235,149 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         const int r = q / CPR, ch = q % CPR;
         int n = n0 + r;
         n = n < N ? n : N - 1;
-        rw[i] = load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w);
+        rw[set][i] = ALIGNED ? load_chunk_aligned<DT>(W, n, ldw, k0 + ch * T::kChunk, K)
+                             : load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w);
       }
     }
   };
-  auto lstore = [&](int buf) {
+  // registers -> LDS.  The aligned path masks chunks beyond K here, at the point of use, so that nothing
+  // touches a loaded register (and forces a wait) while later tiles are still being requested.
+  auto masked = [&](uint4 v, int k) {
+    if (ALIGNED) {
+      const uint32_t keep = k < K ? 0xffffffffu : 0u;
+      v.x &= keep;
+      v.y &= keep;
+      v.z &= keep;
+      v.w &= keep;
+    }
+    return v;
+  };
+  auto lstore = [&](int set, int buf, int k0) {
 #pragma unroll
     for (int i = 0; i < A_PER; ++i) {
       const int q = tid + i * NT;
-      if (A_CHUNKS % NT == 0 || q < A_CHUNKS) *(uint4*)&lds[buf][(q / CPR) * PITCH + (q % CPR) * 16] = ra[i];
+      if (A_CHUNKS % NT == 0 || q < A_CHUNKS)
+        *(uint4*)&lds[buf][(q / CPR) * PITCH + (q % CPR) * 16] = masked(ra[set][i], k0 + (q % CPR) * T::kChunk);
     }
 #pragma unroll
     for (int i = 0; i < W_PER; ++i) {
       const int q = tid + i * NT;
-      if (W_CHUNKS % NT == 0 || q < W_CHUNKS) *(uint4*)&lds[buf][(BM + q / CPR) * PITCH + (q % CPR) * 16] = rw[i];
+      if (W_CHUNKS % NT == 0 || q < W_CHUNKS)
+        *(uint4*)&lds[buf][(BM + q / CPR) * PITCH + (q % CPR) * 16] = masked(rw[set][i], k0 + (q % CPR) * T::kChunk);
     }
   };
 
-  floatx16 acc[TM][TN];
+  // with a single 32x32 block per wave, back-to-back MFMAs into one accumulator would each wait for the
+  // previous result; alternate K steps between two accumulators and add them at the end
+  constexpr int KACC = (TM * TN == 1 && BK / T::kStepK >= 2) ? 2 : 1;
+  floatx16 acc[KACC][TM][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int a = 0; a < KACC; ++a)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][i][j][r] = 0.f;
 
-  const int KT = (K + BK - 1) / BK;
-  gload(0);
-  lstore(0);
-  __syncthreads();
-  const int frag_row = lane & 31, frag_half = lane >> 5;
-  for (int kt = 0; kt < KT; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) gload((kt + 1) * BK);
-    const char* la = &lds[buf][(wm * WTM + frag_row) * PITCH + frag_half * 16];
-    const char* lw = &lds[buf][(BM + wn * WTN + frag_row) * PITCH + frag_half * 16];
-#pragma unroll
-    for (int ks = 0; ks < BK / T::kStepK; ++ks) {
-      uint4 fa[TM], fw[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(la + i * 32 * PITCH + ks * 32);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fw[j] = *(const uint4*)(lw + j * 32 * PITCH + ks * 32);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) T::mma(fa[i], fw[j], acc[i][j]);
-    }
-    if (kt + 1 < KT) lstore(buf ^ 1);
-    __syncthreads();
-  }
-
-  // epilogue: lane owns column n, rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block
+  // per-column epilogue parameters, requested before anything else so their latency hides under the K loop
+  float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn * WTN + j * 32 + (lane & 31);
-    if (n >= N) continue;
-    const float bcol = (ep.bias_rows == 1) ? ep.beta * ep.bias[n] : 0.f;
+    int n = n0 + wn * WTN + j * 32 + (lane & 31);
+    n = n < N ? n : N - 1;
+    cbias[j] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cp0[j] = cp1[j] = cp2[j] = 0.f;
+    if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
+    if (ep.act == BZ_ACT_DICE) {
+      cp0[j] = ep.p0[n];
+      cp1[j] = ep.p1[n];
+      cp2[j] = ep.p2[n];
+    }
+  }
+
+  // The K loop runs over KT rounded up to a multiple of D with no conditionals inside: tiles beyond K are
+  // loaded from a clamped address and zeroed by the mask, so they add nothing.  Straight-line code lets the
+  // compiler count outstanding loads exactly (s_waitcnt vmcnt(n) waits for the oldest set only).
+  const int KT = (K + BK - 1) / BK;
+  const int KTR = (KT + D - 1) / D * D;
+#pragma unroll
+  for (int d = 0; d < D; ++d) gload(d, d * BK);
+  lstore(0, 0, 0);
+  __syncthreads();
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  for (int kt0 = 0; kt0 < KTR; kt0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int kt = kt0 + d;
+      const int buf = kt & 1;
+      gload(d, (kt + D) * BK);  // set d held tile kt, which already sits in LDS
+      const char* la = &lds[buf][(wm * WTM + frag_row) * PITCH + frag_half * 16];
+      const char* lw = &lds[buf][(BM + wn * WTN + frag_row) * PITCH + frag_half * 16];
+#pragma unroll
+      for (int ks = 0; ks < BK / T::kStepK; ++ks) {
+        uint4 fa[TM], fw[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(la + i * 32 * PITCH + ks * 32);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fw[j] = *(const uint4*)(lw + j * 32 * PITCH + ks * 32);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) T::mma(fa[i], fw[j], acc[ks % KACC][i][j]);
+      }
+      lstore((d + 1) % D, buf ^ 1, (kt + 1) * BK);
+      __syncthreads();
+    }
+  }
+
+  if (KACC == 2) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][i][j][r] += acc[KACC - 1][i][j][r];
+  }
+  // epilogue: lane owns column n, rows 8*(r/4) + 4*(lane/32) + r%4 of each 32x32 block.  The activated tile
+  // goes through LDS (free after the K loop) so that global stores are 16 bytes per lane along rows.
+  constexpr int OS = (int)sizeof(OutT);
+  constexpr int OPITCH = BN * OS + 16;
+  static_assert(BM * OPITCH <= (int)sizeof(lds), "output tile must fit the operand buffers");
+  char* lout = &lds[0][0];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int nl = wn * WTN + j * 32 + (lane & 31);
+    const int n = n0 + nl;
+    const bool n_ok = n < N;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < M) {
-          float v = ep.alpha * acc[i][j][r];
+        const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int m = m0 + ml;
+        if (m < M && n_ok) {
+          float v = ep.alpha * acc[0][i][j][r];
           if (ep.bias_rows == 1)
-            v += bcol;
+            v += ep.beta * cbias[j];
           else if (ep.bias_rows > 1)
             v += ep.beta * ep.bias[(int64_t)m * N + n];
-          store_out<OutT>(Y + (int64_t)m * ldy + n, apply_act(v, n, ep));
+          v = apply_act_regs(v, ep, cp0[j], cp1[j], cp2[j]);
+          if (vec_y)
+            store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
+          else
+            store_out<OutT>(Y + (int64_t)m * ldy + n, v);
         }
       }
+    }
+  }
+  if (vec_y) {
+    __syncthreads();
+    constexpr int OCPR = BN * OS / 16;  // 16-byte chunks per tile row
+    for (int q = tid; q < BM * OCPR; q += NT) {
+      const int ml = q / OCPR, ch = q % OCPR;
+      const int m = m0 + ml, n = n0 + ch * (16 / OS);
+      if (m < M && n < N) *(uint4*)((char*)(Y + (int64_t)m * ldy + n)) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
     }
   }
 }
@@ -310,6 +418,20 @@ __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restric
   const int g = tid / lpr, l = tid - g * lpr;
   const int rows_per_wg = 256 / lpr;
   const int nchunks = (K + CH - 1) / CH;
+  // per-column parameters first: their latency hides under the row loads
+  float cb[kSkinnyMaxN], q0[kSkinnyMaxN], q1[kSkinnyMaxN], q2[kSkinnyMaxN];
+#pragma unroll
+  for (int n = 0; n < kSkinnyMaxN; ++n) {
+    const int nn = n < N ? n : N - 1;
+    cb[n] = ep.bias_rows == 1 ? ep.bias[nn] : 0.f;
+    q0[n] = q1[n] = q2[n] = 0.f;
+    if (ep.act == BZ_ACT_PRELU) q0[n] = ep.p0[ep.act_size == 1 ? 0 : nn];
+    if (ep.act == BZ_ACT_DICE) {
+      q0[n] = ep.p0[nn];
+      q1[n] = ep.p1[nn];
+      q2[n] = ep.p2[nn];
+    }
+  }
   for (int64_t m = (int64_t)blockIdx.x * rows_per_wg + g; m < M; m += (int64_t)gridDim.x * rows_per_wg) {
     float acc[kSkinnyMaxN];
 #pragma unroll
@@ -340,7 +462,7 @@ __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restric
         if (n < N) {
           float x = ep.alpha * acc[n];
           if (ep.bias_rows == 1)
-            x += ep.beta * ep.bias[n];
+            x += ep.beta * cb[n];
           else if (ep.bias_rows > 1)
             x += ep.beta * ep.bias[m * N + n];
           v[n] = x;
@@ -364,7 +486,7 @@ __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restric
       } else {
 #pragma unroll
         for (int n = 0; n < kSkinnyMaxN; ++n)
-          if (n < N) v[n] = apply_act(v[n], n, ep);
+          if (n < N) v[n] = apply_act_regs(v[n], ep, q0[n], q1[n], q2[n]);
       }
 #pragma unroll
       for (int n = 0; n < kSkinnyMaxN; ++n)
@@ -388,12 +510,15 @@ __global__ void bz_pack_weight_kernel(const SrcT* __restrict__ src, DstT* __rest
   }
 }
 
-template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN>
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED>
 int launch_mfma(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
   const int tiles_m = (d.m + BM - 1) / BM, tiles_n = (d.n + BN - 1) / BN;
-  hipLaunchKernelGGL((bz_fc_mfma_kernel<DT, OutT, BM, BN, BK, WM, WN>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), 0, st,
+  // output rows 16-byte aligned and N a whole number of 16-byte chunks: coalesced stores through LDS
+  const bool vec_y = ((uintptr_t)d.y % 16 == 0) && ((d.ldy * (int64_t)sizeof(OutT)) % 16 == 0) &&
+                     (d.n % (16 / (int)sizeof(OutT)) == 0);
+  hipLaunchKernelGGL((bz_fc_mfma_kernel<DT, OutT, BM, BN, BK, WM, WN, D, ALIGNED>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), 0, st,
                      (const char*)d.a, (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, vec_a, vec_w,
-                     tiles_m, ep);
+                     vec_y, tiles_m, ep);
   BZ_LAUNCH_OK("bz_fc_mfma_kernel");
   return BZ_OK;
 }
@@ -403,9 +528,12 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
   constexpr int BK = In<DT>::kSize == 2 ? 64 : 32;
   const int64_t wg128 = (int64_t)((d.m + 127) / 128) * ((d.n + 127) / 128);
   const int64_t wg64 = (int64_t)((d.m + 63) / 64) * ((d.n + 63) / 64);
-  if (wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2>(d, ep, vec_a, vec_w, st);
-  if (wg64 >= 256) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2>(d, ep, vec_a, vec_w, st);
-  return launch_mfma<DT, OutT, 32, 64, BK, 1, 2>(d, ep, vec_a, vec_w, st);
+  // rows 16-byte aligned and K a whole number of chunks: branch-free loads, several tiles in flight
+  const bool aligned = vec_a && vec_w && d.k % In<DT>::kChunk == 0;
+  if (!aligned) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 1, false>(d, ep, vec_a, vec_w, st);
+  if (wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2, 2, true>(d, ep, vec_a, vec_w, st);
+  if (wg64 >= 256) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
+  return launch_mfma<DT, OutT, 32, 64, BK, 1, 2, 4, true>(d, ep, vec_a, vec_w, st);
 }
 
 template <int DT, typename OutT>
