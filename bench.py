@@ -29,7 +29,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--pool", type=int, default=32, help="number of distinct pre-generated batches")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-graph", action="store_true", help="launch kernels one by one instead of replaying HIP graphs")
+    ap.add_argument("--graph", action="store_true", help="replay one HIP graph per step instead of launching kernels one by one")
+    ap.add_argument("--streams", type=int, default=4,
+                    help="predictor streams: consecutive batches go round robin to this many HIP streams (the reference "
+                         "runs one Predictor per serving thread, each with its own stream)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one process, no collectives); --gpus %d is not supported" % args.gpus,
@@ -54,7 +57,7 @@ def main():
 
     # one HIP graph per pooled batch: the five launches of a step replay as one submission
     graphs = None
-    if not args.no_graph:
+    if args.graph:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -68,11 +71,19 @@ def main():
                 fwd.step(i)
             graphs.append(g)
 
-    def run_step(i):
+    import ctypes
+    S = max(1, min(args.streams, fwd.n_batches))
+    assert fwd.n_batches % S == 0, "--pool must be a multiple of --streams (a pooled batch always runs on one stream)"
+    streams = [torch.cuda.Stream() for _ in range(S)] if S > 1 else [torch.cuda.current_stream()]
+    stream_ptrs = [ctypes.c_void_p(st.cuda_stream) for st in streams]
+
+    def run_step(i, s=None):
+        s = i % S if s is None else s
         if graphs is not None:
-            graphs[i % fwd.n_batches].replay()
+            with torch.cuda.stream(streams[s]):
+                graphs[i % fwd.n_batches].replay()
         else:
-            fwd.step(i)
+            fwd.step(i, stream_ptrs[s])
 
     # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations
     for i in range(W):
@@ -90,7 +101,7 @@ def main():
     lat = []
     for i in range(min(K, 2000)):
         a = time.perf_counter()
-        run_step(i)
+        run_step(i, 0)
         torch.cuda.synchronize()
         lat.append((time.perf_counter() - a) * 1e3)
     lat = np.sort(np.array(lat))
@@ -182,7 +193,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic (seeded; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
         "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
-                   "batch_pool": fwd.n_batches, "submission": "per-kernel launches" if graphs is None else "hip graph per step",
+                   "batch_pool": fwd.n_batches, "submission": "per-kernel launches" if graphs is None else "hip graph per step", "predictor_streams": S,
                    "device": arch},
         "roofline": roofline,
         "embedding_pool": {"GB/s": round(pool_gbs, 1), "frac_of_hbm_peak": round(pool_gbs / HBM_PEAK_GBS, 5),

@@ -1,0 +1,120 @@
+/*
+ * blaze_c_api.h -- the public C ABI of the predictor, entry point for entry point the one the reference
+ * exports from blaze/api/c_api/c_api_predictor.h:16-105 and c_api_error.h (what its ctypes binding
+ * blaze/binding/python/pyblaze loads).  Conventions kept: opaque void* handles; every call returns 0 on
+ * success and -1 on failure; the message of the last failure is thread local (Blaze_GetLastErrorString,
+ * c_api_error.cc:12-28); name / shape arrays returned by the List*Names, ParamName, *Shape calls point into
+ * thread-local or predictor-owned storage and stay valid until the next such call on that thread / predictor;
+ * Blaze_PredictorOutput copies into caller memory; Blaze_PredictorFeed copies `len` bytes in and requires
+ * len == element count * sizeof(dtype).  A Predictor is not thread safe: one per serving thread.
+ *
+ * device_type for Blaze_PredictorCreate: 1 = the accelerator (MI355X), the value existing callers pass for
+ * the GPU; -1 = probe; 0 (CPU) fails at operator creation: this build has no CPU execution path.
+ *
+ * Not provided by this build (they return -1 with a message): the model importers and the offline optimizer
+ * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze, Blaze_OptimizeBlaze) and the text-to-QED table
+ * builder (Blaze_QuickEmbeddingBuildFp32/Fp16).
+ */
+#ifndef BLAZE_C_API_H_
+#define BLAZE_C_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BLAZE_API __attribute__((visibility("default")))
+
+typedef void* PredictorManagerHandle;
+typedef void* PredictorHandle;
+
+/* c_api_error.h */
+BLAZE_API void Blaze_GetLastErrorString(const char** msg);
+BLAZE_API void Blaze_SetLastErrorString(const char* format, ...);
+
+/* c_api_predictor.h:19-24 -- accepted and ignored: request batching is outside this build */
+BLAZE_API int Blaze_InitScheduler(int enable_batching, int max_batch_size, int batch_timeout_micros, int num_threads_for_cpu,
+                                  int num_threads_for_cuda, int num_threads_for_pipe);
+
+/* c_api_predictor.h:27-42 */
+BLAZE_API int Blaze_PredictorManagerCreate(PredictorManagerHandle* handle);
+BLAZE_API int Blaze_PredictorManagerDelete(PredictorManagerHandle handle);
+BLAZE_API int Blaze_PredictorManagerSetDataType(PredictorManagerHandle handle, int data_type);
+BLAZE_API int Blaze_PredictorManagerSetRunMode(PredictorManagerHandle handle, const char* run_mode);
+BLAZE_API int Blaze_LoadSparseModelWeight(PredictorManagerHandle handle, const char* sparse_model_weight_file);
+/* (sic) the reference spells it Predcitor; both spellings are exported */
+BLAZE_API int Blaze_PredcitorManagerLoadModel(PredictorManagerHandle handle, const char* blaze_model_file, int optimization_pass);
+BLAZE_API int Blaze_PredictorManagerLoadModel(PredictorManagerHandle handle, const char* blaze_model_file, int optimization_pass);
+BLAZE_API int Blaze_PredictorManagerLoadDeepNetModel(PredictorManagerHandle handle, const char* deepnet_conf_file,
+                                                     const char* deepnet_param_file, int optimization_pass);
+
+/* c_api_predictor.h:45-49 */
+BLAZE_API int Blaze_PredictorCreate(PredictorManagerHandle predictor_mgr, int device_type, int device_id, PredictorHandle* handle);
+BLAZE_API int Blaze_PredictorDelete(PredictorHandle handle);
+
+/* c_api_predictor.h:53-61 */
+BLAZE_API int Blaze_PredictorReshapeInput(PredictorHandle handle, const char* name, const int* data, int num);
+BLAZE_API int Blaze_PredictorFeed(PredictorHandle handle, const char* name, void* data, int len);
+BLAZE_API int Blaze_PredictorForward(PredictorHandle handle);
+
+/* c_api_predictor.h:64-74 */
+BLAZE_API int Blaze_PredictorOutputShape(PredictorHandle handle, const char* name, size_t* ndim, size_t** shape);
+BLAZE_API int Blaze_PredictorOutputDataType(PredictorHandle handle, const char* name, int* data_type);
+BLAZE_API int Blaze_PredictorOutput(PredictorHandle handle, const char* name, void* data, size_t len);
+
+/* c_api_predictor.h:77-90 */
+BLAZE_API int Blaze_PredictorParamName(PredictorHandle handle, size_t* ndim, const char*** name);
+BLAZE_API int Blaze_PredictorParamShape(PredictorHandle handle, const char* name, size_t* ndim, size_t** shape);
+BLAZE_API int Blaze_PredictorParamDataType(PredictorHandle handle, const char* name, int* data_type);
+BLAZE_API int Blaze_PredictorParam(PredictorHandle handle, const char* name, void* data, size_t len);
+
+/* c_api_predictor.h:93-98 */
+BLAZE_API int Blaze_PredictorListInputNames(PredictorHandle handle, size_t* ndim, const char*** names);
+BLAZE_API int Blaze_PredictorListOutputNames(PredictorHandle handle, size_t* ndim, const char*** names);
+
+/* c_api_predictor.h:101-107 -- observer "profile": per-operator host wall time as chrome-trace JSON */
+BLAZE_API int Blaze_PredictorRegisterObservers(PredictorHandle handle, size_t ndim, const char** names);
+BLAZE_API int Blaze_PredictorDumpObservers(PredictorHandle handle, size_t* ndim, const char*** key, const char*** value);
+
+/* c_api_blaze_converter.h / c_api_blaze_optimizer.h / c_api_quick_embedding.h: not part of this build */
+BLAZE_API int Blaze_ConvertBlaze(const char* model_conf_file, const char* model_data_file, int model_type, int weight_type,
+                                 int io_type, int x_type_num, const char** x_type_key, const int* x_type_value,
+                                 const char* blaze_model_file, int binary);
+BLAZE_API int Blaze_OptimizeBlaze(const char* raw_model_file, const char* optimized_model_file, int binary);
+BLAZE_API int Blaze_QuickEmbeddingBuildFp32(const char* path, const char* meta, const char* output_file, int thread_num);
+BLAZE_API int Blaze_QuickEmbeddingBuildFp16(const char* path, const char* meta, const char* output_file, int thread_num);
+
+/* ---- extensions (no reference counterpart) ------------------------------------------------------------ */
+
+/*
+ * Register an in-memory table with the manager's device store (created on demand as "qed_hip_sparse_puller")
+ * instead of loading a QED file: synthetic benchmarks, tables generated on the device, int8 tables with a
+ * per-row fp32 scale (a storage format the reference's QED reader rejects, blaze/store/defines.h:29-50).
+ * value_type: 1 fp32, 12 fp16, 7 int8.  rows_ptr: [rows, dim] row major, device memory when on_device else
+ * host memory.  keys: host int64[rows] or NULL (ids are row numbers).  scale: [rows] fp32, same place as rows_ptr.
+ */
+BLAZE_API int Blaze_HipStoreAddTable(PredictorManagerHandle handle, const char* table_name, int value_type, int64_t rows, int dim,
+                                     const void* rows_ptr, int on_device, const int64_t* keys, const float* scale);
+
+/* load a model from memory: a NetDef in protobuf text format (is_text) or proto2 wire format */
+BLAZE_API int Blaze_PredictorManagerLoadModelFromString(PredictorManagerHandle handle, const char* data, size_t len, int is_text);
+
+/*
+ * NetDef text format <-> proto2 wire format, for tools without a protobuf toolchain.  Writes at most cap bytes
+ * to out (may be NULL to query the size) and the full size to *out_len.
+ */
+BLAZE_API int Blaze_ConvertNetDef(const char* in, size_t len, int in_is_text, int out_is_text, char* out, size_t cap, size_t* out_len);
+
+/* device address of an input / output blob after ReshapeInput / Forward, for callers that keep inputs on the device */
+BLAZE_API int Blaze_PredictorInputDevicePtr(PredictorHandle handle, const char* name, void** ptr);
+BLAZE_API int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char* name, void** ptr);
+
+/* run Forward `count` times on the calling thread (benchmark loops without per-call host overhead) */
+BLAZE_API int Blaze_PredictorForwardN(PredictorHandle handle, int count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BLAZE_C_API_H_ */

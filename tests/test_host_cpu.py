@@ -1,0 +1,248 @@
+"""Host-layer checks that need no GPU: exported ABI, NetDef codecs against real protobuf, the QED builder against
+the reference's own store object code, and error conventions of the C API."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header, macro):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(macro + r"\s+[\w\s\*]+?\b(\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    """The shared library loads and exports exactly what include/*.h declares (no compute calls here)."""
+    import blaze_hip
+    import pyblaze_hip
+    lib = C.CDLL(blaze_hip.LIB_PATH)
+    kernel_api = _declared("blaze_hip.h", "BZ_API")
+    predictor_api = _declared("blaze_c_api.h", "BLAZE_API")
+    assert len(kernel_api) >= 11 and len(predictor_api) >= 36
+    for name in kernel_api + predictor_api:
+        assert hasattr(lib, name), "declared in include/ but not exported: " + name
+    assert sorted(kernel_api) == sorted(blaze_hip.EXPORTS)
+    assert sorted(predictor_api) == sorted(pyblaze_hip.EXPORTS)
+
+
+def test_struct_layouts_match_header():
+    """ctypes mirrors of the descriptor structs have the sizes the C compiler gives them."""
+    import subprocess
+    import tempfile
+    import blaze_hip
+    src = ('#include "blaze_hip.h"\n#include <stdio.h>\nint main(){printf("%zu %zu %zu %zu %zu\\n", sizeof(bz_embed_slot), '
+           'sizeof(bz_embed_launch), sizeof(bz_fc_desc), sizeof(bz_bgemm_desc), sizeof(bz_act_desc));return 0;}\n')
+    with tempfile.TemporaryDirectory() as d:
+        open(os.path.join(d, "s.c"), "w").write(src)
+        subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), os.path.join(d, "s.c"), "-o", os.path.join(d, "s")])
+        sizes = [int(x) for x in subprocess.check_output([os.path.join(d, "s")]).split()]
+    assert sizes == [C.sizeof(blaze_hip.EmbedSlot), C.sizeof(blaze_hip.EmbedLaunch), C.sizeof(blaze_hip.FcDesc),
+                     C.sizeof(blaze_hip.BgemmDesc), C.sizeof(blaze_hip.ActDesc)]
+
+
+def _sample_net():
+    import pyblaze_hip as pb
+    nb = pb.NetBuilder("ctr", device_type=1)
+    nb.external_input("101.ids", pb.K_INT64)
+    nb.external_input("101.values", pb.K_FLOAT)
+    nb.external_input("101.segments", pb.K_INT32)
+    nb.external_output("prob")
+    nb.arg("fuse_gemm_activation", 0)
+    nb.constant("w", np.array([[0.5, -1.25], [3.0, 1e-7]], np.float32))
+    nb.constant("i64", np.array([1032342412, 849234344343, -5], np.int64))
+    nb.op("Embedding", ["101.ids", "101.values", "101.segments"], ["block"],
+          embedding_config=pb.embedding_config_text([("101", "a_01", 2)], [[dict(fg="101", udf=0)]]))
+    nb.op("Gemm", ["block", "w"], ["fc"], transB=True, alpha=0.75)
+    nb.op("Softmax", ["fc"], ["prob"], axis=1)
+    return nb.text()
+
+
+def test_netdef_text_to_wire_matches_protobuf():
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    wire = pb.convert_netdef(_sample_net(), True, False)
+    net = NetDef()
+    net.ParseFromString(wire)
+    assert net.name == "ctr" and net.run_mode == "simple" and net.device_option.device_type == 1
+    assert [o.type for o in net.op] == ["ConstantFill", "ConstantFill", "Embedding", "Gemm", "Softmax"]
+    assert [v.name for v in net.external_input] == ["101.ids", "101.values", "101.segments"]
+    assert [v.dtype for v in net.external_input] == [10, 1, 2]
+    fill = {a.name: a for a in net.op[0].arg}
+    assert list(fill["shape"].ints) == [2, 2] and fill["dtype"].i == 1
+    assert np.array_equal(np.array(fill["value"].floats, np.float32), np.array([0.5, -1.25, 3.0, 1e-7], np.float32))
+    assert list({a.name: a for a in net.op[1].arg}["value"].ints) == [1032342412, 849234344343, -5]
+    gemm = {a.name: a for a in net.op[3].arg}
+    assert gemm["transB"].i == 1 and gemm["alpha"].f == 0.75
+    cfg = {a.name: a for a in net.op[2].arg}["embedding_config"].s.decode()
+    assert 'table_name : "a_01"' in cfg and "\n" in cfg
+    assert {a.name: a.i for a in net.arg} == {"fuse_gemm_activation": 0}
+
+
+def test_netdef_wire_to_text_round_trip_through_protobuf():
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    from google.protobuf import text_format
+    ref = NetDef()
+    ref.name = "rt"
+    ref.run_mode = "dag"
+    ref.version = 1007
+    ref.device_option.device_type = 1
+    ref.device_option.device_id = 3
+    op = ref.op.add()
+    op.type, op.name = "Gemm", 'quote"and\\slash'
+    op.input.extend(["a", "b"])
+    op.output.append("y")
+    op.device_option.device_type = 0
+    op.device_option.device_id = 0
+    a = op.arg.add()
+    a.name, a.f = "alpha", 0.1
+    a = op.arg.add()
+    a.name = "blob"
+    a.s = bytes(range(256))
+    a.floats.extend([1.5, -2.25e-30, 3e38])
+    a.ints.extend([0, -1, 2**62, -2**63])
+    a.strings.extend([b"x", b""])
+    vi = ref.external_input.add()
+    vi.name, vi.dtype, vi.level, vi.input_type, vi.feature_name = "in", 12, 1, 3, "feat"
+    vi.tensor_shape.dims.extend([7, 9])
+    vo = ref.external_output.add()  # scalar fields are written out with their values whether or not they were set
+    vo.name, vo.dtype, vo.level, vo.input_type = "y", 1, 0, 0
+    wire = ref.SerializeToString()
+    text = pb.convert_netdef(wire, False, True).decode("latin-1")
+    back = NetDef()
+    text_format.Parse(text, back)
+    assert back == ref
+    # and C++ wire writer -> protobuf reader
+    again = NetDef()
+    again.ParseFromString(pb.convert_netdef(wire, False, False))
+    assert again == ref
+
+
+def test_malformed_models_are_rejected():
+    import pyblaze_hip as pb
+    with pytest.raises(pb.BlazeError):
+        pb.convert_netdef(b"\x0a\xff\xff\xff\xff\x0f", False, True)  # length runs past the buffer
+    with pytest.raises(pb.BlazeError):
+        pb.convert_netdef('op { type : "Gemm" ', True, False)  # missing brace
+    with pytest.raises(pb.BlazeError):
+        pb.convert_netdef('op { type : "Gemm" arg { name : "alpha" f : abc } }', True, False)
+    pm = pb.PredictorManager()
+    with pytest.raises(pb.BlazeError, match="can not open|failed"):
+        pm.load_model("/nonexistent/model.blaze")
+    with pytest.raises(pb.BlazeError, match="importer|failed"):
+        pm.load_deepnet_model("a.conf", "a.dat")
+    with pytest.raises(pb.BlazeError):
+        pm.load_sparse_model_weight("/nonexistent/qed.bin")
+
+
+def test_cpu_predictor_fails_loudly():
+    """device_type 0 is accepted by the API but no operator of the path has a CPU implementation here."""
+    import pyblaze_hip as pb
+    pm = pb.PredictorManager()
+    pm.load_model_from_string(_sample_net(), True)
+    with pytest.raises(pb.BlazeError, match="no CPU fallback|not registered"):
+        pm.create_predictor(device_type=0)
+
+
+def test_null_handles_return_minus_one():
+    import pyblaze_hip as pb
+    l = pb.lib()
+    assert l.Blaze_PredictorForward(None) == -1
+    assert l.Blaze_PredictorDelete(None) == -1
+    assert l.Blaze_PredictorFeed(None, b"x", None, 0) == -1
+    assert l.Blaze_LoadSparseModelWeight(None, b"x") == -1
+    assert l.Blaze_ConvertBlaze(None, None, 0, 0, 0, 0, None, None, None, 0) == -1
+    assert "not part of this build" in pb.last_error()
+
+
+# ---------------------------------------------------------------- QED builder
+def _write_tables(tmp_path, tables):
+    names = []
+    for name, (keys, rows) in tables.items():
+        with open(tmp_path / name, "w") as f:
+            for k, r in zip(keys, rows):
+                f.write(",".join([str(int(k))] + [repr(float(x)) for x in r]) + "\n")
+        names.append(name)
+    with open(tmp_path / "meta", "w") as f:
+        f.write("\n".join(names) + "\n")
+
+
+def _parse_qed(path):
+    """Independent python reader of the QED container, returns (version, trie bytes, [(gid, hash image, blob image)])."""
+    data = open(path, "rb").read()
+    assert data[:31] == b"ALIMAMA_MODEL_SERVING_EMBEDDING"
+    version = int.from_bytes(data[31:35], "little")
+    pos = 35
+    tlen = int.from_bytes(data[pos:pos + 8], "little")
+    trie = data[pos:pos + 8 + tlen]
+    pos += 8 + tlen
+    tables = []
+    while pos < len(data):
+        gid = int.from_bytes(data[pos:pos + 2], "little")
+        pos += 2
+        nb = int.from_bytes(data[pos:pos + 4], "little")
+        pb_ = int.from_bytes(data[pos + 4 + 8 * nb:pos + 12 + 8 * nb], "little")
+        hlen = 4 + 8 * nb + 8 + pb_
+        himg = data[pos:pos + hlen]
+        pos += hlen
+        blen = int.from_bytes(data[pos:pos + 8], "little")
+        bimg = data[pos:pos + 8 + blen]
+        pos += 8 + blen
+        tables.append((gid, himg, bimg))
+    return version, trie, tables
+
+
+def test_qed_builder_file_image(tmp_path, oracle):
+    import pyblaze_hip as pb
+    rng = np.random.default_rng(12)
+    tables = {}
+    for name, n, dim in (("a_01", 60, 4), ("a_02", 1, 8), ("104_7", 200, 6)):
+        keys = np.unique(rng.integers(-2**62, 2**62, size=n * 2, dtype=np.int64))[:n]
+        tables[name] = (keys, rng.standard_normal((n, dim)).astype(np.float32))
+    _write_tables(tmp_path, tables)
+    out = str(tmp_path / "qed.bin")
+    pb.build_qed(str(tmp_path), "meta", out)
+    version, trie, parsed = _parse_qed(out)
+    assert version == 2000 and [g for g, _, _ in parsed] == [0, 1, 2]
+    for (name, (keys, rows)), (gid, himg, bimg) in zip(tables.items(), parsed):
+        dim = rows.shape[1]
+        # hash image: the oracle's restatement (itself byte-equal to the reference's HashTable::Dump)
+        mine = oracle.HashTable(keys.astype(np.uint64), 1 + 4 * dim * np.arange(len(keys), dtype=np.uint64))
+        assert bytes(mine.dump()) == himg
+        assert int.from_bytes(bimg[:8], "little") == 1 + rows.nbytes
+        assert bimg[9:] == rows.tobytes()
+        if oracle.have_ref():
+            ref = oracle.RefStore(keys, rows)
+            assert bytes(ref.hash_dump()) == himg, "differs from the reference's HashTable::Dump"
+            rb = bytes(ref.blob_dump())
+            assert rb[:8] == bimg[:8] and rb[9:] == bimg[9:], "differs from the reference's WeightBlob::Dump"
+    if oracle.have_ref():
+        rt = oracle.RefTrie(list(tables.keys()), [0, 1, 2])
+        assert bytes(rt.dump()) == trie, "differs from the reference's Trie::Dump"
+    # fp16 flavour: same index, narrowed rows
+    out16 = str(tmp_path / "qed16.bin")
+    pb.build_qed(str(tmp_path), "meta", out16, fp16=True)
+    v16, trie16, parsed16 = _parse_qed(out16)
+    assert v16 == 2001 and trie16 == trie
+    rows0 = tables["a_01"][1]
+    assert parsed16[0][2][9:] == rows0.astype(np.float16).tobytes()
+
+
+def test_qed_builder_meta_quirk_and_errors(tmp_path):
+    """A last meta line without newline is dropped, as the reference's ParseMeta does; a missing table fails."""
+    import pyblaze_hip as pb
+    open(tmp_path / "t1", "w").write("1,0.5\n2,0.25\n")
+    open(tmp_path / "t2", "w").write("1,0.5\n")
+    open(tmp_path / "meta", "w").write("t1\nt2")
+    out = str(tmp_path / "q.bin")
+    pb.build_qed(str(tmp_path), "meta", out)
+    _, _, parsed = _parse_qed(out)
+    assert len(parsed) == 1
+    open(tmp_path / "meta2", "w").write("t1\nmissing\n")
+    with pytest.raises(pb.BlazeError, match="can not open"):
+        pb.build_qed(str(tmp_path), "meta2", out)

@@ -1,0 +1,294 @@
+"""GPU tests of the drop-in boundary: operators run through Predictor / the Blaze_* C ABI.
+
+The reference's operator tests build a net from a text NetDef whose inputs are ConstantFill ops, run it and compare
+outputs with |d| <= 1e-6 (test/operator/operator_test_common.h:20-84).  The same is done here from the same data
+(tests/golden/reference_kats.json), through Blaze_PredictorManagerLoadModelFromString / Blaze_PredictorCreate /
+Blaze_PredictorForward / Blaze_PredictorOutput on device_type 1.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pb():
+    import torch
+    import blaze_hip
+    import pyblaze_hip
+    assert torch.cuda.is_available(), "no GPU visible"
+    blaze_hip.device_check()
+    return pyblaze_hip
+
+
+def _np_dtype(code):
+    return {1: np.float32, 2: np.int32, 10: np.int64, 12: np.float16}[code]
+
+
+def _net_from_kat(pb, case, skip_types=()):
+    nb = pb.NetBuilder("kat", device_type=1)
+    for name, t in case["tensors"].items():
+        nb.constant(name, np.array(t["values"], _np_dtype(t["dtype"])).reshape(t["shape"]), dtype=t["dtype"])
+    for op in case["ops"]:
+        args = {}
+        for k, v in op["args"].items():
+            if k in ("store_name", "store_type", "store_url"):
+                continue
+            if k in ("alpha", "beta"):
+                v = float(v)
+            args[k] = v
+        nb.op(op["type"], op["inputs"], op["outputs"], **args)
+    for name, e in case["expected"].items():
+        nb.external_output(name, e["dtype"])
+    return nb.text()
+
+
+DENSE = ["gemm_net_v1_cpu", "prelu_net_v1_cpu", "dice_net_v1_cpu", "leaky_relu_net_v1_cpu", "sigmoid_net_v1_cpu",
+         "softmax_net_v1_cpu", "matmul_net_v1_cpu", "fused_parallel_gemm_net_v1_cpu", "fused_parallel_gemm_net_v2_cpu",
+         "fused_parallel_gemm_net_v3_cpu", "fused_parallel_gemm_net_v4_cpu", "fused_parallel_gemm_net_v5_cpu",
+         "fused_parallel_matmul_net_v1_cpu", "fused_parallel_matmul_net_v2_cpu", "fused_parallel_matmul_net_v3_cpu"]
+
+
+@pytest.mark.parametrize("name", DENSE)
+def test_reference_operator_kats_through_predictor(pb, kats, name):
+    case = kats[name]
+    pm = pb.PredictorManager()
+    pm.load_model_from_string(_net_from_kat(pb, case), True)
+    p = pm.create_predictor(1, 0)
+    print("case", name, flush=True)
+    p.forward()
+    for out_name, e in case["expected"].items():
+        got = p.output_asnumpy(out_name)
+        assert list(got.shape) == e["shape"]
+        np.testing.assert_allclose(got, np.array(e["values"], np.float32).reshape(e["shape"]), rtol=0, atol=1e-6)
+
+
+def test_reference_embedding_kat_through_predictor(pb, kats):
+    """embedding_v1.conf: the reference runs it over its mock puller (every key -> a row of ones); here the device
+    store gets tables of ones keyed by every id of the fixture."""
+    case = kats["embedding_v1"]
+    pm = pb.PredictorManager()
+    for fg, table, dim in (("101", "a_01", 4), ("102", "a_02", 8), ("104_7", "a_03", 6)):
+        ids = np.unique(np.array(case["tensors"][fg + ".ids"]["values"], np.int64))
+        pm.add_table(table, np.ones((ids.size, dim), np.float32), keys=ids)
+    pm.load_model_from_string(_net_from_kat(pb, case), True)
+    p = pm.create_predictor(1, 0)
+    p.forward()
+    for out_name, e in case["expected"].items():
+        got = p.output_asnumpy(out_name)
+        assert list(got.shape) == e["shape"] and got.dtype == np.float32
+        np.testing.assert_allclose(got, np.array(e["values"], np.float32).reshape(e["shape"]), rtol=0, atol=1e-6)
+
+
+def _write_csv(path, keys, rows):
+    with open(path, "w") as f:
+        for k, r in zip(keys, rows):
+            f.write(",".join([str(int(k))] + [repr(float(x)) for x in r]) + "\n")
+
+
+def _ctr_text(pb, fgs, blocks, dims_in, layers, acts, dtype, fuse, dense_name="dense"):
+    """Embedding -> Concat(dense, block) -> [Gemm + activation]* ; returns (text, weights)."""
+    code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
+    nb = pb.NetBuilder("ctr", device_type=1)
+    inputs = []
+    for fg, _, _ in fgs:
+        nb.external_input(fg + ".ids", pb.K_INT64)
+        nb.external_input(fg + ".values", pb.K_FLOAT)
+        nb.external_input(fg + ".segments", pb.K_INT32)
+        inputs += [fg + ".ids", fg + ".values", fg + ".segments"]
+    nb.external_input(dense_name, code)
+    nb.external_output("prob", code)
+    nb.arg("fuse_gemm_activation", int(fuse))
+    rng = np.random.default_rng(77)
+    weights = []
+    for li in range(len(layers) - 1):
+        k, n = layers[li], layers[li + 1]
+        w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+        b = (rng.standard_normal(n) * 0.1).astype(np.float32)
+        extra = ()
+        if acts[li] == "PRelu":
+            extra = (rng.uniform(0.1, 0.4, n).astype(np.float32), )
+        elif acts[li] == "Dice":
+            extra = ((rng.standard_normal(n) * 0.1).astype(np.float32), (rng.standard_normal(n) * 0.1).astype(np.float32),
+                     rng.uniform(0.5, 1.5, n).astype(np.float32))
+        weights.append((w, b, extra))
+        nb.constant("w%d" % li, w, dtype=code)
+        nb.constant("b%d" % li, b, dtype=code)
+        for j, e in enumerate(extra):
+            nb.constant("p%d_%d" % (li, j), e, dtype=code)
+    nb.op("Embedding", inputs, ["block"], embedding_config=pb.embedding_config_text(fgs, blocks),
+          **({"out_dtype": code} if dtype == np.float16 else {}))
+    nb.op("Concat", [dense_name, "block"], ["x0"], axis=1)
+    for li in range(len(layers) - 1):
+        last = li == len(layers) - 2
+        nb.op("Gemm", ["x%d" % li, "w%d" % li, "b%d" % li], ["h%d" % li])
+        out = "prob" if last else "x%d" % (li + 1)
+        if acts[li] == "Softmax":
+            nb.op("Softmax", ["h%d" % li], [out], axis=1)
+        elif acts[li] == "LeakyRelu":
+            nb.op("LeakyRelu", ["h%d" % li], [out], alpha=0.0)
+        elif acts[li] == "Sigmoid":
+            nb.op("Sigmoid", ["h%d" % li], [out])
+        else:
+            nb.op(acts[li], ["h%d" % li] + ["p%d_%d" % (li, j) for j in range(len(weights[li][2]))], [out])
+    return nb.text(), weights
+
+
+def _oracle_ctr(oracle, tables, fgs, blocks, inputs, dense, weights, acts, r):
+    """The same net on the CPU oracle; r rounds to the model's storage type after every op (identity for fp32)."""
+    outs = oracle.embedding_op({fg: (t, d) for fg, t, d in fgs}, blocks, inputs, tables)
+    h = np.concatenate([r(dense), r(outs[0])], axis=1)
+    for (w, b, extra), act in zip(weights, acts):
+        y = r(oracle.gemm_op(h, r(w), r(b)))
+        if act == "PRelu":
+            y = oracle.prelu(y, r(extra[0]))
+        elif act == "Dice":
+            y = oracle.dice(y, *[r(e) for e in extra])
+        elif act == "LeakyRelu":
+            y = oracle.leaky_relu(y, 0.0)
+        elif act == "Sigmoid":
+            y = oracle.sigmoid(y)
+        else:
+            y = oracle.softmax(y, 1)
+        h = r(y)
+    return h
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("acts", [("PRelu", "Dice", "Softmax"), ("LeakyRelu", "Sigmoid", "Softmax")])
+def test_ctr_model_from_qed_file_fused_and_unfused(pb, oracle, tmp_path, dtype, acts):
+    """Text tables -> Blaze_QuickEmbeddingBuild* -> Blaze_LoadSparseModelWeight -> Embedding + Concat + FC stack.
+    With and without folding the activations into the Gemm epilogue; both against the oracle."""
+    rng = np.random.default_rng(5)
+    fgs = [("101", "t_a", 8), ("102", "t_b", 16), ("103", "t_c", 8)]
+    blocks = [[dict(fg="101", udf=0), dict(fg="102", udf=1), dict(fg="103", udf=0)]]
+    tabs, oracle_tabs = {}, {}
+    for _, tname, dim in fgs:
+        n = int(rng.integers(30, 120))
+        keys = np.unique(rng.integers(-2**40, 2**40, n * 2, dtype=np.int64))[:n]
+        rows = (rng.standard_normal((n, dim)) * 0.5).astype(np.float32)
+        _write_csv(tmp_path / tname, keys, rows)
+        tabs[tname] = (keys, rows)
+    open(tmp_path / "meta", "w").write("".join(t + "\n" for _, t, _ in fgs))
+    qed = str(tmp_path / "model.qed")
+    pb.build_qed(str(tmp_path), "meta", qed, fp16=(dtype == np.float16))
+    for tname, (keys, rows) in tabs.items():
+        # what the builder parsed back from text (repr round-trips fp32 exactly), narrowed for the fp16 file
+        oracle_tabs[tname] = oracle.Table(rows.astype(np.float16) if dtype == np.float16 else rows, keys=keys)
+    batch, dense_dim = 37, 5
+    layers = (dense_dim + 32, 24, 16, 2)
+    inputs = {}
+    for fg, tname, _ in fgs:
+        seg = rng.integers(0, 6, batch).astype(np.int32)
+        pool = np.concatenate([tabs[tname][0], rng.integers(-2**40, 2**40, 10, dtype=np.int64)])
+        ids = rng.choice(pool, int(seg.sum()))
+        inputs[fg] = (ids.astype(np.int64), rng.standard_normal(ids.size).astype(np.float32), seg)
+    dense = rng.standard_normal((batch, dense_dim)).astype(np.float32)
+    r = (lambda x: np.asarray(x, np.float32).astype(np.float16).astype(np.float32)) if dtype == np.float16 else (lambda x: x)
+    results = []
+    for fuse in (True, False):
+        text, weights = _ctr_text(pb, fgs, blocks, dense_dim, layers, acts, dtype, fuse)
+        pm = pb.PredictorManager()
+        pm.load_sparse_model_weight(qed)
+        pm.load_model_from_string(text, True)
+        p = pm.create_predictor(1, 0)
+        assert p.list_input_names() == [n for fg, _, _ in fgs for n in (fg + ".ids", fg + ".values", fg + ".segments")] + ["dense"]
+        assert p.list_output_names() == ["prob"]
+        for fg, (ids, vals, seg) in inputs.items():
+            p.feed(fg + ".ids", ids)
+            p.feed(fg + ".values", vals)
+            p.feed(fg + ".segments", seg)
+        p.feed("dense", dense.astype(dtype))
+        print("case dtype=%s acts=%s fuse=%s" % (dtype.__name__, acts, fuse), flush=True)
+        p.forward()
+        got = p.output_asnumpy("prob")
+        assert got.shape == (batch, 2) and got.dtype == dtype
+        results.append(got.astype(np.float32))
+        p.forward()  # a second run reuses cached descriptors and packed weights
+        assert np.array_equal(p.output_asnumpy("prob").astype(np.float32), results[-1])
+    want = _oracle_ctr(oracle, oracle_tabs, fgs, blocks, inputs, dense, weights, acts, r)
+    tol = 2e-3 if dtype == np.float16 else 1e-5
+    for got in results:
+        np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
+    np.testing.assert_allclose(results[0], results[1], rtol=tol, atol=tol)
+    names = p.list_internal_names()
+    assert "w0" in names and p.internal_shape("w0") == (layers[0], layers[1])
+    np.testing.assert_array_equal(p.internal_asnumpy("w0"), weights[0][0].astype(dtype))
+
+
+def test_feed_and_forward_error_conventions(pb):
+    pm = pb.PredictorManager()
+    nb = pb.NetBuilder("err", device_type=1)
+    nb.external_input("x", pb.K_FLOAT)
+    nb.external_output("y")
+    nb.constant("w", np.ones((4, 3), np.float32))
+    nb.op("Gemm", ["x", "w"], ["y"])
+    pm.load_model_from_string(nb.text(), True)
+    p = pm.create_predictor(1, 0)
+    x = np.ones((2, 4), np.float32)
+    p.reshape_input("x", x.shape)
+    with pytest.raises(pb.BlazeError, match="Feed x failed"):
+        p.feed_raw("x", x, x.nbytes - 4)  # len must equal size * sizeof(dtype)
+    with pytest.raises(pb.BlazeError, match="Feed nope failed"):
+        p.feed_raw("nope", x, x.nbytes)
+    p.feed("x", x)
+    p.forward()
+    np.testing.assert_array_equal(p.output_asnumpy("y"), np.full((2, 3), 4, np.float32))
+    p.feed("x", np.ones((2, 5), np.float32))  # inner dimension no longer matches the weight
+    with pytest.raises(pb.BlazeError, match="Forward failed.*a_k=5 b_k=4"):
+        p.forward()
+    p.feed("x", x)  # the predictor stays usable after a failed run
+    p.forward()
+    np.testing.assert_array_equal(p.output_asnumpy("y"), np.full((2, 3), 4, np.float32))
+    p.register_observers(["profile"])
+    p.forward()
+    trace = json.loads(p.dump_observers()["profile"])
+    assert [e["name"].split(":")[0] for e in trace["traceEvents"]] == ["ConstantFill", "Gemm"]
+
+
+def test_embedding_operator_errors(pb):
+    cfg = pb.embedding_config_text([("101", "t", 4)], [[dict(fg="101", udf=0)]])
+
+    def build(cfg_text, store=True, inputs=("101.ids", "101.values", "101.segments")):
+        pm = pb.PredictorManager()
+        if store:
+            pm.add_table("t", np.ones((3, 4), np.float32))
+        nb = pb.NetBuilder("e", device_type=1)
+        for n, dt in zip(inputs, (pb.K_INT64, pb.K_FLOAT, pb.K_INT32)):
+            nb.external_input(n, dt)
+        nb.external_output("block")
+        nb.op("Embedding", list(inputs), ["block"], embedding_config=cfg_text)
+        pm.load_model_from_string(nb.text(), True)
+        return pm
+
+    with pytest.raises(pb.BlazeError, match="Parse embedding config failed"):
+        build("feature_group_config { feature_group : ").create_predictor(1, 0)
+    with pytest.raises(pb.BlazeError, match="feature group config not exist"):
+        build(pb.embedding_config_text([("101", "t", 4)], [[dict(fg="999", udf=0)]])).create_predictor(1, 0)
+    with pytest.raises(pb.BlazeError, match="id input name"):
+        build(cfg, inputs=("101.ids", "102.values", "101.segments")).create_predictor(1, 0)
+    p = build(cfg, store=False).create_predictor(1, 0)
+    p.feed("101.ids", np.array([0, 1], np.int64))
+    p.feed("101.values", np.ones(2, np.float32))
+    p.feed("101.segments", np.array([2], np.int32))
+    with pytest.raises(pb.BlazeError, match="no sparse puller"):
+        p.forward()
+    p = build(cfg).create_predictor(1, 0)
+    p.feed("101.ids", np.array([0, 1], np.int64))
+    p.feed("101.values", np.ones(3, np.float32))  # ids / values disagree
+    p.feed("101.segments", np.array([2], np.int32))
+    with pytest.raises(pb.BlazeError, match="id_blob->size"):
+        p.forward()
+    p.feed("101.values", np.array([2.0, 3.0], np.float32))
+    p.forward()
+    np.testing.assert_array_equal(p.output_asnumpy("block"), np.full((1, 4), 5.0, np.float32))
+    # unknown table name: the block stays zero
+    p = build(pb.embedding_config_text([("101", "unknown_table", 4)], [[dict(fg="101", udf=0)]])).create_predictor(1, 0)
+    p.feed("101.ids", np.array([0, 1], np.int64))
+    p.feed("101.values", np.ones(2, np.float32))
+    p.feed("101.segments", np.array([2], np.int32))
+    p.forward()
+    assert not p.output_asnumpy("block").any()

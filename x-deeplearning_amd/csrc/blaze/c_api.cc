@@ -1,0 +1,382 @@
+// c_api.cc -- the Blaze_* C ABI over Predictor / PredictorManager (include/blaze_c_api.h).
+#include "blaze_c_api.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "blaze/predictor.h"
+#include "blaze/qed_builder.h"
+#include "blaze/qed_store.h"
+
+using blaze::Predictor;
+using blaze::PredictorManager;
+
+namespace {
+
+// thread-local message buffer (the reference keeps 4 MB per thread; messages here are short)
+struct ErrorEntry {
+  char last_string[16384];
+};
+ErrorEntry* ErrorStore() {
+  static thread_local ErrorEntry e = {{0}};
+  return &e;
+}
+
+// thread-local storage behind the string arrays the List*/Param*/DumpObservers calls hand out
+struct StringVectorEntry {
+  std::vector<std::string> strings, values;
+  std::vector<const char*> names, keys, vals;
+};
+StringVectorEntry* StringStore() {
+  static thread_local StringVectorEntry e;
+  return &e;
+}
+
+int Fail(const char* what) {
+  const std::string& why = blaze::last_error_for_thread();
+  if (why.empty())
+    Blaze_SetLastErrorString("%s", what);
+  else
+    Blaze_SetLastErrorString("%s: %s", what, why.c_str());
+  blaze::last_error_for_thread().clear();
+  return -1;
+}
+
+int ReturnNames(const std::vector<std::string>& src, size_t* ndim, const char*** names) {
+  StringVectorEntry* e = StringStore();
+  e->strings = src;
+  e->names.clear();
+  for (const auto& s : e->strings) e->names.push_back(s.c_str());
+  *ndim = e->names.size();
+  *names = e->names.data();
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+void Blaze_GetLastErrorString(const char** msg) { *msg = ErrorStore()->last_string; }
+
+void Blaze_SetLastErrorString(const char* format, ...) {
+  va_list ap;
+  va_start(ap, format);
+  vsnprintf(ErrorStore()->last_string, sizeof(ErrorStore()->last_string), format, ap);
+  va_end(ap);
+}
+
+int Blaze_InitScheduler(int enable_batching, int max_batch_size, int batch_timeout_micros, int num_threads_for_cpu,
+                        int num_threads_for_cuda, int num_threads_for_pipe) {
+  if (!blaze::InitScheduler(enable_batching, max_batch_size, batch_timeout_micros, num_threads_for_cpu, num_threads_for_cuda,
+                            num_threads_for_pipe))
+    return Fail("InitScheduler Failed");
+  return 0;
+}
+
+int Blaze_PredictorManagerCreate(PredictorManagerHandle* handle) {
+  if (handle == nullptr) return Fail("Create PredictorManager Failed");
+  *handle = new PredictorManager();
+  return 0;
+}
+int Blaze_PredictorManagerDelete(PredictorManagerHandle handle) {
+  delete reinterpret_cast<PredictorManager*>(handle);
+  return 0;
+}
+int Blaze_PredictorManagerSetDataType(PredictorManagerHandle handle, int data_type) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr) return Fail("SetDataType: the predict manager is nullptr");
+  pm->SetDataType(static_cast<blaze::PredictDataType>(data_type));
+  return 0;
+}
+int Blaze_PredictorManagerSetRunMode(PredictorManagerHandle handle, const char* run_mode) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr) return Fail("SetRunMode: the predict manager is nullptr");
+  pm->SetRunMode(run_mode);
+  return 0;
+}
+int Blaze_LoadSparseModelWeight(PredictorManagerHandle handle, const char* file) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr || file == nullptr) return Fail("Load sparse model weight failed");
+  if (!pm->LoadSparseModelWeight(file)) return Fail("Load sparse model weight failed");
+  return 0;
+}
+int Blaze_PredictorManagerLoadModel(PredictorManagerHandle handle, const char* file, int optimization_pass) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr || file == nullptr) return Fail("Load blaze model failed");
+  if (!pm->LoadModel(file, optimization_pass != 0)) return Fail("Load blaze model failed");
+  return 0;
+}
+int Blaze_PredcitorManagerLoadModel(PredictorManagerHandle handle, const char* file, int optimization_pass) {
+  return Blaze_PredictorManagerLoadModel(handle, file, optimization_pass);
+}
+int Blaze_PredictorManagerLoadDeepNetModel(PredictorManagerHandle handle, const char* conf, const char* param, int optimization_pass) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr) return Fail("The predict manager is nullptr");
+  if (!pm->LoadDeepNetModel(conf, param, optimization_pass != 0)) return Fail("Load deepnet model failed");
+  return 0;
+}
+int Blaze_PredictorManagerLoadModelFromString(PredictorManagerHandle handle, const char* data, size_t len, int is_text) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr || data == nullptr) return Fail("The predict manager is nullptr");
+  try {
+    blaze::NetDef def;
+    if (is_text) {
+      blaze::ParseNetDefText(std::string(data, len), &def);
+    } else if (!blaze::ParseNetDefBinary(data, len, &def)) {
+      return Fail("malformed NetDef");
+    }
+    if (!pm->LoadNetDef(def)) return Fail("LoadNetDef failed");
+  } catch (std::exception& e) {
+    blaze::last_error_for_thread() = e.what();
+    return Fail("Load model from string failed");
+  }
+  return 0;
+}
+
+int Blaze_PredictorCreate(PredictorManagerHandle mgr, int device_type, int device_id, PredictorHandle* handle) {
+  auto* pm = reinterpret_cast<PredictorManager*>(mgr);
+  if (pm == nullptr || handle == nullptr) return Fail("Create Predictor Failed");
+  Predictor* p = pm->CreatePredictor(static_cast<blaze::PredictDeviceType>(device_type), device_id);
+  if (p == nullptr) return Fail("Create Predictor Failed");
+  *handle = p;
+  return 0;
+}
+int Blaze_PredictorDelete(PredictorHandle handle) {
+  if (handle == nullptr) return -1;
+  delete reinterpret_cast<Predictor*>(handle);
+  return 0;
+}
+
+int Blaze_PredictorReshapeInput(PredictorHandle handle, const char* name, const int* data, int num) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return Fail("The predictor is nullptr");
+  std::vector<size_t> shape;
+  for (int i = 0; i < num; ++i) shape.push_back((size_t)data[i]);
+  if (!p->ReshapeInput(name, shape)) {
+    Blaze_SetLastErrorString("Reshape input: %s failed", name);
+    return -1;
+  }
+  return 0;
+}
+int Blaze_PredictorFeed(PredictorHandle handle, const char* name, void* data, int len) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return Fail("The predictor is nullptr");
+  if (!p->Feed(name, data, (size_t)len)) {
+    Blaze_SetLastErrorString("Feed %s failed", name);
+    return -1;
+  }
+  return 0;
+}
+int Blaze_PredictorForward(PredictorHandle handle) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  if (!p->Forward()) return Fail("Forward failed");
+  return 0;
+}
+int Blaze_PredictorForwardN(PredictorHandle handle, int count) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  for (int i = 0; i < count; ++i)
+    if (!p->Forward()) return Fail("Forward failed");
+  return 0;
+}
+
+int Blaze_PredictorOutputShape(PredictorHandle handle, const char* name, size_t* ndim, size_t** nshape) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  try {
+    const std::vector<size_t>& shape = p->OutputShape(name);
+    *ndim = shape.size();
+    *nshape = const_cast<size_t*>(shape.data());
+  } catch (std::exception& e) {
+    Blaze_SetLastErrorString("%s", e.what());
+    return -1;
+  }
+  return 0;
+}
+int Blaze_PredictorOutputDataType(PredictorHandle handle, const char* name, int* data_type) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  *data_type = p->OutputDataType(name);
+  return *data_type < 0 ? Fail("not an output of the net") : 0;
+}
+int Blaze_PredictorOutput(PredictorHandle handle, const char* name, void* data, size_t len) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  size_t slen = 0;
+  void* dptr = nullptr;
+  if (!p->Output(name, &dptr, &slen)) {
+    Blaze_SetLastErrorString("Output %s failed", name);
+    return -1;
+  }
+  if (slen > len) {
+    Blaze_SetLastErrorString("Output %s needs %zu bytes, caller gave %zu", name, slen, len);
+    return -1;
+  }
+  memcpy(data, dptr, slen);
+  return 0;
+}
+
+int Blaze_PredictorParamName(PredictorHandle handle, size_t* ndim, const char*** name) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  return ReturnNames(p->ListInternalName(), ndim, name);
+}
+int Blaze_PredictorParamShape(PredictorHandle handle, const char* name, size_t* ndim, size_t** nshape) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  try {
+    const std::vector<size_t>& shape = p->InternalShape(name);
+    *ndim = shape.size();
+    *nshape = const_cast<size_t*>(shape.data());
+  } catch (std::exception& e) {
+    Blaze_SetLastErrorString("%s", e.what());
+    return -1;
+  }
+  return 0;
+}
+int Blaze_PredictorParamDataType(PredictorHandle handle, const char* name, int* data_type) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  *data_type = p->InternalDataType(name);
+  return *data_type < 0 ? Fail("not a parameter of the net") : 0;
+}
+int Blaze_PredictorParam(PredictorHandle handle, const char* name, void* data, size_t len) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  size_t slen = 0;
+  void* dptr = nullptr;
+  if (!p->InternalParam(name, &dptr, &slen) || slen > len) {
+    Blaze_SetLastErrorString("Param %s failed", name);
+    return -1;
+  }
+  memcpy(data, dptr, slen);
+  return 0;
+}
+
+int Blaze_PredictorListInputNames(PredictorHandle handle, size_t* ndim, const char*** names) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  return ReturnNames(p->ListInputName(), ndim, names);
+}
+int Blaze_PredictorListOutputNames(PredictorHandle handle, size_t* ndim, const char*** names) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  return ReturnNames(p->ListOutputName(), ndim, names);
+}
+
+int Blaze_PredictorRegisterObservers(PredictorHandle handle, size_t ndim, const char** names) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  std::vector<std::string> v;
+  for (size_t i = 0; i < ndim; ++i) v.push_back(names[i]);
+  p->RegisterObservers(v);
+  return 0;
+}
+int Blaze_PredictorDumpObservers(PredictorHandle handle, size_t* ndim, const char*** key, const char*** value) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  std::unordered_map<std::string, std::string> dump;
+  p->DumpObservers(&dump);
+  StringVectorEntry* e = StringStore();
+  e->strings.clear();
+  e->values.clear();
+  for (const auto& kv : dump) {
+    e->strings.push_back(kv.first);
+    e->values.push_back(kv.second);
+  }
+  e->keys.clear();
+  e->vals.clear();
+  for (size_t i = 0; i < e->strings.size(); ++i) {
+    e->keys.push_back(e->strings[i].c_str());
+    e->vals.push_back(e->values[i].c_str());
+  }
+  *ndim = e->keys.size();
+  *key = e->keys.data();
+  *value = e->vals.data();
+  return 0;
+}
+
+int Blaze_ConvertBlaze(const char*, const char*, int, int, int, int, const char**, const int*, const char*, int) {
+  Blaze_SetLastErrorString("Blaze_ConvertBlaze: the model importers are not part of this build");
+  return -1;
+}
+int Blaze_OptimizeBlaze(const char*, const char*, int) {
+  Blaze_SetLastErrorString("Blaze_OptimizeBlaze: the offline optimizer is not part of this build");
+  return -1;
+}
+int Blaze_QuickEmbeddingBuildFp32(const char* path, const char* meta, const char* output_file, int thread_num) {
+  std::string err;
+  if (!blaze::store::BuildQuickEmbedding(path, meta, output_file, blaze::kFloat, thread_num, &err)) {
+    Blaze_SetLastErrorString("QuickEmbeddingBuildFp32 failed: %s", err.c_str());
+    return -1;
+  }
+  return 0;
+}
+int Blaze_QuickEmbeddingBuildFp16(const char* path, const char* meta, const char* output_file, int thread_num) {
+  std::string err;
+  if (!blaze::store::BuildQuickEmbedding(path, meta, output_file, blaze::kFloat16, thread_num, &err)) {
+    Blaze_SetLastErrorString("QuickEmbeddingBuildFp16 failed: %s", err.c_str());
+    return -1;
+  }
+  return 0;
+}
+
+int Blaze_HipStoreAddTable(PredictorManagerHandle handle, const char* table_name, int value_type, int64_t rows, int dim,
+                           const void* rows_ptr, int on_device, const int64_t* keys, const float* scale) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr || table_name == nullptr) return Fail("The predict manager is nullptr");
+  try {
+    auto& puller = pm->EnsureSparsePuller("qed_hip_sparse_puller");
+    auto* qed = dynamic_cast<blaze::store::QedHipSparsePuller*>(puller.get());
+    if (qed == nullptr) return Fail("the manager's sparse puller is not the device store");
+    if (qed->AddTable(table_name, value_type, rows, dim, rows_ptr, on_device != 0, keys, scale) != blaze::store::kOK)
+      return Fail("AddTable failed");
+  } catch (std::exception& e) {
+    blaze::last_error_for_thread() = e.what();
+    return Fail("AddTable failed");
+  }
+  return 0;
+}
+
+int Blaze_ConvertNetDef(const char* in, size_t len, int in_is_text, int out_is_text, char* out, size_t cap, size_t* out_len) {
+  if (in == nullptr || out_len == nullptr) return Fail("null argument");
+  try {
+    blaze::NetDef def;
+    if (in_is_text) {
+      blaze::ParseNetDefText(std::string(in, len), &def);
+    } else if (!blaze::ParseNetDefBinary(in, len, &def)) {
+      return Fail("malformed NetDef");
+    }
+    std::string s;
+    if (out_is_text)
+      blaze::SerializeNetDefText(def, &s);
+    else
+      blaze::SerializeNetDefBinary(def, &s);
+    *out_len = s.size();
+    if (out != nullptr) {
+      if (cap < s.size()) return Fail("output buffer too small");
+      memcpy(out, s.data(), s.size());
+    }
+  } catch (std::exception& e) {
+    blaze::last_error_for_thread() = e.what();
+    return Fail("convert failed");
+  }
+  return 0;
+}
+
+int Blaze_PredictorInputDevicePtr(PredictorHandle handle, const char* name, void** ptr) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr || ptr == nullptr) return -1;
+  *ptr = p->InputDevicePtr(name);
+  return *ptr ? 0 : Fail("not an input of the net");
+}
+int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char* name, void** ptr) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr || ptr == nullptr) return -1;
+  *ptr = p->OutputDevicePtr(name);
+  return *ptr ? 0 : Fail("not an output of the net");
+}
+
+}  // extern "C"

@@ -1,0 +1,601 @@
+// dense_ops.cc -- Gemm, MatMul, FusedParallelGemm, FusedParallelMatMul on the accelerator.
+//
+// Operator-level behaviour (argument names and defaults, shape rules, error messages) follows the reference:
+//   Gemm                 blaze/operator/op/gemm_op.h:21-153       (transA, transB, alpha=1, beta=1; 2-D or 3-D A)
+//   MatMul               blaze/operator/op/matmul_op.h:21-171     (transA, transB, from_deepnet; numpy broadcast, outer rank <= 1)
+//   FusedParallelGemm    blaze/operator/fused_op/fused_parallel_gemm_op.h:32-184
+//   FusedParallelMatMul  blaze/operator/fused_op/fused_parallel_matmul_op.h:24-200
+// The arithmetic goes to the kernel layer (include/blaze_hip.h): an FC is one bz_fc_fused launch (MFMA, fp32
+// accumulate, bias and -- when the following activation operator was folded in -- activation in the epilogue);
+// batched products are bz_gemm_strided_batched.
+#include "blaze/graph.h"
+#include "blaze/operator.h"
+#include "blaze_hip.h"
+
+namespace blaze {
+
+namespace {
+
+int BzType(int data_type) {
+  switch (data_type) {
+    case kFloat: return BZ_F32;
+    case kFloat16: return BZ_F16;
+    default: BLAZE_THROW("Unsupported type: ", data_type);
+  }
+}
+
+// A device buffer derived from a blob (packed weight, fp32 copy of a parameter), rebuilt when the blob moves.
+struct Derived {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  const Blob* src = nullptr;
+  uint64_t version = ~0ull;
+  ~Derived() {
+    if (ptr) (void)hipFree(ptr);
+  }
+  bool Stale(const Blob* b) const { return ptr == nullptr || src != b || version != b->version(); }
+  void Resize(size_t n) {
+    if (n > bytes) {
+      if (ptr) (void)hipFree(ptr);
+      HIP_CHECK(hipMalloc(&ptr, n));
+      bytes = n;
+    }
+  }
+  void Mark(const Blob* b) {
+    src = b;
+    version = b->version();
+  }
+};
+
+// fp32 view of a parameter blob (bias, PRelu slope, Dice gamma/mean/var): fp32 blobs are used in place, fp16
+// ones are widened once on the device (exact) and cached.  Constant blobs are immutable after load; for other
+// producers the copy is redone every run.
+const float* AsFloatParam(Blob* b, Derived* cache, bool constant, hipStream_t st) {
+  if (b->data_type() == kFloat) return b->as<float>();
+  BLAZE_CONDITION_THROW(b->data_type() == kFloat16, "Unsupported type: ", b->data_type());
+  if (!constant || cache->Stale(b)) {
+    const int n = (int)b->size();
+    const int64_t ld = (n + 7) / 8 * 8;
+    cache->Resize(ld * sizeof(float));
+    BZ_CHECK(bz_fc_pack_weight(b->data(), BZ_F16, 1, n, 1, cache->ptr, BZ_F32, ld, st));
+    cache->Mark(b);
+  }
+  return (const float*)cache->ptr;
+}
+
+// One FC:  y[M,N] = act(alpha * op(A) * op(B) + beta * bias) through bz_fc_fused.
+struct FcCall {
+  // operands
+  const void* a = nullptr;
+  int a_rows = 0, a_cols = 0;  // as stored
+  bool trans_a = false;
+  Blob* b_blob = nullptr;
+  const void* b = nullptr;     // b_blob->data() + offset
+  int b_rows = 0, b_cols = 0;  // as stored
+  bool trans_b = false;
+  bool b_constant = false;
+  int dtype = kFloat;
+  const float* bias = nullptr;
+  int bias_rows = 0;
+  void* y = nullptr;
+  int y_dtype = kFloat;
+  float alpha = 1.f, beta = 1.f;
+  // epilogue
+  int act = BZ_ACT_NONE;
+  const float *p0 = nullptr, *p1 = nullptr, *p2 = nullptr;
+  int act_size = 0;
+  bool dice_nosqrt = false;
+  float act_alpha = 0.f;
+};
+
+void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st) {
+  const int M = c.trans_a ? c.a_cols : c.a_rows;
+  const int K = c.trans_a ? c.a_rows : c.a_cols;
+  const int N = c.trans_b ? c.b_rows : c.b_cols;
+  const int bt = BzType(c.dtype);
+  const int es = (int)DataTypeSize(c.dtype);
+  const int chunk = 16 / es;
+  bz_fc_desc d;
+  memset(&d, 0, sizeof(d));
+  // A: row major [M,K] is used in place; a transposed A is re-laid out K-contiguous first
+  if (c.trans_a) {
+    const int64_t lda = (K + 7) / 8 * 8;
+    packed_a->Resize((size_t)M * lda * es);
+    BZ_CHECK(bz_fc_pack_weight(c.a, bt, 0, K, M, packed_a->ptr, bt, lda, st));
+    d.a = packed_a->ptr;
+    d.lda = lda;
+  } else {
+    d.a = c.a;
+    d.lda = K;
+  }
+  // W: [N,K] with aligned rows is used in place, anything else is packed (once for constants)
+  if (c.trans_b && (K % chunk == 0) && ((uintptr_t)c.b % 16 == 0)) {
+    d.w = c.b;
+    d.ldw = K;
+  } else {
+    const int64_t ldw = (K + 7) / 8 * 8;
+    const bool redo = !c.b_constant || packed_b->Stale(c.b_blob) || packed_b->bytes < (size_t)N * ldw * es;
+    if (redo) {
+      packed_b->Resize((size_t)N * ldw * es);
+      BZ_CHECK(bz_fc_pack_weight(c.b, bt, c.trans_b ? 1 : 0, K, N, packed_b->ptr, bt, ldw, st));
+      packed_b->Mark(c.b_blob);
+    }
+    d.w = packed_b->ptr;
+    d.ldw = ldw;
+  }
+  d.bias = c.bias;
+  d.bias_rows = c.bias_rows;
+  d.y = c.y;
+  d.ldy = N;
+  d.m = M;
+  d.n = N;
+  d.k = K;
+  d.in_dtype = bt;
+  d.out_dtype = BzType(c.y_dtype);
+  d.act = c.act;
+  d.act_p0 = c.p0;
+  d.act_p1 = c.p1;
+  d.act_p2 = c.p2;
+  d.act_size = c.act_size;
+  d.dice_nosqrt = c.dice_nosqrt ? 1 : 0;
+  d.alpha = c.alpha;
+  d.beta = c.bias ? c.beta : 0.f;
+  d.act_alpha = c.act_alpha;
+  BZ_CHECK(bz_fc_fused(&d, st));
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------ Gemm
+template <class Context>
+class GemmOp : public Operator<Context>, public FusableProducer {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+
+  GemmOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
+    transa_ = OperatorBase::GetSingleArgument<bool>("transA", false);
+    transb_ = OperatorBase::GetSingleArgument<bool>("transB", false);
+    alpha_ = OperatorBase::GetSingleArgument<float>("alpha", 1.0);
+    beta_ = OperatorBase::GetSingleArgument<float>("beta", 1.0);
+    b_constant_ = workspace->HasConstantBlob(def.input(1));
+    for (int i = 2; i < def.input_size(); ++i) c_constant_ = workspace->HasConstantBlob(def.input(i));
+  }
+
+  // Fold the activation operator that consumes this Gemm's output into the epilogue.  Only shapes the epilogue
+  // expresses exactly are accepted: per-column parameters of size N (or a single PRelu slope).
+  bool TryFuse(OperatorBase* consumer) override {
+    if (!b_constant_ || this->Input(1)->shape().size() != 2) return false;
+    const int N = (int)(transb_ ? this->Input(1)->shape()[0] : this->Input(1)->shape()[1]);
+    const std::string& t = consumer->type();
+    auto param_ok = [&](int idx, bool scalar_ok) {
+      Blob* p = consumer->Input(idx);
+      if (!this->workspace_->HasConstantBlob(consumer->operator_def().input(idx))) return false;
+      return (int)p->size() == N || (scalar_ok && p->size() == 1);
+    };
+    if (t == "PRelu") {
+      if (!param_ok(1, true)) return false;
+      fused_act_ = BZ_ACT_PRELU;
+    } else if (t == "Dice") {
+      if (!param_ok(1, false) || !param_ok(2, false) || !param_ok(3, false)) return false;
+      fused_act_ = BZ_ACT_DICE;
+      fused_nosqrt_ = ArgumentHelper::GetSingle<bool>(consumer->operator_def().arg(), "nosqrt", false);
+    } else if (t == "LeakyRelu") {
+      fused_act_ = BZ_ACT_LEAKY_RELU;
+      fused_alpha_ = ArgumentHelper::GetSingle<float>(consumer->operator_def().arg(), "alpha", 0.01f);
+    } else if (t == "Sigmoid") {
+      fused_act_ = BZ_ACT_SIGMOID;
+    } else if (t == "Softmax") {
+      const size_t axis = ArgumentHelper::GetSingle<size_t>(consumer->operator_def().arg(), "axis", 1);
+      if (N > 8 || axis != 1 || this->Input(0)->shape().size() == 3) return false;
+      fused_act_ = BZ_ACT_SOFTMAX;
+    } else {
+      return false;
+    }
+    fused_ = consumer;
+    return true;
+  }
+
+  bool RunOnDevice() override {
+    CheckValid();
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->InputSize() > 2 ? this->Input(2) : nullptr;
+    Blob* y = fused_ ? fused_->Output(0) : this->Output(0);
+    const auto& a_shape = a->shape();
+    const auto& b_shape = b->shape();
+    TIndex M = a_shape.size() == 3 ? a_shape[1] : a_shape[0];
+    TIndex K = a_shape.size() == 3 ? a_shape[2] : a_shape[1];
+    if (transa_) std::swap(M, K);
+    const TIndex N = transb_ ? b_shape[0] : b_shape[1];
+    TIndex rows = M;  // rows of the one 2-D product that realises the op
+    if (a_shape.size() == 3) {
+      y->Reshape({a_shape[0], M, N});
+      // M == 1 collapses to a 2-D Gemm with M = batch (gemm_op.h:54-55); M > 1 with a shared weight is the
+      // strided-batched case (stride_b = 0, :77-91), which over contiguous slices is again one 2-D product
+      BLAZE_CONDITION_THROW(!transa_ || a_shape[0] == 1, "3-D Gemm with transA is not supported on this device");
+      rows = a_shape[0] * M;
+    } else {
+      y->Reshape({M, N});
+    }
+    hipStream_t st = context_.hip_stream();
+    FcCall call;
+    call.a = a->data();
+    call.a_rows = transa_ ? (int)K : (int)rows;
+    call.a_cols = transa_ ? (int)rows : (int)K;
+    call.trans_a = transa_;
+    call.b_blob = b;
+    call.b = b->data();
+    call.b_rows = (int)b_shape[0];
+    call.b_cols = (int)b_shape[1];
+    call.trans_b = transb_;
+    call.b_constant = b_constant_;
+    call.dtype = a->data_type();
+    call.y = y->data();
+    call.y_dtype = y->data_type();
+    call.alpha = alpha_;
+    call.beta = beta_;
+    if (c != nullptr) {
+      call.bias = AsFloatParam(c, &bias_f32_, c_constant_, st);
+      if (c->shape().size() == 2 && c->shape()[0] != 1) {
+        // a full [M,N] bias; under a 3-D A it repeats for every batch slice (DimEqualBroadcastAssign)
+        BLAZE_CONDITION_THROW(a_shape.size() != 3 || a_shape[0] == 1, "3-D Gemm with an [M,N] bias is not supported on this device");
+        call.bias_rows = (int)rows;
+      } else {
+        call.bias_rows = 1;
+      }
+    }
+    if (fused_) {
+      call.act = fused_act_;
+      call.dice_nosqrt = fused_nosqrt_;
+      call.act_alpha = fused_alpha_;
+      if (fused_act_ == BZ_ACT_PRELU) {
+        call.p0 = AsFloatParam(fused_->Input(1), &p_f32_[0], true, st);
+        call.act_size = (int)fused_->Input(1)->size();
+      } else if (fused_act_ == BZ_ACT_DICE) {
+        for (int i = 0; i < 3; ++i) {
+          const float* p = AsFloatParam(fused_->Input(1 + i), &p_f32_[i], true, st);
+          (i == 0 ? call.p0 : (i == 1 ? call.p1 : call.p2)) = p;
+        }
+        call.act_size = (int)N;
+      }
+    }
+    RunFc(call, &packed_b_, &packed_a_, st);
+    return true;
+  }
+
+ protected:
+  void CheckValid() {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->InputSize() > 2 ? this->Input(2) : nullptr;
+    BLAZE_CONDITION_THROW(a->shape().size() == 2 || a->shape().size() == 3, "a->shape.size()=", a->shape().size());
+    BLAZE_CONDITION_THROW(b->shape().size() == 2, "b->shape.size()=", b->shape().size(), " ", this->def_.DebugString());
+    if (c != nullptr) BLAZE_CONDITION_THROW(c->shape().size() <= 2, "c->shape().size()=", c->shape().size());
+    BLAZE_CONDITION_THROW(a->data_type() == b->data_type(), "a->data_type()=", a->data_type(), " b->data_type()=", b->data_type());
+    const auto& a_shape = a->shape();
+    const auto& b_shape = b->shape();
+    TIndex a_m = a_shape.size() == 3 ? a_shape[1] : a_shape[0];
+    TIndex a_k = a_shape.size() == 3 ? a_shape[2] : a_shape[1];
+    if (transa_) std::swap(a_m, a_k);
+    TIndex b_k = b_shape[0], b_n = b_shape[1];
+    if (transb_) std::swap(b_k, b_n);
+    BLAZE_CONDITION_THROW(a_k == b_k, "a_k=", a_k, " b_k=", b_k, " ", this->def_.DebugString());
+    if (c != nullptr) {
+      if (c->shape().size() == 2) {
+        BLAZE_CONDITION_THROW(a_m == c->shape()[0], "a_m=", a_m, " c->shape()[0]=", c->shape()[0]);
+        BLAZE_CONDITION_THROW(b_n == c->shape()[1], "b_n=", b_n, " c->shape()[1]=", c->shape()[1]);
+      } else {
+        BLAZE_CONDITION_THROW(b_n == c->shape()[0], "b_n=", b_n, " c->shape()[0]=", c->shape()[0]);
+      }
+    }
+  }
+
+  float alpha_, beta_;
+  bool transa_, transb_;
+  bool b_constant_ = false, c_constant_ = false;
+  Derived packed_b_, packed_a_, bias_f32_, p_f32_[3];
+  OperatorBase* fused_ = nullptr;
+  int fused_act_ = BZ_ACT_NONE;
+  bool fused_nosqrt_ = false;
+  float fused_alpha_ = 0.f;
+};
+
+REGISTER_HIP_OPERATOR(Gemm, GemmOp<HIPContext>);
+
+// Input: A, B, [C]  Output: Y
+OPERATOR_SCHEMA(Gemm)
+    .NumInputs(2, 3)
+    .NumOutputs(1)
+    .IdenticalTypeOfInput(0)
+    .SetDoc("General Matrix multiplication: Y = alpha * op(A) * op(B) + beta * C, with a 2-D or 3-D A");
+
+// ------------------------------------------------------------------------------------------ batched helpers
+namespace {
+
+void StridedBatched(bool ta, bool tb, int M, int N, int K, float alpha, const void* A, int64_t sa, const void* B, int64_t sb,
+                    float beta, void* C, int64_t sc, int batch, int data_type, hipStream_t st) {
+  bz_bgemm_desc d;
+  memset(&d, 0, sizeof(d));
+  d.a = A;
+  d.b = B;
+  d.c = C;
+  d.stride_a = sa;
+  d.stride_b = sb;
+  d.stride_c = sc;
+  d.trans_a = ta;
+  d.trans_b = tb;
+  d.m = M;
+  d.n = N;
+  d.k = K;
+  d.batch = batch;
+  d.dtype = BzType(data_type);
+  d.alpha = alpha;
+  d.beta = beta;
+  BZ_CHECK(bz_gemm_strided_batched(&d, st));
+}
+
+TIndex Prod(const std::vector<TIndex>& v) {
+  TIndex p = 1;
+  for (auto d : v) p *= d;
+  return p;
+}
+
+// ULF batchdot compatibility: 2-D B [b,k] -> [b,1,k], 2-D A [b,k] -> [b,k,1] (matmul_op.h:147-165)
+void UlfCompatibleReshape(Blob* a, Blob* b) {
+  if (b->shape().size() == 2) b->Reshape({b->shape()[0], 1, b->shape()[1]});
+  if (a->shape().size() == 2) a->Reshape({a->shape()[0], a->shape()[1], 1});
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------ MatMul
+template <class Context>
+class MatMulOp : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  MatMulOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
+    transa_ = OperatorBase::GetSingleArgument<bool>("transA", false);
+    transb_ = OperatorBase::GetSingleArgument<bool>("transB", false);
+    from_deepnet_ = OperatorBase::GetSingleArgument<bool>("from_deepnet", false);
+  }
+
+  bool RunOnDevice() override {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->Output(0);
+    Setup();
+    std::vector<TIndex> a_outer(a->shape().begin(), a->shape().end() - 2);
+    std::vector<TIndex> b_outer(b->shape().begin(), b->shape().end() - 2);
+    int M = (int)a->shape()[a->shape().size() - 2], K = (int)a->shape()[a->shape().size() - 1];
+    if (transa_) std::swap(M, K);
+    const int N = (int)(transb_ ? b->shape()[b->shape().size() - 2] : b->shape()[b->shape().size() - 1]);
+    // BroadcastGemm is instantiated for outer rank <= 1 only (math/broadcast.h:236-246)
+    BLAZE_CONDITION_THROW(a_outer.size() <= 1 && b_outer.size() <= 1, "Not Implemented BroadcastGemm!");
+    const TIndex a_size = Prod(a_outer), b_size = Prod(b_outer);
+    if (a_size != 1 && b_size != 1) BLAZE_CONDITION_THROW(a_size == b_size, "a_size=", a_size, " b_size=", b_size);
+    // BroadcastGemm_NxN (math/broadcast.h:157-222): a side with one matrix is shared by the whole batch
+    StridedBatched(transa_, transb_, M, N, K, 1.0f, a->data(), a_size == 1 ? 0 : (int64_t)M * K, b->data(),
+                   b_size == 1 ? 0 : (int64_t)K * N, 0.f, c->data(), (int64_t)M * N, (int)std::max(a_size, b_size),
+                   a->data_type(), context_.hip_stream());
+    return true;
+  }
+
+ protected:
+  void Setup() {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->Output(0);
+    if (from_deepnet_) UlfCompatibleReshape(a, b);
+    BLAZE_CONDITION_THROW(a->shape().size() >= 2, "a->shape().size()=", a->shape().size());
+    BLAZE_CONDITION_THROW(b->shape().size() >= 2, "b->shape().size()=", b->shape().size());
+    BLAZE_CONDITION_THROW(a->data_type() == b->data_type(), "a->data_type()=", a->data_type(), " b->data_type()=", b->data_type());
+    Blob *min = a, *max = b;
+    if (a->shape().size() > b->shape().size()) std::swap(min, max);
+    std::vector<TIndex> shape = max->shape();
+    const size_t off = max->shape().size() - min->shape().size();
+    for (size_t k = 0; k + 2 < min->shape().size(); ++k) {
+      const TIndex dim_min = min->shape()[k], dim_max = max->shape()[off + k];
+      BLAZE_CONDITION_THROW(dim_min == dim_max || dim_min == 1 || dim_max == 1, "dim_min=", dim_min, " dim_max=", dim_max,
+                            " op=", this->def_.name());
+      if (dim_max == 1) shape[off + k] = dim_min;
+    }
+    const size_t ar = a->shape().size(), br = b->shape().size();
+    const TIndex a_k = transa_ ? a->shape()[ar - 2] : a->shape()[ar - 1];
+    const TIndex b_k = transb_ ? b->shape()[br - 1] : b->shape()[br - 2];
+    BLAZE_CONDITION_THROW(a_k == b_k, "a_k=", a_k, " b_k=", b_k);
+    shape[shape.size() - 2] = transa_ ? a->shape()[ar - 1] : a->shape()[ar - 2];
+    shape[shape.size() - 1] = transb_ ? b->shape()[br - 2] : b->shape()[br - 1];
+    c->Reshape(shape);
+  }
+  bool transa_, transb_, from_deepnet_;
+};
+
+REGISTER_HIP_OPERATOR(MatMul, MatMulOp<HIPContext>);
+
+OPERATOR_SCHEMA(MatMul).NumInputs(2).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("Matrix product that behaves like numpy.matmul");
+
+// ------------------------------------------------------------------------------------------ FusedParallelGemm
+template <class Context>
+class FusedParallelGemmOp : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  FusedParallelGemmOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
+    parallel_num_ = OperatorBase::GetSingleArgument<int>("parallel_num", 2);
+    transa_ = OperatorBase::GetSingleArgument<bool>("transA", false);
+    transb_ = OperatorBase::GetSingleArgument<bool>("transB", false);
+    alpha_ = OperatorBase::GetSingleArgument<float>("alpha", 1.0);
+    beta_ = OperatorBase::GetSingleArgument<float>("beta", 1.0);
+    BLAZE_CONDITION_THROW(parallel_num_ > 0, "parallel_num=", parallel_num_);
+    b_constant_ = workspace->HasConstantBlob(def.input(1));
+    if (def.input_size() > 2) c_constant_ = workspace->HasConstantBlob(def.input(2));
+    packed_b_.resize(parallel_num_);
+  }
+
+  bool RunOnDevice() override {
+    CheckValid();
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->InputSize() > 2 ? this->Input(2) : nullptr;
+    Blob* y = this->Output(0);
+    const auto& a_shape = a->shape();
+    const auto& b_shape = b->shape();
+    const int P = parallel_num_;
+    TIndex M = a_shape.size() == 3 ? a_shape[1] : a_shape[0];
+    TIndex K = a_shape.size() == 3 ? a_shape[2] : a_shape[1];
+    if (transa_) std::swap(M, K);
+    const TIndex N = transb_ ? b_shape[0] / P : b_shape[1];
+    TIndex rows = M;
+    if (a_shape.size() == 3) {
+      y->Reshape({a_shape[0] * P, M, N});
+      BLAZE_CONDITION_THROW(!transa_ || a_shape[0] == 1, "3-D FusedParallelGemm with transA is not supported on this device");
+      rows = a_shape[0] * M;
+    } else {
+      y->Reshape({M * P, N});
+    }
+    hipStream_t st = context_.hip_stream();
+    const float* bias = c ? AsFloatParam(c, &bias_f32_, c_constant_, st) : nullptr;
+    const bool full_bias = c && c->shape().size() == 2 && c->shape()[0] != (TIndex)P;
+    if (full_bias)
+      BLAZE_CONDITION_THROW(a_shape.size() != 3 || a_shape[0] == 1, "3-D FusedParallelGemm with a [P*M,N] bias is not supported on this device");
+    const size_t es = DataTypeSize(a->data_type());
+    // the P sibling FCs share the input; slice p owns weights [K,N] (or [N,K]), bias and output slice p
+    for (int p = 0; p < P; ++p) {
+      FcCall call;
+      call.a = a->data();
+      call.a_rows = transa_ ? (int)K : (int)rows;
+      call.a_cols = transa_ ? (int)rows : (int)K;
+      call.trans_a = transa_;
+      call.b_blob = b;
+      call.b = (const char*)b->data() + (size_t)p * K * N * es;
+      call.b_rows = transb_ ? (int)N : (int)K;
+      call.b_cols = transb_ ? (int)K : (int)N;
+      call.trans_b = transb_;
+      call.b_constant = b_constant_;
+      call.dtype = a->data_type();
+      call.y = (char*)y->data() + (size_t)p * rows * N * DataTypeSize(y->data_type());
+      call.y_dtype = y->data_type();
+      call.alpha = alpha_;
+      call.beta = beta_;
+      if (bias) {
+        call.bias = bias + (full_bias ? (size_t)p * rows * N : (size_t)p * N);
+        call.bias_rows = full_bias ? (int)rows : 1;
+      }
+      RunFc(call, &packed_b_[p], &packed_a_, st);
+    }
+    return true;
+  }
+
+ protected:
+  void CheckValid() {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->InputSize() > 2 ? this->Input(2) : nullptr;
+    BLAZE_CONDITION_THROW(a->shape().size() == 2 || a->shape().size() == 3, "a->shape().size()=", a->shape().size());
+    BLAZE_CONDITION_THROW(b->shape().size() == 2, "b->shape().size()=", b->shape().size());
+    if (c != nullptr) BLAZE_CONDITION_THROW(c->shape().size() <= 2, "c->shape().size()=", c->shape().size());
+    const auto& a_shape = a->shape();
+    const auto& b_shape = b->shape();
+    TIndex a_m = a_shape.size() == 3 ? a_shape[1] : a_shape[0];
+    TIndex a_k = a_shape.size() == 3 ? a_shape[2] : a_shape[1];
+    if (transa_) std::swap(a_m, a_k);
+    // the P weights are stacked on dim 0: [P*K, N], or [P*N, K] under transB
+    TIndex b_k = transb_ ? b_shape[1] : b_shape[0] / parallel_num_;
+    TIndex b_n = transb_ ? b_shape[0] / parallel_num_ : b_shape[1];
+    BLAZE_CONDITION_THROW(a_k == b_k, "a_k=", a_k, " b_k=", b_k);
+    if (c != nullptr) {
+      if (c->shape().size() == 2) {
+        BLAZE_CONDITION_THROW(a_m == c->shape()[0] / parallel_num_, "a_m=", a_m, " c->shape()[0]=", c->shape()[0],
+                              " parallel_num_=", parallel_num_);
+        BLAZE_CONDITION_THROW(b_n == c->shape()[1], "b_n=", b_n, " c->shape()[1]=", c->shape()[1]);
+      } else {
+        BLAZE_CONDITION_THROW(b_n == c->shape()[0] / parallel_num_, "b_n=", b_n, " c->shape()[0]=", c->shape()[0]);
+      }
+    }
+  }
+  int parallel_num_;
+  bool transa_, transb_;
+  float alpha_, beta_;
+  bool b_constant_ = false, c_constant_ = false;
+  std::vector<Derived> packed_b_;
+  Derived packed_a_, bias_f32_;
+};
+
+REGISTER_HIP_OPERATOR(FusedParallelGemm, FusedParallelGemmOp<HIPContext>);
+
+OPERATOR_SCHEMA(FusedParallelGemm)
+    .NumInputs(2, 3)
+    .NumOutputs(1)
+    .IdenticalTypeOfInput(0)
+    .SetDoc("parallel_num sibling Gemms that share one input, weights stacked on dim 0");
+
+// ------------------------------------------------------------------------------------------ FusedParallelMatMul
+template <class Context>
+class FusedParallelMatMulOp : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  FusedParallelMatMulOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
+    parallel_num_ = OperatorBase::GetSingleArgument<int>("parallel_num", 2);
+    from_deepnet_ = OperatorBase::GetSingleArgument<bool>("from_deepnet", false);
+    transa_ = OperatorBase::GetSingleArgument<bool>("transA", false);
+    transb_ = OperatorBase::GetSingleArgument<bool>("transB", false);
+    BLAZE_CONDITION_THROW(parallel_num_ > 0, "parallel_num=", parallel_num_);
+  }
+
+  bool RunOnDevice() override {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->Output(0);
+    if (from_deepnet_) UlfCompatibleReshape(a, b);
+    BLAZE_CONDITION_THROW(a->shape().size() >= 2, "a->shape().size()=", a->shape().size());
+    BLAZE_CONDITION_THROW(b->shape().size() >= 2, "b->shape().size()=", b->shape().size());
+    std::vector<TIndex> a_shape = a->shape(), b_shape = b->shape();
+    const int P = parallel_num_;
+    BLAZE_CONDITION_THROW(a_shape[0] % P == 0, "a_shape[0]=", a_shape[0], " parallel_num=", P);
+    BLAZE_CONDITION_THROW(b_shape[0] % P == 0, "b_shape[0]=", b_shape[0], " parallel_num=", P);
+    a_shape[0] /= P;
+    b_shape[0] /= P;
+    int M = (int)a_shape[a_shape.size() - 2], K = (int)a_shape[a_shape.size() - 1];
+    if (transa_) std::swap(M, K);
+    const int N = (int)(transb_ ? b_shape[b_shape.size() - 2] : b_shape[b_shape.size() - 1]);
+    const TIndex b_k = transb_ ? b_shape[b_shape.size() - 1] : b_shape[b_shape.size() - 2];
+    BLAZE_CONDITION_THROW((TIndex)K == b_k, "a_k=", K, " b_k=", b_k);
+    a_shape.resize(a_shape.size() - 2);
+    b_shape.resize(b_shape.size() - 2);
+    BLAZE_CONDITION_THROW(a_shape.size() <= 1 && b_shape.size() <= 1, "Not Implemented BatchedBroadcastGemm!");
+    const TIndex a_size = Prod(a_shape), b_size = Prod(b_shape);
+    if (a_size != 1 && b_size != 1) BLAZE_CONDITION_THROW(a_size == b_size, "a_size=", a_size, " b_size=", b_size);
+    BLAZE_CONDITION_THROW(a_size == b_size || a_size == 1 || b_size == 1, "a_size=", a_size, " b_size=", b_size);
+    const TIndex cb = std::max(a_size, b_size);
+    c->Reshape({(TIndex)P * cb, (TIndex)M, (TIndex)N});
+    const size_t es = DataTypeSize(a->data_type());
+    hipStream_t st = context_.hip_stream();
+    if (a_size == b_size) {
+      // one batch over every slice of every parallel group (math/broadcast.h:282-317)
+      StridedBatched(transa_, transb_, M, N, K, 1.f, a->data(), (int64_t)M * K, b->data(), (int64_t)K * N, 0.f, c->data(),
+                     (int64_t)M * N, (int)(a_size * P), a->data_type(), st);
+    } else {
+      // per parallel group, the single matrix of one side is shared by the group's batch (:340-378; the
+      // N == 1 shortcut of :319-338 is the same products computed through a transposed Gemm)
+      for (int p = 0; p < P; ++p)
+        StridedBatched(transa_, transb_, M, N, K, 1.f, (const char*)a->data() + (size_t)p * a_size * M * K * es,
+                       a_size == 1 ? 0 : (int64_t)M * K, (const char*)b->data() + (size_t)p * b_size * K * N * es,
+                       b_size == 1 ? 0 : (int64_t)K * N, 0.f, (char*)c->data() + (size_t)p * cb * M * N * es, (int64_t)M * N,
+                       (int)cb, a->data_type(), st);
+    }
+    return true;
+  }
+
+ protected:
+  bool transa_, transb_, from_deepnet_;
+  int parallel_num_;
+};
+
+REGISTER_HIP_OPERATOR(FusedParallelMatMul, FusedParallelMatMulOp<HIPContext>);
+
+OPERATOR_SCHEMA(FusedParallelMatMul)
+    .NumInputs(2)
+    .NumOutputs(1)
+    .IdenticalTypeOfInput(0)
+    .SetDoc("parallel_num sibling MatMuls stacked on dim 0");
+
+}  // namespace blaze

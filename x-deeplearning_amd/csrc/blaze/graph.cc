@@ -1,0 +1,226 @@
+#include "blaze/graph.h"
+
+#include <stdlib.h>
+
+#include <chrono>
+#include <fstream>
+
+namespace blaze {
+
+// ------------------------------------------------------------------------------------------ workspace
+Workspace::~Workspace() {
+  std::set<Blob*> removed;
+  for (auto& it : blob_map_) removed.insert(it.second);
+  for (auto* b : blob_recycle_bins_) removed.insert(b);
+  for (auto* b : removed) delete b;
+  for (auto& it : constant_fill_blob_map_) delete it.second;
+}
+
+Blob* Workspace::CreateConstantBlob(const std::string& name, const DeviceOption& device_option, bool* newblob) {
+  auto it = constant_fill_blob_map_.find(name);
+  if (it == constant_fill_blob_map_.end()) {
+    it = constant_fill_blob_map_.emplace(name, new Blob(device_option)).first;
+    if (newblob) *newblob = true;
+  } else if (newblob) {
+    *newblob = false;
+  }
+  return it->second;
+}
+
+Blob* Workspace::CreateBlob(const std::string& name, const DeviceOption& device_option, bool* newblob) {
+  auto c = constant_fill_blob_map_.find(name);
+  if (c != constant_fill_blob_map_.end()) {
+    if (newblob) *newblob = false;
+    return c->second;
+  }
+  auto it = blob_map_.find(name);
+  if (it == blob_map_.end()) {
+    it = blob_map_.emplace(name, new Blob(device_option)).first;
+    if (newblob) *newblob = true;
+  } else if (newblob) {
+    *newblob = false;
+  }
+  return it->second;
+}
+
+void Workspace::Init(const NetDef& net_def) {
+  std::unique_lock<std::mutex> lock(mutex_);
+  net_def_.reset(new NetDef(net_def));
+  input_data_type_map_.clear();
+  input_info_map_.clear();
+  for (const auto& in : net_def_->external_input_) {
+    input_data_type_map_[in.name()] = in.dtype();
+    input_info_map_[in.name()] = in;
+  }
+}
+
+void Workspace::RecycleBlobMap() {
+  for (auto& it : blob_map_) blob_recycle_bins_.insert(it.second);
+  blob_map_.clear();
+}
+
+std::shared_ptr<Net> Workspace::CreateNet() {
+  std::unique_lock<std::mutex> lock(mutex_);
+  BLAZE_CONDITION_THROW(net_def_ != nullptr, "Workspace::Init was not called");
+  RecycleBlobMap();  // every net (= predictor) gets its own activation blobs; constants stay shared
+  std::string run_mode = net_def_->run_mode();
+  if (!NetRegistry()->Has(run_mode)) {
+    LOG_INFO("run_mode %s is not available in this build, using the simple executor", run_mode.c_str());
+    run_mode = "simple";
+  }
+  return NetRegistry()->Create(run_mode, net_def_, this);
+}
+
+std::shared_ptr<Net> Workspace::CreateNet(const char* net_file) {
+  NetDef def;
+  std::string err;
+  if (!LoadNetDefFromFile(net_file, &def, &err)) BLAZE_THROW("Open net_file: ", net_file, " failed: ", err);
+  Init(def);
+  return CreateNet();
+}
+
+DataType Workspace::input_data_type(const std::string& input_name) const {
+  auto it = input_data_type_map_.find(input_name);
+  BLAZE_CONDITION_THROW(it != input_data_type_map_.end(), "input_name: ", input_name, " data_type not defined");
+  return it->second;
+}
+
+const ValueInfo& Workspace::input_info(const std::string& input_name) const {
+  auto it = input_info_map_.find(input_name);
+  BLAZE_CONDITION_THROW(it != input_info_map_.end(), "input_name=", input_name, " is not input name");
+  return it->second;
+}
+
+// ------------------------------------------------------------------------------------------ net
+NetRegistryType* NetRegistry() {
+  static NetRegistryType* r = new NetRegistryType();
+  return r;
+}
+
+Net::Net(const std::shared_ptr<const NetDef>& def, Workspace* ws) : name_(def->name()), net_def_(def), workspace_(ws) {
+  BLAZE_CONDITION_THROW(net_def_->has_device_option(), "net has no device option");
+  // external inputs: tensors consumed before any operator produced them, in order of first use; external
+  // outputs: the declared ones, else tensors nobody consumes
+  std::set<std::string> produced, consumed;
+  for (const auto& op : def->op()) {
+    for (const auto& in : op.input()) {
+      if (!produced.count(in) && !consumed.count(in)) external_input_.push_back(in);
+      consumed.insert(in);
+    }
+    for (const auto& out : op.output()) produced.insert(out);
+  }
+  if (def->external_output_size() > 0) {
+    for (const auto& v : def->external_output_) external_output_.push_back(v.name());
+  } else {
+    for (const auto& op : def->op())
+      for (const auto& out : op.output())
+        if (!consumed.count(out)) external_output_.push_back(out);
+  }
+  if (def->external_input_size() > 0) {
+    for (const auto& in : external_input_) {
+      bool declared = false;
+      for (const auto& v : def->external_input_) declared |= v.name() == in;
+      BLAZE_CONDITION_THROW(declared, "Source for input ", in, " is unkown for net ", def->name());
+    }
+  }
+}
+
+Blob* Net::external_input_blob(const std::string& name) const {
+  auto it = external_input_blob_.find(name);
+  return it == external_input_blob_.end() ? nullptr : it->second;
+}
+Blob* Net::external_output_blob(const std::string& name) const {
+  auto it = external_output_blob_.find(name);
+  return it == external_output_blob_.end() ? nullptr : it->second;
+}
+
+bool Net::Run() {
+  if (!RunImpl()) {
+    LOG_ERROR("Failed to run impl");
+    return false;
+  }
+  // all operators run on stream 0 of this thread: waiting for that stream waits for the net (simple_net.cc:27-32)
+  if (!operators_.empty()) operators_.back()->WaitStream();
+  return true;
+}
+
+std::string Net::DumpProfile() const {
+  std::stringstream ss;
+  ss << "{\"traceEvents\":[";
+  double t = 0;
+  bool first = true;
+  for (const auto& op : operators_) {
+    if (!first) ss << ",";
+    first = false;
+    ss << "{\"name\":\"" << op->type() << ":" << op->name() << "\",\"ph\":\"X\",\"pid\":0,\"tid\":0,\"ts\":" << t
+       << ",\"dur\":" << op->last_run_us() << "}";
+    t += op->last_run_us();
+  }
+  ss << "]}";
+  return ss.str();
+}
+
+SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws) : Net(net_def, ws) {
+  const bool net_has_device_option = net_def->has_device_option();
+  for (int idx = 0; idx < net_def->op_size(); ++idx) {
+    OperatorDef def(net_def->op(idx));
+    if (!def.has_device_option() && net_has_device_option) *def.mutable_device_option() = net_def->device_option();
+    std::unique_ptr<OperatorBase> op = CreateOperator(def, ws, idx);
+    for (int i = 0; i < def.input_size(); ++i)
+      for (const auto& ei : external_input_)
+        if (ei == def.input(i)) external_input_blob_[ei] = op->Input(i);
+    for (int i = 0; i < def.output_size(); ++i)
+      for (const auto& eo : external_output_)
+        if (eo == def.output(i)) external_output_blob_[eo] = op->Output(i);
+    operators_.emplace_back(std::move(op));
+  }
+  skipped_.assign(operators_.size(), false);
+  // Gemm -> activation folding: the consumer must be the only reader of the producer's output
+  const Argument* fuse_arg = ArgumentHelper::Find(net_def->arg_, "fuse_gemm_activation");
+  const char* env = getenv("BLAZE_NO_FUSION");
+  const bool fuse = !(env && atoi(env) != 0) && !(fuse_arg && fuse_arg->has_i && fuse_arg->i == 0);
+  if (fuse) {
+    for (size_t i = 0; i + 1 < operators_.size(); ++i) {
+      auto* producer = dynamic_cast<FusableProducer*>(operators_[i].get());
+      if (!producer || skipped_[i]) continue;
+      const OperatorDef& pd = operators_[i]->operator_def();
+      const OperatorDef& cd = operators_[i + 1]->operator_def();
+      if (pd.output_size() != 1 || cd.input_size() < 1 || cd.input(0) != pd.output(0)) continue;
+      const std::string& mid = pd.output(0);
+      bool other_reader = false;
+      for (size_t j = 0; j < operators_.size(); ++j) {
+        if (j == i + 1) continue;
+        for (const auto& in : operators_[j]->operator_def().input()) other_reader |= (j != i && in == mid);
+      }
+      bool is_output = false;
+      for (const auto& eo : external_output_) is_output |= (eo == mid && cd.output(0) != mid);
+      if (other_reader || is_output) continue;
+      if (producer->TryFuse(operators_[i + 1].get())) skipped_[i + 1] = true;
+    }
+  }
+}
+
+bool SimpleNet::RunImpl() {
+  for (size_t i = 0; i < operators_.size(); ++i) {
+    if (skipped_[i]) continue;
+    auto& op = operators_[i];
+    bool res;
+    if (profile_) {
+      auto t0 = std::chrono::steady_clock::now();
+      res = op->Run();
+      op->WaitStream();
+      op->set_last_run_us(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+    } else {
+      res = op->Run();
+    }
+    if (!res) {
+      LOG_ERROR("Operator failed, name=%s type=%s", op->name().c_str(), op->type().c_str());
+      return false;
+    }
+  }
+  return true;
+}
+
+REGISTER_NET(simple, SimpleNet);
+
+}  // namespace blaze

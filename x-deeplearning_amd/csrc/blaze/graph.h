@@ -1,0 +1,118 @@
+// graph.h -- Workspace (blob ownership per model / per predictor) and the sequential executor.
+//
+// Minimal re-creation of the callers of the operator boundary: blaze/graph/workspace.h:24-196 (constants are
+// shared by every net of a workspace, activations belong to one net), blaze/graph/net.h:21-178 and
+// blaze/graph/simple_net.cc:9-46 (create one operator per OperatorDef, run them in order on stream 0, wait
+// for the stream).  The DAG / hybrid executors, observers beyond a wall-clock profile, and the batching
+// schedulers are not part of this build; run_mode strings other than "simple" fall back to this executor.
+#pragma once
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <set>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "blaze/operator.h"
+#include "blaze/sparse_puller.h"
+
+namespace blaze {
+
+class Net;
+
+class Workspace {
+ public:
+  ~Workspace();
+  Blob* CreateConstantBlob(const std::string& name, const DeviceOption& device_option, bool* newblob = nullptr);
+  Blob* CreateBlob(const std::string& name, const DeviceOption& device_option, bool* newblob = nullptr);
+  bool HasConstantBlob(const std::string& name) const { return constant_fill_blob_map_.count(name) != 0; }
+  const std::map<std::string, Blob*>& constant_blobs() const { return constant_fill_blob_map_; }
+
+  void SetSparsePuller(std::shared_ptr<store::SparsePuller> p) { sparse_puller_ = p; }
+  std::shared_ptr<store::SparsePuller>& GetSparsePuller() { return sparse_puller_; }
+
+  void Init(const NetDef& net_def);
+  std::shared_ptr<Net> CreateNet();
+  std::shared_ptr<Net> CreateNet(const char* net_file);  // text or binary NetDef (tests, small models)
+
+  DataType input_data_type(const std::string& input_name) const;
+  bool has_input_info(const std::string& input_name) const { return input_info_map_.count(input_name) != 0; }
+  const ValueInfo& input_info(const std::string& input_name) const;
+  std::shared_ptr<NetDef>& net_def() { return net_def_; }
+
+ private:
+  void RecycleBlobMap();
+  std::map<std::string, Blob*> constant_fill_blob_map_;  // shared by all predictors of the model
+  std::map<std::string, Blob*> blob_map_;                // the blobs of the net being built
+  std::set<Blob*> blob_recycle_bins_;                    // blobs of nets built earlier
+  std::shared_ptr<NetDef> net_def_;
+  std::map<std::string, DataType> input_data_type_map_;
+  std::unordered_map<std::string, ValueInfo> input_info_map_;
+  std::shared_ptr<store::SparsePuller> sparse_puller_;
+  std::mutex mutex_;
+};
+
+class Net {
+ public:
+  Net(const std::shared_ptr<const NetDef>& net_def, Workspace* ws);
+  virtual ~Net() noexcept {}
+  // reset, run every operator, wait for the device (net.h:33-49); exceptions propagate to the Predictor
+  virtual bool Run();
+  const std::vector<std::string>& external_input() const { return external_input_; }
+  const std::vector<std::string>& external_output() const { return external_output_; }
+  Blob* external_input_blob(const std::string& name) const;
+  Blob* external_output_blob(const std::string& name) const;
+  const ValueInfo& external_input_info(const std::string& name) const { return workspace_->input_info(name); }
+  bool has_external_input_info(const std::string& name) const { return workspace_->has_input_info(name); }
+  std::vector<std::unique_ptr<OperatorBase>>& GetOperators() { return operators_; }
+  Workspace* workspace() { return workspace_; }
+  // "profile" observer: per-operator host wall time of the last Run, as chrome-trace JSON
+  void set_profile(bool on) { profile_ = on; }
+  std::string DumpProfile() const;
+  const std::string& name() const { return name_; }
+
+ protected:
+  virtual bool RunImpl() = 0;
+  std::string name_;
+  std::shared_ptr<const NetDef> net_def_;
+  Workspace* workspace_;
+  std::vector<std::unique_ptr<OperatorBase>> operators_;
+  std::vector<std::string> external_input_, external_output_;
+  std::map<std::string, Blob*> external_input_blob_, external_output_blob_;
+  bool profile_ = false;
+};
+
+class SimpleNet : public Net {
+ public:
+  SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws);
+
+ protected:
+  bool RunImpl() override;
+  std::vector<bool> skipped_;  // ops folded into their producer's epilogue
+};
+
+typedef Registry<std::shared_ptr<Net>, const std::shared_ptr<const NetDef>&, Workspace*> NetRegistryType;
+NetRegistryType* NetRegistry();
+#define REGISTER_NET(name, ...)                                                                                    \
+  namespace {                                                                                                      \
+  static ::blaze::Registerer<std::shared_ptr<::blaze::Net>, const std::shared_ptr<const ::blaze::NetDef>&,         \
+                             ::blaze::Workspace*>                                                                  \
+      ANONYMOUS_VARIABLE(g_net_##name)(#name, ::blaze::NetRegistry(),                                              \
+                                       [](const std::shared_ptr<const ::blaze::NetDef>& d, ::blaze::Workspace* w) { \
+                                         return std::shared_ptr<::blaze::Net>(new __VA_ARGS__(d, w));              \
+                                       });                                                                         \
+  }
+
+// An operator whose kernel can apply the following activation operator in its epilogue.  SimpleNet offers each
+// (producer, consumer) pair; when TryFuse accepts, the consumer is skipped at run time.  The reference fuses
+// sibling GEMMs but never GEMM + activation (blaze/graph/pattern/); numerically the fused result equals the
+// composition Activation(Gemm(x, W, b)).
+class FusableProducer {
+ public:
+  virtual ~FusableProducer() {}
+  virtual bool TryFuse(OperatorBase* consumer) = 0;
+};
+
+}  // namespace blaze

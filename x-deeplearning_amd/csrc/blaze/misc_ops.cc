@@ -1,0 +1,310 @@
+// misc_ops.cc -- the operators around the Gemms in CTR / DIN graphs: PRelu, Dice, LeakyRelu, Sigmoid, Softmax
+// (used stand-alone when they cannot ride in a Gemm epilogue), ConstantFill (weights) and Concat.
+//
+// Formulas and argument names follow the reference's operators:
+//   PRelu        blaze/operator/op/prelu_op.cc:11-73     slope broadcast over the trailing dims
+//   Dice         blaze/operator/op/dice_op.{h,cc}        inputs X, gamma, mean, var; arg nosqrt
+//   LeakyRelu    blaze/operator/op/leaky_relu_op.cc      arg alpha
+//   Sigmoid      blaze/operator/op/sigmoid_op.cc:15-38
+//   Softmax      blaze/operator/op/softmax_op.cc:13-78   arg axis (default 1)
+//   ConstantFill blaze/operator/op/constant_fill_op.h:13-57  args shape, dtype, value
+//   Concat       blaze/operator/op/concat_op.h           arg axis (default 1)
+#include "blaze/graph.h"
+#include "blaze/operator.h"
+#include "blaze_hip.h"
+
+#include <type_traits>
+
+namespace blaze {
+
+namespace {
+
+int BzType(int data_type) {
+  switch (data_type) {
+    case kFloat: return BZ_F32;
+    case kFloat16: return BZ_F16;
+    default: BLAZE_THROW("Unsupported type: ", data_type);
+  }
+}
+
+// fp32 device copy of a small parameter blob (the activation kernels read fp32 parameters)
+struct ParamF32 {
+  float* ptr = nullptr;
+  size_t cap = 0;
+  ~ParamF32() {
+    if (ptr) (void)hipFree(ptr);
+  }
+  const float* Get(Blob* b, hipStream_t st) {
+    if (b->data_type() == kFloat) return b->as<float>();
+    BLAZE_CONDITION_THROW(b->data_type() == kFloat16, "Unsupported type: ", b->data_type());
+    const int n = (int)b->size();
+    const int64_t ld = (n + 7) / 8 * 8;
+    if ((size_t)ld > cap) {
+      if (ptr) (void)hipFree(ptr);
+      HIP_CHECK(hipMalloc((void**)&ptr, ld * sizeof(float)));
+      cap = ld;
+    }
+    BZ_CHECK(bz_fc_pack_weight(b->data(), BZ_F16, 1, n, 1, ptr, BZ_F32, ld, st));
+    return ptr;
+  }
+};
+
+void RunActivation(Blob* x, Blob* y, int act, const float* p0, const float* p1, const float* p2, int act_size, bool nosqrt,
+                   float alpha, int64_t rows, int64_t cols, hipStream_t st) {
+  bz_act_desc d;
+  memset(&d, 0, sizeof(d));
+  d.x = x->data();
+  d.y = y->data();
+  d.p0 = p0;
+  d.p1 = p1;
+  d.p2 = p2;
+  d.rows = rows;
+  d.cols = cols;
+  d.dtype = BzType(x->data_type());
+  d.act = act;
+  d.act_size = act_size;
+  d.dice_nosqrt = nosqrt ? 1 : 0;
+  d.act_alpha = alpha;
+  BZ_CHECK(bz_activation(&d, st));
+}
+
+}  // namespace
+
+template <class Context>
+class PReluOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  PReluOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {}
+  bool RunOnDevice() override {
+    Blob* X = this->Input(0);
+    Blob* W = this->Input(1);
+    Blob* Y = this->Output(0);
+    BLAZE_CONDITION_THROW(W->size() > 0 && X->size() % W->size() == 0, "X->size()=", X->size(), " W->size()=", W->size());
+    Y->Reshape(X->shape());
+    if (X->size() == 0) return true;
+    hipStream_t st = context_.hip_stream();
+    // the slope is the "inner" broadcast: element i uses w[i % W.size] (prelu_op.cc:13-29)
+    RunActivation(X, Y, BZ_ACT_PRELU, w_.Get(W, st), nullptr, nullptr, (int)W->size(), false, 0.f, (int64_t)(X->size() / W->size()),
+                  (int64_t)W->size(), st);
+    return true;
+  }
+
+ private:
+  ParamF32 w_;
+};
+REGISTER_HIP_OPERATOR(PRelu, PReluOp<HIPContext>);
+OPERATOR_SCHEMA(PRelu).NumInputs(2).NumOutputs(1).AllowInplace({{0, 0}}).IdenticalTypeOfInput(0).SetDoc(
+    "f(x) = slope * x for x < 0, f(x) = x for x >= 0");
+
+template <class Context>
+class DiceOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  DiceOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    nosqrt_ = OperatorBase::GetSingleArgument<bool>("nosqrt", false);
+  }
+  bool RunOnDevice() override {
+    Blob* x = this->Input(0);
+    Blob* gamma = this->Input(1);
+    Blob* mean = this->Input(2);
+    Blob* var = this->Input(3);
+    Blob* y = this->Output(0);
+    const int dt[4] = {x->data_type(), gamma->data_type(), mean->data_type(), var->data_type()};
+    for (int k = 1; k < 4; ++k)
+      BLAZE_CONDITION_THROW(dt[k] == dt[k - 1], "data_type[", k, "]=", dt[k], " data_type[", k - 1, "]=", dt[k - 1]);
+    BLAZE_CONDITION_THROW(gamma->size() == mean->size() && mean->size() == var->size(), "size[gamma]=", gamma->size(),
+                          " size[mean]=", mean->size(), " size[var]=", var->size());
+    BLAZE_CONDITION_THROW(gamma->size() > 0 && x->size() % gamma->size() == 0, "x->size()=", x->size(), " gamma->size()=", gamma->size());
+    y->Reshape(x->shape());
+    if (x->size() == 0) return true;
+    hipStream_t st = context_.hip_stream();
+    RunActivation(x, y, BZ_ACT_DICE, p_[0].Get(gamma, st), p_[1].Get(mean, st), p_[2].Get(var, st), (int)gamma->size(), nosqrt_, 0.f,
+                  (int64_t)(x->size() / gamma->size()), (int64_t)gamma->size(), st);
+    return true;
+  }
+
+ private:
+  bool nosqrt_ = false;
+  ParamF32 p_[3];
+};
+REGISTER_HIP_OPERATOR(Dice, DiceOp<HIPContext>);
+OPERATOR_SCHEMA(Dice).NumInputs(4).NumOutputs(1).AllowInplace({{0, 0}}).IdenticalTypeOfInput(0).SetDoc(
+    "Dice activation (https://arxiv.org/pdf/1706.06978.pdf), inference form with fixed mean/var");
+
+template <class Context>
+class LeakyReluOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  LeakyReluOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    alpha_ = OperatorBase::GetSingleArgument<float>("alpha", 0.01f);
+  }
+  bool RunOnDevice() override {
+    Blob* X = this->Input(0);
+    Blob* Y = this->Output(0);
+    Y->Reshape(X->shape());
+    if (X->size() == 0) return true;
+    RunActivation(X, Y, BZ_ACT_LEAKY_RELU, nullptr, nullptr, nullptr, 0, false, alpha_, 1, (int64_t)X->size(), context_.hip_stream());
+    return true;
+  }
+
+ private:
+  float alpha_;
+};
+REGISTER_HIP_OPERATOR(LeakyRelu, LeakyReluOp<HIPContext>);
+OPERATOR_SCHEMA(LeakyRelu).NumInputs(1).NumOutputs(1).AllowInplace({{0, 0}}).IdenticalTypeOfInput(0).SetDoc(
+    "f(x) = alpha * x for x < 0, f(x) = x for x >= 0");
+
+template <class Context>
+class SigmoidOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  SigmoidOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {}
+  bool RunOnDevice() override {
+    Blob* X = this->Input(0);
+    Blob* Y = this->Output(0);
+    Y->Reshape(X->shape());
+    if (X->size() == 0) return true;
+    RunActivation(X, Y, BZ_ACT_SIGMOID, nullptr, nullptr, nullptr, 0, false, 0.f, 1, (int64_t)X->size(), context_.hip_stream());
+    return true;
+  }
+};
+REGISTER_HIP_OPERATOR(Sigmoid, SigmoidOp<HIPContext>);
+OPERATOR_SCHEMA(Sigmoid).NumInputs(1).NumOutputs(1).AllowInplace({{0, 0}}).IdenticalTypeOfInput(0).SetDoc("y = 1 / (1 + exp(-x))");
+
+template <class Context>
+class SoftmaxOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  SoftmaxOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    axis_ = OperatorBase::GetSingleArgument<size_t>("axis", 1);
+  }
+  bool RunOnDevice() override {
+    Blob* X = this->Input(0);
+    Blob* Y = this->Output(0);
+    BLAZE_CONDITION_THROW(axis_ < X->shape().size(), "axis=", axis_, " X->shape().size()=", X->shape().size());
+    // softmax over `axis` with W trailing elements (softmax_op.cc:23-26); the device kernel covers W == 1,
+    // which is every head on this path ([batch, classes])
+    const TIndex W = X->size((int)axis_ + 1, (int)X->shape().size());
+    BLAZE_CONDITION_THROW(W == 1, "Softmax over a non-innermost axis (inner size ", W, ") is not supported on this device");
+    Y->Reshape(X->shape());
+    if (X->size() == 0) return true;
+    const int64_t C = (int64_t)X->shape()[axis_];
+    RunActivation(X, Y, BZ_ACT_SOFTMAX, nullptr, nullptr, nullptr, 0, false, 0.f, (int64_t)X->size() / C, C, context_.hip_stream());
+    return true;
+  }
+
+ private:
+  size_t axis_;
+};
+REGISTER_HIP_OPERATOR(Softmax, SoftmaxOp<HIPContext>);
+OPERATOR_SCHEMA(Softmax).NumInputs(1).NumOutputs(1).AllowInplace({{0, 0}}).IdenticalTypeOfInput(0).SetDoc("softmax over axis");
+
+// ------------------------------------------------------------------------------------------ ConstantFill
+template <class Context>
+class ConstantFillOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  ConstantFillOp(const OperatorDef& def, Workspace* ws)
+      : Operator<Context>(def, ws, false), shape_(OperatorBase::GetRepeatedArgument<TIndex>("shape")) {
+    const DataType dtype = (DataType)OperatorBase::GetSingleArgument<int>("dtype", kFloat);
+    for (const std::string& out : def.output()) this->outputs_.push_back(ws->CreateConstantBlob(out, this->device_option_));
+    Blob* output = this->Output(0);
+    output->set_data_type(dtype);
+    output->Reshape(shape_);
+    const size_t n = output->size();
+    std::vector<unsigned char> host(n * DataTypeSize(dtype));
+    switch (dtype) {  // CONSTANT_FILL_TYPE_SWITCH
+      case kFloat: {
+        const auto v = OperatorBase::GetRepeatedArgument<float>("value");
+        CheckCount(v.size(), n);
+        memcpy(host.data(), v.data(), host.size());
+        break;
+      }
+      case kFloat16: {  // stored as floats in the model, narrowed per element with round-to-nearest-even
+        const auto v = OperatorBase::GetRepeatedArgument<float>("value");
+        CheckCount(v.size(), n);
+        uint16_t* h = (uint16_t*)host.data();
+        for (size_t i = 0; i < n; ++i) h[i] = FloatToHalf(v[i]);
+        break;
+      }
+      case kInt32: {
+        const auto v = OperatorBase::GetRepeatedArgument<int>("value");
+        CheckCount(v.size(), n);
+        memcpy(host.data(), v.data(), host.size());
+        break;
+      }
+      case kInt64: {
+        const auto v = OperatorBase::GetRepeatedArgument<int64_t>("value");
+        CheckCount(v.size(), n);
+        memcpy(host.data(), v.data(), host.size());
+        break;
+      }
+      default:
+        BLAZE_THROW("Unsupported type: ", dtype);
+    }
+    // one-time upload, synchronous: the blob is shared by every predictor created afterwards
+    if constexpr (std::is_same<Context, HIPContext>::value) {
+      context_.Activate();
+      HIP_CHECK(hipMemcpy(output->data(), host.data(), host.size(), hipMemcpyHostToDevice));
+    } else {
+      memcpy(output->data(), host.data(), host.size());
+    }
+  }
+  bool RunOnDevice() override { return true; }
+
+ private:
+  void CheckCount(size_t have, size_t want) {
+    BLAZE_CONDITION_THROW(have == want, "value.size()=", have, " output->size()=", want, " ", this->def_.DebugString());
+  }
+  std::vector<TIndex> shape_;
+};
+REGISTER_HIP_OPERATOR(ConstantFill, ConstantFillOp<HIPContext>);
+REGISTER_CPU_OPERATOR(ConstantFill, ConstantFillOp<CPUContext>);
+OPERATOR_SCHEMA(ConstantFill).NumInputs(0).NumOutputs(1).SetDoc("a constant tensor: args shape, dtype, value");
+
+
+// ------------------------------------------------------------------------------------------ Concat
+template <class Context>
+class ConcatOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  ConcatOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    axis_ = OperatorBase::GetSingleArgument<int>("axis", 1);
+  }
+  bool RunOnDevice() override {
+    Blob* x0 = this->Input(0);
+    const size_t rank = x0->shape().size();
+    BLAZE_CONDITION_THROW(axis_ >= 0 && (size_t)axis_ < rank, "axis=", axis_, " rank=", rank);
+    std::vector<TIndex> shape = x0->shape();
+    TIndex total = 0;
+    for (int i = 0; i < this->InputSize(); ++i) {
+      Blob* x = this->Input(i);
+      BLAZE_CONDITION_THROW(x->shape().size() == rank && x->data_type() == x0->data_type(), "concat input ", i, " has another rank or type");
+      for (size_t k = 0; k < rank; ++k)
+        if ((int)k != axis_) BLAZE_CONDITION_THROW(x->shape()[k] == shape[k], "concat input ", i, " dim ", k, " mismatch");
+      total += x->shape()[axis_];
+    }
+    shape[axis_] = total;
+    Blob* y = this->Output(0);
+    y->Reshape(shape);
+    const size_t es = DataTypeSize(y->data_type());
+    const TIndex outer = y->size(0, axis_), inner = y->size(axis_ + 1, (int)rank);
+    hipStream_t st = context_.hip_stream();
+    size_t col = 0;
+    for (int i = 0; i < this->InputSize(); ++i) {
+      Blob* x = this->Input(i);
+      const size_t width = x->shape()[axis_] * inner * es;
+      if (width > 0 && outer > 0)
+        HIP_CHECK(hipMemcpy2DAsync((char*)y->data() + col, total * inner * es, x->data(), width, width, outer, hipMemcpyDeviceToDevice, st));
+      col += width;
+    }
+    return true;
+  }
+
+ private:
+  int axis_;
+};
+REGISTER_HIP_OPERATOR(Concat, ConcatOp<HIPContext>);
+OPERATOR_SCHEMA(Concat).NumInputs(1, INT_MAX).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("concatenate along axis");
+
+}  // namespace blaze

@@ -1,0 +1,328 @@
+#include "blaze/predictor.h"
+
+#include "blaze/qed_store.h"
+
+namespace blaze {
+
+Predictor::Predictor(std::shared_ptr<Net> net) : net_(net) {
+  for (const auto& name : net_->external_output()) {
+    Blob* b = net_->external_output_blob(name);
+    BLAZE_CONDITION_THROW(b != nullptr, "external_output: ", name, " is not in external_output_blob");
+    output_index_[name] = (int)external_output_blob_.size();
+    external_output_blob_.push_back(b);
+    DeviceOption cpu;
+    cpu.set_device_type(kCPU);
+    output_cpu_.push_back(std::make_shared<Blob>(cpu));
+    output_cpu_.back()->set_data_type((DataType)b->data_type());
+  }
+  for (const auto& name : net_->external_input()) {
+    Blob* b = net_->external_input_blob(name);
+    BLAZE_CONDITION_THROW(b != nullptr, "external_input: ", name, " is not in external_input_blob");
+    input_index_[name] = (int)external_input_blob_.size();
+    external_input_blob_.push_back(b);
+  }
+}
+
+int Predictor::InputName2Idx(const char* name) const {
+  auto it = input_index_.find(name);
+  return it == input_index_.end() ? -1 : it->second;
+}
+int Predictor::OutputName2Idx(const char* name) const {
+  auto it = output_index_.find(name);
+  return it == output_index_.end() ? -1 : it->second;
+}
+
+bool Predictor::ReshapeInput(const char* name, const std::vector<size_t>& shape) {
+  const int idx = InputName2Idx(name);
+  if (idx < 0) {
+    LOG_ERROR("The name: %s is not The input of net", name);
+    return false;
+  }
+  return ReshapeInput((size_t)idx, shape);
+}
+bool Predictor::ReshapeInput(size_t idx, const std::vector<size_t>& shape) {
+  if (idx >= external_input_blob_.size()) {
+    LOG_ERROR("The idx=%zu exceed size=%zu", idx, external_input_blob_.size());
+    return false;
+  }
+  try {
+    external_input_blob_[idx]->Reshape(shape);
+  } catch (std::exception& e) {
+    LOG_ERROR("reshape failed: %s", e.what());
+    return false;
+  }
+  return true;
+}
+
+bool Predictor::Feed(const char* name, const void* data, size_t len) {
+  const int idx = InputName2Idx(name);
+  if (idx < 0) {
+    LOG_ERROR("The name: %s is not The input of net", name);
+    return false;
+  }
+  return Feed((size_t)idx, data, len);
+}
+bool Predictor::Feed(size_t idx, const void* data, size_t len) {
+  if (idx >= external_input_blob_.size()) {
+    LOG_ERROR("The idx=%zu exceed size=%zu", idx, external_input_blob_.size());
+    return false;
+  }
+  Blob* blob = external_input_blob_[idx];
+  const size_t need = blob->size() * DataTypeSize(blob->data_type());
+  if (len != need) {
+    LOG_ERROR("The len=%zu need size=%zu blob->size()=%zu", len, need, (size_t)blob->size());
+    return false;
+  }
+  try {
+    if (blob->device_type() == kCPU) {
+      memcpy(blob->data(), data, need);
+    } else {
+      HIPContext ctx(blob->device_option());
+      ctx.Activate();
+      CopyBytes(blob->data(), kHIP, data, kCPU, need, ctx.hip_stream());
+    }
+  } catch (std::exception& e) {
+    LOG_ERROR("feed failed: %s", e.what());
+    return false;
+  }
+  return true;
+}
+
+int Predictor::InputDataType(const char* name) const {
+  const int idx = InputName2Idx(name);
+  return idx < 0 ? (int)kPDT_Invalid : external_input_blob_[idx]->data_type();
+}
+
+bool Predictor::Forward(const PredictorCallback&& cb) {
+  try {
+    if (!net_->Run()) return false;
+    if (cb) cb();
+    return true;
+  } catch (std::exception& e) {
+    LOG_ERROR("failed: %s", e.what());
+    last_error_for_thread() = e.what();
+    return false;
+  }
+}
+
+bool Predictor::Output(const char* name, void** data, size_t* len) {
+  const int idx = OutputName2Idx(name);
+  if (idx < 0) {
+    LOG_ERROR("The name: %s is not The output of net", name);
+    return false;
+  }
+  return Output((size_t)idx, data, len);
+}
+bool Predictor::Output(size_t idx, void** data, size_t* len) {
+  if (idx >= external_output_blob_.size()) {
+    LOG_ERROR("The idx=%zu exceed size=%zu", idx, external_output_blob_.size());
+    return false;
+  }
+  Blob* blob = external_output_blob_[idx];
+  const size_t bytes = blob->size() * DataTypeSize(blob->data_type());
+  try {
+    if (blob->device_type() == kCPU) {
+      *data = blob->data();
+    } else {
+      std::shared_ptr<Blob>& cpu = output_cpu_[idx];
+      cpu->set_data_type((DataType)blob->data_type());
+      cpu->Reshape(blob->shape());
+      HIPContext ctx(blob->device_option());
+      ctx.Activate();
+      CopyBytes(cpu->data(), kCPU, blob->data(), kHIP, bytes, ctx.hip_stream());
+      *data = cpu->data();
+    }
+  } catch (std::exception& e) {
+    LOG_ERROR("output failed: %s", e.what());
+    return false;
+  }
+  if (len) *len = bytes;
+  return true;
+}
+
+const std::vector<size_t>& Predictor::OutputShape(size_t idx) const {
+  BLAZE_CONDITION_THROW(idx < external_output_blob_.size(), "The idx=", idx, " blob is null");
+  return external_output_blob_[idx]->shape();
+}
+const std::vector<size_t>& Predictor::OutputShape(const char* name) const {
+  const int idx = OutputName2Idx(name);
+  BLAZE_CONDITION_THROW(idx >= 0, "The name ", name, " is not Output of net");
+  return OutputShape((size_t)idx);
+}
+int Predictor::OutputDataType(const char* name) const {
+  const int idx = OutputName2Idx(name);
+  return idx < 0 ? (int)kPDT_Invalid : external_output_blob_[idx]->data_type();
+}
+
+std::vector<std::string> Predictor::ListInternalName() const {
+  std::vector<std::string> names;
+  for (const auto& it : net_->workspace()->constant_blobs()) names.push_back(it.first);
+  return names;
+}
+bool Predictor::InternalParam(const char* name, void** data, size_t* len) {
+  const auto& m = net_->workspace()->constant_blobs();
+  auto it = m.find(name);
+  if (it == m.end()) return false;
+  Blob* blob = it->second;
+  const size_t bytes = blob->size() * DataTypeSize(blob->data_type());
+  try {
+    if (blob->device_type() == kCPU) {
+      *data = blob->data();
+    } else {
+      DeviceOption cpu_opt;
+      cpu_opt.set_device_type(kCPU);
+      auto& cpu = param_cpu_[name];
+      if (!cpu) cpu = std::make_shared<Blob>(cpu_opt);
+      cpu->set_data_type((DataType)blob->data_type());
+      cpu->Reshape(blob->shape());
+      HIPContext ctx(blob->device_option());
+      ctx.Activate();
+      CopyBytes(cpu->data(), kCPU, blob->data(), kHIP, bytes, ctx.hip_stream());
+      *data = cpu->data();
+    }
+  } catch (std::exception& e) {
+    LOG_ERROR("param copy failed: %s", e.what());
+    return false;
+  }
+  if (len) *len = bytes;
+  return true;
+}
+const std::vector<size_t>& Predictor::InternalShape(const char* name) const {
+  const auto& m = net_->workspace()->constant_blobs();
+  auto it = m.find(name);
+  BLAZE_CONDITION_THROW(it != m.end(), "The name ", name, " is not a parameter of net");
+  return it->second->shape();
+}
+int Predictor::InternalDataType(const char* name) const {
+  const auto& m = net_->workspace()->constant_blobs();
+  auto it = m.find(name);
+  return it == m.end() ? (int)kPDT_Invalid : it->second->data_type();
+}
+
+void Predictor::RegisterObservers(const std::vector<std::string>& names) {
+  for (const auto& n : names)
+    if (n == "profile") net_->set_profile(true);
+}
+void Predictor::DumpObservers(std::unordered_map<std::string, std::string>* dump_map) {
+  (*dump_map)["profile"] = net_->DumpProfile();
+}
+
+void* Predictor::InputDevicePtr(const char* name) {
+  const int idx = InputName2Idx(name);
+  return idx < 0 ? nullptr : external_input_blob_[idx]->data();
+}
+void* Predictor::OutputDevicePtr(const char* name) {
+  const int idx = OutputName2Idx(name);
+  return idx < 0 ? nullptr : external_output_blob_[idx]->data();
+}
+
+std::string& last_error_for_thread() {
+  static thread_local std::string s;
+  return s;
+}
+
+// ------------------------------------------------------------------------------------------ manager
+std::shared_ptr<store::SparsePuller>& PredictorManager::EnsureSparsePuller(const char* type) {
+  if (!sparse_puller_) sparse_puller_.reset(store::SparsePullerCreationRegisterer::Get()->CreateSparsePuller(type));
+  return sparse_puller_;
+}
+
+bool PredictorManager::LoadSparseModelWeight(const char* uri, const char* type) {
+  try {
+    sparse_puller_.reset(store::SparsePullerCreationRegisterer::Get()->CreateSparsePuller(type));
+    if (store::kOK != sparse_puller_->Load(uri)) {
+      LOG_ERROR("load sparse model %s failed", uri);
+      return false;
+    }
+  } catch (std::exception& e) {
+    LOG_ERROR("load sparse model %s failed: %s", uri, e.what());
+    last_error_for_thread() = e.what();
+    return false;
+  }
+  return true;
+}
+
+bool PredictorManager::LoadModel(const char* filename, bool optimization_pass) {
+  return LoadModel(filename, "", kBlaze, optimization_pass);
+}
+bool PredictorManager::LoadDeepNetModel(const char* model_conf, const char* model_data, bool optimization_pass) {
+  return LoadModel(model_conf, model_data, kUlf, optimization_pass);
+}
+bool PredictorManager::LoadModel(const char* conf_file, const char*, ModelType model_type, bool) {
+  if (model_type != kBlaze) {
+    LOG_ERROR("model type %d needs an importer that is not part of this build; convert the model to a Blaze NetDef first", model_type);
+    last_error_for_thread() = "unsupported model type";
+    return false;
+  }
+  std::string err;
+  NetDef def;
+  if (!LoadNetDefFromFile(conf_file, &def, &err)) {
+    LOG_ERROR("Load model %s failed: %s", conf_file, err.c_str());
+    last_error_for_thread() = err;
+    return false;
+  }
+  return LoadNetDef(def);
+}
+bool PredictorManager::LoadNetDef(const NetDef& net_def) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  net_def_ = net_def;
+  if (!run_mode_.empty()) net_def_.run_mode_ = run_mode_;
+  has_net_ = true;
+  workspace_.clear();
+  return true;
+}
+
+Predictor* PredictorManager::CreatePredictor(PredictDeviceType predict_device, int device_id) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  try {
+    BLAZE_CONDITION_THROW(has_net_, "no model loaded");
+    if (device_id < 0) device_id = 0;
+    DeviceOption device_option;
+    switch (predict_device) {
+      case kPDT_CPU:
+        device_option.set_device_type(kCPU);
+        device_option.set_device_id(0);
+        break;
+      case kPDT_HIP:
+        device_option.set_device_type(kHIP);
+        device_option.set_device_id(device_id);
+        break;
+      default: {  // ProbeDevice (predictor_manager_impl.cc:162-177): round robin over the visible accelerators
+        static int next = 0;
+        int count = 0;
+        HIP_CHECK(hipGetDeviceCount(&count));
+        BLAZE_CONDITION_THROW(count > 0, "no accelerator visible and this build has no CPU path");
+        device_option.set_device_type(kHIP);
+        device_option.set_device_id(next++ % count);
+      }
+    }
+    const int dt = device_option.device_type(), di = device_option.device_id();
+    auto& ws = workspace_[dt][di];
+    if (!ws) {
+      ws.reset(new Workspace());
+      ws->Init(net_def_);
+      auto* opt = ws->net_def()->mutable_device_option();
+      opt->set_device_type(dt);
+      opt->set_device_id(di);
+      // the device of the predictor overrides what individual operators were exported with
+      for (auto& op : ws->net_def()->op_) {
+        if (op.has_device_option()) {
+          op.device_option_.set_device_type(dt);
+          op.device_option_.set_device_id(di);
+        }
+      }
+      ws->SetSparsePuller(sparse_puller_);
+    }
+    std::shared_ptr<Net> net = ws->CreateNet();
+    BLAZE_CONDITION_THROW(net != nullptr, "net creation failed");
+    return new Predictor(net);
+  } catch (std::exception& e) {
+    LOG_ERROR("Create Model Predictor failed, msg=%s", e.what());
+    last_error_for_thread() = e.what();
+    return nullptr;
+  }
+}
+
+bool InitScheduler(bool, int, int, int, int, int) { return true; }
+
+}  // namespace blaze

@@ -1,0 +1,76 @@
+#include "blaze/runtime.h"
+
+#include <stdlib.h>
+
+namespace blaze {
+
+void* Alloc(size_t bytes, int device_type, int device_id) {
+  if (bytes == 0) bytes = 16;
+  void* p = nullptr;
+  if (device_type == kCPU) {
+    p = malloc(bytes);
+    BLAZE_CONDITION_THROW(p != nullptr, "malloc of ", bytes, " bytes failed");
+    return p;
+  }
+  int cur = 0;
+  HIP_CHECK(hipGetDevice(&cur));
+  if (cur != device_id) HIP_CHECK(hipSetDevice(device_id));
+  HIP_CHECK(hipMalloc(&p, bytes));
+  if (cur != device_id) HIP_CHECK(hipSetDevice(cur));
+  return p;
+}
+
+void Free(void* ptr, int device_type, int) {
+  if (ptr == nullptr) return;
+  if (device_type == kCPU) {
+    free(ptr);
+  } else {
+    (void)hipFree(ptr);
+  }
+}
+
+void HIPContext::Activate() const {
+  static thread_local int current = -1;
+  if (current != device_id_) {
+    HIP_CHECK(hipSetDevice(device_id_));
+    current = device_id_;
+  }
+}
+
+hipStream_t HIPContext::hip_stream(int device_id, int stream_id) {
+  struct Streams {
+    std::vector<std::vector<hipStream_t>> per_device;
+    ~Streams() {
+      for (auto& v : per_device)
+        for (auto s : v)
+          if (s) (void)hipStreamDestroy(s);
+    }
+  };
+  static thread_local Streams tls;
+  BLAZE_CONDITION_THROW(stream_id >= 0 && stream_id < kMaxStreamNum, "stream_id=", stream_id);
+  if ((int)tls.per_device.size() <= device_id) tls.per_device.resize(device_id + 1);
+  auto& v = tls.per_device[device_id];
+  if (v.empty()) v.resize(kMaxStreamNum, nullptr);
+  if (v[stream_id] == nullptr) {
+    int cur = 0;
+    HIP_CHECK(hipGetDevice(&cur));
+    if (cur != device_id) HIP_CHECK(hipSetDevice(device_id));
+    HIP_CHECK(hipStreamCreateWithFlags(&v[stream_id], hipStreamNonBlocking));  // default priority
+    if (cur != device_id) HIP_CHECK(hipSetDevice(cur));
+  }
+  return v[stream_id];
+}
+
+void CopyBytes(void* dst, int dst_device_type, const void* src, int src_device_type, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return;
+  if (dst_device_type == kCPU && src_device_type == kCPU) {
+    memcpy(dst, src, bytes);
+    return;
+  }
+  hipMemcpyKind kind = dst_device_type == kCPU ? hipMemcpyDeviceToHost
+                                               : (src_device_type == kCPU ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice);
+  HIP_CHECK(hipMemcpyAsync(dst, src, bytes, kind, stream));
+  HIP_CHECK(hipStreamSynchronize(stream));
+}
+
+}  // namespace blaze

@@ -1,0 +1,145 @@
+// runtime.h -- Blob (typed buffer that owns its memory) and the device contexts.
+//
+// Follows the ownership rules of the reference (blaze/common/blob.h:17-103): Reshape grows capacity and never
+// shrinks it, RefReshape borrows foreign memory, operators never free their inputs.  The accelerator context
+// replaces CUDAContext (blaze/common/context.h:123-182): streams are thread local per (device, stream id), so a
+// serving thread that owns a Predictor owns its stream, and kernels are stream ordered with no device
+// synchronisation inside operators.
+#pragma once
+
+#include <memory>
+#include <vector>
+
+#include "blaze/common.h"
+#include "blaze/proto.h"
+
+namespace blaze {
+
+// cudaMalloc / malloc twins of blaze/common/allocator.h:33-71.  Host memory for device_type kCPU is pinned
+// (hipHostMalloc) when `pinned`, so Feed/Output copies run at full PCIe rate.
+void* Alloc(size_t bytes, int device_type, int device_id);
+void Free(void* ptr, int device_type, int device_id);
+
+class Blob {
+ public:
+  explicit Blob(const DeviceOption& device_option) : device_option_(device_option) {}
+  Blob(const DeviceOption& device_option, const std::vector<TIndex>& dims, DataType data_type)
+      : device_option_(device_option), data_type_(data_type) {
+    Reshape(dims);
+  }
+  ~Blob() { Destroy(); }
+  Blob(const Blob&) = delete;
+  Blob& operator=(const Blob&) = delete;
+
+  void Reshape(const std::vector<TIndex>& dims) {
+    TIndex n = 1;
+    for (auto d : dims) n *= d;
+    size_ = n;
+    if (size_ > capacity_ || !own_handle_) {
+      Destroy();
+      own_handle_ = true;
+      capacity_ = size_;
+      data_ = blaze::Alloc(capacity_ * DataTypeSize(data_type_), device_option_.device_type(), device_option_.device_id());
+      ++version_;
+    }
+    dims_ = dims;
+  }
+  void RefReshape(const std::vector<TIndex>& dims, void* handle) {
+    Destroy();
+    own_handle_ = false;
+    TIndex n = 1;
+    for (auto d : dims) n *= d;
+    size_ = capacity_ = n;
+    dims_ = dims;
+    data_ = handle;
+    ++version_;
+  }
+  const DeviceOption& device_option() const { return device_option_; }
+  int device_type() const { return device_option_.device_type(); }
+  int device_id() const { return device_option_.device_id(); }
+  // changing the element type of a blob that already holds memory re-sizes its capacity in elements
+  void set_data_type(DataType t) {
+    if (t != data_type_ && data_ != nullptr && own_handle_) capacity_ = capacity_ * DataTypeSize(data_type_) / DataTypeSize(t);
+    data_type_ = t;
+  }
+  int data_type() const { return data_type_; }
+  std::vector<TIndex>& shape() { return dims_; }
+  const std::vector<TIndex>& shape() const { return dims_; }
+  TIndex capacity() const { return capacity_; }
+  TIndex size() const { return size_; }
+  TIndex size(int start, int end) const {
+    TIndex s = 1;
+    for (int k = start; k < end; ++k) s *= dims_[k];
+    return s;
+  }
+  TIndex dim(size_t index) const {
+    BLAZE_CONDITION_THROW(index < dims_.size(), "index=", index, " dims_.size()=", dims_.size());
+    return dims_[index];
+  }
+  template <typename T>
+  T* as() { return reinterpret_cast<T*>(data_); }
+  void* data() { return data_; }
+  const void* data() const { return data_; }
+  // bumps whenever the buffer address may have changed: lets operators cache descriptors that embed pointers
+  uint64_t version() const { return version_; }
+
+ private:
+  void Destroy() {
+    if (data_ != nullptr && own_handle_)
+      blaze::Free(data_, device_option_.device_type(), device_option_.device_id());
+    data_ = nullptr;
+    capacity_ = 0;
+  }
+  DeviceOption device_option_;
+  void* data_ = nullptr;
+  TIndex capacity_ = 0, size_ = 0;
+  std::vector<TIndex> dims_;
+  DataType data_type_ = kFloat;
+  bool own_handle_ = true;
+  uint64_t version_ = 0;
+};
+
+constexpr int kMaxStreamNum = 4;  // blaze/common/context.h:121
+
+class CPUContext {
+ public:
+  explicit CPUContext(const DeviceOption& option) : device_option_(option) {}
+  void SwitchToDevice(int) {}
+  void FinishDeviceComputation() {}
+  int device_type() const { return kCPU; }
+  int stream_id() const { return 0; }
+  const DeviceOption& device_option() const { return device_option_; }
+
+ private:
+  DeviceOption device_option_;
+};
+
+class HIPContext {
+ public:
+  explicit HIPContext(const DeviceOption& option) : device_option_(option), device_id_(option.device_id()) {}
+  void SwitchToDevice(int stream_id) {
+    stream_id_ = stream_id;
+    Activate();
+  }
+  void Activate() const;                 // hipSetDevice when the thread is on another device
+  hipStream_t hip_stream() const { return hip_stream(device_id_, stream_id_); }
+  static hipStream_t hip_stream(int device_id, int stream_id);  // thread-local, created on first use
+  void FinishDeviceComputation() {
+    Activate();
+    HIP_CHECK(hipStreamSynchronize(hip_stream()));
+  }
+  int device_type() const { return kHIP; }
+  int device_id() const { return device_id_; }
+  int stream_id() const { return stream_id_; }
+  const DeviceOption& device_option() const { return device_option_; }
+
+ private:
+  DeviceOption device_option_;
+  int device_id_ = 0;
+  int stream_id_ = 0;
+};
+
+// copies between blobs of any two devices on `stream` (nullptr: the thread's stream 0), synchronous on return
+void CopyBytes(void* dst, int dst_device_type, const void* src, int src_device_type, size_t bytes, hipStream_t stream);
+
+}  // namespace blaze

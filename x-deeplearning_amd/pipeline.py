@@ -84,8 +84,8 @@ class CtrForward:
         d = self.steps[i % self.n_batches]["descs"][layer]
         bz.check(self.lib.bz_fc_fused(C.byref(d), st or self._stream()))
 
-    def step(self, i):
-        st = self._stream()
+    def step(self, i, st=None):
+        st = st or self._stream()
         if not self.fused_scan:
             self.scan(i, st)
         self.pool(i, st)
