@@ -5,7 +5,9 @@
 
 A step is one forward pass (Embedding gather/pool -> FC 896-512-256-2 with PReLU -> softmax) over one
 synthetic batch of 2048 samples (config 2), inputs already resident in HBM.  A pool of pre-generated
-batches is cycled so the id stream is not one cached batch.  Prints ONE JSON line.
+batches is cycled so the id stream is not one cached batch.  By default the step is Predictor.Forward through
+the Blaze_* C ABI (the drop-in path), issued by a few serving threads with one Predictor set and HIP stream
+each, as the reference is deployed.  Prints ONE JSON line.
 """
 import argparse
 import json
@@ -29,10 +31,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--pool", type=int, default=32, help="number of distinct pre-generated batches")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--graph", action="store_true", help="replay one HIP graph per step instead of launching kernels one by one")
-    ap.add_argument("--streams", type=int, default=4,
-                    help="predictor streams: consecutive batches go round robin to this many HIP streams (the reference "
-                         "runs one Predictor per serving thread, each with its own stream)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
+                         "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
+    ap.add_argument("--threads", type=int, default=8,
+                    help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
+                         "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
+    ap.add_argument("--kernel-api", action="store_true",
+                    help="drive the kernel-layer C ABI directly instead of Predictor.Forward (lower host overhead)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (one process, no collectives); --gpus %d is not supported" % args.gpus,
@@ -47,62 +53,94 @@ def main():
 
     assert torch.cuda.is_available(), "no GPU visible"
     arch = bz.device_check()
+    if args.calibrate_copy:
+        import ctypes
+        rows, width = 65536, 4096
+        src = torch.ones(rows * width, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        d = bz.ConcatDesc()
+        d.src[0], d.width[0], d.dst, d.dst_pitch, d.rows, d.n = src.data_ptr(), width, dst.data_ptr(), width, rows, 1
+        for _ in range(5):
+            bz.check(bz.lib().bz_concat_cols(ctypes.byref(d), None))
+        torch.cuda.synchronize()
+        assert bool((dst == 1).all())
+        print(json.dumps({"calibration": "bz_concat_kernel", "launches": 5, "bytes_read_per_launch": rows * width,
+                          "bytes_written_per_launch": rows * width}))
+        return
     cfg = Config2()
     tables = cfg.tables()
     mlp = cfg.mlp()
     sparse, dense = cfg.batches(args.pool)
+    # kernel-layer harness: per-kernel timing below, and the whole step in --kernel-api mode
     fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16")
     torch.cuda.synchronize()
     K, W = args.steps, args.warmup
+    T = max(1, min(args.threads, fwd.n_batches))
+    assert fwd.n_batches % T == 0, "--pool must be a multiple of --threads (a pooled batch always runs on one thread)"
 
-    # one HIP graph per pooled batch: the five launches of a step replay as one submission
-    graphs = None
-    if args.graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            fwd.step(0)
-        torch.cuda.current_stream().wait_stream(side)
+    predictors = None
+    if not args.kernel_api:
+        # the drop-in path: one Predictor per pooled batch (inputs fed once = resident in HBM), Forward through
+        # the Blaze_* C ABI; consecutive steps go round robin over T serving threads
+        from ctr_model import build_manager, make_predictor
+        pm, fgs = build_manager(cfg, tables, mlp, np.float16)
+        predictors = [make_predictor(pm, fgs, sparse[b], dense[b], np.float16) for b in range(fwd.n_batches)]
+        predictors[0].forward()
+        ref = fwd.output(0)
+        fwd.step(0)
         torch.cuda.synchronize()
-        graphs = []
-        for i in range(fwd.n_batches):
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                fwd.step(i)
-            graphs.append(g)
+        # (the fp16 model's output blob is fp16; the harness keeps the last layer's probabilities in fp32)
+        assert np.allclose(predictors[0].output_asnumpy("prob").astype(np.float32), ref.cpu().numpy(), atol=1e-3), \
+            "Predictor and kernel-layer harness disagree"
 
     import ctypes
-    S = max(1, min(args.streams, fwd.n_batches))
-    assert fwd.n_batches % S == 0, "--pool must be a multiple of --streams (a pooled batch always runs on one stream)"
-    streams = [torch.cuda.Stream() for _ in range(S)] if S > 1 else [torch.cuda.current_stream()]
+    import threading
+    streams = [torch.cuda.Stream() for _ in range(T)]
     stream_ptrs = [ctypes.c_void_p(st.cuda_stream) for st in streams]
 
-    def run_step(i, s=None):
-        s = i % S if s is None else s
-        if graphs is not None:
-            with torch.cuda.stream(streams[s]):
-                graphs[i % fwd.n_batches].replay()
+    def run_step(i, t):
+        if predictors is not None:
+            predictors[i % fwd.n_batches].forward()  # launches on the calling thread's stream and waits for it
         else:
-            fwd.step(i, stream_ptrs[s])
+            fwd.step(i, stream_ptrs[t])
 
     # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations
-    for i in range(W):
-        run_step(i)
-    torch.cuda.synchronize()
+    start = threading.Barrier(T + 1)
+    errors = []
+
+    def worker(t):
+        try:
+            for i in range(t, W, T):
+                run_step(i, t)
+            torch.cuda.synchronize()
+            start.wait()
+            for i in range(t, K, T):
+                run_step(W - (W % T) + i, t)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+            start.abort()
+
+    threads = [threading.Thread(target=worker, args=(t, )) for t in range(T)]
+    for th in threads:
+        th.start()
+    start.wait()
     t0 = time.perf_counter()
-    for i in range(K):
-        run_step(W + i)
+    for th in threads:
+        th.join()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    if errors:
+        raise errors[0]
     ms_per_step = (t1 - t0) * 1e3 / K
     samples_per_s = cfg.batch * K / (t1 - t0)
 
-    # ---- latency: each step submitted and waited for on its own
+    # ---- latency: one batch at a time on one thread, each step submitted and waited for on its own
     lat = []
     for i in range(min(K, 2000)):
         a = time.perf_counter()
         run_step(i, 0)
-        torch.cuda.synchronize()
+        if predictors is None:
+            torch.cuda.synchronize()
         lat.append((time.perf_counter() - a) * 1e3)
     lat = np.sort(np.array(lat))
     p50, p99 = float(lat[len(lat) // 2]), float(lat[int(len(lat) * 0.99)])
@@ -193,7 +231,9 @@ def main():
         "dtype": "f16",
         "data": "synthetic (seeded; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
         "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
-                   "batch_pool": fwd.n_batches, "submission": "per-kernel launches" if graphs is None else "hip graph per step", "predictor_streams": S,
+                   "batch_pool": fwd.n_batches,
+                   "path": "kernel-layer C ABI (bz_*)" if predictors is None else "Predictor.Forward via Blaze_* C ABI",
+                   "serving_threads": T,
                    "device": arch},
         "roofline": roofline,
         "embedding_pool": {"GB/s": round(pool_gbs, 1), "frac_of_hbm_peak": round(pool_gbs / HBM_PEAK_GBS, 5),

@@ -260,6 +260,25 @@ typedef struct bz_act_desc {
 
 BZ_API int bz_activation(const bz_act_desc* desc, bz_stream_t stream);
 
+/*
+ * Concatenate up to BZ_CONCAT_MAX row-major 2-D pieces side by side in ONE launch:
+ * dst[r, col_k .. col_k + width_k) = src_k[r, 0 .. width_k), widths in bytes.  Stands in for Concat along the
+ * last axis (blaze/operator/op/concat_op.cu:33), the op that joins the dense features with the embedding block
+ * in CTR graphs.
+ */
+#define BZ_CONCAT_MAX 16
+typedef struct bz_concat_desc {
+  const void* src[BZ_CONCAT_MAX];
+  int64_t width[BZ_CONCAT_MAX]; /* bytes per row of each piece (its rows are contiguous) */
+  void* dst;
+  int64_t dst_pitch;            /* bytes per output row */
+  int64_t rows;
+  int32_t n;
+  int32_t reserved_;
+} bz_concat_desc;
+
+BZ_API int bz_concat_cols(const bz_concat_desc* desc, bz_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,7 +21,7 @@ ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 
 EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
-    "bz_activation"
+    "bz_activation", "bz_concat_cols"
 ]
 
 
@@ -61,6 +61,11 @@ class ActDesc(C.Structure):
                 ("act_size", C.c_int32), ("dice_nosqrt", C.c_int32), ("act_alpha", C.c_float), ("reserved_", C.c_int32)]
 
 
+class ConcatDesc(C.Structure):
+    _fields_ = [("src", C.c_void_p * 16), ("width", C.c_int64 * 16), ("dst", C.c_void_p), ("dst_pitch", C.c_int64),
+                ("rows", C.c_int64), ("n", C.c_int32), ("reserved_", C.c_int32)]
+
+
 class BlazeHipError(RuntimeError):
     pass
 
@@ -91,6 +96,7 @@ def lib():
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
         l.bz_activation.argtypes = [C.POINTER(ActDesc), vp]
+        l.bz_concat_cols.argtypes = [C.POINTER(ConcatDesc), vp]
         _lib = l
     return _lib
 

@@ -94,7 +94,52 @@ __global__ __launch_bounds__(256) void bz_softmax_kernel(const T* __restrict__ x
   for (int64_t c = lane; c < cols; c += 64) stf<T>(yr + c, expf(ldf<T>(xr + c) - mx) / sum);
 }
 
+// side-by-side concatenation: blockIdx.y picks the piece, threads copy 16 bytes each when every address allows
+__global__ __launch_bounds__(256) void bz_concat_kernel(bz_concat_desc d) {
+  const int k = blockIdx.y;
+  const char* src = (const char*)d.src[k];
+  const int64_t width = d.width[k];
+  int64_t col = 0;
+  for (int i = 0; i < k; ++i) col += d.width[i];
+  char* dst = (char*)d.dst + col;
+  const bool vec = ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) && (width % 16 == 0) && (d.dst_pitch % 16 == 0);
+  if (vec) {
+    const int64_t cpr = width / 16, total = cpr * d.rows;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+      const int64_t r = i / cpr, c = i - r * cpr;
+      *(uint4*)(dst + r * d.dst_pitch + c * 16) = *(const uint4*)(src + r * width + c * 16);
+    }
+  } else {
+    const int64_t total = width * d.rows;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+      const int64_t r = i / width, c = i - r * width;
+      dst[r * d.dst_pitch + c] = src[r * width + c];
+    }
+  }
+}
+
 }  // namespace
+
+extern "C" int bz_concat_cols(const bz_concat_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_concat_cols: null descriptor");
+  const bz_concat_desc& d = *desc;
+  BZ_REQUIRE(d.n > 0 && d.n <= BZ_CONCAT_MAX && d.dst != nullptr && d.rows >= 0, "bz_concat_cols: n=%d rows=%lld", d.n,
+             (long long)d.rows);
+  int64_t total = 0, widest = 0;
+  for (int i = 0; i < d.n; ++i) {
+    BZ_REQUIRE(d.width[i] >= 0 && (d.width[i] == 0 || d.src[i] != nullptr), "bz_concat_cols: piece %d is null", i);
+    total += d.width[i];
+    widest = d.width[i] > widest ? d.width[i] : widest;
+  }
+  BZ_REQUIRE(total <= d.dst_pitch, "bz_concat_cols: pieces are %lld bytes wide, output rows only %lld", (long long)total,
+             (long long)d.dst_pitch);
+  if (d.rows == 0 || widest == 0) return BZ_OK;
+  const int64_t work = (widest / 16 + 1) * d.rows;
+  const int gx = (int)(((work + 255) / 256) < 2048 ? ((work + 255) / 256) : 2048);
+  hipLaunchKernelGGL(bz_concat_kernel, dim3(gx, d.n), dim3(256), 0, bz::as_stream(stream), d);
+  BZ_LAUNCH_OK("bz_concat_kernel");
+  return BZ_OK;
+}
 
 extern "C" int bz_activation(const bz_act_desc* desc, bz_stream_t stream) {
   BZ_REQUIRE(desc != nullptr, "bz_activation: null descriptor");

@@ -13,6 +13,7 @@
 #include "blaze/operator.h"
 #include "blaze_hip.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace blaze {
@@ -290,13 +291,24 @@ class ConcatOp final : public Operator<Context> {
     const size_t es = DataTypeSize(y->data_type());
     const TIndex outer = y->size(0, axis_), inner = y->size(axis_ + 1, (int)rank);
     hipStream_t st = context_.hip_stream();
+    // one launch per group of BZ_CONCAT_MAX pieces
     size_t col = 0;
-    for (int i = 0; i < this->InputSize(); ++i) {
-      Blob* x = this->Input(i);
-      const size_t width = x->shape()[axis_] * inner * es;
-      if (width > 0 && outer > 0)
-        HIP_CHECK(hipMemcpy2DAsync((char*)y->data() + col, total * inner * es, x->data(), width, width, outer, hipMemcpyDeviceToDevice, st));
-      col += width;
+    for (int i0 = 0; i0 < this->InputSize(); i0 += BZ_CONCAT_MAX) {
+      bz_concat_desc d;
+      memset(&d, 0, sizeof(d));
+      d.n = std::min(BZ_CONCAT_MAX, this->InputSize() - i0);
+      size_t group = 0;
+      for (int i = 0; i < d.n; ++i) {
+        Blob* x = this->Input(i0 + i);
+        d.src[i] = x->data();
+        d.width[i] = (int64_t)(x->shape()[axis_] * inner * es);
+        group += (size_t)d.width[i];
+      }
+      d.dst = (char*)y->data() + col;  // this group starts `col` bytes into every output row
+      d.dst_pitch = (int64_t)(total * inner * es);
+      d.rows = (int64_t)outer;
+      BZ_CHECK(bz_concat_cols(&d, st));
+      col += group;
     }
     return true;
   }
