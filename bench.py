@@ -22,6 +22,11 @@ sys.path.insert(1, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
+# HBM-side bytes per launch of the pooling kernel on this exact workload (default seed, pool of 32 batches), from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, averaged over 1704 dispatches) scaled by what the same
+# counters read for a plain 256 MiB copy (`--calibrate-copy`: FETCH_SIZE reads 0.5 of the bytes, WRITE_SIZE all of them):
+# fetch 11983.05 KiB x 2.0 + write 3335.43 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
+POOL_TRAFFIC_BYTES = int((11983.05 * 2.0 + 3335.43) * 1024)
 
 
 def main():
@@ -37,6 +42,9 @@ def main():
     ap.add_argument("--threads", type=int, default=8,
                     help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
                          "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
+    ap.add_argument("--with-feed", action="store_true",
+                    help="also time steps that Feed every input from host memory and copy the output back (the "
+                         "PCIe-inclusive rate; reported as an extra key, never as `value`)")
     ap.add_argument("--kernel-api", action="store_true",
                     help="drive the kernel-layer C ABI directly instead of Predictor.Forward (lower host overhead)")
     args = ap.parse_args()
@@ -145,6 +153,37 @@ def main():
     lat = np.sort(np.array(lat))
     p50, p99 = float(lat[len(lat) // 2]), float(lat[int(len(lat) * 0.99)])
 
+    # ---- PCIe-inclusive rate: every step feeds all 79 inputs from pageable host memory and copies the output back
+    feed_rate = None
+    if args.with_feed and predictors is not None:
+        fT = T
+        n_feed = max(fT, min(K, 400) // fT * fT)
+        fbar = threading.Barrier(fT + 1)
+
+        def feed_worker(t):
+            from ctr_model import feed_inputs
+            for i in range(t, n_feed + 2 * fT, fT):
+                if i == t + 2 * fT:
+                    fbar.wait()
+                b = i % fwd.n_batches
+                feed_inputs(predictors[b], fgs, sparse[b], dense[b], np.float16)
+                predictors[b].forward()
+                predictors[b].output_asnumpy("prob")
+
+        ths = [threading.Thread(target=feed_worker, args=(t, )) for t in range(fT)]
+        for th in ths:
+            th.start()
+        fbar.wait()
+        f0 = time.perf_counter()
+        for th in ths:
+            th.join()
+        f1 = time.perf_counter()
+        in_bytes = float(np.mean([sum(a.nbytes for trip in sparse[b] for a in trip) + dense[b].size * 2
+                                  for b in range(fwd.n_batches)]))
+        feed_rate = {"samples/s": round(cfg.batch * n_feed / (f1 - f0), 1), "ms_per_step": round((f1 - f0) * 1e3 / n_feed, 4),
+                     "host_bytes_per_step": int(in_bytes), "steps": n_feed, "threads": fT,
+                     "note": "Feed of every input from pageable host memory + Forward + Output copy, per step"}
+
     # ---- per-kernel durations: HIP events on the launch stream around a replayed HIP graph that holds
     # R back-to-back launches of the one kernel (over the pooled batches), so host launch cost is not in it
     def timed(fn, reps):
@@ -184,7 +223,8 @@ def main():
                     "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK_TFLOPS, 5), "traffic": None}
     else:
         roofline = {"kernel": "bz_embed_pool_kernel", "bound": "hbm", "achieved": round(pool_gbs, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(pool_gbs / HBM_PEAK_GBS, 5), "traffic": None,
+                    "unit": "GB/s", "frac": round(pool_gbs / HBM_PEAK_GBS, 5),
+                    "traffic": POOL_TRAFFIC_BYTES if args.pool == 32 else None,
                     "algorithmic_bytes_per_launch": int(emb_bytes), "avg_launch_us": round(pool_us, 2)}
 
     # ---- CPU baseline: the oracle (a scalar port of the reference's CPU path), one predictor per thread
@@ -196,7 +236,7 @@ def main():
         tabs = [orc.Table(t.cpu().numpy()) for t in tables]
         mlp_np = [(w.cpu().numpy(), b.cpu().numpy(), s.cpu().numpy()) for (w, b, s) in mlp]
         threads = max(1, min(16, len(os.sched_getaffinity(0))))
-        per_thread = 1
+        per_thread = 2
         def worker(t):
             for j in range(per_thread):
                 b = (t * per_thread + j) % len(sparse)
@@ -243,6 +283,8 @@ def main():
         "kernel_us": {k: round(v, 2) for k, v in kern_us.items()},
         "cpu_baseline": cpu,
     }
+    if feed_rate is not None:
+        out["with_host_feed"] = feed_rate
     print(json.dumps(out))
 
 

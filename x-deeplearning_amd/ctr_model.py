@@ -51,9 +51,13 @@ def build_manager(cfg, tables, mlp, dtype=np.float16):
 
 def make_predictor(pm, fgs, sparse, dense, dtype=np.float16):
     p = pm.create_predictor(1, 0)
+    feed_inputs(p, fgs, sparse, dense, dtype)
+    return p
+
+
+def feed_inputs(p, fgs, sparse, dense, dtype=np.float16):
     for (fg, _, _), (ids, vals, seg) in zip(fgs, sparse):
         p.feed(fg + ".ids", ids)
         p.feed(fg + ".values", vals)
         p.feed(fg + ".segments", seg)
     p.feed("dense", dense.astype(dtype))
-    return p
