@@ -1,0 +1,192 @@
+"""The benchmark configurations at their full sizes, as parity cases (GPU).
+
+config 1 (fp32, batch 128) runs through Predictor.Forward and is compared with the CPU oracle end to end:
+pooled block bit-exact, probabilities rel 1e-5.  config 4 (int8 + per-row scale, 34 GB of tables) and
+config 5 (fp16 tables, 102 GB; bf16 MLP whose first layer is 215 GFLOP) are generated on the device; the
+oracle sees only the rows a batch touches (copied back and indexed by key).  Tolerance for the fp16 / bf16 /
+int8 paths: 2e-3 against the fp32 oracle fed the same rounded inputs.  Size-independent properties checked at
+full size: scaling all values by 2 doubles every pooled element exactly; an empty segment gives a zero row.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def bz():
+    import torch
+    import blaze_hip
+    assert torch.cuda.is_available(), "no GPU visible"
+    blaze_hip.device_check()
+    return blaze_hip
+
+
+def _touched_table(oracle, dev_rows, ids, dev_scale=None):
+    """Oracle table holding only the rows `ids` name, keyed by id (the device indexes the full table by row)."""
+    import torch
+    uniq = np.unique(ids)
+    idx = torch.from_numpy(uniq).cuda()
+    rows = dev_rows[idx].cpu().numpy()
+    scale = None if dev_scale is None else dev_scale[idx].cpu().numpy()
+    return oracle.Table(rows, scale=scale, keys=uniq.astype(np.uint64))
+
+
+def _bf16_round(x):
+    """fp32 -> nearest-even bf16, back to fp32 (numpy)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16
+    return r.astype(np.uint32).view(np.float32)
+
+
+def test_config1_fp32_end_to_end_through_predictor(oracle):
+    import torch
+    from ctr_model import build_manager, make_predictor
+    from pipeline import oracle_forward
+    from synth import Config1
+    cfg = Config1()
+    print("config1 full size: batch %d, %d x [%d,%d] fp32" % (cfg.batch, cfg.slots, cfg.rows, cfg.dim), flush=True)
+    tables, mlp = cfg.tables(), cfg.mlp()
+    sparse, dense = cfg.batches(2)
+    pm, fgs = build_manager(cfg, tables, mlp, np.float32, expose_block=True)
+    tabs = [oracle.Table(t.cpu().numpy()) for t in tables]
+    mlp_np = [(w.cpu().numpy(), b.cpu().numpy(), s.cpu().numpy()) for (w, b, s) in mlp]
+    for b in range(2):
+        p = make_predictor(pm, fgs, sparse[b], dense[b], np.float32)
+        p.forward()
+        prob = p.output_asnumpy("prob")
+        block = p.output_asnumpy("block")
+        want_pooled, want_prob = oracle_forward(oracle, cfg, tabs, mlp_np, sparse[b], dense[b])
+        # pooled block: bit-exact (same summation order, unfused multiply/add)
+        assert np.array_equal(block.view(np.uint32), want_pooled[:, cfg.dense:].view(np.uint32))
+        assert prob.shape == (cfg.batch, 2)
+        np.testing.assert_allclose(prob, want_prob, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(prob.sum(1), 1.0, rtol=1e-5)
+    torch.cuda.synchronize()
+
+
+@pytest.mark.timeout(400)
+def test_config4_int8_kavg_full_size(bz, oracle):
+    import torch
+    torch.cuda.empty_cache()
+    from synth import Config4
+    cfg = Config4()
+    free, _ = torch.cuda.mem_get_info()
+    need = cfg.slots * cfg.rows * (cfg.dim + 4)
+    if free < need * 1.1:
+        pytest.skip("needs %.0f GB of free HBM" % (need / 1e9))
+    print("config4 full size: batch %d, %d x [%d,%d] int8 + scale" % (cfg.batch, cfg.slots, cfg.rows, cfg.dim), flush=True)
+    tables = cfg.tables()
+    # Poisson(20) practically never draws 0: empty every 97th segment so that the zero-row case is in
+    rng = np.random.default_rng(44)
+    sparse = []
+    for ids, vals, seg in cfg.batch_inputs():
+        off = np.concatenate([[0], np.cumsum(seg)])
+        drop = np.zeros(ids.size, bool)
+        for b in range(int(rng.integers(0, 97)), cfg.batch, 97):
+            drop[off[b]:off[b + 1]] = True
+            seg[b] = 0
+        sparse.append((ids[~drop], vals[~drop], seg))
+    dts = [bz.DeviceTable(q, scale=sc) for q, sc in tables]
+    B, D = cfg.batch, cfg.dim
+
+    def run(scale_values, out_dtype):
+        out = torch.full((B, cfg.slots * D), float("nan"), dtype=out_dtype, device="cuda")
+        items, keep = [], []
+        for s, (ids, vals, seg) in enumerate(sparse):
+            t = [torch.from_numpy(ids).cuda(), torch.from_numpy(vals * np.float32(scale_values)).cuda(), torch.from_numpy(seg).cuda()]
+            keep.append(t)
+            items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=out, col=s * D, udf=bz.AVG))
+        bz.EmbeddingPlan(items).run()
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    got32 = run(1.0, torch.float32)
+    got16 = run(1.0, torch.float16)
+    want = np.zeros((B, cfg.slots * D), np.float32)
+    for s, (ids, vals, seg) in enumerate(sparse):
+        tab = _touched_table(oracle, tables[s][0], ids, tables[s][1])
+        oracle.embed_get(tab, ids, vals, seg, [(1, 0, 0, want, s * D)])
+    # fp32 block: the int8 extension is defined as w = scale*(float)q, then the reference's kavg: bit-exact
+    assert np.array_equal(got32.view(np.uint32), want.view(np.uint32))
+    # fp16 block = that result rounded to nearest even (contract 2e-3)
+    assert np.array_equal(got16.view(np.uint16), want.astype(np.float16).view(np.uint16))
+    np.testing.assert_allclose(got16.astype(np.float32), want, rtol=2e-3, atol=2e-3 * np.abs(want).max())
+    # empty segments are zero rows
+    for s, (_, _, seg) in enumerate(sparse[:5]):
+        empty = np.nonzero(seg == 0)[0]
+        assert empty.size and not got32[empty, s * D:(s + 1) * D].any()
+    # linearity in the values (a power of two is exact): pool(2*v) == 2*pool(v)
+    got2 = run(2.0, torch.float32)
+    assert np.array_equal(got2.view(np.uint32), (got32 * np.float32(2.0)).view(np.uint32))
+
+
+@pytest.mark.timeout(400)
+def test_config5_fp16_tables_bf16_tower_full_size(bz, oracle):
+    import torch
+    torch.cuda.empty_cache()
+    from synth import Config5
+    cfg = Config5()
+    free, _ = torch.cuda.mem_get_info()
+    need = cfg.slots * cfg.rows * cfg.dim * 2
+    if free < need * 1.6:  # generation goes through an fp32 temporary of one table
+        pytest.skip("needs %.0f GB of free HBM" % (need * 1.6 / 1e9))
+    print("config5 full size: batch %d, %d x [%d,%d] fp16, MLP %s bf16" % (cfg.batch, cfg.slots, cfg.rows, cfg.dim, cfg.layers),
+          flush=True)
+    tables = cfg.tables()
+    sparse = cfg.batch_inputs()
+    mlp = cfg.mlp()
+    dts = [bz.DeviceTable(t) for t in tables]
+    B, D = cfg.batch, cfg.dim
+    pooled32 = torch.full((B, cfg.slots * D), float("nan"), dtype=torch.float32, device="cuda")
+    pooled = torch.full((B, cfg.slots * D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    keep = []
+    for out in (pooled32, pooled):
+        items = []
+        for s, (ids, vals, seg) in enumerate(sparse):
+            t = [torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(), torch.from_numpy(seg).cuda()]
+            keep.append(t)
+            items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=out, col=s * D, udf=bz.SUM))
+        bz.EmbeddingPlan(items).run()
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(5)
+    rows = np.sort(rng.choice(B, 64, replace=False))
+    # oracle pooling of every sample for 8 slots, of the 64 sampled rows for all slots
+    want_rows = np.zeros((64, cfg.slots * D), np.float32)
+    got32 = pooled32.cpu().numpy()
+    for s, (ids, vals, seg) in enumerate(sparse):
+        off = np.concatenate([[0], np.cumsum(seg)])
+        if s % 25 == 0:
+            full = np.zeros((B, D), np.float32)
+            oracle.embed_get(_touched_table(oracle, tables[s], ids), ids, vals, seg, [(0, 0, 0, full, 0)])
+            assert np.array_equal(got32[:, s * D:(s + 1) * D].view(np.uint32), full.view(np.uint32))
+        sel = np.concatenate([np.arange(off[r], off[r + 1]) for r in rows])
+        sub = np.zeros((64, D), np.float32)
+        oracle.embed_get(_touched_table(oracle, tables[s], ids[sel]), ids[sel], vals[sel], seg[rows], [(0, 0, 0, sub, 0)])
+        want_rows[:, s * D:(s + 1) * D] = sub
+    assert np.array_equal(got32[rows].view(np.uint32), want_rows.view(np.uint32))  # fp32 block: bit-exact
+    x0 = _bf16_round(want_rows)
+    assert np.array_equal(pooled[torch.from_numpy(rows).cuda()].float().cpu().numpy().view(np.uint32), x0.view(np.uint32))
+
+    # MLP in bf16 (fp32 accumulate); oracle: fp32 path fed the same bf16-rounded inputs, first layer also in fp64
+    x = pooled
+    h = x0
+    n_layers = len(mlp)
+    for li, (w, b) in enumerate(mlp):
+        last = li == n_layers - 1
+        wp = bz.pack_weight(w, False, bz.BF16)
+        y = torch.empty((B, w.shape[1]), dtype=torch.float32 if last else torch.bfloat16, device="cuda")
+        print("fc layer %d: %dx%d . %dx%d" % (li, B, w.shape[0], w.shape[0], w.shape[1]), flush=True)
+        bz.fc_fused(x, wp, w.shape[0], bias=b, act=bz.ACT_SIGMOID if last else bz.ACT_LEAKY_RELU, act_alpha=0.0, out=y)
+        torch.cuda.synchronize()
+        w_r = _bf16_round(w.cpu().numpy())
+        got = y[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+        if li == 0:
+            ref64 = h.astype(np.float64) @ w_r.astype(np.float64) + b.cpu().numpy().astype(np.float64)
+            ref64 = np.where(ref64 >= 0, ref64, 0.0)
+            np.testing.assert_allclose(got, ref64, rtol=2e-3, atol=2e-3 * np.abs(ref64).max())
+        want = oracle.fc(h, w_r, b.cpu().numpy(), act="sigmoid" if last else "relu")
+        np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3 * max(1e-3, float(np.abs(want).max())))
+        h = want if last else _bf16_round(want)
+        x = y
+    assert got.shape == (64, 1) and np.all((got > 0) & (got < 1))

@@ -158,6 +158,13 @@ __device__ __forceinline__ int64_t resolve_row(const bz_embed_slot& s, int64_t i
   return (id >= 0 && id < s.rows) ? id : -1;
 }
 
+// fp32 -> bf16 bit pattern, round to nearest even; NaN stays a quiet NaN
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
 // Store `nvalid` fp32 results as the slot's output dtype at element pointer `dst`
 // using the widest store the address allows.
 template <int N>
@@ -173,13 +180,19 @@ __device__ __forceinline__ void store_elems(void* dst_base, int64_t elem_off, co
       for (int i = 0; i < N; ++i)
         if (i < nvalid) dst[i] = v[i];
     }
-  } else {  // BZ_F16, round to nearest even
-    __half* dst = (__half*)dst_base + elem_off;
+  } else {  // BZ_F16 / BZ_BF16, round to nearest even
+    __half* dst = (__half*)dst_base + elem_off;  // (a 16-bit slot; bf16 bits travel through the same stores)
     uint32_t pk[N / 2];
 #pragma unroll
     for (int i = 0; i < N / 2; ++i) {
-      uint32_t lo = __half_as_ushort(__float2half_rn(v[2 * i]));
-      uint32_t hi = __half_as_ushort(__float2half_rn(v[2 * i + 1]));
+      uint32_t lo, hi;
+      if (out_dtype == BZ_F16) {
+        lo = __half_as_ushort(__float2half_rn(v[2 * i]));
+        hi = __half_as_ushort(__float2half_rn(v[2 * i + 1]));
+      } else {
+        lo = f32_to_bf16_bits(v[2 * i]);
+        hi = f32_to_bf16_bits(v[2 * i + 1]);
+      }
       pk[i] = lo | (hi << 16);
     }
     const uintptr_t a = (uintptr_t)dst;
@@ -527,7 +540,8 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
     bz_embed_slot& s = slots[i];
     BZ_REQUIRE(s.table_dtype == BZ_F32 || s.table_dtype == BZ_F16 || s.table_dtype == BZ_I8,
                "slot %d: unsupported table dtype %d", i, s.table_dtype);
-    BZ_REQUIRE(s.out_dtype == BZ_F32 || s.out_dtype == BZ_F16, "slot %d: unsupported out dtype %d", i, s.out_dtype);
+    BZ_REQUIRE(s.out_dtype == BZ_F32 || s.out_dtype == BZ_F16 || s.out_dtype == BZ_BF16, "slot %d: unsupported out dtype %d", i,
+               s.out_dtype);
     BZ_REQUIRE(s.udf == BZ_SUM || s.udf == BZ_AVG || s.udf == BZ_ASSIGN, "slot %d: Unsupported udf type: %d", i, s.udf);
     BZ_REQUIRE(s.dim > 0 && s.batch >= 0, "slot %d: dim=%d batch=%d", i, s.dim, s.batch);
     if (s.udf == BZ_ASSIGN)

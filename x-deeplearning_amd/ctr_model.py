@@ -10,8 +10,9 @@ import numpy as np
 import pyblaze_hip as pb
 
 
-def build_manager(cfg, tables, mlp, dtype=np.float16):
-    """tables: list of torch cuda tensors [rows, dim]; mlp: [(W [K,N], b, slope)] torch tensors."""
+def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False):
+    """tables: list of torch cuda tensors [rows, dim]; mlp: [(W [K,N], b, slope)] torch tensors.
+    expose_block: also declare the pooled Embedding block an output of the net (for parity checks)."""
     code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
     pm = pb.PredictorManager()
     fgs = []
@@ -28,6 +29,8 @@ def build_manager(cfg, tables, mlp, dtype=np.float16):
         inputs += [fg + ".ids", fg + ".values", fg + ".segments"]
     nb.external_input("dense", code)
     nb.external_output("prob", pb.K_FLOAT)
+    if expose_block:
+        nb.external_output("block", code)
     for li, (w, b, slope) in enumerate(mlp):
         nb.constant("w%d" % li, w.float().cpu().numpy(), dtype=code)
         nb.constant("b%d" % li, b.float().cpu().numpy(), dtype=pb.K_FLOAT if li == len(mlp) - 1 else code)
