@@ -67,7 +67,8 @@ def main():
         src = torch.ones(rows * width, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
         d = bz.ConcatDesc()
-        d.src[0], d.width[0], d.dst, d.dst_pitch, d.rows, d.n = src.data_ptr(), width, dst.data_ptr(), width, rows, 1
+        d.src[0], d.width[0], d.src_pitch[0] = src.data_ptr(), width, width
+        d.dst, d.dst_pitch, d.rows, d.n = dst.data_ptr(), width, rows, 1
         for _ in range(5):
             bz.check(bz.lib().bz_concat_cols(ctypes.byref(d), None))
         torch.cuda.synchronize()

@@ -269,7 +269,9 @@ BZ_API int bz_activation(const bz_act_desc* desc, bz_stream_t stream);
 #define BZ_CONCAT_MAX 16
 typedef struct bz_concat_desc {
   const void* src[BZ_CONCAT_MAX];
-  int64_t width[BZ_CONCAT_MAX]; /* bytes per row of each piece (its rows are contiguous) */
+  int64_t width[BZ_CONCAT_MAX];     /* bytes per row of each piece */
+  int64_t src_pitch[BZ_CONCAT_MAX]; /* bytes between rows of each piece; 0 repeats its one row for every output row
+                                       (Fuse, blaze/operator/op/fuse_op.cc:11-33) */
   void* dst;
   int64_t dst_pitch;            /* bytes per output row */
   int64_t rows;
@@ -278,6 +280,67 @@ typedef struct bz_concat_desc {
 } bz_concat_desc;
 
 BZ_API int bz_concat_cols(const bz_concat_desc* desc, bz_stream_t stream);
+
+/*
+ * Elementwise ops with multidirectional broadcasting, the shape rule of blaze/math/broadcast.h:39-67:
+ * Add / Sub / Mul / Div (blaze/operator/op/elementwise_op.cc:28-165, elementwise_op.cu:55-140),
+ * BroadcastTo (elementwise_op.h:193-226) and Where (elementwise_op.h:228-283; condition int32 | int64, nonzero
+ * picks x).  Operands are described by element strides over the OUTPUT's dims (0 on a broadcast dim), so any
+ * operand layout that is a strided view works.  One fp32 operation per element; fp16 / bf16 tensors are widened,
+ * computed in fp32 and rounded once.
+ */
+#define BZ_MAX_RANK 6
+typedef enum bz_ew_op { BZ_EW_ADD = 0, BZ_EW_SUB = 1, BZ_EW_MUL = 2, BZ_EW_DIV = 3, BZ_EW_ASSIGN = 4, BZ_EW_WHERE = 5 } bz_ew_op;
+typedef struct bz_bcast_desc {
+  const void* a;    /* first operand; the condition for BZ_EW_WHERE */
+  const void* b;    /* second operand (unused by BZ_EW_ASSIGN); x for BZ_EW_WHERE */
+  const void* c;    /* y for BZ_EW_WHERE, else unused */
+  void* out;        /* contiguous, row major over dims[] */
+  int64_t dims[BZ_MAX_RANK];
+  int64_t a_stride[BZ_MAX_RANK];
+  int64_t b_stride[BZ_MAX_RANK];
+  int64_t c_stride[BZ_MAX_RANK];
+  int32_t rank;
+  int32_t op;       /* bz_ew_op */
+  int32_t dtype;    /* BZ_F32 | BZ_F16 | BZ_BF16: type of the value operands and of out */
+  int32_t cond_dtype; /* BZ_I32 | BZ_I64 (BZ_EW_WHERE) */
+} bz_bcast_desc;
+
+BZ_API int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream);
+
+/*
+ * ReduceSum over the middle axis of a contiguous [outer, dim, inner] tensor -> [outer, inner], added in ascending
+ * order of the axis like blaze/math/reduce.cc:13-29 (fp32 accumulate; bit-exact for fp32 tensors).
+ */
+BZ_API int bz_reduce_sum(const void* x, void* y, int64_t outer, int64_t dim, int64_t inner, int dtype, bz_stream_t stream);
+
+/*
+ * BatchNormalization, inference form (blaze/operator/op/batch_normalization_op.cc:11-18):
+ * y = gamma[c] * (x - mean[c]) / (nosqrt ? var[c] : sqrtf(var[c] + eps)) + beta[c], c = flat index % channels.
+ * Parameters are fp32 vectors of `channels` elements.
+ */
+typedef struct bz_bn_desc {
+  const void* x;
+  void* y;
+  const float* gamma;
+  const float* beta;
+  const float* mean;
+  const float* var;
+  int64_t size;
+  int64_t channels;
+  int32_t dtype;  /* BZ_F32 | BZ_F16 | BZ_BF16 */
+  int32_t nosqrt;
+  float eps;
+  int32_t reserved_;
+} bz_bn_desc;
+
+BZ_API int bz_batch_norm(const bz_bn_desc* desc, bz_stream_t stream);
+
+/*
+ * Softmax over the middle axis of a contiguous [outer, c, inner] tensor (blaze/operator/op/softmax_op.cc:21-78:
+ * max-subtracted, exp, sum in ascending order of the axis, divide).  inner == 1 is the row softmax of bz_activation.
+ */
+BZ_API int bz_softmax_axis(const void* x, void* y, int64_t outer, int64_t c, int64_t inner, int dtype, bz_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -633,3 +633,28 @@ ORC_API void orc_softmax(const float* x, float* y, int64_t n, int64_t c, int64_t
     }
   }
 }
+
+/* ReduceSum over the middle axis of [outer, dim, inner]: math/reduce.cc:13-29 (y zeroed, then rows of
+ * `inner` added in ascending j). */
+ORC_API void orc_reduce_sum(const float* x, int64_t outer, int64_t dim, int64_t inner, float* y) {
+  for (int64_t i = 0; i < outer; ++i) {
+    for (int64_t k = 0; k < inner; ++k) y[k] = 0.f;
+    for (int64_t j = 0; j < dim; ++j) {
+      for (int64_t k = 0; k < inner; ++k) y[k] = y[k] + x[k];
+      x += inner;
+    }
+    y += inner;
+  }
+}
+
+/* BatchNormalization (inference): operator/op/batch_normalization_op.cc:11-18; channel = flat index % c. */
+ORC_API void orc_batch_norm(const float* x, int64_t size, const float* gamma, const float* beta, const float* mean,
+                            const float* var, int64_t c, int nosqrt, float eps, float* y) {
+  for (int64_t i = 0; i < size; ++i) {
+    int64_t o = i % c;
+    float den = nosqrt ? var[o] : sqrtf(var[o] + eps);
+    float xn = (x[i] - mean[o]) / den;
+    float g = gamma[o] * xn;
+    y[i] = g + beta[o];
+  }
+}

@@ -90,6 +90,8 @@ def _declare(l):
     l.orc_leaky_relu.argtypes = [vp, vp, i64, f32]
     l.orc_sigmoid.argtypes = [vp, vp, i64]
     l.orc_softmax.argtypes = [vp, vp, i64, i64, i64]
+    l.orc_reduce_sum.argtypes = [vp, i64, i64, i64, vp]
+    l.orc_batch_norm.argtypes = [vp, i64, vp, vp, vp, vp, i64, C.c_int, f32, vp]
 
 
 def _p(a):
@@ -392,6 +394,117 @@ def softmax(x, axis=1):
     w = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
     y = np.empty_like(x)
     lib().orc_softmax(_p(x), _p(y), n, c, w)
+    return y
+
+
+# ------------------------------------------------------------- shape / elementwise ops around the attention unit
+def reshape(x, shape):
+    """Reshape op (operator/op/reshape_op.h:22-52): 0 keeps the input's dim at that position, one negative
+    entry is inferred; the output aliases the input."""
+    x = np.asarray(x)
+    new = []
+    unknown = -1
+    known = 1
+    for i, d in enumerate(shape):
+        if d == 0:
+            new.append(x.shape[i])
+            known *= new[-1]
+        elif d < 0:
+            assert unknown < 0, "can not support two unknown dims"
+            unknown = i
+            new.append(-1)
+        else:
+            new.append(int(d))
+            known *= int(d)
+    if unknown >= 0:
+        new[unknown] = x.size // known
+    else:
+        assert known == x.size
+    return x.reshape(new)
+
+
+def concat(xs, axis=1):
+    """Concat op (operator/op/concat_op.h:46-121, concat_op.cc): same rank, equal dims off the axis."""
+    xs = [np.asarray(x) for x in xs]
+    assert all(x.ndim == xs[0].ndim and x.dtype == xs[0].dtype for x in xs) and axis < xs[0].ndim
+    return np.concatenate(xs, axis=axis)
+
+
+def _broadcast_shape(a, b):
+    """MBroadcasting::BroadcastShape (math/broadcast.h:39-67): right-aligned, dims equal or one of them 1."""
+    n = max(len(a), len(b))
+    a = (1, ) * (n - len(a)) + tuple(a)
+    b = (1, ) * (n - len(b)) + tuple(b)
+    out = []
+    for x, y in zip(a, b):
+        assert x == y or x == 1 or y == 1, "not equal or meet broadcast rule"
+        out.append(max(x, y))
+    return tuple(out)
+
+
+def elementwise(op, a, b):
+    """Add / Sub / Mul / Div ops (operator/op/elementwise_op.cc:28-165): one IEEE fp32 operation per output
+    element under multidirectional broadcasting."""
+    a, b = _f32(a), _f32(b)
+    shape = _broadcast_shape(a.shape, b.shape)
+    a, b = np.broadcast_to(a, shape), np.broadcast_to(b, shape)
+    with np.errstate(all="ignore"):
+        y = {"Add": np.add, "Sub": np.subtract, "Mul": np.multiply, "Div": np.divide}[op](a, b, dtype=np.float32)
+    return np.ascontiguousarray(y)
+
+
+def broadcast_to(a, like=None, shape=None):
+    """BroadcastTo op (operator/op/elementwise_op.h:193-226): to the shape of a second input, or to the `shape`
+    argument where entries > 0 replace the input's dim (same rank)."""
+    a = np.asarray(a)
+    if like is not None:
+        target = tuple(np.asarray(like).shape)
+    else:
+        assert len(shape) == a.ndim
+        target = tuple(int(s) if s > 0 else a.shape[i] for i, s in enumerate(shape))
+    return np.ascontiguousarray(np.broadcast_to(a, target))
+
+
+def where(cond, x, y):
+    """Where op (operator/op/elementwise_op.h:228-283, elementwise_op.cc WhereKernel): nonzero condition
+    (int32 | int64) picks x, else y, all three broadcast together."""
+    cond, x, y = np.asarray(cond), _f32(x), _f32(y)
+    assert cond.dtype in (np.int32, np.int64)
+    shape = _broadcast_shape(_broadcast_shape(cond.shape, x.shape), y.shape)
+    return np.ascontiguousarray(np.where(np.broadcast_to(cond, shape) != 0, np.broadcast_to(x, shape), np.broadcast_to(y, shape)))
+
+
+def reduce_sum(x, axis=0, keepdims=1):
+    """ReduceSum op (operator/op/reduce_sum_op.h:17-58)."""
+    x = _f32(x)
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    dim = x.shape[axis]
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    shape = list(x.shape[:axis]) + ([1] if keepdims else []) + list(x.shape[axis + 1:])
+    y = np.empty(shape, np.float32)
+    lib().orc_reduce_sum(_p(x), outer, dim, inner, _p(y))
+    return y
+
+
+def fuse(x1, x2, comm_index=0):
+    """Fuse op (operator/op/fuse_op.h:35-75, fuse_op.cc:11-33): column concat of two 2-D inputs where the
+    `comm_index` one has a single row that is repeated for every row of the other."""
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    assert x1.ndim == 2 and x2.ndim == 2 and (x1, x2)[comm_index].shape[0] == 1
+    m = max(x1.shape[0], x2.shape[0])
+    if x1.shape[0] == 1:
+        x1 = np.broadcast_to(x1, (m, x1.shape[1]))
+    else:
+        x2 = np.broadcast_to(x2[:1], (m, x2.shape[1]))
+    return np.ascontiguousarray(np.concatenate([x1, x2], axis=1))
+
+
+def batch_norm(x, gamma, beta, mean, var, eps=0.001, nosqrt=False):
+    """BatchNormalization op, inference form (operator/op/batch_normalization_op.cc:11-45)."""
+    x, gamma, beta, mean, var = _f32(x), _f32(gamma), _f32(beta), _f32(mean), _f32(var)
+    assert gamma.size == beta.size == mean.size == var.size
+    y = np.empty_like(x)
+    lib().orc_batch_norm(_p(x), x.size, _p(gamma), _p(beta), _p(mean), _p(var), gamma.size, int(nosqrt), eps, _p(y))
     return y
 
 

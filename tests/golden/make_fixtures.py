@@ -37,6 +37,24 @@ CASES = [
     "fused_op/fused_parallel_matmul/fused_parallel_matmul_net_v2_cpu.conf",
     "fused_op/fused_parallel_matmul/fused_parallel_matmul_net_v3_cpu.conf",
     "sparse_op/embedding/embedding_v1.conf",
+    "op/concat/concat_net_v1_cpu.conf",
+    "op/concat/concat_net_v2_cpu.conf",
+    "op/reduce_sum/reduce_sum_net_v1_cpu.conf",
+    "op/fuse/fuse_net_v1_cpu.conf",
+    "op/fuse/fuse_net_v2_cpu.conf",
+    "op/reshape/reshape_net_v1_cpu.conf",
+    "op/batch_normalization/batch_normalization_net_v1_cpu.conf",
+    "op/elementwise/elementwise_add_net_v1_cpu.conf",
+    "op/elementwise/elementwise_add_net_v2_cpu.conf",
+    "op/elementwise/elementwise_sub_net_v1_cpu.conf",
+    "op/elementwise/elementwise_sub_net_v2_cpu.conf",
+    "op/elementwise/elementwise_mul_net_v1_cpu.conf",
+    "op/elementwise/elementwise_mul_net_v2_cpu.conf",
+    "op/elementwise/elementwise_div_net_v1_cpu.conf",
+    "op/elementwise/elementwise_div_net_v2_cpu.conf",
+    "op/elementwise/elementwise_broadcast_to_net_v1_cpu.conf",
+    "op/elementwise/elementwise_broadcast_to_net_v2_cpu.conf",
+    "op/elementwise/elementwise_where_net_v1_cpu.conf",
 ]
 
 _TOK = re.compile(r'\s*(?:(#[^\n]*)|("(?:\\.|[^"\\])*")|([{}:])|([^\s{}:"#]+))')

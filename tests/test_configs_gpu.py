@@ -190,3 +190,57 @@ def test_config5_fp16_tables_bf16_tower_full_size(bz, oracle):
         h = want if last else _bf16_round(want)
         x = y
     assert got.shape == (64, 1) and np.all((got > 0) & (got < 1))
+
+
+@pytest.mark.timeout(400)
+def test_config3_din_attention_end_to_end_through_predictor(oracle):
+    """config 3 at full size through Predictor.Forward: two Embedding ops (ksum target, kassign history), the
+    attention unit built from Reshape / Concat / Sub / Mul / BroadcastTo / 3-D Gemm + Dice / Mul(mask) / MatMul /
+    ReduceSum, the main MLP with Dice, softmax.  fp16 model against the fp32 oracle fed the same fp16-rounded
+    tables, weights and intermediate tensors: 2e-3."""
+    import torch
+    import din_model
+    torch.cuda.empty_cache()
+    cfg = din_model.Config3()
+    print("config3 full size: batch %d, history %d, 3 x [%d,%d] fp16" % (cfg.batch, cfg.T, cfg.rows, cfg.dim), flush=True)
+    tables = cfg.tables()
+    weights = cfg.weights()
+    batch = cfg.batch_inputs()
+    expose = ("q", "his", "score", "att", "hsum")
+    pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=expose)
+    p = pm.create_predictor(1, 0)
+    din_model.feed(p, inputs, batch, np.float16)
+    p.forward()
+    got = {name: p.output_asnumpy(name).astype(np.float32) for name in expose + ("prob", )}
+    tabs = {}
+    for k, t in zip(din_model.KINDS, tables):
+        ids = np.concatenate([batch[k + ".ids"], batch[k + "_his.ids"]])
+        tabs[k] = _touched_table(oracle, t, ids)
+    rnd = lambda a: np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
+    want = din_model.oracle_forward(oracle, cfg, tabs, weights, batch, rnd)
+    B, T, D3 = cfg.batch, cfg.T, 3 * cfg.dim
+    # pooled blocks: exactly the oracle's fp32 result rounded to fp16
+    assert np.array_equal(got["q"], want["q"])
+    assert got["his"].shape == (B, T, D3) and np.array_equal(got["his"], want["his"])
+    # positions past a sample's history are zero rows
+    seg = batch["item_his.segments"]
+    pad = np.arange(T)[None, :] >= seg[:, None]
+    assert not got["his"][pad].any()
+    np.testing.assert_allclose(got["hsum"], want["hsum"], rtol=2e-3, atol=2e-3 * np.abs(want["hsum"]).max())
+    assert got["score"].shape == (B, T, 1)
+    np.testing.assert_allclose(got["score"], want["score"], rtol=2e-3, atol=2e-3 * np.abs(want["score"]).max())
+    assert got["att"].shape == (B, D3)
+    np.testing.assert_allclose(got["att"], want["att"], rtol=2e-3, atol=2e-3 * np.abs(want["att"]).max())
+    assert got["prob"].shape == (B, 2)
+    np.testing.assert_allclose(got["prob"], want["prob"], rtol=2e-3, atol=2e-3)
+    # the same model with Gemm+Dice folding switched off gives the same probabilities at that tolerance
+    import os
+    os.environ["BLAZE_NO_FUSION"] = "1"
+    try:
+        pm2, _ = din_model.build_manager(cfg, tables, weights, np.float16)
+        p2 = pm2.create_predictor(1, 0)
+        din_model.feed(p2, inputs, batch, np.float16)
+        p2.forward()
+        np.testing.assert_allclose(p2.output_asnumpy("prob").astype(np.float32), want["prob"], rtol=2e-3, atol=2e-3)
+    finally:
+        del os.environ["BLAZE_NO_FUSION"]

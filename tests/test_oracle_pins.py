@@ -45,10 +45,34 @@ def _run_op(oracle, case):
         return oracle.sigmoid(ins[0])
     if ty == "Softmax":
         return oracle.softmax(ins[0], a.get("axis", 1))
+    if ty in ("Add", "Sub", "Mul", "Div"):
+        return oracle.elementwise(ty, ins[0], ins[1])
+    if ty == "BroadcastTo":
+        return oracle.broadcast_to(ins[0], like=ins[1]) if len(ins) > 1 else oracle.broadcast_to(ins[0], shape=a["shape"])
+    if ty == "Where":
+        return oracle.where(ins[0], ins[1], ins[2])
+    if ty == "Concat":
+        return oracle.concat(ins, a.get("axis", 1))
+    if ty == "ReduceSum":
+        return oracle.reduce_sum(ins[0], a.get("axis", 0), a.get("keepdims", 1))
+    if ty == "Fuse":
+        return oracle.fuse(ins[0], ins[1], a.get("comm_index", 0))
+    if ty == "Reshape":
+        return oracle.reshape(ins[0], [int(v) for v in ins[1].reshape(-1)])
+    if ty == "BatchNormalization":
+        return oracle.batch_norm(ins[0], ins[1], ins[2], ins[3], ins[4], a.get("eps", 0.001), bool(a.get("nosqrt", 0)))
     raise KeyError(ty)
 
 
-DENSE_CASES = [
+SHAPE_CASES = [
+    "concat_net_v1_cpu", "concat_net_v2_cpu", "reduce_sum_net_v1_cpu", "fuse_net_v1_cpu", "fuse_net_v2_cpu",
+    "reshape_net_v1_cpu", "batch_normalization_net_v1_cpu", "elementwise_add_net_v1_cpu", "elementwise_add_net_v2_cpu",
+    "elementwise_sub_net_v1_cpu", "elementwise_sub_net_v2_cpu", "elementwise_mul_net_v1_cpu", "elementwise_mul_net_v2_cpu",
+    "elementwise_div_net_v1_cpu", "elementwise_div_net_v2_cpu", "elementwise_broadcast_to_net_v1_cpu",
+    "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu"
+]
+
+DENSE_CASES = SHAPE_CASES + [
     "gemm_net_v1_cpu", "prelu_net_v1_cpu", "dice_net_v1_cpu", "leaky_relu_net_v1_cpu", "sigmoid_net_v1_cpu",
     "softmax_net_v1_cpu", "matmul_net_v1_cpu", "fused_parallel_gemm_net_v1_cpu", "fused_parallel_gemm_net_v2_cpu",
     "fused_parallel_gemm_net_v3_cpu", "fused_parallel_gemm_net_v4_cpu", "fused_parallel_gemm_net_v5_cpu",

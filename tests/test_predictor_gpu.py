@@ -49,7 +49,12 @@ def _net_from_kat(pb, case, skip_types=()):
 DENSE = ["gemm_net_v1_cpu", "prelu_net_v1_cpu", "dice_net_v1_cpu", "leaky_relu_net_v1_cpu", "sigmoid_net_v1_cpu",
          "softmax_net_v1_cpu", "matmul_net_v1_cpu", "fused_parallel_gemm_net_v1_cpu", "fused_parallel_gemm_net_v2_cpu",
          "fused_parallel_gemm_net_v3_cpu", "fused_parallel_gemm_net_v4_cpu", "fused_parallel_gemm_net_v5_cpu",
-         "fused_parallel_matmul_net_v1_cpu", "fused_parallel_matmul_net_v2_cpu", "fused_parallel_matmul_net_v3_cpu"]
+         "fused_parallel_matmul_net_v1_cpu", "fused_parallel_matmul_net_v2_cpu", "fused_parallel_matmul_net_v3_cpu",
+         "concat_net_v1_cpu", "concat_net_v2_cpu", "reduce_sum_net_v1_cpu", "fuse_net_v1_cpu", "fuse_net_v2_cpu",
+         "reshape_net_v1_cpu", "batch_normalization_net_v1_cpu", "elementwise_add_net_v1_cpu", "elementwise_add_net_v2_cpu",
+         "elementwise_sub_net_v1_cpu", "elementwise_sub_net_v2_cpu", "elementwise_mul_net_v1_cpu", "elementwise_mul_net_v2_cpu",
+         "elementwise_div_net_v1_cpu", "elementwise_div_net_v2_cpu", "elementwise_broadcast_to_net_v1_cpu",
+         "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu"]
 
 
 @pytest.mark.parametrize("name", DENSE)

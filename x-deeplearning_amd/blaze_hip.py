@@ -21,8 +21,10 @@ ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 
 EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
-    "bz_activation", "bz_concat_cols"
+    "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis"
 ]
+EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
+MAX_RANK = 6
 
 
 class EmbedSlot(C.Structure):
@@ -62,8 +64,20 @@ class ActDesc(C.Structure):
 
 
 class ConcatDesc(C.Structure):
-    _fields_ = [("src", C.c_void_p * 16), ("width", C.c_int64 * 16), ("dst", C.c_void_p), ("dst_pitch", C.c_int64),
-                ("rows", C.c_int64), ("n", C.c_int32), ("reserved_", C.c_int32)]
+    _fields_ = [("src", C.c_void_p * 16), ("width", C.c_int64 * 16), ("src_pitch", C.c_int64 * 16), ("dst", C.c_void_p),
+                ("dst_pitch", C.c_int64), ("rows", C.c_int64), ("n", C.c_int32), ("reserved_", C.c_int32)]
+
+
+class BcastDesc(C.Structure):
+    _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p), ("out", C.c_void_p), ("dims", C.c_int64 * 6),
+                ("a_stride", C.c_int64 * 6), ("b_stride", C.c_int64 * 6), ("c_stride", C.c_int64 * 6), ("rank", C.c_int32),
+                ("op", C.c_int32), ("dtype", C.c_int32), ("cond_dtype", C.c_int32)]
+
+
+class BnDesc(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("gamma", C.c_void_p), ("beta", C.c_void_p), ("mean", C.c_void_p),
+                ("var", C.c_void_p), ("size", C.c_int64), ("channels", C.c_int64), ("dtype", C.c_int32), ("nosqrt", C.c_int32),
+                ("eps", C.c_float), ("reserved_", C.c_int32)]
 
 
 class BlazeHipError(RuntimeError):
@@ -97,6 +111,10 @@ def lib():
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
         l.bz_activation.argtypes = [C.POINTER(ActDesc), vp]
         l.bz_concat_cols.argtypes = [C.POINTER(ConcatDesc), vp]
+        l.bz_broadcast_op.argtypes = [C.POINTER(BcastDesc), vp]
+        l.bz_reduce_sum.argtypes = [vp, vp, i64, i64, i64, C.c_int, vp]
+        l.bz_batch_norm.argtypes = [C.POINTER(BnDesc), vp]
+        l.bz_softmax_axis.argtypes = [vp, vp, i64, i64, i64, C.c_int, vp]
         _lib = l
     return _lib
 
@@ -340,3 +358,70 @@ def activation(x, act, params=(), out=None, act_alpha=0.0, dice_nosqrt=False, st
     d.dice_nosqrt, d.act_alpha = int(dice_nosqrt), act_alpha
     check(lib().bz_activation(C.byref(d), _stream_ptr(stream)))
     return out
+
+
+def _bcast_strides(t, out_shape):
+    """Element strides of torch tensor `t` seen through `out_shape` (right aligned; 0 on broadcast dims)."""
+    n = len(out_shape)
+    off = n - t.dim()
+    st = [0] * n
+    for k in range(t.dim()):
+        st[off + k] = 0 if t.shape[k] == 1 else t.stride(k)
+    return st
+
+
+def broadcast_op(op, a, b=None, c=None, out_shape=None, stream=None):
+    """Add / Sub / Mul / Div (a, b), BroadcastTo (a -> out_shape), Where (a = int condition, b = x, c = y)."""
+    import torch
+    ops = [t for t in (a, b, c) if t is not None]
+    if out_shape is None:
+        out_shape = torch.broadcast_shapes(*[tuple(t.shape) for t in ops])
+    val = b if op == EW_WHERE else a
+    out = torch.empty(tuple(out_shape), dtype=val.dtype, device=val.device)
+    d = BcastDesc()
+    d.a, d.out = a.data_ptr(), out.data_ptr()
+    d.rank, d.op, d.dtype = len(out_shape), op, bz_dtype(val.dtype)
+    for k, n in enumerate(out_shape):
+        d.dims[k] = n
+    for name, t in (("a_stride", a), ("b_stride", b), ("c_stride", c)):
+        if t is not None:
+            for k, s in enumerate(_bcast_strides(t, out_shape)):
+                getattr(d, name)[k] = s
+    if b is not None:
+        d.b = b.data_ptr()
+    if c is not None:
+        d.c = c.data_ptr()
+    if op == EW_WHERE:
+        d.cond_dtype = bz_dtype(a.dtype)
+    check(lib().bz_broadcast_op(C.byref(d), _stream_ptr(stream)))
+    return out
+
+
+def reduce_sum(x, axis, keepdims=True, stream=None):
+    import torch
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    shape = list(x.shape[:axis]) + ([1] if keepdims else []) + list(x.shape[axis + 1:])
+    y = torch.empty(shape, dtype=x.dtype, device=x.device)
+    check(lib().bz_reduce_sum(x.data_ptr(), y.data_ptr(), outer, x.shape[axis], inner, bz_dtype(x.dtype), _stream_ptr(stream)))
+    return y
+
+
+def batch_norm(x, gamma, beta, mean, var, eps=0.001, nosqrt=False, stream=None):
+    import torch
+    y = torch.empty_like(x)
+    d = BnDesc()
+    d.x, d.y = x.data_ptr(), y.data_ptr()
+    d.gamma, d.beta, d.mean, d.var = gamma.data_ptr(), beta.data_ptr(), mean.data_ptr(), var.data_ptr()
+    d.size, d.channels, d.dtype, d.nosqrt, d.eps = x.numel(), gamma.numel(), bz_dtype(x.dtype), int(nosqrt), eps
+    check(lib().bz_batch_norm(C.byref(d), _stream_ptr(stream)))
+    return y
+
+
+def softmax_axis(x, axis, stream=None):
+    import torch
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    y = torch.empty_like(x)
+    check(lib().bz_softmax_axis(x.data_ptr(), y.data_ptr(), outer, x.shape[axis], inner, bz_dtype(x.dtype), _stream_ptr(stream)))
+    return y

@@ -102,18 +102,20 @@ __global__ __launch_bounds__(256) void bz_concat_kernel(bz_concat_desc d) {
   int64_t col = 0;
   for (int i = 0; i < k; ++i) col += d.width[i];
   char* dst = (char*)d.dst + col;
-  const bool vec = ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) && (width % 16 == 0) && (d.dst_pitch % 16 == 0);
+  const int64_t sp = d.src_pitch[k];
+  const bool vec = ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) && (width % 16 == 0) && (d.dst_pitch % 16 == 0) &&
+                   (sp % 16 == 0);
   if (vec) {
     const int64_t cpr = width / 16, total = cpr * d.rows;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
       const int64_t r = i / cpr, c = i - r * cpr;
-      *(uint4*)(dst + r * d.dst_pitch + c * 16) = *(const uint4*)(src + r * width + c * 16);
+      *(uint4*)(dst + r * d.dst_pitch + c * 16) = *(const uint4*)(src + r * sp + c * 16);
     }
   } else {
     const int64_t total = width * d.rows;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
       const int64_t r = i / width, c = i - r * width;
-      dst[r * d.dst_pitch + c] = src[r * width + c];
+      dst[r * d.dst_pitch + c] = src[r * sp + c];
     }
   }
 }
@@ -128,6 +130,8 @@ extern "C" int bz_concat_cols(const bz_concat_desc* desc, bz_stream_t stream) {
   int64_t total = 0, widest = 0;
   for (int i = 0; i < d.n; ++i) {
     BZ_REQUIRE(d.width[i] >= 0 && (d.width[i] == 0 || d.src[i] != nullptr), "bz_concat_cols: piece %d is null", i);
+    BZ_REQUIRE(d.src_pitch[i] == 0 || d.src_pitch[i] >= d.width[i], "bz_concat_cols: piece %d has pitch %lld < width %lld", i,
+               (long long)d.src_pitch[i], (long long)d.width[i]);
     total += d.width[i];
     widest = d.width[i] > widest ? d.width[i] : widest;
   }

@@ -10,6 +10,7 @@
 //   ConstantFill blaze/operator/op/constant_fill_op.h:13-57  args shape, dtype, value
 //   Concat       blaze/operator/op/concat_op.h           arg axis (default 1)
 #include "blaze/graph.h"
+#include "blaze/op_util.h"
 #include "blaze/operator.h"
 #include "blaze_hip.h"
 
@@ -19,36 +20,6 @@
 namespace blaze {
 
 namespace {
-
-int BzType(int data_type) {
-  switch (data_type) {
-    case kFloat: return BZ_F32;
-    case kFloat16: return BZ_F16;
-    default: BLAZE_THROW("Unsupported type: ", data_type);
-  }
-}
-
-// fp32 device copy of a small parameter blob (the activation kernels read fp32 parameters)
-struct ParamF32 {
-  float* ptr = nullptr;
-  size_t cap = 0;
-  ~ParamF32() {
-    if (ptr) (void)hipFree(ptr);
-  }
-  const float* Get(Blob* b, hipStream_t st) {
-    if (b->data_type() == kFloat) return b->as<float>();
-    BLAZE_CONDITION_THROW(b->data_type() == kFloat16, "Unsupported type: ", b->data_type());
-    const int n = (int)b->size();
-    const int64_t ld = (n + 7) / 8 * 8;
-    if ((size_t)ld > cap) {
-      if (ptr) (void)hipFree(ptr);
-      HIP_CHECK(hipMalloc((void**)&ptr, ld * sizeof(float)));
-      cap = ld;
-    }
-    BZ_CHECK(bz_fc_pack_weight(b->data(), BZ_F16, 1, n, 1, ptr, BZ_F32, ld, st));
-    return ptr;
-  }
-};
 
 void RunActivation(Blob* x, Blob* y, int act, const float* p0, const float* p1, const float* p2, int act_size, bool nosqrt,
                    float alpha, int64_t rows, int64_t cols, hipStream_t st) {
@@ -183,14 +154,13 @@ class SoftmaxOp final : public Operator<Context> {
     Blob* X = this->Input(0);
     Blob* Y = this->Output(0);
     BLAZE_CONDITION_THROW(axis_ < X->shape().size(), "axis=", axis_, " X->shape().size()=", X->shape().size());
-    // softmax over `axis` with W trailing elements (softmax_op.cc:23-26); the device kernel covers W == 1,
-    // which is every head on this path ([batch, classes])
+    // softmax over `axis` with W trailing elements (softmax_op.cc:23-26)
     const TIndex W = X->size((int)axis_ + 1, (int)X->shape().size());
-    BLAZE_CONDITION_THROW(W == 1, "Softmax over a non-innermost axis (inner size ", W, ") is not supported on this device");
     Y->Reshape(X->shape());
     if (X->size() == 0) return true;
     const int64_t C = (int64_t)X->shape()[axis_];
-    RunActivation(X, Y, BZ_ACT_SOFTMAX, nullptr, nullptr, nullptr, 0, false, 0.f, (int64_t)X->size() / C, C, context_.hip_stream());
+    BZ_CHECK(bz_softmax_axis(X->data(), Y->data(), (int64_t)(X->size() / (C * W)), C, (int64_t)W, BzType(X->data_type()),
+                             context_.hip_stream()));
     return true;
   }
 
@@ -302,6 +272,7 @@ class ConcatOp final : public Operator<Context> {
         Blob* x = this->Input(i0 + i);
         d.src[i] = x->data();
         d.width[i] = (int64_t)(x->shape()[axis_] * inner * es);
+        d.src_pitch[i] = d.width[i];
         group += (size_t)d.width[i];
       }
       d.dst = (char*)y->data() + col;  // this group starts `col` bytes into every output row

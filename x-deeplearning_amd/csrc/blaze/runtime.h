@@ -45,14 +45,16 @@ class Blob {
     dims_ = dims;
   }
   void RefReshape(const std::vector<TIndex>& dims, void* handle) {
-    Destroy();
-    own_handle_ = false;
+    if (own_handle_ || data_ != handle) {  // (re-aliasing the same buffer keeps the version)
+      Destroy();
+      own_handle_ = false;
+      data_ = handle;
+      ++version_;
+    }
     TIndex n = 1;
     for (auto d : dims) n *= d;
     size_ = capacity_ = n;
     dims_ = dims;
-    data_ = handle;
-    ++version_;
   }
   const DeviceOption& device_option() const { return device_option_; }
   int device_type() const { return device_option_.device_type(); }

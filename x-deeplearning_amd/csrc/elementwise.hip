@@ -1,0 +1,300 @@
+// elementwise.hip -- the shape / elementwise operators around DIN's attention unit, for gfx950.
+//
+// Add / Sub / Mul / Div / BroadcastTo / Where with multidirectional broadcasting
+// (blaze/operator/op/elementwise_op.{h,cc,cu}, shape rule blaze/math/broadcast.h:39-67), ReduceSum
+// (blaze/operator/op/reduce_sum_op.h:17-58, blaze/math/reduce.cc:13-29), BatchNormalization in its inference
+// form (blaze/operator/op/batch_normalization_op.cc:11-18) and Softmax over an inner axis
+// (blaze/operator/op/softmax_op.cc:21-78).  All of them are one read and one write per element: HBM bound.
+//
+// Broadcast kernel: the host merges adjacent output dims whose operand strides allow it, then dispatches on
+// the merged dims (up to 6).  A thread owns `VEC` consecutive elements of the innermost merged dim, so the index
+// decomposition is paid once per VEC elements.
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "bz_common.h"
+
+namespace {
+
+template <typename T>
+__device__ __forceinline__ float ldv(const T* p);
+template <>
+__device__ __forceinline__ float ldv<float>(const float* p) {
+  return *p;
+}
+template <>
+__device__ __forceinline__ float ldv<__half>(const __half* p) {
+  return __half2float(*p);
+}
+template <>
+__device__ __forceinline__ float ldv<__hip_bfloat16>(const __hip_bfloat16* p) {
+  return __bfloat162float(*p);
+}
+template <typename T>
+__device__ __forceinline__ void stv(T* p, float v);
+template <>
+__device__ __forceinline__ void stv<float>(float* p, float v) {
+  *p = v;
+}
+template <>
+__device__ __forceinline__ void stv<__half>(__half* p, float v) {
+  *p = __float2half_rn(v);
+}
+template <>
+__device__ __forceinline__ void stv<__hip_bfloat16>(__hip_bfloat16* p, float v) {
+  *p = __float2bfloat16(v);
+}
+
+struct BcastP {
+  int64_t dims[BZ_MAX_RANK];  // merged, outermost first; only [0, rank) valid
+  int64_t sa[BZ_MAX_RANK], sb[BZ_MAX_RANK], sc[BZ_MAX_RANK];
+  int rank;
+  int op;
+  int64_t total;  // number of output elements
+};
+
+// VEC consecutive output elements of the innermost dim per thread (the host picks a VEC that divides that dim).
+template <typename T, typename CondT, int VEC>
+__global__ __launch_bounds__(256) void bz_bcast_kernel(const void* __restrict__ a_, const T* __restrict__ b, const T* __restrict__ c,
+                                                       T* __restrict__ out, BcastP p) {
+  const int64_t nvec = p.total / VEC;
+  for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    int64_t lin = v * VEC;
+    int64_t oa = 0, ob = 0, oc = 0;
+    int64_t rem = lin;
+#pragma unroll
+    for (int d = BZ_MAX_RANK - 1; d >= 0; --d) {
+      if (d < p.rank) {
+        const int64_t q = rem / p.dims[d];
+        const int64_t i = rem - q * p.dims[d];
+        rem = q;
+        oa += i * p.sa[d];
+        ob += i * p.sb[d];
+        oc += i * p.sc[d];
+      }
+    }
+    const int last = p.rank - 1;
+    const int64_t ia = p.sa[last], ib = p.sb[last], ic = p.sc[last];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float r;
+      if (p.op == BZ_EW_WHERE) {
+        const CondT cond = ((const CondT*)a_)[oa + e * ia];
+        r = cond != 0 ? ldv<T>(b + ob + e * ib) : ldv<T>(c + oc + e * ic);
+      } else {
+        const float x = ldv<T>((const T*)a_ + oa + e * ia);
+        if (p.op == BZ_EW_ASSIGN) {
+          r = x;
+        } else {
+          const float y = ldv<T>(b + ob + e * ib);
+          r = p.op == BZ_EW_ADD ? __fadd_rn(x, y) : p.op == BZ_EW_SUB ? __fsub_rn(x, y) : p.op == BZ_EW_MUL ? __fmul_rn(x, y) : __fdiv_rn(x, y);
+        }
+      }
+      stv<T>(out + lin + e, r);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bz_reduce_sum_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t outer, int64_t dim,
+                                                            int64_t inner) {
+  const int64_t total = outer * inner;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t o = i / inner, k = i - o * inner;
+    const T* p = x + o * dim * inner + k;
+    float acc = 0.f;
+    int64_t j = 0;
+    for (; j + 4 <= dim; j += 4) {  // four loads in flight, added in order
+      const float v0 = ldv<T>(p + (j + 0) * inner), v1 = ldv<T>(p + (j + 1) * inner);
+      const float v2 = ldv<T>(p + (j + 2) * inner), v3 = ldv<T>(p + (j + 3) * inner);
+      acc = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(acc, v0), v1), v2), v3);
+    }
+    for (; j < dim; ++j) acc = __fadd_rn(acc, ldv<T>(p + j * inner));
+    stv<T>(y + i, acc);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bz_batch_norm_kernel(const T* __restrict__ x, T* __restrict__ y, bz_bn_desc d) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < d.size; i += (int64_t)gridDim.x * 256) {
+    const int64_t c = i % d.channels;
+    const float den = d.nosqrt ? d.var[c] : __fsqrt_rn(__fadd_rn(d.var[c], d.eps));
+    const float xn = __fdiv_rn(__fsub_rn(ldv<T>(x + i), d.mean[c]), den);
+    stv<T>(y + i, __fadd_rn(__fmul_rn(d.gamma[c], xn), d.beta[c]));
+  }
+}
+
+// one thread per (outer, inner) column of the axis: three passes over c values that stay in L1/L2
+template <typename T>
+__global__ __launch_bounds__(256) void bz_softmax_axis_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t outer, int64_t c,
+                                                              int64_t inner) {
+  const int64_t total = outer * inner;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t o = i / inner, k = i - o * inner;
+    const T* xp = x + o * c * inner + k;
+    T* yp = y + o * c * inner + k;
+    float mx = ldv<T>(xp);
+    for (int64_t j = 1; j < c; ++j) mx = fmaxf(mx, ldv<T>(xp + j * inner));
+    float sum = 0.f;
+    for (int64_t j = 0; j < c; ++j) sum += expf(ldv<T>(xp + j * inner) - mx);
+    for (int64_t j = 0; j < c; ++j) stv<T>(yp + j * inner, expf(ldv<T>(xp + j * inner) - mx) / sum);
+  }
+}
+
+int grid_for(int64_t work) {
+  const int64_t want = (work + 255) / 256;
+  return (int)(want < 1 ? 1 : (want < 256 * 32 ? want : 256 * 32));
+}
+
+template <typename T, typename CondT>
+int launch_bcast(const bz_bcast_desc& d, const BcastP& p, int vec, hipStream_t s) {
+  const int grid = grid_for(p.total / vec);
+  const T* b = (const T*)d.b;
+  const T* c = (const T*)d.c;
+  T* out = (T*)d.out;
+  switch (vec) {
+    case 8:
+      hipLaunchKernelGGL((bz_bcast_kernel<T, CondT, 8>), dim3(grid), dim3(256), 0, s, d.a, b, c, out, p);
+      break;
+    case 4:
+      hipLaunchKernelGGL((bz_bcast_kernel<T, CondT, 4>), dim3(grid), dim3(256), 0, s, d.a, b, c, out, p);
+      break;
+    case 2:
+      hipLaunchKernelGGL((bz_bcast_kernel<T, CondT, 2>), dim3(grid), dim3(256), 0, s, d.a, b, c, out, p);
+      break;
+    default:
+      hipLaunchKernelGGL((bz_bcast_kernel<T, CondT, 1>), dim3(grid), dim3(256), 0, s, d.a, b, c, out, p);
+      break;
+  }
+  BZ_LAUNCH_OK("bz_bcast_kernel");
+  return BZ_OK;
+}
+
+template <typename T>
+int launch_bcast_t(const bz_bcast_desc& d, const BcastP& p, int vec, hipStream_t s) {
+  if (d.op == BZ_EW_WHERE && d.cond_dtype == BZ_I64) return launch_bcast<T, int64_t>(d, p, vec, s);
+  return launch_bcast<T, int32_t>(d, p, vec, s);
+}
+
+}  // namespace
+
+extern "C" int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_broadcast_op: null descriptor");
+  const bz_bcast_desc& d = *desc;
+  BZ_REQUIRE(d.rank >= 1 && d.rank <= BZ_MAX_RANK, "bz_broadcast_op: rank %d outside 1..%d", d.rank, BZ_MAX_RANK);
+  BZ_REQUIRE(d.op >= BZ_EW_ADD && d.op <= BZ_EW_WHERE, "bz_broadcast_op: unknown op %d", d.op);
+  BZ_REQUIRE(d.dtype == BZ_F32 || d.dtype == BZ_F16 || d.dtype == BZ_BF16, "bz_broadcast_op: unsupported dtype %d", d.dtype);
+  BZ_REQUIRE(d.a != nullptr && d.out != nullptr, "bz_broadcast_op: null operand");
+  BZ_REQUIRE(d.op == BZ_EW_ASSIGN || d.b != nullptr, "bz_broadcast_op: null second operand");
+  if (d.op == BZ_EW_WHERE) {
+    BZ_REQUIRE(d.c != nullptr, "bz_broadcast_op: Where needs three operands");
+    BZ_REQUIRE(d.cond_dtype == BZ_I32 || d.cond_dtype == BZ_I64, "bz_broadcast_op: condition dtype %d", d.cond_dtype);
+  }
+  const bool use_b = d.op != BZ_EW_ASSIGN, use_c = d.op == BZ_EW_WHERE;
+  int64_t total = 1;
+  for (int i = 0; i < d.rank; ++i) {
+    BZ_REQUIRE(d.dims[i] >= 0, "bz_broadcast_op: dim %d is %lld", i, (long long)d.dims[i]);
+    BZ_REQUIRE(d.a_stride[i] >= 0 && d.b_stride[i] >= 0 && d.c_stride[i] >= 0, "bz_broadcast_op: negative stride");
+    total *= d.dims[i];
+  }
+  if (total == 0) return BZ_OK;
+  // merge adjacent dims: dims (outer, inner) fuse when every operand has stride_outer == stride_inner * dim_inner
+  // (which covers "both broadcast": 0 == 0 * n); dims of size 1 are dropped
+  BcastP p = {};
+  int r = 0;
+  for (int i = 0; i < d.rank; ++i) {
+    if (d.dims[i] == 1) continue;
+    const int64_t sa = d.a_stride[i], sb = use_b ? d.b_stride[i] : 0, sc = use_c ? d.c_stride[i] : 0;
+    if (r > 0 && p.sa[r - 1] == sa * d.dims[i] && p.sb[r - 1] == sb * d.dims[i] && p.sc[r - 1] == sc * d.dims[i]) {
+      p.dims[r - 1] *= d.dims[i];
+      p.sa[r - 1] = sa;
+      p.sb[r - 1] = sb;
+      p.sc[r - 1] = sc;
+    } else {
+      p.dims[r] = d.dims[i];
+      p.sa[r] = sa;
+      p.sb[r] = sb;
+      p.sc[r] = sc;
+      ++r;
+    }
+  }
+  if (r == 0) {  // a single element
+    p.dims[0] = 1;
+    r = 1;
+  }
+  p.rank = r;
+  p.op = d.op;
+  p.total = total;
+  // a thread takes `vec` consecutive elements of the innermost dim: needs the dim to divide evenly
+  int vec = 8;
+  while (vec > 1 && p.dims[r - 1] % vec != 0) vec >>= 1;
+  hipStream_t s = bz::as_stream(stream);
+  if (d.dtype == BZ_F32) return launch_bcast_t<float>(d, p, vec > 4 ? 4 : vec, s);
+  if (d.dtype == BZ_F16) return launch_bcast_t<__half>(d, p, vec, s);
+  return launch_bcast_t<__hip_bfloat16>(d, p, vec, s);
+}
+
+extern "C" int bz_reduce_sum(const void* x, void* y, int64_t outer, int64_t dim, int64_t inner, int dtype, bz_stream_t stream) {
+  BZ_REQUIRE(x != nullptr && y != nullptr, "bz_reduce_sum: null operand");
+  BZ_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, "bz_reduce_sum: negative size");
+  BZ_REQUIRE(dtype == BZ_F32 || dtype == BZ_F16 || dtype == BZ_BF16, "bz_reduce_sum: unsupported dtype %d", dtype);
+  if (outer * inner == 0) return BZ_OK;
+  hipStream_t s = bz::as_stream(stream);
+  const int grid = grid_for(outer * inner);
+  if (dtype == BZ_F32)
+    hipLaunchKernelGGL(bz_reduce_sum_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)x, (float*)y, outer, dim, inner);
+  else if (dtype == BZ_F16)
+    hipLaunchKernelGGL(bz_reduce_sum_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)x, (__half*)y, outer, dim, inner);
+  else
+    hipLaunchKernelGGL(bz_reduce_sum_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, s, (const __hip_bfloat16*)x,
+                       (__hip_bfloat16*)y, outer, dim, inner);
+  BZ_LAUNCH_OK("bz_reduce_sum_kernel");
+  return BZ_OK;
+}
+
+extern "C" int bz_batch_norm(const bz_bn_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_batch_norm: null descriptor");
+  const bz_bn_desc& d = *desc;
+  BZ_REQUIRE(d.x && d.y && d.gamma && d.beta && d.mean && d.var, "bz_batch_norm: null operand");
+  BZ_REQUIRE(d.size >= 0 && d.channels > 0, "bz_batch_norm: size=%lld channels=%lld", (long long)d.size, (long long)d.channels);
+  BZ_REQUIRE(d.dtype == BZ_F32 || d.dtype == BZ_F16 || d.dtype == BZ_BF16, "bz_batch_norm: unsupported dtype %d", d.dtype);
+  if (d.size == 0) return BZ_OK;
+  hipStream_t s = bz::as_stream(stream);
+  const int grid = grid_for(d.size);
+  if (d.dtype == BZ_F32)
+    hipLaunchKernelGGL(bz_batch_norm_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)d.x, (float*)d.y, d);
+  else if (d.dtype == BZ_F16)
+    hipLaunchKernelGGL(bz_batch_norm_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)d.x, (__half*)d.y, d);
+  else
+    hipLaunchKernelGGL(bz_batch_norm_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, s, (const __hip_bfloat16*)d.x,
+                       (__hip_bfloat16*)d.y, d);
+  BZ_LAUNCH_OK("bz_batch_norm_kernel");
+  return BZ_OK;
+}
+
+extern "C" int bz_softmax_axis(const void* x, void* y, int64_t outer, int64_t c, int64_t inner, int dtype, bz_stream_t stream) {
+  BZ_REQUIRE(x != nullptr && y != nullptr, "bz_softmax_axis: null operand");
+  BZ_REQUIRE(outer >= 0 && c > 0 && inner > 0, "bz_softmax_axis: outer=%lld c=%lld inner=%lld", (long long)outer, (long long)c,
+             (long long)inner);
+  BZ_REQUIRE(dtype == BZ_F32 || dtype == BZ_F16, "bz_softmax_axis: unsupported dtype %d", dtype);
+  if (outer == 0) return BZ_OK;
+  if (inner == 1) {  // rows of c contiguous values: one wave per row
+    bz_act_desc a = {};
+    a.x = x;
+    a.y = y;
+    a.rows = outer;
+    a.cols = c;
+    a.dtype = dtype;
+    a.act = BZ_ACT_SOFTMAX;
+    return bz_activation(&a, stream);
+  }
+  hipStream_t s = bz::as_stream(stream);
+  const int grid = grid_for(outer * inner);
+  if (dtype == BZ_F32)
+    hipLaunchKernelGGL(bz_softmax_axis_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)x, (float*)y, outer, c, inner);
+  else
+    hipLaunchKernelGGL(bz_softmax_axis_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)x, (__half*)y, outer, c, inner);
+  BZ_LAUNCH_OK("bz_softmax_axis_kernel");
+  return BZ_OK;
+}

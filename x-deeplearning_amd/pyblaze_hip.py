@@ -315,6 +315,10 @@ class NetBuilder:
             elif isinstance(v, str):
                 esc = v.replace("\\", "\\\\").replace('"', '\\"').replace("\n", "\\n")
                 parts.append('arg { name : "%s" s : "%s" }' % (k, esc))
+            elif isinstance(v, (list, tuple)) and all(isinstance(e, int) for e in v):
+                parts.append('arg { name : "%s" %s }' % (k, " ".join("ints : %d" % e for e in v)))
+            elif isinstance(v, (list, tuple)):
+                parts.append('arg { name : "%s" %s }' % (k, " ".join("floats : %s" % _fmt_float(float(e)) for e in v)))
             else:
                 raise TypeError((k, v))
         parts.append("}")
