@@ -81,7 +81,7 @@ def main():
     mlp = cfg.mlp()
     sparse, dense = cfg.batches(args.pool)
     # kernel-layer harness: per-kernel timing below, and the whole step in --kernel-api mode
-    fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16")
+    fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16", fused_mlp=bool(int(os.environ.get("BZ_FUSED_MLP", "0"))))
     torch.cuda.synchronize()
     K, W = args.steps, args.warmup
     T = max(1, min(args.threads, fwd.n_batches))
@@ -113,33 +113,45 @@ def main():
         else:
             fwd.step(i, stream_ptrs[t])
 
-    # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations
-    start = threading.Barrier(T + 1)
-    errors = []
+    # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations.  The Predictor path is
+    # driven by the library's own serving threads (Blaze_ServePool*: a C++ loop per thread, as a serving binary
+    # would run it); the kernel-layer path by Python threads.
+    if predictors is not None:
+        from pyblaze_hip import ServePool
+        pool = ServePool(T)
+        pool.run(predictors, W)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        pool.run(predictors, K)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    else:
+        start = threading.Barrier(T + 1)
+        errors = []
 
-    def worker(t):
-        try:
-            for i in range(t, W, T):
-                run_step(i, t)
-            torch.cuda.synchronize()
-            start.wait()
-            for i in range(t, K, T):
-                run_step(W - (W % T) + i, t)
-        except Exception as e:  # noqa: BLE001
-            errors.append(e)
-            start.abort()
+        def worker(t):
+            try:
+                for i in range(t, W, T):
+                    run_step(i, t)
+                torch.cuda.synchronize()
+                start.wait()
+                for i in range(t, K, T):
+                    run_step(W - (W % T) + i, t)
+            except Exception as e:  # noqa: BLE001
+                errors.append(e)
+                start.abort()
 
-    threads = [threading.Thread(target=worker, args=(t, )) for t in range(T)]
-    for th in threads:
-        th.start()
-    start.wait()
-    t0 = time.perf_counter()
-    for th in threads:
-        th.join()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    if errors:
-        raise errors[0]
+        threads = [threading.Thread(target=worker, args=(t, )) for t in range(T)]
+        for th in threads:
+            th.start()
+        start.wait()
+        t0 = time.perf_counter()
+        for th in threads:
+            th.join()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        if errors:
+            raise errors[0]
     ms_per_step = (t1 - t0) * 1e3 / K
     samples_per_s = cfg.batch * K / (t1 - t0)
 

@@ -114,6 +114,17 @@ BLAZE_API int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char*
 /* run Forward `count` times on the calling thread (benchmark loops without per-call host overhead) */
 BLAZE_API int Blaze_PredictorForwardN(PredictorHandle handle, int count);
 
+/*
+ * A pool of serving threads (no counterpart in the reference's C API; its C++ example runs one loop per thread,
+ * blaze/example/cpp/predictor_example.cc).  Blaze_ServePoolRun runs `steps` forward passes: pass i runs predictor
+ * i % n_predictors on thread i % n_threads, and returns when all of them have finished on the device.  n_predictors
+ * must be a multiple of the pool's thread count so that a predictor only ever runs on one thread.
+ */
+typedef void* ServePoolHandle;
+BLAZE_API int Blaze_ServePoolCreate(int n_threads, ServePoolHandle* handle);
+BLAZE_API int Blaze_ServePoolRun(ServePoolHandle handle, PredictorHandle* predictors, int n_predictors, int64_t steps);
+BLAZE_API int Blaze_ServePoolDelete(ServePoolHandle handle);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,6 +5,11 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+#include <condition_variable>
+#include <mutex>
+#include <thread>
+
 #include "blaze/predictor.h"
 #include "blaze/qed_builder.h"
 #include "blaze/qed_store.h"
@@ -179,6 +184,100 @@ int Blaze_PredictorForwardN(PredictorHandle handle, int count) {
   if (p == nullptr) return -1;
   for (int i = 0; i < count; ++i)
     if (!p->Forward()) return Fail("Forward failed");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Serving pool: n persistent threads, each driving its own predictors -- the reference's deployment model (one
+// Predictor per thread, api/cpp_api/predictor.h:90-92; example/cpp/predictor_example.cc runs one loop per thread).
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+struct ServePool {
+  std::vector<std::thread> threads;
+  std::mutex mu;
+  std::condition_variable cv_work, cv_done;
+  uint64_t generation = 0;
+  int pending = 0;
+  bool stop = false;
+  // the job of the current generation
+  Predictor** handles = nullptr;
+  int n_handles = 0;
+  int64_t steps = 0;
+  std::atomic<int> failed{0};
+  std::string error;
+
+  explicit ServePool(int n) {
+    for (int t = 0; t < n; ++t) threads.emplace_back([this, t] { Loop(t); });
+  }
+  ~ServePool() {
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      stop = true;
+    }
+    cv_work.notify_all();
+    for (auto& th : threads) th.join();
+  }
+  void Loop(int t) {
+    uint64_t seen = 0;
+    for (;;) {
+      int n_threads;
+      {
+        std::unique_lock<std::mutex> lock(mu);
+        cv_work.wait(lock, [&] { return stop || generation != seen; });
+        if (stop) return;
+        seen = generation;
+        n_threads = (int)threads.size();
+      }
+      // step i of the job runs predictor i % n_handles; thread t takes the steps i == t (mod n_threads), so a
+      // predictor is only ever used by one thread when n_handles is a multiple of n_threads
+      for (int64_t i = t; i < steps && !failed.load(std::memory_order_relaxed); i += n_threads) {
+        if (!handles[i % n_handles]->Forward()) {
+          if (!failed.exchange(1)) {
+            std::lock_guard<std::mutex> lock(mu);
+            error = blaze::last_error_for_thread();
+          }
+        }
+      }
+      {
+        std::lock_guard<std::mutex> lock(mu);
+        if (--pending == 0) cv_done.notify_all();
+      }
+    }
+  }
+  bool Run(Predictor** h, int n, int64_t k) {
+    std::unique_lock<std::mutex> lock(mu);
+    handles = h;
+    n_handles = n;
+    steps = k;
+    failed = 0;
+    error.clear();
+    pending = (int)threads.size();
+    ++generation;
+    cv_work.notify_all();
+    cv_done.wait(lock, [&] { return pending == 0; });
+    return failed.load() == 0;
+  }
+};
+}  // namespace
+
+int Blaze_ServePoolCreate(int n_threads, ServePoolHandle* handle) {
+  if (handle == nullptr || n_threads < 1 || n_threads > 256) return Fail("ServePoolCreate: bad arguments");
+  *handle = new ServePool(n_threads);
+  return 0;
+}
+int Blaze_ServePoolRun(ServePoolHandle handle, PredictorHandle* predictors, int n_predictors, int64_t steps) {
+  auto* pool = reinterpret_cast<ServePool*>(handle);
+  if (pool == nullptr || predictors == nullptr || n_predictors < 1 || steps < 0) return Fail("ServePoolRun: bad arguments");
+  if (n_predictors % (int)pool->threads.size() != 0)
+    return Fail("ServePoolRun: the number of predictors must be a multiple of the pool's threads (a predictor belongs to one thread)");
+  if (!pool->Run(reinterpret_cast<Predictor**>(predictors), n_predictors, steps)) {
+    Blaze_SetLastErrorString("Forward failed in the serving pool: %s", pool->error.c_str());
+    return -1;
+  }
+  return 0;
+}
+int Blaze_ServePoolDelete(ServePoolHandle handle) {
+  delete reinterpret_cast<ServePool*>(handle);
   return 0;
 }
 

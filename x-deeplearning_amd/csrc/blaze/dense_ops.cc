@@ -148,7 +148,7 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
 
 // ------------------------------------------------------------------------------------------ Gemm
 template <class Context>
-class GemmOp : public Operator<Context>, public FusableProducer {
+class GemmOp : public Operator<Context>, public FusableProducer, public StackableFc {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
 
@@ -195,7 +195,115 @@ class GemmOp : public Operator<Context>, public FusableProducer {
     return true;
   }
 
+  // ---- StackableFc: a chain of FC layers as one launch
+  bool StackEligible(int* k_in, int* n_out) override {
+    Blob* b = this->Input(1);
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || b->data_type() != kFloat16) return false;
+    const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
+    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
+    if (this->InputSize() > 2) {
+      Blob* c = this->Input(2);
+      if (!c_constant_ || (int)c->size() != N) return false;  // a per-column bias only
+    }
+    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX && N > BZ_MLP_MAX_HEAD) return false;
+    *k_in = K;
+    *n_out = N;
+    return true;
+  }
+  OperatorBase* StackOutputOp() override { return fused_ ? fused_ : this; }
+  void AbsorbStack(const std::vector<StackableFc*>& followers) override {
+    stack_.clear();
+    for (StackableFc* f : followers) stack_.push_back(static_cast<GemmOp*>(f));
+  }
+
   bool RunOnDevice() override {
+    if (!stack_.empty()) {
+      if (RunStack()) return true;
+      // an input the fused kernel does not take (3-D, unaligned, another type): layer by layer
+      if (!RunSelf()) return false;
+      for (GemmOp* f : stack_)
+        if (!f->RunSelf()) return false;
+      return true;
+    }
+    return RunSelf();
+  }
+
+ protected:
+  // this layer's entry of the fused stack: packed weight, bias and epilogue parameters
+  void FillStackLayer(bz_mlp_layer* L, bool head, hipStream_t st) {
+    Blob* b = this->Input(1);
+    const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
+    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
+    const int64_t ldw = (K + 7) / 8 * 8;
+    if (packed_b_.Stale(b) || packed_b_.bytes < (size_t)N * ldw * 2) {
+      packed_b_.Resize((size_t)N * ldw * 2);
+      BZ_CHECK(bz_fc_pack_weight(b->data(), BZ_F16, transb_ ? 1 : 0, K, N, packed_b_.ptr, BZ_F16, ldw, st));
+      packed_b_.Mark(b);
+      stack_pack_.src = nullptr;
+    }
+    memset(L, 0, sizeof(*L));
+    if (head) {
+      L->w = packed_b_.ptr;
+      L->ldw = (int)ldw;
+    } else {
+      if (stack_pack_.Stale(b)) {
+        stack_pack_.Resize((size_t)bz_mlp_packed_elems(K, N) * 2);
+        BZ_CHECK(bz_mlp_pack_weight(packed_b_.ptr, BZ_F16, K, N, ldw, stack_pack_.ptr, st));
+        stack_pack_.Mark(b);
+      }
+      L->w = stack_pack_.ptr;
+    }
+    L->n = N;
+    L->k = K;
+    if (this->InputSize() > 2) L->bias = AsFloatParam(this->Input(2), &bias_f32_, true, st);
+    L->alpha = alpha_;
+    L->beta = beta_;
+    L->act = fused_ ? fused_act_ : BZ_ACT_NONE;
+    L->dice_nosqrt = fused_nosqrt_ ? 1 : 0;
+    L->act_alpha = fused_alpha_;
+    if (fused_ && fused_act_ == BZ_ACT_PRELU) {
+      L->p0 = AsFloatParam(fused_->Input(1), &p_f32_[0], true, st);
+      L->act_size = (int)fused_->Input(1)->size();
+    } else if (fused_ && fused_act_ == BZ_ACT_DICE) {
+      L->p0 = AsFloatParam(fused_->Input(1), &p_f32_[0], true, st);
+      L->p1 = AsFloatParam(fused_->Input(2), &p_f32_[1], true, st);
+      L->p2 = AsFloatParam(fused_->Input(3), &p_f32_[2], true, st);
+      L->act_size = N;
+    }
+  }
+
+  bool RunStack() {
+    Blob* a = this->Input(0);
+    if (a->shape().size() != 2 || a->data_type() != kFloat16) return false;
+    const TIndex M = a->shape()[0], K = a->shape()[1];
+    if (K % 8 != 0 || (uintptr_t)a->data() % 16 != 0) return false;
+    GemmOp* last = stack_.back();
+    Blob* y = last->StackOutputOp()->Output(0);
+    Blob* lb = last->Input(1);
+    const TIndex n_last = last->transb_ ? lb->shape()[0] : lb->shape()[1];
+    const bool head = n_last <= BZ_MLP_MAX_HEAD;
+    if (!(y->data_type() == kFloat16 || (head && y->data_type() == kFloat))) return false;
+    if (!head && n_last % 8 != 0) return false;
+    CheckValid();
+    y->Reshape({M, n_last});
+    hipStream_t st = context_.hip_stream();
+    bz_mlp_desc d;
+    memset(&d, 0, sizeof(d));
+    d.x = a->data();
+    d.ldx = (int64_t)K;
+    d.y = y->data();
+    d.ldy = (int64_t)n_last;
+    d.m = (int)M;
+    d.n_layers = 1 + (int)stack_.size();
+    d.dtype = BZ_F16;
+    d.out_dtype = BzType(y->data_type());
+    FillStackLayer(&d.layer[0], false, st);
+    for (size_t i = 0; i < stack_.size(); ++i) stack_[i]->FillStackLayer(&d.layer[1 + i], head && i + 1 == stack_.size(), st);
+    BZ_CHECK(bz_mlp_fused(&d, st));
+    return true;
+  }
+
+  bool RunSelf() {
     CheckValid();
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -294,6 +402,8 @@ class GemmOp : public Operator<Context>, public FusableProducer {
   bool transa_, transb_;
   bool b_constant_ = false, c_constant_ = false;
   Derived packed_b_, packed_a_, bias_f32_, p_f32_[3];
+  Derived stack_pack_;           // this layer's weight in the fragment-major pack of bz_mlp_fused
+  std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
   OperatorBase* fused_ = nullptr;
   int fused_act_ = BZ_ACT_NONE;
   bool fused_nosqrt_ = false;

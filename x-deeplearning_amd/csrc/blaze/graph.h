@@ -90,7 +90,8 @@ class SimpleNet : public Net {
 
  protected:
   bool RunImpl() override;
-  std::vector<bool> skipped_;  // ops folded into their producer's epilogue
+  void StackFcLayers();
+  std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
 typedef Registry<std::shared_ptr<Net>, const std::shared_ptr<const NetDef>&, Workspace*> NetRegistryType;
@@ -113,6 +114,21 @@ class FusableProducer {
  public:
   virtual ~FusableProducer() {}
   virtual bool TryFuse(OperatorBase* consumer) = 0;
+};
+
+// An FC operator (Gemm, with or without a folded activation) that can hand its work to the FC before it, so that a
+// chain of FC layers runs as one launch (bz_mlp_fused: the batch rows stay on chip from the first layer to the
+// last).  SimpleNet links consecutive eligible operators whose only connection is producer -> consumer; the head
+// of the chain then runs all of them and the followers are skipped.  Same results as layer-by-layer execution:
+// hidden activations are rounded to the tensor type where the separate operators would have stored them.
+class StackableFc {
+ public:
+  virtual ~StackableFc() {}
+  // static eligibility (constant fp16 weight and bias, no transposed A, ...); reports the layer's widths
+  virtual bool StackEligible(int* k_in, int* n_out) = 0;
+  // the operator whose Output(0) receives this layer's result (the folded activation, else the operator itself)
+  virtual OperatorBase* StackOutputOp() = 0;
+  virtual void AbsorbStack(const std::vector<StackableFc*>& followers) = 0;
 };
 
 }  // namespace blaze

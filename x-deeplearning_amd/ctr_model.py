@@ -10,9 +10,10 @@ import numpy as np
 import pyblaze_hip as pb
 
 
-def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False):
+def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False, fc_stack=False):
     """tables: list of torch cuda tensors [rows, dim]; mlp: [(W [K,N], b, slope)] torch tensors.
-    expose_block: also declare the pooled Embedding block an output of the net (for parity checks)."""
+    expose_block: also declare the pooled Embedding block an output of the net (for parity checks).
+    fc_stack: ask the net to run the chain of FC layers as one launch (net argument fuse_fc_stack)."""
     code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
     pm = pb.PredictorManager()
     fgs = []
@@ -29,6 +30,8 @@ def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False):
         inputs += [fg + ".ids", fg + ".values", fg + ".segments"]
     nb.external_input("dense", code)
     nb.external_output("prob", pb.K_FLOAT)
+    if fc_stack:
+        nb.arg("fuse_fc_stack", 1)
     if expose_block:
         nb.external_output("block", code)
     for li, (w, b, slope) in enumerate(mlp):

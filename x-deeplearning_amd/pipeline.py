@@ -14,10 +14,12 @@ import blaze_hip as bz
 
 
 class CtrForward:
-    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True):
+    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True, fused_mlp=False):
+        """fused_mlp: run the FC stack as one bz_mlp_fused launch instead of one bz_fc_fused launch per layer."""
         import torch
         self.cfg = cfg
         self.fused_scan = fused_scan
+        self.fused_mlp = None
         self.lib = bz.lib()
         tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
         bdt = {"f16": bz.F16, "bf16": bz.BF16, "f32": bz.F32}[dtype]
@@ -26,6 +28,10 @@ class CtrForward:
         for (w, b, slope) in mlp:
             self.weights.append((bz.pack_weight(w, False, bdt), b.float().contiguous(), slope.float().contiguous(),
                                  w.shape[0]))
+        if fused_mlp:
+            n = len(mlp)
+            self.fused_mlp = bz.FusedMlp([dict(w=w, bias=b, act=bz.ACT_SOFTMAX if li == n - 1 else bz.ACT_PRELU,
+                                               params=() if li == n - 1 else (slope, )) for li, (w, b, slope) in enumerate(mlp)], bdt)
         self.n_batches = len(sparse_batches)
         self.steps = []
         self.nnz = []
@@ -84,11 +90,21 @@ class CtrForward:
         d = self.steps[i % self.n_batches]["descs"][layer]
         bz.check(self.lib.bz_fc_fused(C.byref(d), st or self._stream()))
 
+    def mlp(self, i, st=None):
+        s = self.steps[i % self.n_batches]
+        d = self.fused_mlp.desc
+        x, y = s["x"], s["acts"][-1]
+        d.x, d.y, d.ldx, d.ldy, d.m, d.out_dtype = x.data_ptr(), y.data_ptr(), x.stride(0), y.stride(0), x.shape[0], bz.bz_dtype(y.dtype)
+        bz.check(self.lib.bz_mlp_fused(C.byref(d), st or self._stream()))
+
     def step(self, i, st=None):
         st = st or self._stream()
         if not self.fused_scan:
             self.scan(i, st)
         self.pool(i, st)
+        if self.fused_mlp is not None:
+            self.mlp(i, st)
+            return
         for layer in range(len(self.weights)):
             self.fc(i, layer, st)
 

@@ -27,7 +27,8 @@ EXPORTS = [
     "Blaze_PredictorListOutputNames", "Blaze_PredictorRegisterObservers", "Blaze_PredictorDumpObservers",
     "Blaze_ConvertBlaze", "Blaze_OptimizeBlaze", "Blaze_QuickEmbeddingBuildFp32", "Blaze_QuickEmbeddingBuildFp16",
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
-    "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef"
+    "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
+    "Blaze_ServePoolRun", "Blaze_ServePoolDelete"
 ]
 
 
@@ -77,6 +78,9 @@ def lib():
         l.Blaze_ConvertNetDef.argtypes = [cp, sz, i, i, vp, sz, C.POINTER(sz)]
         l.Blaze_PredictorInputDevicePtr.argtypes = [vp, cp, C.POINTER(vp)]
         l.Blaze_PredictorOutputDevicePtr.argtypes = [vp, cp, C.POINTER(vp)]
+        l.Blaze_ServePoolCreate.argtypes = [i, C.POINTER(vp)]
+        l.Blaze_ServePoolRun.argtypes = [vp, C.POINTER(vp), i, C.c_int64]
+        l.Blaze_ServePoolDelete.argtypes = [vp]
         _lib = l
     return _lib
 
@@ -189,6 +193,25 @@ class Predictor(object):
         p = C.c_void_p()
         check_call(lib().Blaze_PredictorOutputDevicePtr(self.handle, name.encode(), C.byref(p)))
         return p.value
+
+
+class ServePool(object):
+    """Persistent serving threads inside the library; run(predictors, steps) executes pass i on predictor
+    i % len(predictors) and thread i % n_threads, returning when all passes have finished on the device."""
+
+    def __init__(self, n_threads):
+        self.handle = C.c_void_p()
+        self.n_threads = n_threads
+        check_call(lib().Blaze_ServePoolCreate(n_threads, C.byref(self.handle)))
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib().Blaze_ServePoolDelete(self.handle)
+            self.handle = None
+
+    def run(self, predictors, steps):
+        arr = (C.c_void_p * len(predictors))(*[getattr(p.handle, "value", p.handle) for p in predictors])
+        check_call(lib().Blaze_ServePoolRun(self.handle, arr, len(predictors), steps))
 
 
 class PredictorManager(object):
