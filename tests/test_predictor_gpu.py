@@ -321,3 +321,37 @@ def test_fc_stack_as_one_launch_matches_layer_by_layer(pb, oracle):
     assert probs[True].shape == (300, 2)
     np.testing.assert_allclose(probs[True], probs[False], rtol=2e-3, atol=2e-3)
     np.testing.assert_allclose(probs[True].sum(1), 1.0, rtol=2e-3)
+
+
+def test_concat_inputs_written_in_place_give_identical_results(pb):
+    """Concat(dense, block) whose inputs are an external input and an Embedding block read by nothing else: both
+    live inside the Concat's output (the Feed copies rows at that tensor's pitch, the pooling kernel writes at it)
+    and nothing is copied.  Bit-identical to the net with the aliasing switched off, also after the batch size and
+    the fed data change."""
+    import torch
+    from ctr_model import build_manager, feed_inputs
+    from synth import Config2
+    cfg = Config2(batch=257, rows=3000, slots=26)
+    tables, mlp = cfg.tables(), cfg.mlp()
+    sparse, dense = cfg.batches(2)
+    small = Config2(batch=64, rows=3000, slots=26)
+    sparse_s, dense_s = small.batches(1, seed_offset=9)
+    outs = {}
+    for alias in (1, 0):
+        pm, fgs = build_manager(cfg, tables, mlp, np.float16, net_args={"alias_concat_inputs": alias})
+        p = pm.create_predictor(1, 0)
+        got = []
+        for sp, dn in ((sparse[0], dense[0]), (sparse_s[0], dense_s[0]), (sparse[1], dense[1])):  # batch 257 -> 64 -> 257
+            feed_inputs(p, fgs, sp, dn, np.float16)
+            p.forward()
+            got.append(p.output_asnumpy("prob").copy())
+        outs[alias] = got
+        if alias:
+            with pytest.raises(pb.BlazeError):
+                p.input_device_ptr("dense")  # a strided input has no plain buffer to hand out
+        else:
+            assert p.input_device_ptr("dense")
+    torch.cuda.synchronize()
+    for a, b in zip(outs[1], outs[0]):
+        assert a.shape == b.shape and np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    assert outs[1][0].shape == (257, 2) and outs[1][1].shape == (64, 2)

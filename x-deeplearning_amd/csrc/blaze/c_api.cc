@@ -469,7 +469,7 @@ int Blaze_PredictorInputDevicePtr(PredictorHandle handle, const char* name, void
   auto* p = reinterpret_cast<Predictor*>(handle);
   if (p == nullptr || ptr == nullptr) return -1;
   *ptr = p->InputDevicePtr(name);
-  return *ptr ? 0 : Fail("not an input of the net");
+  return *ptr ? 0 : Fail("not an input of the net (or an input that lives inside a Concat output and has no plain buffer)");
 }
 int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char* name, void** ptr) {
   auto* p = reinterpret_cast<Predictor*>(handle);

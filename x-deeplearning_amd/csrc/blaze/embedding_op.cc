@@ -141,6 +141,10 @@ class EmbeddingOp final : public Operator<Context> {
     }
   }
 
+  TIndex StaticOutputCols(int idx) const override {
+    return idx >= 0 && (size_t)idx < config_.block_config.size() ? (TIndex)config_.block_config[idx].stride : 0;
+  }
+
   void RunEmbedding(int key_type, int value_type, int num_type) {
     const size_t n_fg = config_.feature_group_config.size();
     std::vector<store::SparsePullerInput> inputs(n_fg);
@@ -180,14 +184,19 @@ class EmbeddingOp final : public Operator<Context> {
         Blob* block = this->Output(bi.block_idx);
         out.out_type = block->data_type();
         out.out_item[j].out = (char*)block->data() + item.offset * DataTypeSize(block->data_type());
-        out.out_item[j].stride = config_.block_config[bi.block_idx].stride;
+        // a block that lives inside a Concat's output has that tensor's row pitch
+        out.out_item[j].stride = block->pitch() ? (int)block->pitch() : config_.block_config[bi.block_idx].stride;
       }
     }
     hipStream_t st = context_.hip_stream();
     for (size_t b = 0; b < needs_zero_.size(); ++b)
       if (needs_zero_[b]) {
         Blob* block = this->Output((int)b);
-        HIP_CHECK(hipMemsetAsync(block->data(), 0, block->size() * DataTypeSize(block->data_type()), st));
+        const size_t es = DataTypeSize(block->data_type());
+        if (block->pitch())
+          HIP_CHECK(hipMemset2DAsync(block->data(), block->pitch() * es, 0, block->shape()[1] * es, block->shape()[0], st));
+        else
+          HIP_CHECK(hipMemsetAsync(block->data(), 0, block->size() * es, st));
       }
     auto status = sparse_puller_->GetOnStream(inputs, outputs, st, &cache_);
     BLAZE_CONDITION_THROW(status == store::kOK, "pull data failed, status=", status);

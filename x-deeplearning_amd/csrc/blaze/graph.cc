@@ -199,6 +199,51 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
       if (producer->TryFuse(operators_[i + 1].get())) skipped_[i + 1] = true;
     }
     StackFcLayers();
+    AliasConcatInputs();
+  }
+}
+
+// Concat along the last axis of 2-D tensors whose inputs are all either blocks of an Embedding operator or
+// external inputs, each read by nothing else: the inputs become column slices of the Concat's output (their
+// producers write in place) and the Concat has nothing left to copy.
+void SimpleNet::AliasConcatInputs() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "alias_concat_inputs");
+  if (arg && arg->has_i && arg->i == 0) return;
+  for (size_t c = 0; c < operators_.size(); ++c) {
+    if (skipped_[c] || operators_[c]->type() != "Concat") continue;
+    const OperatorDef& cd = operators_[c]->operator_def();
+    if (ArgumentHelper::GetSingle<int>(cd.arg(), "axis", 1) != 1 || cd.input_size() < 1) continue;
+    std::vector<Blob*> children;
+    std::vector<TIndex> widths;
+    bool ok = true;
+    for (int i = 0; i < cd.input_size() && ok; ++i) {
+      const std::string& name = cd.input(i);
+      int readers = 0;
+      for (size_t j = 0; j < operators_.size(); ++j)
+        for (const auto& in : operators_[j]->operator_def().input()) readers += (in == name);
+      for (const auto& eo : external_output_) readers += (eo == name);
+      if (readers != 1 || workspace_->HasConstantBlob(name)) {
+        ok = false;
+        break;
+      }
+      TIndex w = 0;
+      bool produced = false;
+      for (size_t j = 0; j < c && !produced; ++j) {
+        const OperatorDef& pd = operators_[j]->operator_def();
+        for (int o = 0; o < pd.output_size(); ++o) {
+          if (pd.output(o) != name) continue;
+          produced = true;
+          w = operators_[j]->StaticOutputCols(o);
+          if (operators_[j]->type() != "Embedding" || w == 0) ok = false;
+        }
+      }
+      bool external = false;
+      for (const auto& ei : external_input_) external |= (ei == name);
+      if (!produced && !external) ok = false;
+      children.push_back(operators_[c]->Input(i));
+      widths.push_back(w);
+    }
+    if (ok) Blob::LinkColumnSlices(operators_[c]->Output(0), children, widths);
   }
 }
 

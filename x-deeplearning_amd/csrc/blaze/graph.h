@@ -91,6 +91,7 @@ class SimpleNet : public Net {
  protected:
   bool RunImpl() override;
   void StackFcLayers();
+  void AliasConcatInputs();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 

@@ -261,26 +261,34 @@ class ConcatOp final : public Operator<Context> {
     const size_t es = DataTypeSize(y->data_type());
     const TIndex outer = y->size(0, axis_), inner = y->size(axis_ + 1, (int)rank);
     hipStream_t st = context_.hip_stream();
-    // one launch per group of BZ_CONCAT_MAX pieces
+    // pieces that already live in the output (column-slice views their producers wrote in place) are skipped;
+    // the others are copied, one launch per group of BZ_CONCAT_MAX
+    bz_concat_desc d;
+    memset(&d, 0, sizeof(d));
     size_t col = 0;
-    for (int i0 = 0; i0 < this->InputSize(); i0 += BZ_CONCAT_MAX) {
-      bz_concat_desc d;
-      memset(&d, 0, sizeof(d));
-      d.n = std::min(BZ_CONCAT_MAX, this->InputSize() - i0);
-      size_t group = 0;
-      for (int i = 0; i < d.n; ++i) {
-        Blob* x = this->Input(i0 + i);
-        d.src[i] = x->data();
-        d.width[i] = (int64_t)(x->shape()[axis_] * inner * es);
-        d.src_pitch[i] = d.width[i];
-        group += (size_t)d.width[i];
-      }
-      d.dst = (char*)y->data() + col;  // this group starts `col` bytes into every output row
+    auto flush = [&]() {
+      if (d.n == 0) return;
       d.dst_pitch = (int64_t)(total * inner * es);
       d.rows = (int64_t)outer;
       BZ_CHECK(bz_concat_cols(&d, st));
-      col += group;
+      memset(&d, 0, sizeof(d));
+    };
+    for (int i = 0; i < this->InputSize(); ++i) {
+      Blob* x = this->Input(i);
+      const size_t width = (size_t)(x->shape()[axis_] * inner * es);
+      const bool in_place = rank == 2 && axis_ == 1 && x->IsColumnSliceOf(y, (TIndex)(col / es));
+      if (in_place || d.n == BZ_CONCAT_MAX) flush();
+      if (!in_place) {
+        BLAZE_CONDITION_THROW(x->pitch() == 0, "concat input ", i, " is a strided view of another tensor");
+        if (d.n == 0) d.dst = (char*)y->data() + col;  // this group starts `col` bytes into every output row
+        d.src[d.n] = x->data();
+        d.width[d.n] = (int64_t)width;
+        d.src_pitch[d.n] = (int64_t)width;
+        ++d.n;
+      }
+      col += width;
     }
+    flush();
     return true;
   }
 

@@ -127,6 +127,8 @@ class OperatorBase {
 
   virtual bool Run(int stream_id = 0) = 0;
   virtual void WaitStream(int stream_id = -1) {}
+  // columns of 2-D output `idx` when they are fixed by the operator's arguments (else 0)
+  virtual TIndex StaticOutputCols(int idx) const { return 0; }
 
   const DeviceOption& device_option() const { return device_option_; }
   void set_net_position(int p) { net_position_ = p; }

@@ -79,7 +79,14 @@ bool Predictor::Feed(size_t idx, const void* data, size_t len) {
     } else {
       HIPContext ctx(blob->device_option());
       ctx.Activate();
-      CopyBytes(blob->data(), kHIP, data, kCPU, need, ctx.hip_stream());
+      if (blob->pitch() != 0) {  // the input lives inside a Concat's output: rows are `pitch` elements apart
+        const size_t es = DataTypeSize(blob->data_type()), w = blob->shape()[1] * es;
+        HIP_CHECK(hipMemcpy2DAsync(blob->data(), blob->pitch() * es, data, w, w, blob->shape()[0], hipMemcpyHostToDevice,
+                                   ctx.hip_stream()));
+        HIP_CHECK(hipStreamSynchronize(ctx.hip_stream()));
+      } else {
+        CopyBytes(blob->data(), kHIP, data, kCPU, need, ctx.hip_stream());
+      }
     }
   } catch (std::exception& e) {
     LOG_ERROR("feed failed: %s", e.what());
@@ -209,7 +216,8 @@ void Predictor::DumpObservers(std::unordered_map<std::string, std::string>* dump
 
 void* Predictor::InputDevicePtr(const char* name) {
   const int idx = InputName2Idx(name);
-  return idx < 0 ? nullptr : external_input_blob_[idx]->data();
+  // (a strided input -- one that lives inside a Concat's output -- has no plain buffer to hand out)
+  return idx < 0 || external_input_blob_[idx]->pitch() != 0 ? nullptr : external_input_blob_[idx]->data();
 }
 void* Predictor::OutputDevicePtr(const char* name) {
   const int idx = OutputName2Idx(name);

@@ -32,15 +32,19 @@ class Blob {
   Blob& operator=(const Blob&) = delete;
 
   void Reshape(const std::vector<TIndex>& dims) {
+    if (slices_ && slices_->parent != this && ReshapeAsSlice(dims)) return;
     TIndex n = 1;
     for (auto d : dims) n *= d;
     size_ = n;
     if (size_ > capacity_ || !own_handle_) {
       Destroy();
       own_handle_ = true;
+      slice_view_ = false;
+      pitch_ = 0;
       capacity_ = size_;
       data_ = blaze::Alloc(capacity_ * DataTypeSize(data_type_), device_option_.device_type(), device_option_.device_id());
       ++version_;
+      if (slices_ && slices_->parent == this) RefreshSlices();
     }
     dims_ = dims;
   }
@@ -51,10 +55,39 @@ class Blob {
       data_ = handle;
       ++version_;
     }
+    pitch_ = 0;
+    slice_view_ = false;
     TIndex n = 1;
     for (auto d : dims) n *= d;
     size_ = capacity_ = n;
     dims_ = dims;
+  }
+
+  // ---- column slices: the inputs of a Concat along the last axis of 2-D tensors living directly in the
+  // Concat's output, so that their producers write in place and the Concat has nothing to copy.  `children` are
+  // the Concat's inputs in order; widths[i] is child i's column count (0 = not known yet).  A child becomes a
+  // view (row pitch = the parent's width) when it is reshaped to 2-D while every width is known; any other
+  // Reshape gives it memory of its own again.  The parent refreshes the views whenever its buffer moves.
+  struct SliceGroup {
+    Blob* parent = nullptr;
+    std::vector<Blob*> children;
+    std::vector<TIndex> widths;
+  };
+  static void LinkColumnSlices(Blob* parent, const std::vector<Blob*>& children, const std::vector<TIndex>& static_widths) {
+    auto g = std::make_shared<SliceGroup>();
+    g->parent = parent;
+    g->children = children;
+    g->widths = static_widths;
+    parent->slices_ = g;
+    for (Blob* c : children) c->slices_ = g;
+  }
+  // elements between consecutive rows when this blob is a column slice, else 0 (rows are contiguous)
+  TIndex pitch() const { return pitch_; }
+  // whether this blob currently is the view of `parent`'s columns [col, col + shape[1])
+  bool IsColumnSliceOf(const Blob* parent, TIndex col) const {
+    return slice_view_ && slices_ && slices_->parent == parent && parent->data_ != nullptr &&
+           parent->dims_.size() == 2 && pitch_ == parent->dims_[1] &&
+           data_ == (const char*)parent->data_ + col * DataTypeSize(data_type_);
   }
   const DeviceOption& device_option() const { return device_option_; }
   int device_type() const { return device_option_.device_type(); }
@@ -86,6 +119,43 @@ class Blob {
   uint64_t version() const { return version_; }
 
  private:
+  bool ReshapeAsSlice(const std::vector<TIndex>& dims) {
+    SliceGroup& g = *slices_;
+    size_t me = 0;
+    while (me < g.children.size() && g.children[me] != this) ++me;
+    if (me == g.children.size() || dims.size() != 2 || g.parent->data_type_ != data_type_) return false;
+    g.widths[me] = dims[1];
+    TIndex total = 0;
+    for (TIndex w : g.widths) {
+      if (w == 0) return false;
+      total += w;
+    }
+    if (own_handle_) Destroy();
+    if (!slice_view_) data_ = nullptr;
+    own_handle_ = false;
+    slice_view_ = true;
+    dims_ = dims;
+    size_ = capacity_ = dims[0] * dims[1];
+    g.parent->Reshape({dims[0], total});  // grows the buffer when needed
+    g.parent->RefreshSlices();            // widths may have moved every view
+    return true;
+  }
+  void RefreshSlices() {
+    SliceGroup& g = *slices_;
+    TIndex total = 0;
+    for (TIndex w : g.widths) total += w;
+    TIndex col = 0;
+    for (size_t i = 0; i < g.children.size(); ++i) {
+      Blob* c = g.children[i];
+      if (c->slice_view_) {
+        void* p = (char*)data_ + col * DataTypeSize(data_type_);
+        if (c->data_ != p || c->pitch_ != total) ++c->version_;
+        c->data_ = p;
+        c->pitch_ = total;
+      }
+      col += g.widths[i];
+    }
+  }
   void Destroy() {
     if (data_ != nullptr && own_handle_)
       blaze::Free(data_, device_option_.device_type(), device_option_.device_id());
@@ -99,6 +169,9 @@ class Blob {
   DataType data_type_ = kFloat;
   bool own_handle_ = true;
   uint64_t version_ = 0;
+  TIndex pitch_ = 0;
+  bool slice_view_ = false;
+  std::shared_ptr<SliceGroup> slices_;
 };
 
 constexpr int kMaxStreamNum = 4;  // blaze/common/context.h:121
