@@ -302,7 +302,7 @@ void SimpleNet::StackFcLayers() {
       int need[2] = {lds[0], lds[1]};
       int hb = 0;
       if (is_head)
-        hb = n2 * k2 * 2;
+        hb = n2 * k2 * 2 + 128;
       else
         need[chain.size() & 1] = std::max(need[chain.size() & 1], 64 * (n2 * 2 + 16));
       if (2 * 64 * (64 * 2 + 16) + need[0] + need[1] + hb > 160 * 1024) break;

@@ -25,6 +25,8 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "bz_common.h"
 
 namespace {
@@ -90,6 +92,25 @@ __device__ __forceinline__ float apply_act_regs(float v, const Epilogue& e, floa
     }
     default:
       return v;
+  }
+}
+
+template <int ACT>
+__device__ __forceinline__ float apply_act_t(float v, const Epilogue& e, float p0, float p1, float p2) {
+  if constexpr (ACT == BZ_ACT_PRELU) {
+    return v * ((float)(v > 0.f) + (float)(v < 0.f) * p0);
+  } else if constexpr (ACT == BZ_ACT_DICE) {
+    const float den = e.dice_nosqrt ? p2 : sqrtf(p2 + kDiceEps);
+    const float t = expf(-1.f * (v - p1) / den);
+    const float p = 1.f / (1.f + t);
+    return (1.f - p) * p0 * v + p * v;
+  } else if constexpr (ACT == BZ_ACT_LEAKY_RELU) {
+    return v >= 0.f ? v : e.act_alpha * v;
+  } else if constexpr (ACT == BZ_ACT_SIGMOID) {
+    const float t = expf(v);
+    return t / (1.f + t);
+  } else {
+    return v;
   }
 }
 
@@ -345,31 +366,53 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   constexpr int OPITCH = BN * OS + 16;
   static_assert(BM * OPITCH <= (int)sizeof(lds), "output tile must fit the operand buffers");
   char* lout = &lds[0][0];
+  // The activation is a compile-time parameter of the element loop: a run-time switch per element would turn the
+  // unrolled epilogue into a string of taken branches over far more code than the loop needs.
+  auto epilogue = [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int nl = wn * WTN + j * 32 + (lane & 31);
-    const int n = n0 + nl;
-    const bool n_ok = n < N;
+    for (int j = 0; j < TN; ++j) {
+      const int nl = wn * WTN + j * 32 + (lane & 31);
+      const int n = n0 + nl;
+      const bool n_ok = n < N;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        const int m = m0 + ml;
-        if (m < M && n_ok) {
-          float v = ep.alpha * acc[0][i][j][r];
-          if (ep.bias_rows == 1)
-            v += ep.beta * cbias[j];
-          else if (ep.bias_rows > 1)
-            v += ep.beta * ep.bias[(int64_t)m * N + n];
-          v = apply_act_regs(v, ep, cp0[j], cp1[j], cp2[j]);
-          if (vec_y)
-            store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
-          else
-            store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+        for (int r = 0; r < 16; ++r) {
+          const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int m = m0 + ml;
+          if (m < M && n_ok) {
+            float v = ep.alpha * acc[0][i][j][r];
+            if (ep.bias_rows == 1)
+              v += ep.beta * cbias[j];
+            else if (ep.bias_rows > 1)
+              v += ep.beta * ep.bias[(int64_t)m * N + n];
+            v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
+            if (vec_y)
+              store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
+            else
+              store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+          }
         }
       }
     }
+  };
+  switch (ep.act) {
+    case BZ_ACT_PRELU:
+      epilogue(std::integral_constant<int, BZ_ACT_PRELU>());
+      break;
+    case BZ_ACT_DICE:
+      epilogue(std::integral_constant<int, BZ_ACT_DICE>());
+      break;
+    case BZ_ACT_LEAKY_RELU:
+      epilogue(std::integral_constant<int, BZ_ACT_LEAKY_RELU>());
+      break;
+    case BZ_ACT_SIGMOID:
+      epilogue(std::integral_constant<int, BZ_ACT_SIGMOID>());
+      break;
+    default:
+      epilogue(std::integral_constant<int, BZ_ACT_NONE>());
+      break;
   }
   if (vec_y) {
     __syncthreads();

@@ -318,83 +318,72 @@ __device__ __forceinline__ void wide_layer_any(const MlpP& P, const LayerP& L, i
   }
 }
 
-// The head: N <= 8 outputs per row from the activations in LDS.  Four lanes share a row (a quarter of K each),
-// reduce by shuffles, then every lane of the group holds the row's N values for the softmax.
+// The head: N <= 8 outputs per row from the activations in LDS.  Four lanes share a row (a quarter of K each) and
+// reduce by shuffles; the logits go through a small LDS scratch, then one lane per row applies the activation /
+// softmax.  Loops over the outputs are kept rolled: this code runs once per launch, and unrolled it would cost more
+// in instruction fetch than it saves in issue slots.
 template <int DT>
 __device__ __forceinline__ void skinny_layer(const MlpP& P, const LayerP& L, int m0, const char* hin, int hin_pitch,
-                                             const char* wl) {
+                                             const char* wl, const float* hp, float* logits) {
   const int tid = threadIdx.x;
   const int row = tid >> 2, part = tid & 3;
   const int K = L.k;  // a multiple of 128
+  const int N = L.n;
+  const int act = L.act;
+  const float alpha = L.alpha, beta = L.bias ? L.beta : 0.f;
   const int kq = K / 4;
-  float dot[BZ_MLP_MAX_HEAD];
+  const char* ap = hin + row * hin_pitch + part * kq * 2;
+  const char* wp = wl + part * kq * 2;
+#pragma unroll 1
+  for (int j = 0; j < N; ++j) {
+    float dot = 0.f;
+    for (int c = 0; c < kq; c += 8) {
+      const uint4 av = *(const uint4*)(ap + c * 2);
+      const uint4 wv = *(const uint4*)(wp + (j * K + c) * 2);
+      const uint32_t ar[4] = {av.x, av.y, av.z, av.w};
+      const uint32_t wr[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
-  for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j) dot[j] = 0.f;
-  for (int c = 0; c < kq; c += 8) {
-    const int k = part * kq + c;
-    const uint4 av = *(const uint4*)(hin + row * hin_pitch + k * 2);
-    const uint32_t ar[4] = {av.x, av.y, av.z, av.w};
-    float a[8];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      a[2 * e] = from_bits<DT>((uint16_t)(ar[e] & 0xffffu));
-      a[2 * e + 1] = from_bits<DT>((uint16_t)(ar[e] >> 16));
-    }
-#pragma unroll
-    for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j) {
-      if (j < L.n) {
-        const uint4 wv = *(const uint4*)(wl + (j * K + k) * 2);
-        const uint32_t wr[4] = {wv.x, wv.y, wv.z, wv.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          dot[j] += a[2 * e] * from_bits<DT>((uint16_t)(wr[e] & 0xffffu));
-          dot[j] += a[2 * e + 1] * from_bits<DT>((uint16_t)(wr[e] >> 16));
-        }
+      for (int e = 0; e < 4; ++e) {
+        dot += from_bits<DT>((uint16_t)(ar[e] & 0xffffu)) * from_bits<DT>((uint16_t)(wr[e] & 0xffffu));
+        dot += from_bits<DT>((uint16_t)(ar[e] >> 16)) * from_bits<DT>((uint16_t)(wr[e] >> 16));
       }
     }
+    dot += __shfl_xor(dot, 1, 64);
+    dot += __shfl_xor(dot, 2, 64);
+    // hp: [bias | p0 | p1 | p2] x 8, staged in LDS at kernel start (zero where a parameter does not apply)
+    if (part == 0) logits[row * BZ_MLP_MAX_HEAD + j] = alpha * dot + beta * hp[j];
   }
-  float v[BZ_MLP_MAX_HEAD];
+  __syncthreads();
+  if (tid >= kBM) return;
+  float* lr = logits + tid * BZ_MLP_MAX_HEAD;
+  const int m = m0 + tid;
   float mx = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j) {
-    float d = dot[j];
-    d += __shfl_xor(d, 1, 64);
-    d += __shfl_xor(d, 2, 64);
-    v[j] = 0.f;
-    if (j < L.n) {
-      float t = L.alpha * d;
-      if (L.bias) t += L.beta * L.bias[j];
-      if (L.act != BZ_ACT_SOFTMAX) {
-        const float p0 = (L.act == BZ_ACT_PRELU) ? L.p0[L.act_size == 1 ? 0 : j] : (L.act == BZ_ACT_DICE ? L.p0[j] : 0.f);
-        const float p1 = L.act == BZ_ACT_DICE ? L.p1[j] : 0.f;
-        const float p2 = L.act == BZ_ACT_DICE ? L.p2[j] : 0.f;
-        t = act_apply(t, L, p0, p1, p2);
-      }
-      v[j] = t;
-      mx = fmaxf(mx, t);
+#pragma unroll 1
+  for (int j = 0; j < N; ++j) {
+    float t = lr[j];
+    if (act != BZ_ACT_SOFTMAX && act != BZ_ACT_NONE) t = act_apply(t, L, hp[8 + j], hp[16 + j], hp[24 + j]);
+    lr[j] = t;
+    mx = fmaxf(mx, t);
+  }
+  float sum = 1.f;
+  if (act == BZ_ACT_SOFTMAX) {  // softmax_op.cc:21-78: subtract the max, exp, divide by the sum
+    sum = 0.f;
+#pragma unroll 1
+    for (int j = 0; j < N; ++j) {
+      const float e = expf(lr[j] - mx);
+      lr[j] = e;
+      sum += e;
     }
   }
-  if (L.act == BZ_ACT_SOFTMAX) {  // softmax_op.cc:21-78: subtract the max, exp, divide by the sum
-    float sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j)
-      if (j < L.n) {
-        v[j] = expf(v[j] - mx);
-        sum += v[j];
-      }
-#pragma unroll
-    for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j) v[j] = v[j] / sum;
-  }
-  const int m = m0 + row;
-  if (part == 0 && m < P.m) {
-#pragma unroll
-    for (int j = 0; j < BZ_MLP_MAX_HEAD; ++j)
-      if (j < L.n) {
-        if (P.out_dtype == BZ_F32)
-          ((float*)P.y)[(int64_t)m * P.ldy + j] = v[j];
-        else
-          ((uint16_t*)P.y)[(int64_t)m * P.ldy + j] = to_bits<DT>(v[j]);
-      }
+  if (m >= P.m) return;
+  const bool f32 = P.out_dtype == BZ_F32;
+#pragma unroll 1
+  for (int j = 0; j < N; ++j) {
+    const float v = act == BZ_ACT_SOFTMAX ? lr[j] / sum : lr[j];
+    if (f32)
+      ((float*)P.y)[(int64_t)m * P.ldy + j] = v;
+    else
+      ((uint16_t*)P.y)[(int64_t)m * P.ldy + j] = to_bits<DT>(v);
   }
 }
 
@@ -419,6 +408,14 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
       hw[i] = *(const uint4*)(H.w + ((int64_t)j * H.ldw + ch * 8) * 2);
     }
   }
+  // ... and its per-output parameters: thread 8*a + j fetches element j of array a (bias, p0, p1, p2)
+  float hp = 0.f;
+  if (P.skinny_last && threadIdx.x < 32) {
+    const int a = threadIdx.x >> 3, j = threadIdx.x & 7;
+    const float* src = a == 0 ? H.bias : (a == 1 ? H.p0 : (a == 2 ? H.p1 : H.p2));
+    const bool used = a == 0 || (a == 1 && (H.act == BZ_ACT_PRELU || H.act == BZ_ACT_DICE)) || (a >= 2 && H.act == BZ_ACT_DICE);
+    if (src != nullptr && used && j < H.n) hp = src[(a == 1 && H.act == BZ_ACT_PRELU && H.act_size == 1) ? 0 : j];
+  }
   for (int li = 0; li < n_wide; ++li) {
     char* hout = lds + P.h_off[li & 1];
     if (li == 0) {
@@ -428,6 +425,7 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
         const int q = threadIdx.x + i * kThreads;
         if (q < head_chunks) *(uint4*)(lds + P.head_off + q * 16) = hw[i];
       }
+      if (P.skinny_last && threadIdx.x < 32) *(float*)(lds + P.head_off + head_chunks * 16 + threadIdx.x * 4) = hp;
     } else {
       wide_layer_any<DT, false>(P, P.l[li], m0, lds, hin, hin_pitch, hout);
     }
@@ -436,7 +434,8 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
     hin_pitch = P.l[li].n * 2 + 16;
   }
   if (P.skinny_last) {
-    skinny_layer<DT>(P, P.l[P.n_layers - 1], m0, hin, hin_pitch, lds + P.head_off);
+    skinny_layer<DT>(P, P.l[P.n_layers - 1], m0, hin, hin_pitch, lds + P.head_off,
+                     (const float*)(lds + P.head_off + head_chunks * 16), (float*)lds);
   } else {
     // the last wide layer's tile: LDS -> global, 16 bytes per lane along rows
     const int n = P.l[n_wide - 1].n;
@@ -569,7 +568,7 @@ extern "C" int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream) {
   P.h_off[0] = a_bytes;
   P.h_off[1] = a_bytes + h_size[0];
   P.head_off = a_bytes + h_size[0] + h_size[1];
-  const int lds_bytes = P.head_off + (skinny_last ? last.n * last.k * 2 : 0);
+  const int lds_bytes = P.head_off + (skinny_last ? last.n * last.k * 2 + 128 : 0);
   BZ_REQUIRE(lds_bytes <= 160 * 1024, "bz_mlp_fused: the stack needs %d bytes of LDS (limit 163840)", lds_bytes);
   hipStream_t st = bz::as_stream(stream);
   const int grid = (d.m + kBM - 1) / kBM;
