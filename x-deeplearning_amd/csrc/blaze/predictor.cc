@@ -1,5 +1,7 @@
 #include "blaze/predictor.h"
 
+#include <algorithm>
+
 #include "blaze/qed_store.h"
 
 namespace blaze {
@@ -20,6 +22,17 @@ Predictor::Predictor(std::shared_ptr<Net> net) : net_(net) {
     BLAZE_CONDITION_THROW(b != nullptr, "external_input: ", name, " is not in external_input_blob");
     input_index_[name] = (int)external_input_blob_.size();
     external_input_blob_.push_back(b);
+    DeviceOption cpu;
+    cpu.set_device_type(kCPU);
+    input_cpu_.push_back(std::make_shared<Blob>(cpu));
+    feed_pending_.push_back(false);
+  }
+}
+
+Predictor::~Predictor() {
+  if (feed_done_) {
+    (void)hipEventSynchronize(feed_done_);
+    (void)hipEventDestroy(feed_done_);
   }
 }
 
@@ -79,14 +92,27 @@ bool Predictor::Feed(size_t idx, const void* data, size_t len) {
     } else {
       HIPContext ctx(blob->device_option());
       ctx.Activate();
+      hipStream_t st = ctx.hip_stream();
+      // stage in pinned memory and queue the transfer; a second Feed of the same input first waits for the first
+      if (feed_done_ == nullptr) HIP_CHECK(hipEventCreateWithFlags(&feed_done_, hipEventDisableTiming));
+      if (feed_pending_[idx]) {
+        HIP_CHECK(hipEventSynchronize(feed_done_));
+        std::fill(feed_pending_.begin(), feed_pending_.end(), false);
+        any_feed_pending_ = false;
+      }
+      Blob* stage = input_cpu_[idx].get();
+      stage->set_data_type((DataType)blob->data_type());
+      stage->Reshape(blob->shape());
+      memcpy(stage->data(), data, need);
       if (blob->pitch() != 0) {  // the input lives inside a Concat's output: rows are `pitch` elements apart
         const size_t es = DataTypeSize(blob->data_type()), w = blob->shape()[1] * es;
-        HIP_CHECK(hipMemcpy2DAsync(blob->data(), blob->pitch() * es, data, w, w, blob->shape()[0], hipMemcpyHostToDevice,
-                                   ctx.hip_stream()));
-        HIP_CHECK(hipStreamSynchronize(ctx.hip_stream()));
-      } else {
-        CopyBytes(blob->data(), kHIP, data, kCPU, need, ctx.hip_stream());
+        HIP_CHECK(hipMemcpy2DAsync(blob->data(), blob->pitch() * es, stage->data(), w, w, blob->shape()[0], hipMemcpyHostToDevice, st));
+      } else if (need > 0) {
+        HIP_CHECK(hipMemcpyAsync(blob->data(), stage->data(), need, hipMemcpyHostToDevice, st));
       }
+      HIP_CHECK(hipEventRecord(feed_done_, st));
+      feed_pending_[idx] = true;
+      any_feed_pending_ = true;
     }
   } catch (std::exception& e) {
     LOG_ERROR("feed failed: %s", e.what());
@@ -102,7 +128,21 @@ int Predictor::InputDataType(const char* name) const {
 
 bool Predictor::Forward(const PredictorCallback&& cb) {
   try {
+    if (any_feed_pending_) {
+      // the transfers were queued on the feeding thread's stream: make this thread's stream wait for them
+      for (Blob* b : external_input_blob_) {
+        if (b->device_type() != kHIP) continue;
+        HIPContext ctx(b->device_option());
+        ctx.Activate();
+        HIP_CHECK(hipStreamWaitEvent(ctx.hip_stream(), feed_done_, 0));
+        break;
+      }
+    }
     if (!net_->Run()) return false;
+    if (any_feed_pending_) {  // Run waited for the stream, which had waited for the transfers
+      std::fill(feed_pending_.begin(), feed_pending_.end(), false);
+      any_feed_pending_ = false;
+    }
     if (cb) cb();
     return true;
   } catch (std::exception& e) {

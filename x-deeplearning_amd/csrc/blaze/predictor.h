@@ -30,6 +30,9 @@ std::string& last_error_for_thread();
 class Predictor {
  public:
   explicit Predictor(std::shared_ptr<Net> net);
+  ~Predictor();
+  Predictor(const Predictor&) = delete;
+  Predictor& operator=(const Predictor&) = delete;
   bool ReshapeInput(const char* name, const std::vector<size_t>& shape);
   bool ReshapeInput(size_t idx, const std::vector<size_t>& shape);
   // copies len bytes in; len must equal size * sizeof(dtype) (predictor_impl.cc:110-138)
@@ -70,6 +73,13 @@ class Predictor {
   std::vector<Blob*> external_input_blob_, external_output_blob_;
   std::unordered_map<std::string, int> input_index_, output_index_;
   std::vector<std::shared_ptr<Blob>> output_cpu_;
+  // pinned staging of fed inputs: Feed copies the caller's bytes here and queues the transfer on the thread's
+  // stream; Forward runs behind it on the same stream.  feed_pending_[i]: input i's staging is still being read.
+  std::vector<std::shared_ptr<Blob>> input_cpu_;
+  std::vector<bool> feed_pending_;
+  bool any_feed_pending_ = false;
+  hipEvent_t feed_done_ = nullptr;  // recorded behind the last queued transfer; Forward's stream waits for it
+                                    // (Feed and Forward may be called from different threads = different streams)
   std::unordered_map<std::string, std::shared_ptr<Blob>> param_cpu_;
 };
 

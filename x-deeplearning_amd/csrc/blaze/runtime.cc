@@ -2,12 +2,31 @@
 
 #include <stdlib.h>
 
+#include <mutex>
+#include <unordered_set>
+
 namespace blaze {
+
+namespace {
+// host blocks that came from hipHostMalloc (the rest came from malloc, when no device is usable)
+std::mutex g_pinned_mu;
+std::unordered_set<void*>& PinnedSet() {
+  static std::unordered_set<void*> s;
+  return s;
+}
+}  // namespace
 
 void* Alloc(size_t bytes, int device_type, int device_id) {
   if (bytes == 0) bytes = 16;
   void* p = nullptr;
   if (device_type == kCPU) {
+    // pinned, so that Feed / Output copies are real DMA transfers instead of the runtime's staged pageable path
+    if (hipHostMalloc(&p, bytes, hipHostMallocDefault) == hipSuccess && p != nullptr) {
+      std::lock_guard<std::mutex> lock(g_pinned_mu);
+      PinnedSet().insert(p);
+      return p;
+    }
+    (void)hipGetLastError();
     p = malloc(bytes);
     BLAZE_CONDITION_THROW(p != nullptr, "malloc of ", bytes, " bytes failed");
     return p;
@@ -23,7 +42,15 @@ void* Alloc(size_t bytes, int device_type, int device_id) {
 void Free(void* ptr, int device_type, int) {
   if (ptr == nullptr) return;
   if (device_type == kCPU) {
-    free(ptr);
+    bool pinned;
+    {
+      std::lock_guard<std::mutex> lock(g_pinned_mu);
+      pinned = PinnedSet().erase(ptr) != 0;
+    }
+    if (pinned)
+      (void)hipHostFree(ptr);
+    else
+      free(ptr);
   } else {
     (void)hipFree(ptr);
   }

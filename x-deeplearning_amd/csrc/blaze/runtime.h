@@ -16,7 +16,7 @@
 namespace blaze {
 
 // cudaMalloc / malloc twins of blaze/common/allocator.h:33-71.  Host memory for device_type kCPU is pinned
-// (hipHostMalloc) when `pinned`, so Feed/Output copies run at full PCIe rate.
+// (hipHostMalloc) whenever a device is usable, so Feed / Output copies run at full PCIe rate; plain malloc otherwise.
 void* Alloc(size_t bytes, int device_type, int device_id);
 void Free(void* ptr, int device_type, int device_id);
 
