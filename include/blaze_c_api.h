@@ -115,14 +115,26 @@ BLAZE_API int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char*
 BLAZE_API int Blaze_PredictorForwardN(PredictorHandle handle, int count);
 
 /*
+ * Forward in two halves (no counterpart in the reference, whose Forward is synchronous): ForwardLaunch queues the whole
+ * pass on the calling thread's stream and returns, ForwardWait (same thread) returns once that pass has finished on
+ * the device.  A thread that owns several predictors can so keep more than one pass queued.  Between the two calls the
+ * predictor must not be fed, read or launched again.
+ */
+BLAZE_API int Blaze_PredictorForwardLaunch(PredictorHandle handle);
+BLAZE_API int Blaze_PredictorForwardWait(PredictorHandle handle);
+
+/*
  * A pool of serving threads (no counterpart in the reference's C API; its C++ example runs one loop per thread,
  * blaze/example/cpp/predictor_example.cc).  Blaze_ServePoolRun runs `steps` forward passes: pass i runs predictor
  * i % n_predictors on thread i % n_threads, and returns when all of them have finished on the device.  n_predictors
- * must be a multiple of the pool's thread count so that a predictor only ever runs on one thread.
+ * must be a multiple of the pool's thread count so that a predictor only ever runs on one thread.  A thread keeps up
+ * to `depth` passes (default 2; 1 = plain synchronous Forward calls) of different predictors queued on its stream,
+ * launching the next before it waits for the oldest; it needs that many predictors per thread to do so.
  */
 typedef void* ServePoolHandle;
 BLAZE_API int Blaze_ServePoolCreate(int n_threads, ServePoolHandle* handle);
 BLAZE_API int Blaze_ServePoolRun(ServePoolHandle handle, PredictorHandle* predictors, int n_predictors, int64_t steps);
+BLAZE_API int Blaze_ServePoolSetDepth(ServePoolHandle handle, int depth);
 BLAZE_API int Blaze_ServePoolDelete(ServePoolHandle handle);
 
 #ifdef __cplusplus

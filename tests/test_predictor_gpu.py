@@ -355,3 +355,44 @@ def test_concat_inputs_written_in_place_give_identical_results(pb):
     for a, b in zip(outs[1], outs[0]):
         assert a.shape == b.shape and np.array_equal(a.view(np.uint16), b.view(np.uint16))
     assert outs[1][0].shape == (257, 2) and outs[1][1].shape == (64, 2)
+
+
+def test_forward_in_two_halves_and_serve_pool_match_plain_forward(pb):
+    """ForwardLaunch / ForwardWait keep two predictors of one thread queued at once, and the serving pool does the
+    same inside the library (depth 2) or calls plain Forward (depth 1): every predictor ends with bit-identical
+    probabilities to its own synchronous Forward.  ForwardWait without a launch is an error, not a hang."""
+    import torch
+    from ctr_model import build_manager, make_predictor
+    from synth import Config2
+    cfg = Config2(batch=200, rows=3000, slots=26)
+    tables, mlp = cfg.tables(), cfg.mlp()
+    sparse, dense = cfg.batches(4)
+    pm, fgs = build_manager(cfg, tables, mlp, np.float16)
+    preds = [make_predictor(pm, fgs, sparse[b], dense[b], np.float16) for b in range(4)]
+    want = []
+    for p in preds:
+        p.forward()
+        want.append(p.output_asnumpy("prob").copy())
+    assert not np.array_equal(want[0], want[1])  # different batches: a mixed-up predictor would show
+
+    with pytest.raises(pb.BlazeError, match="ForwardWait without a ForwardLaunch"):
+        preds[0].forward_wait()
+    preds[0].forward_launch()
+    preds[1].forward_launch()
+    preds[0].forward_wait()
+    preds[1].forward_wait()
+    preds[2].forward_launch()
+    preds[2].forward()  # a launch nobody waited for is waited for by the next Forward
+    for b in range(3):
+        np.testing.assert_array_equal(preds[b].output_asnumpy("prob"), want[b])
+
+    for threads, depth, steps in ((2, 1, 13), (2, 2, 13), (1, 4, 9), (4, 2, 6), (2, 2, 1), (2, 2, 0)):
+        print("serve pool threads=%d depth=%d steps=%d" % (threads, depth, steps), flush=True)
+        pool = pb.ServePool(threads, depth)
+        pool.run(preds, steps)
+        torch.cuda.synchronize()
+        for b in range(4):
+            np.testing.assert_array_equal(preds[b].output_asnumpy("prob"), want[b])
+        del pool
+    with pytest.raises(pb.BlazeError, match="multiple of the pool's threads"):
+        pb.ServePool(3).run(preds, 4)

@@ -203,6 +203,7 @@ struct ServePool {
   Predictor** handles = nullptr;
   int n_handles = 0;
   int64_t steps = 0;
+  int depth = 2;  // passes a thread keeps queued on its stream
   std::atomic<int> failed{0};
   std::string error;
 
@@ -229,13 +230,30 @@ struct ServePool {
         n_threads = (int)threads.size();
       }
       // step i of the job runs predictor i % n_handles; thread t takes the steps i == t (mod n_threads), so a
-      // predictor is only ever used by one thread when n_handles is a multiple of n_threads
-      for (int64_t i = t; i < steps && !failed.load(std::memory_order_relaxed); i += n_threads) {
-        if (!handles[i % n_handles]->Forward()) {
-          if (!failed.exchange(1)) {
-            std::lock_guard<std::mutex> lock(mu);
-            error = blaze::last_error_for_thread();
+      // predictor is only ever used by one thread when n_handles is a multiple of n_threads.  With at least `depth`
+      // predictors per thread, the thread keeps `depth` passes queued on its stream: it launches step j + depth - 1
+      // before it waits for step j, so the device does not idle while the host is woken up and launches again.
+      const int per_thread = n_handles / n_threads;
+      const int64_t d = std::max<int64_t>(1, std::min<int64_t>(depth, per_thread));
+      auto fail = [&] {
+        if (!failed.exchange(1)) {
+          std::lock_guard<std::mutex> lock(mu);
+          error = blaze::last_error_for_thread();
+        }
+      };
+      if (d == 1) {
+        for (int64_t i = t; i < steps && !failed.load(std::memory_order_relaxed); i += n_threads)
+          if (!handles[i % n_handles]->Forward()) fail();
+      } else {
+        int64_t launched = t, waited = t;  // next step to launch / to wait for
+        while (waited < steps) {
+          while (launched < steps && (launched - waited) / n_threads < d && !failed.load(std::memory_order_relaxed)) {
+            if (!handles[launched % n_handles]->ForwardLaunch()) fail();
+            launched += n_threads;
           }
+          if (waited >= launched) break;  // a failure stopped the launches
+          if (!handles[waited % n_handles]->ForwardWait()) fail();
+          waited += n_threads;
         }
       }
       {
@@ -274,6 +292,25 @@ int Blaze_ServePoolRun(ServePoolHandle handle, PredictorHandle* predictors, int 
     Blaze_SetLastErrorString("Forward failed in the serving pool: %s", pool->error.c_str());
     return -1;
   }
+  return 0;
+}
+int Blaze_ServePoolSetDepth(ServePoolHandle handle, int depth) {
+  auto* pool = reinterpret_cast<ServePool*>(handle);
+  if (pool == nullptr || depth < 1 || depth > 64) return Fail("ServePoolSetDepth: bad arguments");
+  std::lock_guard<std::mutex> lock(pool->mu);
+  pool->depth = depth;
+  return 0;
+}
+int Blaze_PredictorForwardLaunch(PredictorHandle handle) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  if (!p->ForwardLaunch()) return Fail("ForwardLaunch failed");
+  return 0;
+}
+int Blaze_PredictorForwardWait(PredictorHandle handle) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr) return -1;
+  if (!p->ForwardWait()) return Fail("ForwardWait failed");
   return 0;
 }
 int Blaze_ServePoolDelete(ServePoolHandle handle) {

@@ -135,11 +135,22 @@ Blob* Net::external_output_blob(const std::string& name) const {
   return it == external_output_blob_.end() ? nullptr : it->second;
 }
 
-bool Net::Run() {
+bool Net::Launch() {
   if (!RunImpl()) {
     LOG_ERROR("Failed to run impl");
     return false;
   }
+  return true;
+}
+
+void* Net::StreamOfLastLaunch() {
+  for (auto it = operators_.rbegin(); it != operators_.rend(); ++it)
+    if (void* st = (*it)->DeviceStream()) return st;
+  return nullptr;
+}
+
+bool Net::Run() {
+  if (!Launch()) return false;
   // all operators run on stream 0 of this thread: waiting for that stream waits for the net (simple_net.cc:27-32)
   if (!operators_.empty()) operators_.back()->WaitStream();
   return true;

@@ -60,6 +60,10 @@ class Net {
   virtual ~Net() noexcept {}
   // reset, run every operator, wait for the device (net.h:33-49); exceptions propagate to the Predictor
   virtual bool Run();
+  // Run in two halves: Launch queues every operator on the calling thread's stream and returns; StreamOfLastLaunch is
+  // that stream (null when the net has no device operator).  Run = Launch + waiting for the stream.
+  bool Launch();
+  void* StreamOfLastLaunch();
   const std::vector<std::string>& external_input() const { return external_input_; }
   const std::vector<std::string>& external_output() const { return external_output_; }
   Blob* external_input_blob(const std::string& name) const;

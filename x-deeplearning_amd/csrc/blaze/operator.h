@@ -127,6 +127,8 @@ class OperatorBase {
 
   virtual bool Run(int stream_id = 0) = 0;
   virtual void WaitStream(int stream_id = -1) {}
+  // the device stream the operator's work is queued on (of the calling thread), null for host operators
+  virtual void* DeviceStream() { return nullptr; }
   // columns of 2-D output `idx` when they are fixed by the operator's arguments (else 0)
   virtual TIndex StaticOutputCols(int idx) const { return 0; }
 
@@ -186,6 +188,7 @@ class Operator : public OperatorBase {
     context_.FinishDeviceComputation();
     context_.SwitchToDevice(old);
   }
+  void* DeviceStream() override { return context_.device_stream(); }
 
  protected:
   Context context_;

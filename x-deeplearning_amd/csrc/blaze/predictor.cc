@@ -30,6 +30,10 @@ Predictor::Predictor(std::shared_ptr<Net> net) : net_(net) {
 }
 
 Predictor::~Predictor() {
+  if (forward_done_) {
+    (void)hipEventSynchronize(forward_done_);
+    (void)hipEventDestroy(forward_done_);
+  }
   if (feed_done_) {
     (void)hipEventSynchronize(feed_done_);
     (void)hipEventDestroy(feed_done_);
@@ -126,8 +130,57 @@ int Predictor::InputDataType(const char* name) const {
   return idx < 0 ? (int)kPDT_Invalid : external_input_blob_[idx]->data_type();
 }
 
+bool Predictor::ForwardLaunch() {
+  try {
+    if (any_feed_pending_) {
+      // the transfers were queued on the feeding thread's stream: make this thread's stream wait for them
+      for (Blob* b : external_input_blob_) {
+        if (b->device_type() != kHIP) continue;
+        HIPContext ctx(b->device_option());
+        ctx.Activate();
+        HIP_CHECK(hipStreamWaitEvent(ctx.hip_stream(), feed_done_, 0));
+        break;
+      }
+    }
+    if (!net_->Launch()) return false;
+    launched_on_ = net_->StreamOfLastLaunch();
+    if (launched_on_ != nullptr) {
+      if (forward_done_ == nullptr) HIP_CHECK(hipEventCreateWithFlags(&forward_done_, hipEventDisableTiming));
+      HIP_CHECK(hipEventRecord(forward_done_, (hipStream_t)launched_on_));
+    }
+    forward_in_flight_ = true;
+    return true;
+  } catch (std::exception& e) {
+    LOG_ERROR("failed: %s", e.what());
+    last_error_for_thread() = e.what();
+    return false;
+  }
+}
+
+bool Predictor::ForwardWait() {
+  try {
+    if (!forward_in_flight_) {
+      last_error_for_thread() = "ForwardWait without a ForwardLaunch before it";
+      return false;
+    }
+    forward_in_flight_ = false;
+    // the event sits behind the net's last operator, which sits behind the queued input transfers
+    if (launched_on_ != nullptr) HIP_CHECK(hipEventSynchronize(forward_done_));
+    if (any_feed_pending_) {
+      std::fill(feed_pending_.begin(), feed_pending_.end(), false);
+      any_feed_pending_ = false;
+    }
+    return true;
+  } catch (std::exception& e) {
+    LOG_ERROR("failed: %s", e.what());
+    last_error_for_thread() = e.what();
+    return false;
+  }
+}
+
 bool Predictor::Forward(const PredictorCallback&& cb) {
   try {
+    if (forward_in_flight_ && !ForwardWait()) return false;  // a launch the caller never waited for
     if (any_feed_pending_) {
       // the transfers were queued on the feeding thread's stream: make this thread's stream wait for them
       for (Blob* b : external_input_blob_) {

@@ -43,6 +43,11 @@ class Predictor {
   const std::vector<std::string>& ListInputName() const { return net_->external_input(); }
 
   bool Forward(const PredictorCallback&& cb = nullptr);
+  // extension: Forward in two halves, so that one thread can keep several of its predictors in flight.
+  // ForwardLaunch queues the net on the calling thread's stream and returns; ForwardWait (same thread) returns once
+  // that pass has finished on the device.  Feed / Output / another launch on this predictor only after the wait.
+  bool ForwardLaunch();
+  bool ForwardWait();
 
   // pointer to a host copy owned by the predictor, valid until the next Output call on it (:194-224)
   bool Output(const char* name, void** data, size_t* len);
@@ -80,6 +85,9 @@ class Predictor {
   bool any_feed_pending_ = false;
   hipEvent_t feed_done_ = nullptr;  // recorded behind the last queued transfer; Forward's stream waits for it
                                     // (Feed and Forward may be called from different threads = different streams)
+  hipEvent_t forward_done_ = nullptr;  // recorded behind the last operator of a ForwardLaunch
+  void* launched_on_ = nullptr;
+  bool forward_in_flight_ = false;
   std::unordered_map<std::string, std::shared_ptr<Blob>> param_cpu_;
 };
 

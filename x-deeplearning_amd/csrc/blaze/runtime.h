@@ -181,6 +181,7 @@ class CPUContext {
   explicit CPUContext(const DeviceOption& option) : device_option_(option) {}
   void SwitchToDevice(int) {}
   void FinishDeviceComputation() {}
+  void* device_stream() const { return nullptr; }
   int device_type() const { return kCPU; }
   int stream_id() const { return 0; }
   const DeviceOption& device_option() const { return device_option_; }
@@ -198,6 +199,7 @@ class HIPContext {
   }
   void Activate() const;                 // hipSetDevice when the thread is on another device
   hipStream_t hip_stream() const { return hip_stream(device_id_, stream_id_); }
+  void* device_stream() const { return (void*)hip_stream(); }
   static hipStream_t hip_stream(int device_id, int stream_id);  // thread-local, created on first use
   void FinishDeviceComputation() {
     Activate();

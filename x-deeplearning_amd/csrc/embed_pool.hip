@@ -329,6 +329,8 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
   }
   // base = sum of the counts before b0 (independent coalesced reads), local = this thread's sample
   // (8 loads in flight per thread: a rolled loop would wait for each load before issuing the next)
+  // this thread's own count is requested first so that it travels with the counts summed below
+  const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)s.segments[b0 + tid] : 0;
   int64_t part = 0;
   for (int64_t i0 = 0; i0 < b0; i0 += 8 * kThreads) {
     int32_t c[8];
@@ -340,7 +342,6 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
 #pragma unroll
     for (int k = 0; k < 8; ++k) part += c[k];
   }
-  const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)s.segments[b0 + tid] : 0;
   int64_t base = part;
 #pragma unroll
   for (int d = bz::kWave / 2; d > 0; d >>= 1) base += __shfl_xor(base, d, bz::kWave);
@@ -418,7 +419,9 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
 #pragma unroll
     for (int k = 0; k < KPL; ++k) {
       row_own[k] = (l < SRC && k * SRC + l < cnt) ? (int)resolve_row(s, id_next[k]) : -1;
-      val_own[k] = val_next[k];
+      // an id without a row contributes value 0 times a zero row: adding +0 leaves the running sum as it is (the
+      // sum starts at +0 and so is never -0), which lets the accumulation below run without the row numbers
+      val_own[k] = row_own[k] >= 0 ? val_next[k] : 0.f;
     }
     if (j + kBlockIds < end) fetch_ids(j + kBlockIds);
     int row[kBlockIds];
@@ -441,13 +444,11 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
     }
 #pragma unroll
     for (int u = 0; u < kBlockIds; ++u) {
-      if (row[u] >= 0) {
-        float w[CE];
-        widen<DT>(raw[u], sc[u], w);
-        // out = out + value * w: two roundings, never an FMA (udf_processor.h:66)
+      float w[CE];
+      widen<DT>(raw[u], sc[u], w);
+      // out = out + value * w: two roundings, never an FMA (udf_processor.h:66)
 #pragma unroll
-        for (int i = 0; i < CE; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(val[u], w[i]));
-      }
+      for (int i = 0; i < CE; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(val[u], w[i]));
     }
   }
   if (s.udf == BZ_AVG) {

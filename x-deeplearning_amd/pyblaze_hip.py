@@ -28,7 +28,8 @@ EXPORTS = [
     "Blaze_ConvertBlaze", "Blaze_OptimizeBlaze", "Blaze_QuickEmbeddingBuildFp32", "Blaze_QuickEmbeddingBuildFp16",
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
-    "Blaze_ServePoolRun", "Blaze_ServePoolDelete"
+    "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_PredictorForwardLaunch",
+    "Blaze_PredictorForwardWait"
 ]
 
 
@@ -81,6 +82,9 @@ def lib():
         l.Blaze_ServePoolCreate.argtypes = [i, C.POINTER(vp)]
         l.Blaze_ServePoolRun.argtypes = [vp, C.POINTER(vp), i, C.c_int64]
         l.Blaze_ServePoolDelete.argtypes = [vp]
+        l.Blaze_ServePoolSetDepth.argtypes = [vp, i]
+        l.Blaze_PredictorForwardLaunch.argtypes = [vp]
+        l.Blaze_PredictorForwardWait.argtypes = [vp]
         _lib = l
     return _lib
 
@@ -108,7 +112,7 @@ class Predictor(object):
         self.handle = handle
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:  # module globals are gone at interpreter exit
             lib().Blaze_PredictorDelete(self.handle)
             self.handle = None
 
@@ -128,6 +132,13 @@ class Predictor(object):
 
     def forward(self):
         check_call(lib().Blaze_PredictorForward(self.handle))
+
+    def forward_launch(self):
+        """Queue the pass on the calling thread's stream; forward_wait (same thread) returns when it has finished."""
+        check_call(lib().Blaze_PredictorForwardLaunch(self.handle))
+
+    def forward_wait(self):
+        check_call(lib().Blaze_PredictorForwardWait(self.handle))
 
     def forward_n(self, count):
         check_call(lib().Blaze_PredictorForwardN(self.handle, count))
@@ -199,13 +210,16 @@ class ServePool(object):
     """Persistent serving threads inside the library; run(predictors, steps) executes pass i on predictor
     i % len(predictors) and thread i % n_threads, returning when all passes have finished on the device."""
 
-    def __init__(self, n_threads):
+    def __init__(self, n_threads, depth=None):
+        """depth: passes a thread keeps queued on its stream (library default 2; 1 = synchronous Forward calls)."""
         self.handle = C.c_void_p()
         self.n_threads = n_threads
         check_call(lib().Blaze_ServePoolCreate(n_threads, C.byref(self.handle)))
+        if depth is not None:
+            check_call(lib().Blaze_ServePoolSetDepth(self.handle, depth))
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib().Blaze_ServePoolDelete(self.handle)
             self.handle = None
 
@@ -220,7 +234,7 @@ class PredictorManager(object):
         check_call(lib().Blaze_PredictorManagerCreate(C.byref(self.handle)))
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib().Blaze_PredictorManagerDelete(self.handle)
             self.handle = None
 
