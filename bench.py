@@ -25,7 +25,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
 # HBM-side bytes per launch of the pooling kernel on this exact workload (default seed, pool of 32 batches), from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, averaged over 1704 dispatches) scaled by what the same
 # counters read for a plain 256 MiB copy (`--calibrate-copy`: FETCH_SIZE reads 0.5 of the bytes, WRITE_SIZE all of them):
-# fetch 11986.46 KiB x 2.0 + write 3333.70 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
+# fetch 11984.86 KiB x 2.0 + write 3329.19 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
 POOL_TRAFFIC_BYTES = int((11984.86 * 2.0 + 3329.19) * 1024)
 
 
