@@ -271,44 +271,44 @@ __device__ __forceinline__ void pool_sum(const bz_embed_slot& s, int64_t start, 
 
 // kassign: position p of the output holds id j = p (in order) or num - trunc + p (reverse);
 // positions without an id, and ids absent from the table, are zero (udf_processor.h:103-131).
+// One call fills chunk c of position p of sample b: the positions of a sample are independent of each other,
+// so the kernel spreads them over lane groups instead of walking them one dependent load after the other.
 template <int DT>
-__device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b) {
+__device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b, int p) {
   constexpr int CE = RowTraits<DT>::kElems;
   const int64_t num = end - start;
   const int e0 = c * CE;
   const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
   const char* table = (const char*)s.table + (int64_t)c * 16;
   const int64_t shift = (s.trunc_dir == BZ_ORDER) ? 0 : num - (int64_t)s.trunc_num;
-  for (int p = 0; p < s.trunc_num; ++p) {
-    const int64_t j = shift + p;
-    float out[CE];
+  const int64_t j = shift + p;
+  float out[CE];
 #pragma unroll
-    for (int i = 0; i < CE; ++i) out[i] = 0.f;
-    if (j >= 0 && j < num) {
-      const int64_t r = resolve_row(s, s.ids[start + j]);
-      if (r >= 0) {
-        const float val = s.values[start + j];
-        const uint4 raw = *(const uint4*)(table + r * (int64_t)s.pitch);
-        const float sc = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
-        float w[CE];
-        widen<DT>(raw, sc, w);
+  for (int i = 0; i < CE; ++i) out[i] = 0.f;
+  if (j >= 0 && j < num) {
+    const int64_t r = resolve_row(s, s.ids[start + j]);
+    if (r >= 0) {
+      const float val = s.values[start + j];
+      const uint4 raw = *(const uint4*)(table + r * (int64_t)s.pitch);
+      const float sc = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
+      float w[CE];
+      widen<DT>(raw, sc, w);
 #pragma unroll
-        for (int i = 0; i < CE; ++i) out[i] = __fmul_rn(val, w[i]);
-      }
+      for (int i = 0; i < CE; ++i) out[i] = __fmul_rn(val, w[i]);
     }
-    store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * s.dim + e0, out, nvalid, s.out_dtype);
   }
+  store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * s.dim + e0, out, nvalid, s.out_dtype);
 }
 
 // zero fill of one item's columns (unknown table name: quick_embedding_dict.cc:95 leaves the
 // memset block untouched)
-__device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int l, int lpr) {
-  const int width = (s.udf == BZ_ASSIGN) ? s.dim * s.trunc_num : s.dim;
-  for (int e = l; e < width; e += lpr) {
+__device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int p, int l, int lpr) {
+  const int64_t base = b * s.out_stride + (int64_t)p * s.dim;  // p = 0 unless kassign
+  for (int e = l; e < s.dim; e += lpr) {
     if (s.out_dtype == BZ_F32)
-      ((float*)s.out)[b * s.out_stride + e] = 0.f;
+      ((float*)s.out)[base + e] = 0.f;
     else
-      ((__half*)s.out)[b * s.out_stride + e] = __ushort_as_half(0);
+      ((__half*)s.out)[base + e] = __ushort_as_half(0);
   }
 }
 
@@ -494,21 +494,30 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   const int tid = threadIdx.x;
   const int g = tid / lpr;
   const int l = tid - g * lpr;
-  const int64_t b0 = (int64_t)(v - s.wg_begin) * groups;
-  stage_offsets(s, b0, groups, s_off, s_part);
-  const int64_t b = b0 + g;
-  if (b >= s.batch) return;
+  // a lane group owns one item: a sample (ksum / kavg) or one output position of a sample (kassign)
+  const int64_t per = s.udf == BZ_ASSIGN ? s.trunc_num : 1;
+  const int64_t n_items = (int64_t)s.batch * per;
+  const int64_t i0 = (int64_t)(v - s.wg_begin) * groups;
+  int64_t i_last = i0 + groups - 1;
+  if (i_last >= n_items) i_last = n_items - 1;
+  const int64_t b_first = i0 / per;
+  const int n_samples = (int)(i_last / per - b_first) + 1;  // <= groups
+  stage_offsets(s, b_first, n_samples, s_off, s_part);
+  const int64_t item = i0 + g;
+  if (item >= n_items) return;
+  const int64_t b = item / per;
+  const int p = (int)(item - b * per);
   if (s.table == nullptr) {
-    pool_zero(s, b, l, lpr);
+    pool_zero(s, b, p, l, lpr);
     return;
   }
-  const int64_t start = s_off[g], end = s_off[g + 1];
+  const int64_t start = s_off[b - b_first], end = s_off[b - b_first + 1];
   for (int c = l; c < nchunks; c += lpr) {
     if (s.udf == BZ_ASSIGN) {
       switch (s.table_dtype) {
-        case BZ_F32: pool_assign<BZ_F32>(s, start, end, c, b); break;
-        case BZ_F16: pool_assign<BZ_F16>(s, start, end, c, b); break;
-        default: pool_assign<BZ_I8>(s, start, end, c, b); break;
+        case BZ_F32: pool_assign<BZ_F32>(s, start, end, c, b, p); break;
+        case BZ_F16: pool_assign<BZ_F16>(s, start, end, c, b, p); break;
+        default: pool_assign<BZ_I8>(s, start, end, c, b, p); break;
       }
     } else {
       switch (s.table_dtype) {
@@ -567,7 +576,9 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
     const int lpr = kThreads / g;
     const int ce = s.table_dtype == BZ_F32 ? 4 : (s.table_dtype == BZ_F16 ? 8 : 16);
     s.wg_begin = (int32_t)total;
-    s.wg_count = (int32_t)((s.batch + g - 1) / g);
+    const int64_t items = (int64_t)s.batch * (s.udf == BZ_ASSIGN ? s.trunc_num : 1);  // lane groups needed
+    BZ_REQUIRE((items + g - 1) / g < (1ll << 30), "slot %d: too many workgroups", i);
+    s.wg_count = (int32_t)((items + g - 1) / g);
     total += s.wg_count;
     BZ_REQUIRE(total < (1ll << 30), "too many workgroups");
     if (i == 0) lpr0 = lpr;

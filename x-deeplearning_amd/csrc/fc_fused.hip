@@ -574,16 +574,20 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
   // rows 16-byte aligned and K a whole number of chunks: branch-free loads, several tiles in flight
   const bool aligned = vec_a && vec_w && d.k % In<DT>::kChunk == 0;
   if (!aligned) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 1, false>(d, ep, vec_a, vec_w, st);
-  // Largest first.  128x256 with eight waves and three K tiles in flight fills the chip once it has a workgroup per
-  // CU (its fp32 output tile would not fit the operand buffers it is staged in, so 2-byte outputs only); below
-  // that, 128x128; then 64x128 while that still gives two workgroups per CU; then the latency-bound small tiles.
+  // Largest first, and never a tile much wider than N.  128x256 with eight waves and three K tiles in flight fills the
+  // chip once it has a workgroup per CU (its fp32 output tile would not fit the operand buffers it is staged in, so
+  // 2-byte outputs only); below that, 128x128; then 64x128 while that still gives two workgroups per CU; then the
+  // latency-bound small tiles.
   const int64_t wg128x256 = (int64_t)((d.m + 127) / 128) * ((d.n + 255) / 256);
   const int64_t wg64x128 = (int64_t)((d.m + 63) / 64) * ((d.n + 127) / 128);
   if constexpr (sizeof(OutT) == 2) {
-    if (wg128x256 >= 256) return launch_mfma<DT, OutT, 128, 256, BK, 2, 4, 3, true>(d, ep, vec_a, vec_w, st);
+    if (d.n > 128 && wg128x256 >= 256) return launch_mfma<DT, OutT, 128, 256, BK, 2, 4, 3, true>(d, ep, vec_a, vec_w, st);
   }
-  if (wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2, 3, true>(d, ep, vec_a, vec_w, st);
-  if (wg64x128 >= 512) return launch_mfma<DT, OutT, 64, 128, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
+  // tall and narrow (the attention MLP over batch x history rows): one 96-wide tile reads A once
+  if (d.n > 64 && d.n <= 96 && (d.m + 127) / 128 >= 256)
+    return launch_mfma<DT, OutT, 128, 96, BK, 4, 1, 2, true>(d, ep, vec_a, vec_w, st);
+  if (d.n > 64 && wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2, 3, true>(d, ep, vec_a, vec_w, st);
+  if (d.n > 64 && wg64x128 >= 512) return launch_mfma<DT, OutT, 64, 128, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
   if (wg64 >= 256) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
   return launch_mfma<DT, OutT, 32, 64, BK, 1, 2, 4, true>(d, ep, vec_a, vec_w, st);
 }
