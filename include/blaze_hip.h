@@ -200,6 +200,20 @@ typedef struct bz_fc_desc {
   float alpha, beta;
   float act_alpha;     /* LEAKY_RELU slope */
   int32_t reserved_;
+  /*
+   * Optional second, skinny layer in the same launch (head_n > 0): Z[M, head_n] = head_act(Y * head_w^T + head_bias),
+   * computed from the rounded tile of Y while it is still on chip -- the Gemm -> activation -> Gemm(N <= 8) ->
+   * Softmax | Sigmoid tail of a CTR tower without the second launch.  Needs 8 < n <= 256 (a workgroup owns whole rows
+   * of Y), out_dtype == in_dtype, 16-byte aligned operand rows.  y may be NULL then (Y is not stored).
+   */
+  const void* head_w;     /* device [head_n, head_ldw], K (= n) contiguous, dtype in_dtype */
+  const float* head_bias; /* device [head_n] or NULL */
+  void* head_y;           /* device [M, head_ldy] */
+  int64_t head_ldw, head_ldy;
+  int32_t head_n;         /* 0 = no head, else 1..8 */
+  int32_t head_act;       /* BZ_ACT_NONE | BZ_ACT_SIGMOID | BZ_ACT_SOFTMAX */
+  int32_t head_out_dtype; /* BZ_F32 | BZ_F16 | BZ_BF16 */
+  int32_t reserved2_;
 } bz_fc_desc;
 
 BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);
@@ -357,6 +371,33 @@ typedef struct bz_bcast_desc {
 } bz_bcast_desc;
 
 BZ_API int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream);
+
+/*
+ * Concat along the last axis whose pieces are computed on the fly: piece p is x[p] (BZ_EW_ASSIGN, a copy or a
+ * row-broadcast), or x[p] (op) y[p] for Add / Sub / Mul / Div.  One launch stands in for the reference's sequence
+ * BroadcastTo / Sub / Mul / ... followed by Concat (blaze/operator/op/elementwise_op.cu:55-140, concat_op.cu:33), the
+ * way a DIN attention unit assembles [q, k, q-k, q*k] (tools/example_model/din/model/graph_ulf.txt), without writing
+ * the intermediate tensors.  Each element is computed exactly as the separate operators do (fp32 operation on the
+ * widened operands, rounded once to dtype).
+ * Rows are indexed by two coordinates, row = i0 * r1 + i1; an operand's element (row, c) is at
+ * base[i0 * stride[0] + i1 * stride[1] + c] (stride 0 = broadcast over that coordinate), c < width[p].
+ */
+#define BZ_CEW_MAX 8
+typedef struct bz_concat_ew_desc {
+  const void* x[BZ_CEW_MAX];
+  const void* y[BZ_CEW_MAX];          /* NULL for BZ_EW_ASSIGN */
+  int64_t x_stride[BZ_CEW_MAX][2];    /* in elements */
+  int64_t y_stride[BZ_CEW_MAX][2];
+  int32_t op[BZ_CEW_MAX];             /* BZ_EW_ADD | SUB | MUL | DIV | ASSIGN */
+  int32_t width[BZ_CEW_MAX];          /* columns of the piece */
+  void* dst;                          /* [r0 * r1, dst_pitch] */
+  int64_t dst_pitch;                  /* elements per output row, >= sum of the widths */
+  int64_t r0, r1;
+  int32_t n;                          /* pieces, 1..BZ_CEW_MAX */
+  int32_t dtype;                      /* BZ_F32 | BZ_F16 | BZ_BF16 */
+} bz_concat_ew_desc;
+
+BZ_API int bz_concat_ew(const bz_concat_ew_desc* desc, bz_stream_t stream);
 
 /*
  * ReduceSum over the middle axis of a contiguous [outer, dim, inner] tensor -> [outer, inner], added in ascending

@@ -244,3 +244,40 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
         np.testing.assert_allclose(p2.output_asnumpy("prob").astype(np.float32), want["prob"], rtol=2e-3, atol=2e-3)
     finally:
         del os.environ["BLAZE_NO_FUSION"]
+
+
+def test_attention_unit_assembled_by_the_concat_equals_the_separate_operators():
+    """The DIN graph's BroadcastTo / Sub / Mul feeding Concat(axis 2): by default the Concat computes those pieces
+    itself in one launch and the three operators never run; with fuse_concat_pieces: 0 each runs and the Concat copies.
+    Same bits in the assembled tensor and in the probabilities, also after the batch shrinks and grows again."""
+    import json
+    import torch
+    import din_model
+    cfg = din_model.Config3(batch=96, rows=5000, T=20)
+    small = din_model.Config3(batch=17, rows=5000, T=20)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=5), cfg.batch_inputs(seed_offset=9)]
+    outs = {}
+    for fuse in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("att_in", ),
+                                             net_args={"fuse_concat_pieces": fuse})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append((p.output_asnumpy("att_in").copy(), p.output_asnumpy("prob").copy()))
+        ran = {e["name"].split(":")[0] for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0}
+        assert ("BroadcastTo" in ran) == (fuse == 0) and ("Sub" in ran) == (fuse == 0), ran
+        assert "Mul" in ran  # Mul(score, mask) is nobody's concat piece
+        outs[fuse] = got
+    torch.cuda.synchronize()
+    D3 = 3 * cfg.dim
+    for (a1, p1), (a0, p0), b in zip(outs[1], outs[0], (96, 17, 96)):
+        assert a1.shape == (b, cfg.T, 4 * D3) and a1.any()
+        assert np.array_equal(a1.view(np.uint16), a0.view(np.uint16))
+        assert np.array_equal(p1, p0)
+        q, k = a1[:, :, :D3].astype(np.float32), a1[:, :, D3:2 * D3].astype(np.float32)
+        assert np.array_equal(a1[:, :, 2 * D3:3 * D3], (q - k).astype(np.float16))
+        assert np.array_equal(a1[:, :, 3 * D3:], (q * k).astype(np.float16))

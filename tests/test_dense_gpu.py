@@ -144,6 +144,75 @@ def test_fc_half(bz, oracle, in_name, out_name, M, N, K, act):
     _fc_case(bz, oracle, M, N, K, in_name, out_name, act, seed=M + N * 3 + K)
 
 
+@pytest.mark.parametrize("in_name", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("M,K,N,N2,act,hact", [
+    (2048, 512, 256, 2, "prelu", "softmax"),   # config 2's last two layers: 32x256 tile
+    (300, 200, 80, 2, "dice", "softmax"),      # DIN main tower tail: 32x128 tile, ragged M
+    (5000, 80, 40, 1, "dice", "none"),         # DIN attention tail: 32x64 tile
+    (17000, 80, 40, 1, "dice", "none"),        # the same with enough rows for the 64x64 tile
+    (513, 128, 128, 8, "relu", "sigmoid"),     # widest head
+    (100, 64, 16, 3, "none", "softmax"),
+])
+def test_fc_with_skinny_head_in_one_launch(bz, oracle, in_name, M, K, N, N2, act, hact):
+    """Layer + skinny head in one launch against the same two layers as two launches.  The one-launch form uses a tile
+    that spans the whole row, so its fp32 sums run in another order: the first layer's output agrees to one rounding
+    of the tensor type, the head to 1e-5 (fp32) / 2e-3 (the head reads the rounded tile as the second launch reads the
+    stored tensor), also when the first layer's output is not stored.  The head against the oracle, computed from
+    the first layer's own stored output: 1e-5 (fp32) / 2e-3 relative to the operand magnitudes."""
+    import torch
+    print("case", in_name, M, K, N, N2, act, hact, flush=True)
+    rng = np.random.default_rng(M + 3 * K + N)
+    tdt, bt = _tdtype(in_name), {"f32": bz.F32, "f16": bz.F16, "bf16": bz.BF16}[in_name]
+    A = _round_to(rng.standard_normal((M, K)), in_name)
+    W1 = _round_to(rng.standard_normal((K, N)) / np.sqrt(K), in_name)
+    W2 = _round_to(rng.standard_normal((N, N2)) / np.sqrt(N), in_name)
+    b1 = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    b2 = (rng.standard_normal(N2) * 0.1).astype(np.float32)
+    params = ()
+    if act == "prelu":
+        params = (rng.uniform(0.1, 0.4, N).astype(np.float32), )
+    elif act == "dice":
+        params = ((rng.standard_normal(N) * 0.1).astype(np.float32), (rng.standard_normal(N) * 0.1).astype(np.float32),
+                  rng.uniform(0.5, 1.5, N).astype(np.float32))
+    a = _dev(A, tdt)
+    w1 = bz.pack_weight(_dev(W1, None if in_name == "f32" else tdt), False, bt)
+    w2 = bz.pack_weight(_dev(W2, None if in_name == "f32" else tdt), False, bt)
+    kw = dict(bias=_dev(b1), act=ACT[act], act_params=tuple(_dev(p) for p in params), out_dtype=bt)
+    y_ref = bz.fc_fused(a, w1, K, **kw)
+    z_ref = bz.fc_fused(y_ref, w2, N, bias=_dev(b2), act=ACT[hact], out_dtype=bz.F32)
+    z1 = torch.full((M, N2), -7.0, dtype=torch.float32, device="cuda")
+    y1, _ = bz.fc_fused(a, w1, K, head=dict(w=w2, bias=_dev(b2), act=ACT[hact], out=z1), **kw)
+    z2 = torch.full((M, N2), -7.0, dtype=tdt, device="cuda")
+    none, _ = bz.fc_fused(a, w1, K, head=dict(w=w2, bias=_dev(b2), act=ACT[hact], out=z2), store_out=False, **kw)
+    torch.cuda.synchronize()
+    assert none is None
+    ulp = {"f32": 1e-5, "f16": 2.0**-10, "bf16": 2.0**-7}[in_name]
+    np.testing.assert_allclose(y1.float().cpu().numpy(), y_ref.float().cpu().numpy(), rtol=ulp, atol=ulp)  # sums of O(1) magnitude: absolute part for cancelled values
+    tol = 1e-5 if in_name == "f32" else 2e-3
+    np.testing.assert_allclose(z1.cpu().numpy(), z_ref.cpu().numpy(), rtol=tol, atol=tol)
+    np.testing.assert_allclose(z2.float().cpu().numpy(), z1.cpu().numpy(), rtol=ulp, atol=1e-6)  # same head, rounded to the type
+    # oracle: second layer in fp64 from the first layer's stored (rounded) output
+    y = y1.float().cpu().numpy().astype(np.float64)
+    pre = (y @ W2.astype(np.float64) + b2).astype(np.float32)
+    want = {"none": pre, "sigmoid": oracle.sigmoid(pre), "softmax": oracle.softmax(pre, 1)}[hact]
+    scale = np.abs(y) @ np.abs(W2).astype(np.float64) + np.abs(b2)
+    assert np.all(np.abs(z1.cpu().numpy() - want) <= 1e-5 * scale + 1e-6)  # fp32 head from the stored tile: fp32 accuracy
+
+
+def test_fc_head_limits_are_refused(bz):
+    import torch
+    a = torch.zeros((64, 512), dtype=torch.float16, device="cuda")
+    w = torch.zeros((512, 512), dtype=torch.float16, device="cuda")
+    h = torch.zeros((2, 512), dtype=torch.float16, device="cuda")
+    z = torch.zeros((64, 2), dtype=torch.float32, device="cuda")
+    with pytest.raises(bz.BlazeHipError, match="n <= 256"):
+        bz.fc_fused(a, w, 512, head=dict(w=h, out=z))
+    w = torch.zeros((128, 512), dtype=torch.float16, device="cuda")
+    h = torch.zeros((9, 128), dtype=torch.float16, device="cuda")
+    with pytest.raises(bz.BlazeHipError, match="head of 9 outputs"):
+        bz.fc_fused(a, w, 512, head=dict(w=h, out=torch.zeros((64, 9), dtype=torch.float32, device="cuda")))
+
+
 @pytest.mark.parametrize("in_name", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("M,N,K,act", [(2048, 2, 256, "softmax"), (128, 2, 80, "softmax"), (5000, 1, 40, "none"),
                                        (8192, 1, 256, "sigmoid"), (7, 8, 1000, "prelu"), (3, 3, 12, "dice")])

@@ -150,6 +150,35 @@ def test_fuse_repeats_the_single_row(bz, oracle):
         assert np.array_equal(out.cpu().numpy(), oracle.fuse(x1, x2, comm))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("r0,r1,w,kshape", [(64, 50, 54, "q"),     # DIN: [q, k, q-k, q*k], q broadcast over the history
+                                            (7, 50, 36, "k"),      # the example graph: one history, 7 candidate ads
+                                            (33, 1, 8, "q"),       # 2-D after merging, widths a multiple of 8
+                                            (5, 3, 7, "q")])       # odd width: one column per thread
+def test_concat_of_pieces_computed_on_the_fly_equals_the_separate_operators(bz, oracle, dtype, r0, r1, w, kshape):
+    """bz_concat_ew against the oracle's BroadcastTo / Sub / Mul / Add / Div followed by Concat: bit-identical
+    (every element is one fp32 operation on the widened operands, rounded once)."""
+    import torch
+    rng = np.random.default_rng(r0 * 1000 + r1 * 10 + w)
+    qs, ks = ((r0, 1, w), (r0, r1, w)) if kshape == "q" else ((r0, 1, w), (1, r1, w))
+    q = rng.standard_normal(qs).astype(dtype)
+    k = (rng.standard_normal(ks) + 2.5).astype(dtype)
+    print("case", dtype.__name__, r0, r1, w, kshape, flush=True)
+    qd, kd = _dev(q), _dev(k)
+    got = bz.concat_ew([(bz.EW_ASSIGN, qd, None), (bz.EW_ASSIGN, kd, None), (bz.EW_SUB, qd, kd), (bz.EW_MUL, qd, kd),
+                        (bz.EW_ADD, kd, qd), (bz.EW_DIV, qd, kd)])
+    torch.cuda.synchronize()
+    rnd = (lambda x: x.astype(dtype).astype(np.float32))
+    qf, kf = q.astype(np.float32), k.astype(np.float32)
+    full = (r0, r1, w)
+    want = oracle.concat([rnd(oracle.broadcast_to(qf, shape=full)), rnd(oracle.broadcast_to(kf, shape=full)),
+                          rnd(oracle.elementwise("Sub", qf, kf)), rnd(oracle.elementwise("Mul", qf, kf)),
+                          rnd(oracle.elementwise("Add", kf, qf)), rnd(oracle.elementwise("Div", qf, kf))], 2).astype(dtype)
+    assert tuple(got.shape) == want.shape
+    view = np.uint32 if dtype == np.float32 else np.uint16
+    assert np.array_equal(got.cpu().numpy().view(view), want.view(view))
+
+
 def test_bad_descriptors_are_refused(bz):
     import ctypes as C
     d = bz.BcastDesc()
@@ -159,3 +188,6 @@ def test_bad_descriptors_are_refused(bz):
     assert b"rank" in bz.lib().bz_last_error()
     assert bz.lib().bz_reduce_sum(None, None, 1, 1, 1, bz.F32, None) != 0
     assert bz.lib().bz_softmax_axis(None, None, 1, 1, 1, bz.F32, None) != 0
+    e = bz.ConcatEwDesc()
+    assert bz.lib().bz_concat_ew(C.byref(e), None) != 0  # no pieces
+    assert b"pieces" in bz.lib().bz_last_error()

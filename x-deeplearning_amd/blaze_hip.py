@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight"
+    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 MAX_RANK = 6
@@ -48,7 +48,9 @@ class FcDesc(C.Structure):
                 ("ldy", C.c_int64), ("m", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("in_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("bias_rows", C.c_int32), ("act", C.c_int32), ("act_size", C.c_int32),
                 ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
-                ("reserved_", C.c_int32)]
+                ("reserved_", C.c_int32), ("head_w", C.c_void_p), ("head_bias", C.c_void_p), ("head_y", C.c_void_p),
+                ("head_ldw", C.c_int64), ("head_ldy", C.c_int64), ("head_n", C.c_int32), ("head_act", C.c_int32),
+                ("head_out_dtype", C.c_int32), ("reserved2_", C.c_int32)]
 
 
 class BgemmDesc(C.Structure):
@@ -73,6 +75,12 @@ class BcastDesc(C.Structure):
     _fields_ = [("a", C.c_void_p), ("b", C.c_void_p), ("c", C.c_void_p), ("out", C.c_void_p), ("dims", C.c_int64 * 6),
                 ("a_stride", C.c_int64 * 6), ("b_stride", C.c_int64 * 6), ("c_stride", C.c_int64 * 6), ("rank", C.c_int32),
                 ("op", C.c_int32), ("dtype", C.c_int32), ("cond_dtype", C.c_int32)]
+
+
+class ConcatEwDesc(C.Structure):
+    _fields_ = [("x", C.c_void_p * 8), ("y", C.c_void_p * 8), ("x_stride", (C.c_int64 * 2) * 8), ("y_stride", (C.c_int64 * 2) * 8),
+                ("op", C.c_int32 * 8), ("width", C.c_int32 * 8), ("dst", C.c_void_p), ("dst_pitch", C.c_int64),
+                ("r0", C.c_int64), ("r1", C.c_int64), ("n", C.c_int32), ("dtype", C.c_int32)]
 
 
 class BnDesc(C.Structure):
@@ -122,6 +130,7 @@ def lib():
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
+        l.bz_concat_ew.argtypes = [C.POINTER(ConcatEwDesc), vp]
         l.bz_activation.argtypes = [C.POINTER(ActDesc), vp]
         l.bz_concat_cols.argtypes = [C.POINTER(ConcatDesc), vp]
         l.bz_broadcast_op.argtypes = [C.POINTER(BcastDesc), vp]
@@ -317,7 +326,10 @@ def pack_weight(w, trans_b, dst_dtype, stream=None):
 
 
 def fc_fused(a, w_packed, k, bias=None, act=ACT_NONE, act_params=(), out=None, out_dtype=None, alpha=1.0, beta=1.0,
-             act_alpha=0.0, dice_nosqrt=False, stream=None):
+             act_alpha=0.0, dice_nosqrt=False, stream=None, head=None, store_out=True):
+    """head: dict(w=packed [n2, ldw] weight of a second layer with n2 <= 8 outputs, bias=fp32 [n2] or None, act=ACT_NONE |
+    ACT_SIGMOID | ACT_SOFTMAX, out=tensor [m, n2]) computed in the same launch; then returns (out, head out), and
+    store_out=False skips storing the first layer's output (out is returned as None)."""
     import torch
     m = a.shape[0]
     n = w_packed.shape[0]
@@ -342,7 +354,19 @@ def fc_fused(a, w_packed, k, bias=None, act=ACT_NONE, act_params=(), out=None, o
     d.act_size = ps[0].numel() if ps[0] is not None else 0
     d.dice_nosqrt = int(dice_nosqrt)
     d.alpha, d.beta, d.act_alpha = alpha, beta, act_alpha
+    if head is not None:
+        hw, hy = head["w"], head["out"]
+        assert hw.dtype == a.dtype and hy.shape[0] == m
+        d.head_w, d.head_y, d.head_ldw, d.head_ldy = hw.data_ptr(), hy.data_ptr(), hw.stride(0), hy.stride(0)
+        d.head_n, d.head_act, d.head_out_dtype = hw.shape[0], head.get("act", ACT_NONE), bz_dtype(hy.dtype)
+        if head.get("bias") is not None:
+            assert head["bias"].dtype == torch.float32
+            d.head_bias = head["bias"].data_ptr()
+        if not store_out:
+            d.y = None
     check(lib().bz_fc_fused(C.byref(d), _stream_ptr(stream)))
+    if head is not None:
+        return (out if store_out else None), head["out"]
     return out
 
 
@@ -411,6 +435,32 @@ def broadcast_op(op, a, b=None, c=None, out_shape=None, stream=None):
     if op == EW_WHERE:
         d.cond_dtype = bz_dtype(a.dtype)
     check(lib().bz_broadcast_op(C.byref(d), _stream_ptr(stream)))
+    return out
+
+
+def concat_ew(pieces, stream=None):
+    """Concat along the last axis of pieces computed on the fly.  pieces: list of (op, x, y) with op one of EW_ADD /
+    EW_SUB / EW_MUL / EW_DIV (y a tensor) or EW_ASSIGN (y None); operands are contiguous tensors [r0 | 1, r1 | 1, w]
+    broadcast over the two row coordinates.  -> tensor [r0, r1, sum of w]."""
+    import torch
+    ops = [t for _, x, y in pieces for t in (x, y) if t is not None]
+    r0 = max(t.shape[0] for t in ops)
+    r1 = max(t.shape[1] for t in ops)
+    total = sum(x.shape[2] for _, x, _ in pieces)
+    out = torch.empty((r0, r1, total), dtype=ops[0].dtype, device=ops[0].device)
+    d = ConcatEwDesc()
+    d.n, d.dtype, d.dst, d.dst_pitch, d.r0, d.r1 = len(pieces), bz_dtype(out.dtype), out.data_ptr(), total, r0, r1
+    for i, (op, x, y) in enumerate(pieces):
+        d.op[i], d.width[i], d.x[i] = op, x.shape[2], x.data_ptr()
+        for name, t in (("x_stride", x), ("y_stride", y)):
+            if t is None:
+                continue
+            assert t.is_contiguous() and t.shape[2] == x.shape[2] and t.shape[0] in (1, r0) and t.shape[1] in (1, r1)
+            getattr(d, name)[i][0] = 0 if t.shape[0] == 1 and r0 > 1 else t.shape[1] * t.shape[2]
+            getattr(d, name)[i][1] = 0 if t.shape[1] == 1 and r1 > 1 else t.shape[2]
+        if y is not None:
+            d.y[i] = y.data_ptr()
+    check(lib().bz_concat_ew(C.byref(d), _stream_ptr(stream)))
     return out
 
 

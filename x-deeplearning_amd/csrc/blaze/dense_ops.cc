@@ -86,6 +86,12 @@ struct FcCall {
   int act_size = 0;
   bool dice_nosqrt = false;
   float act_alpha = 0.f;
+  // a second, skinny layer in the same launch (bz_fc_desc.head_*); y may then be null
+  const void* head_w = nullptr;
+  int64_t head_ldw = 0;
+  const float* head_bias = nullptr;
+  void* head_y = nullptr;
+  int head_n = 0, head_act = BZ_ACT_NONE, head_y_dtype = kFloat;
 };
 
 void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st) {
@@ -141,6 +147,16 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
   d.alpha = c.alpha;
   d.beta = c.bias ? c.beta : 0.f;
   d.act_alpha = c.act_alpha;
+  if (c.head_n > 0) {
+    d.head_w = c.head_w;
+    d.head_ldw = c.head_ldw;
+    d.head_bias = c.head_bias;
+    d.head_y = c.head_y;
+    d.head_ldy = c.head_n;
+    d.head_n = c.head_n;
+    d.head_act = c.head_act;
+    d.head_out_dtype = BzType(c.head_y_dtype);
+  }
   BZ_CHECK(bz_fc_fused(&d, st));
 }
 
@@ -216,16 +232,44 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     for (StackableFc* f : followers) stack_.push_back(static_cast<GemmOp*>(f));
   }
 
+  // ---- a following layer of at most 8 outputs in this operator's launch
+  bool CanHostHead(int* n_out) override {
+    Blob* b = this->Input(1);
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr) return false;
+    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
+    if (N > 256 || N <= 8 || N % 8 != 0) return false;
+    if (this->InputSize() > 2 && (!c_constant_ || (int)this->Input(2)->size() != N)) return false;
+    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX) return false;
+    *n_out = N;
+    return true;
+  }
+  bool CanBeHead(int k_in) override {
+    Blob* b = this->Input(1);
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr) return false;
+    const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
+    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
+    if (K != k_in || N > 8 || alpha_ != 1.f || beta_ != 1.f) return false;
+    if (this->InputSize() > 2 && (!c_constant_ || (int)this->Input(2)->size() != N)) return false;
+    if (fused_ && fused_act_ != BZ_ACT_SOFTMAX && fused_act_ != BZ_ACT_SIGMOID) return false;
+    return true;
+  }
+  void AbsorbHead(StackableFc* head) override { head_ = static_cast<GemmOp*>(head); }
+
   bool RunOnDevice() override {
+    if (head_ != nullptr) {
+      if (RunSelf(true)) return true;
+      // an input the one-launch form does not take (unaligned rows, mixed types): one launch per layer
+      return RunSelf(false) && head_->RunSelf(false);
+    }
     if (!stack_.empty()) {
       if (RunStack()) return true;
       // an input the fused kernel does not take (3-D, unaligned, another type): layer by layer
-      if (!RunSelf()) return false;
+      if (!RunSelf(false)) return false;
       for (GemmOp* f : stack_)
-        if (!f->RunSelf()) return false;
+        if (!f->RunSelf(false)) return false;
       return true;
     }
-    return RunSelf();
+    return RunSelf(false);
   }
 
  protected:
@@ -303,12 +347,21 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     return true;
   }
 
-  bool RunSelf() {
+  // with_head: also compute head_'s layer in this launch and leave this layer's own output unstored; false when the
+  // operands do not allow it (nothing has been launched then)
+  bool RunSelf(bool with_head) {
     CheckValid();
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
     Blob* c = this->InputSize() > 2 ? this->Input(2) : nullptr;
     Blob* y = fused_ ? fused_->Output(0) : this->Output(0);
+    if (with_head) {
+      const size_t es = DataTypeSize(a->data_type());
+      const TIndex k = a->shape().back();
+      if (a->data_type() != y->data_type() || a->data_type() != head_->Input(1)->data_type() || (k * es) % 16 != 0 ||
+          (uintptr_t)a->data() % 16 != 0 || a->pitch() != 0)
+        return false;
+    }
     const auto& a_shape = a->shape();
     const auto& b_shape = b->shape();
     TIndex M = a_shape.size() == 3 ? a_shape[1] : a_shape[0];
@@ -316,12 +369,27 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     if (transa_) std::swap(M, K);
     const TIndex N = transb_ ? b_shape[0] : b_shape[1];
     TIndex rows = M;  // rows of the one 2-D product that realises the op
+    Blob* hy = nullptr;
+    if (with_head) {
+      Blob* hb = head_->Input(1);
+      const TIndex n2 = head_->transb_ ? hb->shape()[0] : hb->shape()[1];
+      hy = head_->fused_ ? head_->fused_->Output(0) : head_->Output(0);
+      if (a_shape.size() == 3)
+        hy->Reshape({a_shape[0], M, n2});
+      else
+        hy->Reshape({M, n2});
+    }
     if (a_shape.size() == 3) {
-      y->Reshape({a_shape[0], M, N});
+      if (with_head)
+        y->SetShapeOnly({a_shape[0], M, N});
+      else
+        y->Reshape({a_shape[0], M, N});
       // M == 1 collapses to a 2-D Gemm with M = batch (gemm_op.h:54-55); M > 1 with a shared weight is the
       // strided-batched case (stride_b = 0, :77-91), which over contiguous slices is again one 2-D product
       BLAZE_CONDITION_THROW(!transa_ || a_shape[0] == 1, "3-D Gemm with transA is not supported on this device");
       rows = a_shape[0] * M;
+    } else if (with_head) {
+      y->SetShapeOnly({M, N});
     } else {
       y->Reshape({M, N});
     }
@@ -338,10 +406,29 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     call.trans_b = transb_;
     call.b_constant = b_constant_;
     call.dtype = a->data_type();
-    call.y = y->data();
+    call.y = with_head ? nullptr : y->data();
     call.y_dtype = y->data_type();
     call.alpha = alpha_;
     call.beta = beta_;
+    if (with_head) {
+      Blob* hb = head_->Input(1);
+      const int n2 = (int)(head_->transb_ ? hb->shape()[0] : hb->shape()[1]);
+      const int es = (int)DataTypeSize(hb->data_type());
+      const int64_t ldw = (N + 7) / 8 * 8;
+      if (head_->packed_b_.Stale(hb) || head_->packed_b_.bytes < (size_t)n2 * ldw * es) {
+        head_->packed_b_.Resize((size_t)n2 * ldw * es);
+        BZ_CHECK(bz_fc_pack_weight(hb->data(), BzType(hb->data_type()), head_->transb_ ? 1 : 0, (int)N, n2, head_->packed_b_.ptr,
+                                   BzType(hb->data_type()), ldw, st));
+        head_->packed_b_.Mark(hb);
+      }
+      call.head_w = head_->packed_b_.ptr;
+      call.head_ldw = ldw;
+      if (head_->InputSize() > 2) call.head_bias = AsFloatParam(head_->Input(2), &head_->bias_f32_, true, st);
+      call.head_y = hy->data();
+      call.head_y_dtype = hy->data_type();
+      call.head_n = n2;
+      call.head_act = head_->fused_ ? head_->fused_act_ : BZ_ACT_NONE;
+    }
     if (c != nullptr) {
       call.bias = AsFloatParam(c, &bias_f32_, c_constant_, st);
       if (c->shape().size() == 2 && c->shape()[0] != 1) {
@@ -404,6 +491,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   Derived packed_b_, packed_a_, bias_f32_, p_f32_[3];
   Derived stack_pack_;           // this layer's weight in the fragment-major pack of bz_mlp_fused
   std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
+  GemmOp* head_ = nullptr;       // the layer of at most 8 outputs computed in this operator's launch
   OperatorBase* fused_ = nullptr;
   int fused_act_ = BZ_ACT_NONE;
   bool fused_nosqrt_ = false;

@@ -210,7 +210,110 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
       if (producer->TryFuse(operators_[i + 1].get())) skipped_[i + 1] = true;
     }
     StackFcLayers();
+    FuseFcHeads();
     AliasConcatInputs();
+    FuseConcatPieces();
+  }
+}
+
+// FC layer (with its folded activation) -> FC layer of at most 8 outputs (with its folded Softmax / Sigmoid), the
+// first one's result read by nothing else: one launch (graph.h, StackableFc::CanHostHead).  Switch: fuse_fc_head: 0.
+void SimpleNet::FuseFcHeads() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_fc_head");
+  if (arg && arg->has_i && arg->i == 0) return;
+  for (size_t i = 0; i < operators_.size(); ++i) {
+    auto* first = skipped_[i] ? nullptr : dynamic_cast<StackableFc*>(operators_[i].get());
+    int n1 = 0;
+    if (!first || !first->CanHostHead(&n1)) continue;
+    size_t j = i + 1;
+    while (j < operators_.size() && skipped_[j]) ++j;  // (the first layer's folded activation)
+    if (j >= operators_.size()) break;
+    auto* second = dynamic_cast<StackableFc*>(operators_[j].get());
+    if (!second || !second->CanBeHead(n1)) continue;
+    const std::string& mid = first->StackOutputOp()->operator_def().output(0);
+    if (operators_[j]->operator_def().input(0) != mid) continue;
+    int readers = 0;
+    for (size_t k = 0; k < operators_.size(); ++k) {
+      if (skipped_[k]) continue;
+      for (const auto& in : operators_[k]->operator_def().input()) readers += (in == mid);
+    }
+    bool is_output = false;
+    for (const auto& eo : external_output_) is_output |= (eo == mid);
+    if (readers != 1 || is_output) continue;
+    first->AbsorbHead(second);
+    skipped_[j] = true;
+  }
+}
+
+// Concat inputs that are outputs of elementwise operators -> pieces computed by the Concat itself (graph.h,
+// ConcatPieceSource).  A producer is taken over when its output is read only by the Concat -- or, as a shape
+// reference (second input of BroadcastTo), by another producer the same Concat takes over -- is neither an output of the
+// net nor written in place, and nothing between the producer and the Concat overwrites the producer's inputs.
+void SimpleNet::FuseConcatPieces() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_concat_pieces");
+  if (arg && arg->has_i && arg->i == 0) return;
+  auto is_external_output = [&](const std::string& name) {
+    for (const auto& eo : external_output_)
+      if (eo == name) return true;
+    return false;
+  };
+  for (size_t c = 0; c < operators_.size(); ++c) {
+    auto* host = skipped_[c] ? nullptr : dynamic_cast<ConcatPieceHost*>(operators_[c].get());
+    if (!host) continue;
+    const OperatorDef& cd = operators_[c]->operator_def();
+    // candidate producer of every input: the last operator before the Concat that writes the name
+    std::vector<int> producer(cd.input_size(), -1);
+    for (int i = 0; i < cd.input_size(); ++i) {
+      int readers_in_concat = 0;
+      for (const auto& in : cd.input()) readers_in_concat += (in == cd.input(i));
+      if (readers_in_concat != 1 || is_external_output(cd.input(i)) || workspace_->HasConstantBlob(cd.input(i))) continue;
+      for (size_t j = 0; j < c; ++j) {
+        if (skipped_[j]) continue;
+        const OperatorDef& pd = operators_[j]->operator_def();
+        for (const auto& out : pd.output())
+          if (out == cd.input(i)) producer[i] = (int)j;
+      }
+      if (producer[i] < 0) continue;
+      const OperatorDef& pd = operators_[producer[i]]->operator_def();
+      bool ok = dynamic_cast<ConcatPieceSource*>(operators_[producer[i]].get()) != nullptr && pd.output_size() == 1;
+      for (const auto& in : pd.input()) ok &= (in != pd.output(0));  // in place: the "intermediate" is somebody's input
+      // nothing between the producer and the Concat may overwrite what the producer reads
+      for (size_t k = producer[i] + 1; k < c && ok; ++k)
+        for (const auto& out : operators_[k]->operator_def().output())
+          for (const auto& in : pd.input()) ok &= (out != in);
+      if (!ok) producer[i] = -1;
+    }
+    // drop candidates whose output has a reader other than the Concat or a shape-only read by another candidate
+    for (bool changed = true; changed;) {
+      changed = false;
+      for (int i = 0; i < cd.input_size(); ++i) {
+        if (producer[i] < 0) continue;
+        bool ok = true;
+        for (size_t j = 0; j < operators_.size() && ok; ++j) {
+          if (j == c) continue;
+          const OperatorDef& rd = operators_[j]->operator_def();
+          for (int k = 0; k < rd.input_size() && ok; ++k) {
+            if (rd.input(k) != cd.input(i)) continue;
+            bool shape_only_by_candidate = rd.type() == "BroadcastTo" && k == 1;
+            bool is_candidate = false;
+            for (int q = 0; q < cd.input_size(); ++q) is_candidate |= (producer[q] == (int)j);
+            ok = shape_only_by_candidate && is_candidate && !skipped_[j];
+          }
+        }
+        if (!ok) {
+          producer[i] = -1;
+          changed = true;
+        }
+      }
+    }
+    int taken = 0;
+    for (int i = 0; i < cd.input_size(); ++i) taken += producer[i] >= 0;
+    if (taken == 0 || cd.input_size() > BZ_CEW_MAX) continue;
+    for (int i = 0; i < cd.input_size(); ++i) {
+      if (producer[i] < 0) continue;
+      host->AdoptProducer(i, operators_[producer[i]].get(), producer[i]);
+      skipped_[producer[i]] = true;
+    }
   }
 }
 

@@ -96,6 +96,8 @@ class SimpleNet : public Net {
   bool RunImpl() override;
   void StackFcLayers();
   void AliasConcatInputs();
+  void FuseConcatPieces();
+  void FuseFcHeads();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -134,6 +136,36 @@ class StackableFc {
   // the operator whose Output(0) receives this layer's result (the folded activation, else the operator itself)
   virtual OperatorBase* StackOutputOp() = 0;
   virtual void AbsorbStack(const std::vector<StackableFc*>& followers) = 0;
+  // A layer of at most 256 outputs followed by a layer of at most 8 (the logit / score of a tower): the second is
+  // computed in the first one's launch from the output tile still on chip (bz_fc_desc.head_*), and what the first
+  // layer would have stored for it is not stored at all.
+  virtual bool CanHostHead(int* n_out) = 0;   // static eligibility of the first layer; reports its width
+  virtual bool CanBeHead(int k_in) = 0;       // static eligibility of the second layer for a first layer of width k_in
+  virtual void AbsorbHead(StackableFc* head) = 0;
+};
+
+// A Concat along the last axis whose inputs are elementwise results (Add / Sub / Mul / Div / BroadcastTo of tensors
+// that differ only by broadcasting over rows) read by nothing else: the Concat computes those pieces while it
+// writes them (bz_concat_ew) and their operators are skipped -- the attention unit's [q, k, q-k, q*k] in one launch
+// without the intermediate tensors.  Same bits as the separate operators.
+struct ConcatPiece {
+  Blob* x = nullptr;
+  Blob* y = nullptr;            // null: the piece is x itself, broadcast over rows where its dims are 1
+  int op = 0;                   // bz_ew_op; BZ_EW_ASSIGN when y is null
+  std::vector<TIndex> shape;    // of the piece
+};
+class ConcatPieceSource {  // implemented by the elementwise operators
+ public:
+  virtual ~ConcatPieceSource() {}
+  // Describes Output(0) without computing it and gives the output blob its shape (no memory), so that operators that
+  // only read that shape still work.  False: this instance cannot be described (in-place output, type mismatch).
+  virtual bool DescribePiece(ConcatPiece* piece) = 0;
+};
+class ConcatPieceHost {  // implemented by Concat
+ public:
+  virtual ~ConcatPieceHost() {}
+  // input `input_idx` is the output of `producer` (net position `position`), which the net will not run any more
+  virtual void AdoptProducer(int input_idx, OperatorBase* producer, int position) = 0;
 };
 
 }  // namespace blaze

@@ -236,13 +236,23 @@ OPERATOR_SCHEMA(ConstantFill).NumInputs(0).NumOutputs(1).SetDoc("a constant tens
 
 // ------------------------------------------------------------------------------------------ Concat
 template <class Context>
-class ConcatOp final : public Operator<Context> {
+class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
   ConcatOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
     axis_ = OperatorBase::GetSingleArgument<int>("axis", 1);
   }
+  void AdoptProducer(int input_idx, OperatorBase* producer, int position) override {
+    producers_.push_back({position, input_idx, producer});
+    std::sort(producers_.begin(), producers_.end(), [](const Adopted& a, const Adopted& b) { return a.position < b.position; });
+  }
   bool RunOnDevice() override {
+    if (!producers_.empty()) {
+      if (RunWithPieces()) return true;
+      // shapes the one-launch form does not take: run the adopted operators after all, in net order, then copy
+      for (const Adopted& a : producers_)
+        if (!a.op->Run(context_.stream_id())) return false;
+    }
     Blob* x0 = this->Input(0);
     const size_t rank = x0->shape().size();
     BLAZE_CONDITION_THROW(axis_ >= 0 && (size_t)axis_ < rank, "axis=", axis_, " rank=", rank);
@@ -293,7 +303,114 @@ class ConcatOp final : public Operator<Context> {
   }
 
  private:
+  struct Adopted {
+    int position;
+    int input_idx;
+    OperatorBase* op;
+  };
+  // The inputs as pieces of one bz_concat_ew launch.  False when the shapes do not fit that kernel's model (concat
+  // along another axis than the last, an operand broadcast along the last axis, or row dims that do not merge into
+  // two coordinates); nothing has been launched then.
+  bool RunWithPieces() {
+    const int n = this->InputSize();
+    std::vector<ConcatPiece> pieces(n);
+    std::vector<bool> described(n, false);
+    for (const Adopted& a : producers_) {  // net order: a BroadcastTo may take its shape from an earlier piece
+      auto* src = dynamic_cast<ConcatPieceSource*>(a.op);
+      if (!src || !src->DescribePiece(&pieces[a.input_idx])) return false;
+      described[a.input_idx] = true;
+    }
+    for (int i = 0; i < n; ++i) {
+      if (described[i]) continue;
+      Blob* x = this->Input(i);
+      if (x->pitch() != 0) return false;
+      pieces[i].x = x;
+      pieces[i].op = BZ_EW_ASSIGN;
+      pieces[i].shape = x->shape();
+    }
+    const size_t rank = pieces[0].shape.size();
+    if (rank < 1 || axis_ != (int)rank - 1) return false;
+    const int dtype = pieces[0].x->data_type();
+    std::vector<TIndex> shape = pieces[0].shape;
+    TIndex total = 0;
+    for (int i = 0; i < n; ++i) {
+      const ConcatPiece& p = pieces[i];
+      BLAZE_CONDITION_THROW(p.shape.size() == rank && p.x->data_type() == dtype && (!p.y || p.y->data_type() == dtype),
+                            "concat input ", i, " has another rank or type");
+      for (size_t k = 0; k + 1 < rank; ++k)
+        BLAZE_CONDITION_THROW(p.shape[k] == shape[k], "concat input ", i, " dim ", k, " mismatch");
+      if (p.shape[rank - 1] <= 0 || p.shape[rank - 1] >= (1ll << 31)) return false;
+      total += p.shape[rank - 1];
+    }
+    // every operand's dims, right aligned to the piece's rank; `bc[k]` collects, per outer dim, which operands are
+    // broadcast along it (one bit per operand): adjacent dims with the same set merge into one row coordinate
+    struct Operand {
+      std::vector<TIndex> dims;
+    };
+    std::vector<Operand> ops;
+    for (int i = 0; i < n; ++i) {
+      for (Blob* b : {pieces[i].x, pieces[i].y}) {
+        Operand o;
+        if (b) {
+          if (b->shape().size() > rank) return false;
+          o.dims.assign(rank - b->shape().size(), 1);
+          o.dims.insert(o.dims.end(), b->shape().begin(), b->shape().end());
+          if (o.dims[rank - 1] != pieces[i].shape[rank - 1]) return false;  // broadcast along the concat axis
+        }
+        ops.push_back(o);
+      }
+    }
+    std::vector<uint32_t> group_sig;
+    std::vector<TIndex> group_size;
+    for (size_t k = 0; k + 1 < rank; ++k) {
+      if (shape[k] == 1) continue;
+      uint32_t sig = 0;
+      for (size_t o = 0; o < ops.size(); ++o)
+        if (!ops[o].dims.empty() && ops[o].dims[k] == 1) sig |= 1u << o;
+      if (!group_sig.empty() && group_sig.back() == sig) {
+        group_size.back() *= shape[k];
+      } else {
+        group_sig.push_back(sig);
+        group_size.push_back(shape[k]);
+      }
+    }
+    if (group_sig.size() > 2) return false;
+    while (group_sig.size() < 2) {
+      group_sig.push_back(0);
+      group_size.push_back(1);
+    }
+    shape[rank - 1] = total;
+    Blob* y = this->Output(0);
+    y->set_data_type((DataType)dtype);
+    y->Reshape(shape);
+    bz_concat_ew_desc d;
+    memset(&d, 0, sizeof(d));
+    d.n = n;
+    d.dtype = BzType(dtype);
+    d.dst = y->data();
+    d.dst_pitch = total;
+    d.r0 = group_size[0];
+    d.r1 = group_size[1];
+    for (int i = 0; i < n; ++i) {
+      const int64_t w = pieces[i].shape[rank - 1];
+      d.op[i] = pieces[i].op;
+      d.width[i] = (int32_t)w;
+      d.x[i] = pieces[i].x->data();
+      d.y[i] = pieces[i].y ? pieces[i].y->data() : nullptr;
+      for (int side = 0; side < 2; ++side) {
+        if (side == 1 && !pieces[i].y) continue;
+        const bool b0 = (group_sig[0] >> (2 * i + side)) & 1, b1 = (group_sig[1] >> (2 * i + side)) & 1;
+        int64_t* st = side == 0 ? d.x_stride[i] : d.y_stride[i];
+        st[0] = b0 ? 0 : (b1 ? 1 : d.r1) * w;
+        st[1] = b1 ? 0 : w;
+      }
+    }
+    BZ_CHECK(bz_concat_ew(&d, context_.hip_stream()));
+    return true;
+  }
+
   int axis_;
+  std::vector<Adopted> producers_;  // inputs computed by this operator instead of by their own (sorted by net position)
 };
 REGISTER_HIP_OPERATOR(Concat, ConcatOp<HIPContext>);
 OPERATOR_SCHEMA(Concat).NumInputs(1, INT_MAX).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("concatenate along axis");

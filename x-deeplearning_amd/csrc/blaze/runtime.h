@@ -48,6 +48,14 @@ class Blob {
     }
     dims_ = dims;
   }
+  // the shape alone, for the output of an operator whose work its consumer has taken over: readers may ask the shape,
+  // nobody reads the data (a later Reshape allocates as usual)
+  void SetShapeOnly(const std::vector<TIndex>& dims) {
+    TIndex n = 1;
+    for (auto d : dims) n *= d;
+    size_ = n;
+    dims_ = dims;
+  }
   void RefReshape(const std::vector<TIndex>& dims, void* handle) {
     if (own_handle_ || data_ != handle) {  // (re-aliasing the same buffer keeps the version)
       Destroy();

@@ -116,10 +116,22 @@ OPERATOR_SCHEMA(Reshape).NumInputs(2).NumOutputs(1).IdenticalTypeOfInput(0).SetD
 
 // ------------------------------------------------------------------------------------------ Add / Sub / Mul / Div
 template <class Context, int OP>
-class ElementwiseOp final : public Operator<Context> {
+class ElementwiseOp final : public Operator<Context>, public ConcatPieceSource {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
   ElementwiseOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {}
+  bool DescribePiece(ConcatPiece* piece) override {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    Blob* c = this->Output(0);
+    if (a->data_type() != b->data_type() || c == a || c == b || a->pitch() != 0 || b->pitch() != 0) return false;
+    piece->x = a;
+    piece->y = b;
+    piece->op = OP;
+    piece->shape = BroadcastShape(a->shape(), b->shape(), this->def_);
+    c->SetShapeOnly(piece->shape);
+    return true;
+  }
   bool RunOnDevice() override {
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -158,30 +170,28 @@ BLAZE_REGISTER_ELEMENTWISE(Div, BZ_EW_DIV, "a / b = c");
 
 // ------------------------------------------------------------------------------------------ BroadcastTo
 template <class Context>
-class BroadcastToOp final : public Operator<Context> {
+class BroadcastToOp final : public Operator<Context>, public ConcatPieceSource {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
   BroadcastToOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
     broadcast_shape_ = OperatorBase::GetRepeatedArgument<int>("shape");
   }
+  bool DescribePiece(ConcatPiece* piece) override {
+    Blob* a = this->Input(0);
+    Blob* y = this->Output(0);
+    if (y == a || a->pitch() != 0) return false;
+    piece->x = a;
+    piece->y = nullptr;
+    piece->op = BZ_EW_ASSIGN;
+    piece->shape = TargetShape();
+    y->SetShapeOnly(piece->shape);
+    return true;
+  }
   bool RunOnDevice() override {
     Blob* a = this->Input(0);
     Blob* y = this->Output(0);
     const std::vector<TIndex> as = a->shape();
-    std::vector<TIndex> out;
-    if (this->InputSize() > 1) {
-      out = this->Input(1)->shape();
-    } else {
-      BLAZE_CONDITION_THROW(as.size() == broadcast_shape_.size(), "a->shape().size()=", as.size(),
-                            " broadcast_shape_.size()=", broadcast_shape_.size());
-      out = as;
-      for (size_t i = 0; i < broadcast_shape_.size(); ++i) {
-        BLAZE_CONDITION_THROW(broadcast_shape_[i] >= 0, "can not support dim < 0");
-        if (broadcast_shape_[i] > 0) out[i] = (TIndex)broadcast_shape_[i];
-      }
-    }
-    BLAZE_CONDITION_THROW(BroadcastShape(as, out, this->def_) == out, "input does not broadcast to the target shape op=",
-                          this->def_.name());
+    const std::vector<TIndex> out = TargetShape();
     BLAZE_CONDITION_THROW(y != a || as == out, "in-place output would grow op=", this->def_.name());
     y->Reshape(out);
     if (y->size() == 0) return true;
@@ -198,6 +208,25 @@ class BroadcastToOp final : public Operator<Context> {
   }
 
  private:
+  // the shape of the second input, or the input's own with the positive entries of `shape` put in
+  std::vector<TIndex> TargetShape() {
+    const std::vector<TIndex> as = this->Input(0)->shape();
+    std::vector<TIndex> out;
+    if (this->InputSize() > 1) {
+      out = this->Input(1)->shape();
+    } else {
+      BLAZE_CONDITION_THROW(as.size() == broadcast_shape_.size(), "a->shape().size()=", as.size(),
+                            " broadcast_shape_.size()=", broadcast_shape_.size());
+      out = as;
+      for (size_t i = 0; i < broadcast_shape_.size(); ++i) {
+        BLAZE_CONDITION_THROW(broadcast_shape_[i] >= 0, "can not support dim < 0");
+        if (broadcast_shape_[i] > 0) out[i] = (TIndex)broadcast_shape_[i];
+      }
+    }
+    BLAZE_CONDITION_THROW(BroadcastShape(as, out, this->def_) == out, "input does not broadcast to the target shape op=",
+                          this->def_.name());
+    return out;
+  }
   std::vector<int> broadcast_shape_;
 };
 REGISTER_HIP_OPERATOR(BroadcastTo, BroadcastToOp<HIPContext>);

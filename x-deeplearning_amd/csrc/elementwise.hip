@@ -147,6 +147,75 @@ int grid_for(int64_t work) {
   return (int)(want < 1 ? 1 : (want < 256 * 32 ? want : 256 * 32));
 }
 
+// ---- concat of pieces computed on the fly -------------------------------------------------------------------
+struct CewP {
+  const void* x[BZ_CEW_MAX];
+  const void* y[BZ_CEW_MAX];
+  int64_t xs[BZ_CEW_MAX][2], ys[BZ_CEW_MAX][2];
+  int32_t op[BZ_CEW_MAX];
+  int32_t col0[BZ_CEW_MAX + 1];  // first output column of each piece; col0[n] = total
+  int n;
+  int64_t rows, r1, dst_pitch;
+};
+
+// VEC consecutive columns of one output row per thread (the host picks a VEC that divides every width).  IdxT is
+// 32-bit whenever the element count allows: the two divisions per thread are the expensive part of this kernel.
+template <typename T, int VEC, typename IdxT>
+__global__ __launch_bounds__(256) void bz_concat_ew_kernel(T* __restrict__ dst, CewP arg) {
+  // the piece table is indexed with a run-time piece number: from LDS, not from a per-lane copy of the arguments
+  __shared__ CewP p;
+  static_assert(sizeof(CewP) % 4 == 0, "copied in 32-bit words");
+  for (int w = threadIdx.x; w < (int)(sizeof(CewP) / 4); w += 256) ((uint32_t*)&p)[w] = ((const uint32_t*)&arg)[w];
+  __syncthreads();
+  const IdxT per_row = (IdxT)(p.col0[p.n] / VEC);
+  const IdxT nvec = (IdxT)p.rows * per_row;
+  const IdxT r1 = (IdxT)p.r1;
+  for (IdxT v = (IdxT)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (IdxT)gridDim.x * 256) {
+    const IdxT row = v / per_row;
+    const int col = (int)(v - row * per_row) * VEC;
+    int k = 0;
+#pragma unroll
+    for (int q = 1; q < BZ_CEW_MAX; ++q) k += (q < p.n && col >= p.col0[q]);
+    const int c = col - p.col0[k];
+    const IdxT i0 = row / r1, i1 = row - i0 * r1;
+    const T* x = (const T*)p.x[k] + (int64_t)i0 * p.xs[k][0] + (int64_t)i1 * p.xs[k][1] + c;
+    T* out = dst + (int64_t)row * p.dst_pitch + col;
+    const int op = p.op[k];
+    if (op == BZ_EW_ASSIGN) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) out[e] = x[e];
+    } else {
+      const T* y = (const T*)p.y[k] + (int64_t)i0 * p.ys[k][0] + (int64_t)i1 * p.ys[k][1] + c;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float a = ldv<T>(x + e), b = ldv<T>(y + e);
+        stv<T>(out + e, op == BZ_EW_ADD ? __fadd_rn(a, b) : op == BZ_EW_SUB ? __fsub_rn(a, b) : op == BZ_EW_MUL ? __fmul_rn(a, b) : __fdiv_rn(a, b));
+      }
+    }
+  }
+}
+
+template <typename T, typename IdxT>
+int launch_concat_ew_i(void* dst, const CewP& p, int vec, hipStream_t s) {
+  const int grid = grid_for(p.rows * (p.col0[p.n] / vec));
+  switch (vec) {
+    case 8: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 8, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
+    case 4: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 4, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
+    case 2: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 2, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
+    default: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 1, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
+  }
+  BZ_LAUNCH_OK("bz_concat_ew_kernel");
+  return BZ_OK;
+}
+
+template <typename T>
+int launch_concat_ew(void* dst, const CewP& p, int vec, hipStream_t s) {
+  const int64_t nvec = p.rows * (p.col0[p.n] / vec);
+  // (the grid-stride loop adds at most 2^21 to an index below nvec)
+  if (nvec < (1ll << 31) - (1ll << 22) && p.r1 < (1ll << 31)) return launch_concat_ew_i<T, uint32_t>(dst, p, vec, s);
+  return launch_concat_ew_i<T, int64_t>(dst, p, vec, s);
+}
+
 template <typename T, typename CondT>
 int launch_bcast(const bz_bcast_desc& d, const BcastP& p, int vec, hipStream_t s) {
   const int grid = grid_for(p.total / vec);
@@ -233,6 +302,60 @@ extern "C" int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream) {
   if (d.dtype == BZ_F32) return launch_bcast_t<float>(d, p, vec > 4 ? 4 : vec, s);
   if (d.dtype == BZ_F16) return launch_bcast_t<__half>(d, p, vec, s);
   return launch_bcast_t<__hip_bfloat16>(d, p, vec, s);
+}
+
+extern "C" int bz_concat_ew(const bz_concat_ew_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_concat_ew: null descriptor");
+  const bz_concat_ew_desc& d = *desc;
+  BZ_REQUIRE(d.n >= 1 && d.n <= BZ_CEW_MAX, "bz_concat_ew: %d pieces outside 1..%d", d.n, BZ_CEW_MAX);
+  BZ_REQUIRE(d.dtype == BZ_F32 || d.dtype == BZ_F16 || d.dtype == BZ_BF16, "bz_concat_ew: unsupported dtype %d", d.dtype);
+  BZ_REQUIRE(d.r0 >= 0 && d.r1 >= 0 && d.dst != nullptr, "bz_concat_ew: r0=%lld r1=%lld or null dst", (long long)d.r0, (long long)d.r1);
+  const int es = bz::dtype_size(d.dtype);
+  CewP p = {};
+  p.n = d.n;
+  p.rows = d.r0 * d.r1;
+  p.r1 = d.r1 > 0 ? d.r1 : 1;
+  p.dst_pitch = d.dst_pitch;
+  int vec = 8;
+  auto fit = [&](int64_t q) {
+    while (vec > 1 && q % vec != 0) vec >>= 1;
+  };
+  int64_t total = 0;
+  for (int i = 0; i < d.n; ++i) {
+    BZ_REQUIRE(d.op[i] >= BZ_EW_ADD && d.op[i] <= BZ_EW_ASSIGN, "bz_concat_ew: piece %d: unknown op %d", i, d.op[i]);
+    BZ_REQUIRE(d.x[i] != nullptr && (d.op[i] == BZ_EW_ASSIGN || d.y[i] != nullptr), "bz_concat_ew: piece %d: null operand", i);
+    BZ_REQUIRE(d.width[i] > 0, "bz_concat_ew: piece %d: width %d", i, d.width[i]);
+    p.x[i] = d.x[i];
+    p.y[i] = d.y[i];
+    p.op[i] = d.op[i];
+    p.col0[i] = (int32_t)total;
+    total += d.width[i];
+    fit(d.width[i]);
+    fit((int64_t)((uintptr_t)d.x[i] / es));
+    BZ_REQUIRE((uintptr_t)d.x[i] % es == 0, "bz_concat_ew: piece %d: misaligned operand", i);
+    for (int k = 0; k < 2; ++k) {
+      BZ_REQUIRE(d.x_stride[i][k] >= 0 && d.y_stride[i][k] >= 0, "bz_concat_ew: piece %d: negative stride", i);
+      p.xs[i][k] = d.x_stride[i][k];
+      p.ys[i][k] = d.y_stride[i][k];
+      fit(d.x_stride[i][k]);
+      if (d.op[i] != BZ_EW_ASSIGN) fit(d.y_stride[i][k]);
+    }
+    if (d.op[i] != BZ_EW_ASSIGN) {
+      BZ_REQUIRE((uintptr_t)d.y[i] % es == 0, "bz_concat_ew: piece %d: misaligned operand", i);
+      fit((int64_t)((uintptr_t)d.y[i] / es));
+    }
+  }
+  BZ_REQUIRE(total <= d.dst_pitch && total < (1ll << 31), "bz_concat_ew: widths sum to %lld, row pitch is %lld", (long long)total,
+             (long long)d.dst_pitch);
+  BZ_REQUIRE((uintptr_t)d.dst % es == 0, "bz_concat_ew: misaligned dst");
+  p.col0[d.n] = (int32_t)total;
+  fit(d.dst_pitch);
+  fit((int64_t)((uintptr_t)d.dst / es));
+  if (p.rows == 0) return BZ_OK;
+  hipStream_t s = bz::as_stream(stream);
+  if (d.dtype == BZ_F32) return launch_concat_ew<float>(d.dst, p, vec, s);
+  if (d.dtype == BZ_F16) return launch_concat_ew<__half>(d.dst, p, vec, s);
+  return launch_concat_ew<__hip_bfloat16>(d.dst, p, vec, s);
 }
 
 extern "C" int bz_reduce_sum(const void* x, void* y, int64_t outer, int64_t dim, int64_t inner, int dtype, bz_stream_t stream) {

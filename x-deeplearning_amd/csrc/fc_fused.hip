@@ -203,14 +203,46 @@ __device__ __forceinline__ uint4 load_chunk_aligned(const char* base, int64_t ro
   return *(const uint4*)(base + (row * ld + kc) * ES);  // caller zeroes chunks with k >= K when it consumes them
 }
 
+constexpr int kSkinnyMaxN = 8;
+
+template <int DT>
+__device__ __forceinline__ void chunk_to_float(const uint4& c, float (&f)[In<DT>::kChunk]) {
+  const uint32_t r[4] = {c.x, c.y, c.z, c.w};
+  if constexpr (DT == BZ_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r[i]);
+  } else if constexpr (DT == BZ_F16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xffffu)));
+      f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
+    }
+  } else {  // bf16: the upper 16 bits of the fp32 pattern
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(r[i] << 16);
+      f[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+  }
+}
+
+// the optional skinny second layer computed from the first layer's output tile while it is still in LDS
+struct HeadArgs {
+  const char* w;      // [n, ldw], K contiguous, the dtype of the first layer's operands
+  const float* bias;  // [n] or null
+  void* y;            // [M, ldy]
+  int64_t ldw, ldy;
+  int n, act, out_dtype;
+};
+
 // ---------------------------------------------------------------------------------------------
 // tiled MFMA kernel
 // ---------------------------------------------------------------------------------------------
-template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED>
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED, bool HEAD>
 __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __restrict__ A, const char* __restrict__ W,
                                                                   OutT* __restrict__ Y, int M, int N, int K, int64_t lda,
                                                                   int64_t ldw, int64_t ldy, bool vec_a, bool vec_w,
-                                                                  bool vec_y, int tiles_m, Epilogue ep) {
+                                                                  bool vec_y, int tiles_m, Epilogue ep, HeadArgs head) {
   using T = In<DT>;
   constexpr int NT = WM * WN * 64;
   constexpr int ES = T::kSize;
@@ -224,6 +256,12 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % T::kStepK == 0, "tile shape");
 
   __shared__ __attribute__((aligned(16))) char lds[2][(BM + BN) * PITCH];
+  // HEAD: the second layer's weight [kSkinnyMaxN, BN], requested now into registers, parked in LDS after the K loop
+  constexpr int HW_ROW = BN * ES;  // bytes
+  constexpr int HW_CHUNKS = HEAD ? kSkinnyMaxN * HW_ROW / 16 : 1;
+  constexpr int HW_PER = (HW_CHUNKS + NT - 1) / NT;
+  __shared__ __attribute__((aligned(16))) char lds_hw[HEAD ? kSkinnyMaxN * HW_ROW : 16];
+  uint4 rhw[HW_PER];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -287,6 +325,17 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         *(uint4*)&lds[buf][(BM + q / CPR) * PITCH + (q % CPR) * 16] = masked(rw[set][i], k0 + (q % CPR) * T::kChunk);
     }
   };
+
+  if constexpr (HEAD) {
+    const int present = N * ES / 16;  // chunks of a weight row that exist (N is a whole number of chunks)
+#pragma unroll
+    for (int i = 0; i < HW_PER; ++i) {
+      const int q = tid + i * NT;
+      const int j = q / (HW_ROW / 16), ch = q % (HW_ROW / 16);
+      rhw[i] = make_uint4(0, 0, 0, 0);
+      if (q < HW_CHUNKS && j < head.n && ch < present) rhw[i] = *(const uint4*)(head.w + (int64_t)j * head.ldw * ES + ch * 16);
+    }
+  }
 
   // with a single 32x32 block per wave, back-to-back MFMAs into one accumulator would each wait for the
   // previous result; alternate K steps between two accumulators and add them at the end
@@ -388,7 +437,7 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
             else if (ep.bias_rows > 1)
               v += ep.beta * ep.bias[(int64_t)m * N + n];
             v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
-            if (vec_y)
+            if (HEAD || vec_y)
               store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
             else
               store_out<OutT>(Y + (int64_t)m * ldy + n, v);
@@ -414,13 +463,97 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
       epilogue(std::integral_constant<int, BZ_ACT_NONE>());
       break;
   }
-  if (vec_y) {
+  if constexpr (HEAD) {
+#pragma unroll
+    for (int i = 0; i < HW_PER; ++i) {
+      const int q = tid + i * NT;
+      if (q < HW_CHUNKS) *(uint4*)&lds_hw[q * 16] = rhw[i];
+    }
+  }
+  if (HEAD || vec_y) {
     __syncthreads();
-    constexpr int OCPR = BN * OS / 16;  // 16-byte chunks per tile row
-    for (int q = tid; q < BM * OCPR; q += NT) {
-      const int ml = q / OCPR, ch = q % OCPR;
-      const int m = m0 + ml, n = n0 + ch * (16 / OS);
-      if (m < M && n < N) *(uint4*)((char*)(Y + (int64_t)m * ldy + n)) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+    if (vec_y) {
+      constexpr int OCPR = BN * OS / 16;  // 16-byte chunks per tile row
+      for (int q = tid; q < BM * OCPR; q += NT) {
+        const int ml = q / OCPR, ch = q % OCPR;
+        const int m = m0 + ml, n = n0 + ch * (16 / OS);
+        if (m < M && n < N) *(uint4*)((char*)(Y + (int64_t)m * ldy + n)) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+      }
+    } else if (Y != nullptr) {  // HEAD with an output that takes no 16-byte stores
+      for (int q = tid; q < BM * BN; q += NT) {
+        const int ml = q / BN, nl = q % BN;
+        if (m0 + ml < M && n0 + nl < N) Y[(int64_t)(m0 + ml) * ldy + n0 + nl] = ((const OutT*)(lout + ml * OPITCH))[nl];
+      }
+    }
+  }
+  if constexpr (HEAD) {
+    // z[m, j] = head_act(sum_n y[m, n] * w2[j, n] + b2[j]) from the rounded tile, as the separate skinny launch
+    // computes it from the stored tensor.  NT / BM lanes share a row; this workgroup owns whole rows (n0 == 0).
+    static_assert(OS == ES, "the head reads the tile with the operand type");
+    constexpr int LPRH = NT / BM;
+    constexpr int CH = In<DT>::kChunk;
+    const int r = tid / LPRH, hl = tid % LPRH;
+    const int m = m0 + r;
+    const int nch = N / CH;
+    float hacc[kSkinnyMaxN];
+#pragma unroll
+    for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] = 0.f;
+    for (int ch = hl; ch < nch; ch += LPRH) {
+      float a[CH];
+      chunk_to_float<DT>(*(const uint4*)(lout + r * OPITCH + ch * 16), a);
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) {
+        if (j < head.n) {
+          float w[CH];
+          chunk_to_float<DT>(*(const uint4*)(lds_hw + j * HW_ROW + ch * 16), w);
+#pragma unroll
+          for (int i = 0; i < CH; ++i) hacc[j] = fmaf(a[i], w[i], hacc[j]);
+        }
+      }
+    }
+#pragma unroll
+    for (int d = LPRH >> 1; d > 0; d >>= 1) {
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] += __shfl_xor(hacc[j], d, 64);
+    }
+    if (hl == 0 && m < M) {
+      float v[kSkinnyMaxN];
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) v[j] = (j < head.n) ? hacc[j] + (head.bias ? head.bias[j] : 0.f) : 0.f;
+      if (head.act == BZ_ACT_SOFTMAX) {  // softmax_op.cc:21-78: subtract max, exp, sum in order, divide
+        float mx = v[0];
+#pragma unroll
+        for (int j = 1; j < kSkinnyMaxN; ++j)
+          if (j < head.n) mx = v[j] > mx ? v[j] : mx;
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j)
+          if (j < head.n) {
+            v[j] = expf(v[j] - mx);
+            sum += v[j];
+          }
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j)
+          if (j < head.n) v[j] = v[j] / sum;
+      } else if (head.act == BZ_ACT_SIGMOID) {
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j) {
+          const float t = expf(v[j]);
+          v[j] = t / (1.f + t);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) {
+        if (j < head.n) {
+          const int64_t at = (int64_t)m * head.ldy + j;
+          if (head.out_dtype == BZ_F32)
+            store_out<float>((float*)head.y + at, v[j]);
+          else if (head.out_dtype == BZ_F16)
+            store_out<__half>((__half*)head.y + at, v[j]);
+          else
+            store_out<__hip_bfloat16>((__hip_bfloat16*)head.y + at, v[j]);
+        }
+      }
     }
   }
 }
@@ -428,29 +561,6 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
 // ---------------------------------------------------------------------------------------------
 // skinny kernel: N <= 8
 // ---------------------------------------------------------------------------------------------
-constexpr int kSkinnyMaxN = 8;
-
-template <int DT>
-__device__ __forceinline__ void chunk_to_float(const uint4& c, float (&f)[In<DT>::kChunk]) {
-  const uint32_t r[4] = {c.x, c.y, c.z, c.w};
-  if constexpr (DT == BZ_F32) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r[i]);
-  } else if constexpr (DT == BZ_F16) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f[2 * i] = __half2float(__ushort_as_half((unsigned short)(r[i] & 0xffffu)));
-      f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(r[i] >> 16)));
-    }
-  } else {  // bf16: the upper 16 bits of the fp32 pattern
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f[2 * i] = __uint_as_float(r[i] << 16);
-      f[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
-    }
-  }
-}
-
 template <int DT, typename OutT>
 __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restrict__ A, const char* __restrict__ W,
                                                            OutT* __restrict__ Y, int M, int N, int K, int64_t lda,
@@ -553,17 +663,41 @@ __global__ void bz_pack_weight_kernel(const SrcT* __restrict__ src, DstT* __rest
   }
 }
 
-template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED>
+template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, bool ALIGNED, bool HEAD = false>
 int launch_mfma(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
   const int tiles_m = (d.m + BM - 1) / BM, tiles_n = (d.n + BN - 1) / BN;
   // output rows 16-byte aligned and N a whole number of 16-byte chunks: coalesced stores through LDS
-  const bool vec_y = ((uintptr_t)d.y % 16 == 0) && ((d.ldy * (int64_t)sizeof(OutT)) % 16 == 0) &&
+  const bool vec_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * (int64_t)sizeof(OutT)) % 16 == 0) &&
                      (d.n % (16 / (int)sizeof(OutT)) == 0);
-  hipLaunchKernelGGL((bz_fc_mfma_kernel<DT, OutT, BM, BN, BK, WM, WN, D, ALIGNED>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), 0, st,
-                     (const char*)d.a, (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, vec_a, vec_w,
-                     vec_y, tiles_m, ep);
+  HeadArgs head = {};
+  if (HEAD) {
+    head.w = (const char*)d.head_w;
+    head.bias = d.head_bias;
+    head.y = d.head_y;
+    head.ldw = d.head_ldw;
+    head.ldy = d.head_ldy;
+    head.n = d.head_n;
+    head.act = d.head_act;
+    head.out_dtype = d.head_out_dtype;
+  }
+  hipLaunchKernelGGL((bz_fc_mfma_kernel<DT, OutT, BM, BN, BK, WM, WN, D, ALIGNED, HEAD>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), 0,
+                     st, (const char*)d.a, (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, vec_a, vec_w, vec_y,
+                     tiles_m, ep, head);
   BZ_LAUNCH_OK("bz_fc_mfma_kernel");
   return BZ_OK;
+}
+
+// Layer + skinny head in one launch: a workgroup owns whole rows of the first layer's output (N <= 256).
+template <int DT, typename OutT>
+int dispatch_head(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
+  constexpr int BK = In<DT>::kSize == 2 ? 64 : 32;
+  if (d.n <= 64) {
+    if ((d.m + 63) / 64 >= 256) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 4, true, true>(d, ep, true, true, st);
+    return launch_mfma<DT, OutT, 32, 64, BK, 1, 2, 4, true, true>(d, ep, true, true, st);
+  }
+  if (d.n <= 128) return launch_mfma<DT, OutT, 32, 128, BK, 1, 4, 4, true, true>(d, ep, true, true, st);
+  // eight waves: with one workgroup per 32 rows only M / 32 CUs work, and each has 288 KB of operands to pull in
+  return launch_mfma<DT, OutT, 32, 256, BK, 1, 8, 4, true, true>(d, ep, true, true, st);
 }
 
 template <int DT, typename OutT>
@@ -630,7 +764,7 @@ extern "C" {
 int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   BZ_REQUIRE(desc != nullptr, "bz_fc_fused: null descriptor");
   const bz_fc_desc& d = *desc;
-  BZ_REQUIRE(d.a && d.w && d.y, "bz_fc_fused: null a/w/y");
+  BZ_REQUIRE(d.a && d.w && (d.y || d.head_n > 0), "bz_fc_fused: null a/w/y");
   BZ_REQUIRE(d.m >= 0 && d.n > 0 && d.k > 0, "bz_fc_fused: bad shape m=%d n=%d k=%d", d.m, d.n, d.k);
   BZ_REQUIRE(d.lda >= d.k && d.ldw >= d.k && d.ldy >= d.n, "bz_fc_fused: leading dimension smaller than row (lda=%lld ldw=%lld ldy=%lld)",
              (long long)d.lda, (long long)d.ldw, (long long)d.ldy);
@@ -674,6 +808,29 @@ int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   const bool vec_a = ((uintptr_t)d.a % 16 == 0) && ((d.lda * es) % 16 == 0);
   const bool vec_w = ((uintptr_t)d.w % 16 == 0) && ((d.ldw * es) % 16 == 0);
   hipStream_t st = bz::as_stream(stream);
+  if (d.head_n != 0) {
+    const int chunk = 16 / es;
+    BZ_REQUIRE(d.head_n > 0 && d.head_n <= kSkinnyMaxN && d.head_w && d.head_y, "bz_fc_fused: head of %d outputs (1..%d) or null head_w/head_y",
+               d.head_n, kSkinnyMaxN);
+    if (d.n > 256 || d.n <= kSkinnyMaxN || d.n % chunk != 0)
+      return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a fused head needs %d < n <= 256 and n a multiple of %d (n=%d)", kSkinnyMaxN, chunk, d.n);
+    if (!(vec_a && vec_w && d.k % chunk == 0))
+      return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a fused head needs 16-byte aligned operand rows and k a multiple of %d", chunk);
+    BZ_REQUIRE(d.out_dtype == d.in_dtype, "bz_fc_fused: with a fused head the layer's output type must be its input type");
+    BZ_REQUIRE(d.act != BZ_ACT_SOFTMAX && (d.bias_rows == 0 || d.bias_rows == 1), "bz_fc_fused: fused head after softmax or a full bias");
+    BZ_REQUIRE(d.head_act == BZ_ACT_NONE || d.head_act == BZ_ACT_SIGMOID || d.head_act == BZ_ACT_SOFTMAX,
+               "bz_fc_fused: head activation %d (none, sigmoid or softmax)", d.head_act);
+    BZ_REQUIRE(d.head_ldw >= d.n && (d.head_ldw * es) % 16 == 0 && (uintptr_t)d.head_w % 16 == 0 && d.head_ldy >= d.head_n,
+               "bz_fc_fused: head_ldw=%lld (>= n, rows 16-byte aligned) head_ldy=%lld (>= head_n)", (long long)d.head_ldw,
+               (long long)d.head_ldy);
+    BZ_REQUIRE(d.head_out_dtype == BZ_F32 || d.head_out_dtype == BZ_F16 || d.head_out_dtype == BZ_BF16, "bz_fc_fused: head out dtype %d",
+               d.head_out_dtype);
+    switch (d.in_dtype) {
+      case BZ_F16: return dispatch_head<BZ_F16, __half>(d, ep, st);
+      case BZ_BF16: return dispatch_head<BZ_BF16, __hip_bfloat16>(d, ep, st);
+      default: return dispatch_head<BZ_F32, float>(d, ep, st);
+    }
+  }
   switch (d.in_dtype) {
     case BZ_F16: return dispatch_out<BZ_F16>(d, ep, vec_a, vec_w, st);
     case BZ_BF16: return dispatch_out<BZ_BF16>(d, ep, vec_a, vec_w, st);

@@ -75,9 +75,10 @@ class Config3:
         return feed
 
 
-def build_manager(cfg, tables, weights, dtype=np.float16, expose=()):
+def build_manager(cfg, tables, weights, dtype=np.float16, expose=(), net_args=None):
     """-> (PredictorManager with the model loaded, list of external input names).  `expose`: names of
-    intermediate blobs also declared as outputs (for parity checks)."""
+    intermediate blobs also declared as outputs (for parity checks).  net_args: integer net arguments, e.g.
+    {"fuse_concat_pieces": 0}."""
     code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
     pm = pb.PredictorManager()
     for k, t in zip(KINDS, tables):
@@ -96,6 +97,8 @@ def build_manager(cfg, tables, weights, dtype=np.float16, expose=()):
     nb.external_output("prob", pb.K_FLOAT)
     for name in expose:
         nb.external_output(name, code)
+    for k, v in (net_args or {}).items():
+        nb.arg(k, int(v))
     for tag in ("att", "main"):
         for li, l in enumerate(weights[tag]):
             p = "%s%d_" % (tag, li)
