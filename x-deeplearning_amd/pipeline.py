@@ -14,11 +14,15 @@ import blaze_hip as bz
 
 
 class CtrForward:
-    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True, fused_mlp=False):
-        """fused_mlp: run the FC stack as one bz_mlp_fused launch instead of one bz_fc_fused launch per layer."""
+    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True, fused_mlp=False,
+                 fused_head=True):
+        """fused_mlp: run the FC stack as one bz_mlp_fused launch instead of one bz_fc_fused launch per layer.
+        fused_head: the last (skinny) layer rides in the launch of the layer before it, as SimpleNet runs the model."""
         import torch
         self.cfg = cfg
         self.fused_scan = fused_scan
+        self.fused_head = fused_head and len(mlp) >= 2
+        self._launches = None
         self.fused_mlp = None
         self.lib = bz.lib()
         tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
@@ -70,7 +74,15 @@ class CtrForward:
                     d.act, d.act_p0, d.act_size = bz.ACT_PRELU, slope.data_ptr(), slope.numel()
                 descs.append(d)
                 acts.append(y)
-            self.steps.append(dict(plan=plan, descs=descs, acts=acts, keep=keep, x=x))
+            head_desc = None
+            if self.fused_head:  # layer n-2 with layer n-1 as its head; the tensor between them is not stored
+                head_desc = bz.FcDesc.from_buffer_copy(descs[-2])
+                last = descs[-1]
+                head_desc.y = None
+                head_desc.head_w, head_desc.head_bias, head_desc.head_y = last.w, last.bias, last.y
+                head_desc.head_ldw, head_desc.head_ldy, head_desc.head_n = last.ldw, last.ldy, last.n
+                head_desc.head_act, head_desc.head_out_dtype = last.act, last.out_dtype
+            self.steps.append(dict(plan=plan, descs=descs, acts=acts, keep=keep, x=x, head_desc=head_desc))
             self.nnz.append(nnz)
 
     # --- launches (current stream) ---------------------------------------------------------------
@@ -90,6 +102,26 @@ class CtrForward:
         d = self.steps[i % self.n_batches]["descs"][layer]
         bz.check(self.lib.bz_fc_fused(C.byref(d), st or self._stream()))
 
+    def fc_with_head(self, i, st=None):
+        """the last two layers in one launch"""
+        d = self.steps[i % self.n_batches]["head_desc"]
+        bz.check(self.lib.bz_fc_fused(C.byref(d), st or self._stream()))
+
+    def launches(self):
+        """[(name, callable(i, stream))] of one step's launches after the pooling kernel"""
+        if getattr(self, "_launches", None) is None:
+            self._launches = self._make_launches()
+        return self._launches
+
+    def _make_launches(self):
+        n = len(self.weights)
+        if self.fused_mlp is not None:
+            return [("bz_mlp_fused", self.mlp)]
+        if self.fused_head:
+            return [("bz_fc[%d]" % li, (lambda i, st=None, li=li: self.fc(i, li, st))) for li in range(n - 2)] + \
+                   [("bz_fc[%d+%d]" % (n - 2, n - 1), self.fc_with_head)]
+        return [("bz_fc[%d]" % li, (lambda i, st=None, li=li: self.fc(i, li, st))) for li in range(n)]
+
     def mlp(self, i, st=None):
         s = self.steps[i % self.n_batches]
         d = self.fused_mlp.desc
@@ -102,11 +134,8 @@ class CtrForward:
         if not self.fused_scan:
             self.scan(i, st)
         self.pool(i, st)
-        if self.fused_mlp is not None:
-            self.mlp(i, st)
-            return
-        for layer in range(len(self.weights)):
-            self.fc(i, layer, st)
+        for _, launch in self._launches or self.launches():
+            launch(i, st)
 
     def output(self, i):
         return self.steps[i % self.n_batches]["acts"][-1]
