@@ -118,7 +118,9 @@ typedef struct bz_embed_launch {
   int32_t variant;      /* 0 = generic kernel; else (table_dtype << 8) | lanes_per_row: the specialised
                            ksum/kavg kernel (all slots share dtype, row width class and are sum/avg) */
   int32_t fused_scan;   /* 1: no slot carries offsets; the pooling kernel scans the segments itself */
-  int32_t reserved_;
+  int32_t scan_first;   /* advice, set with fused_scan: 1 when so many workgroups per slot would each re-read the counts
+                           before their first sample (batch * workgroups * 2 bytes per slot) that scanning once into
+                           slot.offsets (bz_segments_to_offsets_slots) and planning again is the cheaper way */
 } bz_embed_launch;
 
 /*

@@ -249,3 +249,35 @@ def test_qed_builder_meta_quirk_and_errors(tmp_path):
     open(tmp_path / "meta2", "w").write("t1\nmissing\n")
     with pytest.raises(pb.BlazeError, match="can not open"):
         pb.build_qed(str(tmp_path), "meta2", out)
+
+
+def test_embedding_planner_geometry_and_scan_advice():
+    """bz_embed_plan runs on the host only (the pointers are never followed): workgroup counts per slot -- a lane group
+    per sample for ksum / kavg, per output position for kassign -- and the advice to scan the counts in a launch of
+    their own once the fused scan would re-read them too often (config 5's shape), not for config 2's."""
+    import ctypes as C
+    import blaze_hip as bz
+
+    def plan(n_slots, batch, dim, udf=bz.SUM, trunc=0, offsets=False, dtype=bz.F16):
+        slots = (bz.EmbedSlot * n_slots)()
+        for s in slots:
+            s.table, s.ids, s.values, s.segments, s.out = 0x10000, 0x20000, 0x30000, 0x40000, 0x50000
+            s.rows, s.dim, s.pitch = 1000, dim, (dim * 2 + 15) // 16 * 16
+            s.table_dtype, s.out_dtype, s.udf, s.batch = dtype, bz.F16, udf, batch
+            s.trunc_num, s.trunc_dir, s.out_stride = trunc, 0, dim * max(trunc, 1)
+            if offsets:
+                s.offsets = 0x60000
+        launch = bz.EmbedLaunch()
+        assert bz.lib().bz_embed_plan(slots, n_slots, C.byref(launch)) == 0, bz.lib().bz_last_error()
+        return slots, launch
+
+    slots, launch = plan(26, 2048, 32)           # config 2: dim 32 fp16 = 4 chunks -> 64 samples per workgroup
+    assert launch.total_wg == 26 * 32 and launch.wg_per_slot == 32 and launch.fused_scan == 1 and launch.scan_first == 0
+    assert launch.variant == (bz.F16 << 8) | 4
+    assert [s.wg_begin for s in slots][:3] == [0, 32, 64]
+    _, launch = plan(200, 8192, 64)              # config 5: 8 chunks -> 32 samples per workgroup, 256 workgroups a slot
+    assert launch.total_wg == 200 * 256 and launch.fused_scan == 1 and launch.scan_first == 1
+    _, launch = plan(200, 8192, 64, offsets=True)
+    assert launch.fused_scan == 0 and launch.scan_first == 0
+    slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 64 positions per workgroup
+    assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 64] * 3

@@ -429,3 +429,33 @@ def test_skinny_last_layer_rides_in_the_launch_before_it(pb, oracle):
         np.testing.assert_allclose(a, b, rtol=2e-3, atol=2e-3)
         np.testing.assert_allclose(a.sum(1), 1.0, rtol=2e-3)
     assert not np.array_equal(probs[1][0], probs[1][2])
+
+
+def test_embedding_operator_scans_first_when_the_batch_is_large(pb):
+    """A batch so large that every workgroup of the pooling kernel would re-read tens of thousands of counts: the
+    puller follows the planner's advice, scans the segments in a launch of their own and pools from the offsets.
+    Bit-identical block to the one-launch form of the kernel layer."""
+    import torch
+    import blaze_hip as bz
+    from ctr_model import build_manager, make_predictor
+    from synth import Config2
+    cfg = Config2(batch=70000, rows=5000, slots=2)
+    tables, mlp = cfg.tables(), cfg.mlp()
+    sparse, dense = cfg.batches(1)
+    pm, fgs = build_manager(cfg, tables, mlp, np.float16, expose_block=True)
+    p = make_predictor(pm, fgs, sparse[0], dense[0], np.float16)
+    p.forward()
+    got = p.output_asnumpy("block")
+    out = torch.zeros((cfg.batch, cfg.slots * cfg.dim), dtype=torch.float16, device="cuda")
+    items, keep = [], []
+    for s, (ids, vals, seg) in enumerate(sparse[0]):
+        t = [torch.from_numpy(x).cuda() for x in (ids, vals, seg)]
+        keep.append(t)
+        items.append(dict(table=bz.DeviceTable(tables[s]), ids=t[0], values=t[1], segments=t[2], out=out, col=s * cfg.dim, udf=bz.SUM))
+    auto = bz.EmbeddingPlan(items)
+    assert auto.launch.fused_scan == 0  # the same advice the puller received
+    bz.EmbeddingPlan(items, fused_scan=True).run()
+    torch.cuda.synchronize()
+    assert got.shape == (cfg.batch, cfg.slots * cfg.dim) and got.any()
+    assert np.array_equal(got.view(np.uint16), out.cpu().numpy().view(np.uint16))
+    assert p.output_asnumpy("prob").shape == (cfg.batch, 2)

@@ -39,7 +39,7 @@ class EmbedSlot(C.Structure):
 
 class EmbedLaunch(C.Structure):
     _fields_ = [("n_slots", C.c_int32), ("total_wg", C.c_int32), ("wg_per_slot", C.c_int32), ("variant", C.c_int32),
-                ("fused_scan", C.c_int32), ("reserved_", C.c_int32)]
+                ("fused_scan", C.c_int32), ("scan_first", C.c_int32)]
 
 
 class FcDesc(C.Structure):
@@ -243,10 +243,17 @@ class EmbeddingPlan:
     [B, stride]), col (element offset inside the block), udf, trunc_dir, trunc_num, dim}.
     """
 
-    def __init__(self, items, fused_scan=True):
-        """fused_scan: the pooling kernel derives offsets from the segments itself (one launch); otherwise
-        run() first scans every slot's segments into an offsets buffer (two launches)."""
+    def __init__(self, items, fused_scan=None):
+        """fused_scan: True = the pooling kernel derives offsets from the segments itself (one launch); False = run()
+        first scans every slot's segments into an offsets buffer (two launches); None = what bz_embed_plan advises
+        for these shapes (launch.scan_first)."""
         import torch
+        if fused_scan is None:
+            probe = EmbeddingPlan(items, fused_scan=True)
+            if not probe.launch.scan_first:
+                self.__dict__.update(probe.__dict__)
+                return
+            fused_scan = False
         self.items = items
         self.fused_scan = fused_scan
         n = len(items)

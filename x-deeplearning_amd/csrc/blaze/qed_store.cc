@@ -113,9 +113,12 @@ struct SlotCache : SparsePuller::DeviceCache {
   bz_embed_slot* dev = nullptr;
   size_t cap = 0;
   bz_embed_launch launch;
+  int64_t* offsets = nullptr;  // scratch for the separate scan, when the planner advises it
+  size_t offsets_cap = 0;      // in elements
   ~SlotCache() override {
     if (pinned) (void)hipHostFree(pinned);
     if (dev) (void)hipFree(dev);
+    if (offsets) (void)hipFree(offsets);
   }
 };
 
@@ -371,6 +374,22 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
   if (slots.empty()) return kOK;
   BZ_CHECK(bz_embed_plan(slots.data(), (int)slots.size(), &sc->launch));
   hipStream_t st = (hipStream_t)stream;
+  if (sc->launch.scan_first) {
+    // many workgroups per slot: scan every slot's counts once into scratch instead of once per workgroup
+    size_t need = 0;
+    for (const auto& s : slots) need += (size_t)s.batch + 1;
+    if (sc->offsets_cap < need) {
+      if (sc->offsets) HIP_CHECK(hipFree(sc->offsets));  // (its last reader finished: a predictor is waited for before its next pass)
+      HIP_CHECK(hipMalloc((void**)&sc->offsets, need * sizeof(int64_t)));
+      sc->offsets_cap = need;
+    }
+    size_t at = 0;
+    for (auto& s : slots) {
+      s.offsets = sc->offsets + at;
+      at += (size_t)s.batch + 1;
+    }
+    BZ_CHECK(bz_embed_plan(slots.data(), (int)slots.size(), &sc->launch));
+  }
   const size_t bytes = slots.size() * sizeof(bz_embed_slot);
   const bool changed = sc->host.size() != slots.size() || memcmp(sc->host.data(), slots.data(), bytes) != 0;
   if (changed) {
@@ -386,6 +405,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
     HIP_CHECK(hipMemcpyAsync(sc->dev, sc->pinned, bytes, hipMemcpyHostToDevice, st));
     sc->host = slots;
   }
+  if (!sc->launch.fused_scan) BZ_CHECK(bz_segments_to_offsets_slots(sc->dev, (int)slots.size(), st));
   BZ_CHECK(bz_embed_pool(sc->dev, &sc->launch, st));
   return kOK;
 }

@@ -366,6 +366,10 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
 // specialised ksum / kavg kernel: every slot has table dtype DT and LPR lanes per row
 // ---------------------------------------------------------------------------------------------
 constexpr int kBlockIds = 16;  // ids walked per step
+// Above this many bytes of repeated count reads a separate scan launch (about 15 us with its gap) is cheaper than the
+// fused one: config 5 (200 slots x 256 workgroups x batch 8192: 840 MB) pools in 262 + 16 us with offsets against
+// 427 us fused; config 4 (26 MB) and config 2 (3 MB) stay fused.
+constexpr int64_t kScanFirstBytes = 128ll << 20;
 
 template <int DT, int LPR>
 __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
@@ -592,7 +596,10 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
   launch->wg_per_slot = (uniform_wg && slots[0].wg_count > 0) ? slots[0].wg_count : 0;
   launch->variant = (uniform_shape && launch->wg_per_slot > 0) ? ((slots[0].table_dtype << 8) | lpr0) : 0;
   launch->fused_scan = any_offsets ? 0 : 1;
-  launch->reserved_ = 0;
+  // the fused scan reads, per workgroup, the counts before its first sample: on average batch/2 counts of 4 bytes
+  int64_t prefix_bytes = 0;
+  for (int i = 0; i < n_slots; ++i) prefix_bytes += (int64_t)slots[i].wg_count * slots[i].batch * 2;
+  launch->scan_first = (launch->fused_scan && prefix_bytes > kScanFirstBytes) ? 1 : 0;
   return BZ_OK;
 }
 
