@@ -273,7 +273,7 @@ typedef struct bz_mlp_desc {
 
 BZ_API int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream);
 
-/* number of elements of the fragment-major pack of a [k, n] weight (k is padded to a multiple of 128); 0 if n is not
+/* number of elements of the fragment-major pack of a [k, n] weight (k is padded to a multiple of 256); 0 if n is not
  * a multiple of 128 */
 BZ_API int64_t bz_mlp_packed_elems(int k, int n);
 

@@ -47,6 +47,9 @@ CASES = [
     (130, (264, 256, 512, 128, 8), ("relu", "dice", "prelu", "none")),  # four layers, widest hidden, head of 8
     (1, (64, 128, 2), ("sigmoid", "softmax")),
     (77, (1024, 512, 256), ("prelu", "dice")),                     # last layer wide
+    # from 64 workgroups of 64 rows on, the kernel takes 64 rows per workgroup (the cases above take 32)
+    (4133, (896, 512, 256, 2), ("prelu", "prelu", "softmax")),
+    (4096, (136, 256, 128), ("dice", "relu")),
 ]
 
 
@@ -104,5 +107,5 @@ def test_fused_mlp_refuses_shapes_it_cannot_run(bz):
     assert bz.lib().bz_mlp_fused(C.byref(d), None) != 0
     d.dtype, d.n_layers = bz.F32, 1
     assert bz.lib().bz_mlp_fused(C.byref(d), None) != 0 and b"fp16 and bf16 only" in bz.lib().bz_last_error()
-    assert bz.lib().bz_mlp_packed_elems(896, 512) == 896 * 512 and bz.lib().bz_mlp_packed_elems(72, 384) == 128 * 384
+    assert bz.lib().bz_mlp_packed_elems(896, 512) == 1024 * 512 and bz.lib().bz_mlp_packed_elems(72, 384) == 256 * 384
     assert bz.lib().bz_mlp_packed_elems(64, 100) == 0

@@ -31,11 +31,13 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int kBM = 64;              // rows per workgroup
+constexpr int kBM = 64;              // rows per workgroup (32 when that is what it takes to put 64 workgroups on the chip)
 constexpr int kBK = 64;              // K per step
 constexpr int kThreads = 256;
 constexpr int kAPitch = kBK * 2 + 16;  // staged input tile: 64 rows x 128 bytes, padded against bank conflicts
 constexpr float kDiceEps = 1e-8f;    // blaze/operator/common_helper.h:90
+// K steps of a packed weight: a whole number of the longest trip of the K loop (4 steps), zero filled beyond K
+__host__ __device__ constexpr int ktp_of(int k) { return (k + 4 * kBK - 1) / (4 * kBK) * 4; }
 
 struct LayerP {
   const char* w;  // wide layer: fragment-major pack; skinny layer: [n, ldw] K contiguous
@@ -126,22 +128,40 @@ __device__ __forceinline__ float act_apply(float v, const LayerP& L, float p0, f
   }
 }
 
-// One wide layer for this workgroup's 64 rows.  NB = 32-column blocks per wave (N = 128 * NB).
+// f(integral_constant<int, P>) for P = B .. E-1, unrolled at compile time (register sets are indexed by P)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>());
+    static_for<B + 1, E>(f);
+  }
+}
+
+// One wide layer for this workgroup's rows.  NB = 32-column blocks per wave (N = 128 * NB).
 // STREAM_A: operand A is staged from global memory tile by tile (layer 0); otherwise it is read in place from
 // the activation buffer `hin` (pitch hin_pitch bytes).  Output goes to `hout` (pitch N*2 + 16) in the tensor dtype.
-template <int DT, int NB, bool STREAM_A>
+template <int DT, int BM, int NB, bool STREAM_A>
 __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m0, char* lds, const char* hin, int hin_pitch,
                                            char* hout) {
+  constexpr int TMS = BM / 32;                // 32-row blocks per wave
+  constexpr int A_PER = BM * 8 / kThreads;    // 16-byte chunks of one input tile per thread
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int K = L.k;
-  const int KT2 = (K + 2 * kBK - 1) / (2 * kBK) * 2;  // steps, rounded up to even (the pack is zero filled there)
+  // DW register sets of weights: the loads of step s + DW - 1 are issued during step s.  With 32 rows per workgroup
+  // the accumulators leave room for four sets, i.e. three steps (about 1.5 us of MFMA work) of latency cover: the
+  // weights arrive from the last-level cache, not from L2, whenever a pooling kernel ran since their last use.
+  constexpr int DW = (BM == 32 && NB <= 2) ? 4 : 2;  // (four sets of a 4-block layer would not fit the register file)
+  constexpr int DA = DW;  // register sets of input tiles (STREAM_A)
+  const int KT = (K + kBK - 1) / kBK;
+  const int KTP = ktp_of(K);                 // steps in the pack (zero filled beyond K)
+  const int KTR = (KT + DW - 1) / DW * DW;   // steps run: a whole number of trips, <= KTP
   const int frag_row = lane & 31, frag_half = lane >> 5;
 
-  floatx16 acc[2][NB];
+  floatx16 acc[TMS][NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TMS; ++i)
 #pragma unroll
     for (int j = 0; j < NB; ++j)
 #pragma unroll
@@ -163,8 +183,8 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
   }
 
   // weight fragments of step s: NB*4 wave-wide 16-byte loads, each 1 KB contiguous
-  const char* wbase = L.w + ((int64_t)wave * KT2 * NB * 4) * 1024 + lane * 16;
-  uint4 rw[2][NB][4];
+  const char* wbase = L.w + ((int64_t)wave * KTP * NB * 4) * 1024 + lane * 16;
+  uint4 rw[DW][NB][4];
   auto gload_w = [&](int set, int s) {
     const char* p = wbase + (int64_t)s * (NB * 4 * 1024);
 #pragma unroll
@@ -173,11 +193,11 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
       for (int kk = 0; kk < 4; ++kk) rw[set][j][kk] = *(const uint4*)(p + (j * 4 + kk) * 1024);
   };
 
-  // input tile of step s (STREAM_A): 64 rows x 64 k = 512 16-byte chunks, two per thread
-  uint4 ra[2][2];
+  // input tile of step s (STREAM_A): BM rows x 64 k = BM * 8 16-byte chunks, A_PER per thread
+  uint4 ra[DA][A_PER];
   auto gload_a = [&](int set, int s) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < A_PER; ++i) {
       const int q = tid + i * kThreads;
       const int r = q >> 3, ch = q & 7;
       int m = m0 + r;
@@ -189,7 +209,7 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
   };
   auto lstore_a = [&](int set, int buf, int s) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < A_PER; ++i) {
       const int q = tid + i * kThreads;
       const int r = q >> 3, ch = q & 7;
       const uint32_t keep = (s * kBK + ch * 8) < K ? 0xffffffffu : 0u;
@@ -198,19 +218,20 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
       v.y &= keep;
       v.z &= keep;
       v.w &= keep;
-      *(uint4*)(lds + buf * (kBM * kAPitch) + r * kAPitch + ch * 16) = v;
+      *(uint4*)(lds + buf * (BM * kAPitch) + r * kAPitch + ch * 16) = v;
     }
   };
 
-  // One K step: the MFMAs of step s out of rw[set], with the weight loads of step `s_next` into rw[set ^ 1] dealt
-  // among them, one load per two MFMAs.  A wave issues in order, and a wave-wide 16-byte load occupies the CU's
+  // One K step: the MFMAs of step s out of rw[set], with the weight loads of step `s_next` into rw[set_next] dealt
+  // among them, one load per TMS MFMAs.  A wave issues in order, and a wave-wide 16-byte load occupies the CU's
   // address unit for about as long as the matrix unit needs for two MFMAs; a burst of loads in front of the MFMAs
   // would keep the matrix unit idle until the whole burst has been accepted.
-  auto compute = [&](int set, const char* a_base, int a_pitch, int s_next) {
+  auto compute = [&](auto set_c, auto next_c, const char* a_base, int a_pitch, int s_next) {
+    constexpr int set = decltype(set_c)::value, set_next = decltype(next_c)::value;
     // a_base points at this lane's fragment of k-substep 0 in M tile 0
-    uint4 fa[2][4];
+    uint4 fa[TMS][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TMS; ++i)
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) fa[i][kk] = *(const uint4*)(a_base + i * 32 * a_pitch + kk * 32);
     const char* pn = wbase + (int64_t)s_next * (NB * 4 * 1024);
@@ -218,44 +239,48 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
     for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
-        rw[set ^ 1][j][kk] = *(const uint4*)(pn + (j * 4 + kk) * 1024);
-        mma<DT>(fa[0][kk], rw[set][j][kk], acc[0][j]);
-        mma<DT>(fa[1][kk], rw[set][j][kk], acc[1][j]);
+        rw[set_next][j][kk] = *(const uint4*)(pn + (j * 4 + kk) * 1024);
+#pragma unroll
+        for (int i = 0; i < TMS; ++i) mma<DT>(fa[i][kk], rw[set][j][kk], acc[i][j]);
         __builtin_amdgcn_sched_barrier(0);  // pin this order: the scheduler would otherwise regroup loads and MFMAs
       }
     }
   };
+  // DW steps per trip, no conditionals inside: loads are issued in the order they are consumed, so the compiler's
+  // wait counts are exact.  Before step s: rw[s % DW .. (s + DW - 2) % DW] hold the weights of steps s .. s + DW - 2.
+#pragma unroll
+  for (int d = 0; d < DW - 1; ++d) gload_w(d, d < KTR ? d : KTR - 1);
 
   if constexpr (STREAM_A) {
-    // Two steps per trip, no conditionals inside: loads are issued in the order they are consumed, so the
-    // compiler's wait counts are exact.  Before step s: tile s is in LDS buffer s&1, registers ra[(s+1)&1] hold
-    // tile s+1, rw[s&1] holds the weights of step s.
-    gload_a(0, 0);
-    gload_a(1, 1);
-    gload_w(0, 0);
+    // Before step s: tile s is in LDS buffer s & 1, registers ra[(s + 1) % DA ..] hold tiles s + 1 .. s + DA - 1.
+#pragma unroll
+    for (int d = 0; d < DA; ++d) gload_a(d, d);
     lstore_a(0, 0, 0);
     __syncthreads();
-    for (int s0 = 0; s0 < KT2; s0 += 2) {
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
+    for (int s0 = 0; s0 < KTR; s0 += DW) {
+      static_for<0, DW>([&](auto p_c) {
+        constexpr int p = decltype(p_c)::value;
         const int s = s0 + p;
-        gload_a(p, s + 2);
+        gload_a(p % DA, s + DA);  // set p held tile s, which already sits in LDS
         __builtin_amdgcn_sched_barrier(0);
-        compute(p, lds + p * (kBM * kAPitch) + frag_row * kAPitch + frag_half * 16, kAPitch, s + 1 < KT2 ? s + 1 : s);
-        lstore_a(p ^ 1, p ^ 1, s + 1);
+        compute(std::integral_constant<int, p % DW>(), std::integral_constant<int, (p + DW - 1) % DW>(),
+                lds + (p & 1) * (BM * kAPitch) + frag_row * kAPitch + frag_half * 16, kAPitch,
+                s + DW - 1 < KTR ? s + DW - 1 : KTR - 1);
+        lstore_a((p + 1) % DA, (p + 1) & 1, s + 1);
         __syncthreads();
-      }
+      });
     }
   } else {
-    gload_w(0, 0);
-    for (int s0 = 0; s0 < KT2; s0 += 2) {
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
+    for (int s0 = 0; s0 < KTR; s0 += DW) {
+      static_for<0, DW>([&](auto p_c) {
+        constexpr int p = decltype(p_c)::value;
         const int s = s0 + p;
-        // beyond K the pack holds zeros, and the activation buffer's columns beyond K are never read because
-        // K of a later layer is the previous layer's N, a multiple of 128 = two steps
-        compute(p, hin + frag_row * hin_pitch + (s * kBK) * 2 + frag_half * 16, hin_pitch, s + 1 < KT2 ? s + 1 : s);
-      }
+        // steps beyond K multiply zero weights: they read step 0's (this row's own, finite) activations again rather
+        // than whatever lies behind the row in LDS
+        const int sa = s < KT ? s : 0;
+        compute(std::integral_constant<int, p % DW>(), std::integral_constant<int, (p + DW - 1) % DW>(),
+                hin + frag_row * hin_pitch + (sa * kBK) * 2 + frag_half * 16, hin_pitch, s + DW - 1 < KTR ? s + DW - 1 : KTR - 1);
+      });
     }
   }
 
@@ -270,7 +295,7 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
       const int n = wave * (NB * 32) + j * 32 + frag_row;
       const float bj = beta * cbias[j];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < TMS; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = i * 32 + 8 * (r >> 2) + 4 * frag_half + (r & 3);
@@ -299,39 +324,40 @@ __device__ __forceinline__ void wide_layer(const MlpP& P, const LayerP& L, int m
   }
 }
 
-template <int DT, bool STREAM_A>
+template <int DT, int BM, bool STREAM_A>
 __device__ __forceinline__ void wide_layer_any(const MlpP& P, const LayerP& L, int m0, char* lds, const char* hin, int hin_pitch,
                                                char* hout) {
   switch (L.n / 128) {
     case 1:
-      wide_layer<DT, 1, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
+      wide_layer<DT, BM, 1, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
       break;
     case 2:
-      wide_layer<DT, 2, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
+      wide_layer<DT, BM, 2, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
       break;
     case 3:
-      wide_layer<DT, 3, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
+      wide_layer<DT, BM, 3, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
       break;
     default:
-      wide_layer<DT, 4, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
+      wide_layer<DT, BM, 4, STREAM_A>(P, L, m0, lds, hin, hin_pitch, hout);
       break;
   }
 }
 
-// The head: N <= 8 outputs per row from the activations in LDS.  Four lanes share a row (a quarter of K each) and
-// reduce by shuffles; the logits go through a small LDS scratch, then one lane per row applies the activation /
+// The head: N <= 8 outputs per row from the activations in LDS.  kThreads / BM lanes share a row (an equal part of K
+// each) and reduce by shuffles; the logits go through a small LDS scratch, then one lane per row applies the activation /
 // softmax.  Loops over the outputs are kept rolled: this code runs once per launch, and unrolled it would cost more
 // in instruction fetch than it saves in issue slots.
-template <int DT>
+template <int DT, int BM>
 __device__ __forceinline__ void skinny_layer(const MlpP& P, const LayerP& L, int m0, const char* hin, int hin_pitch,
                                              const char* wl, const float* hp, float* logits) {
+  constexpr int LPR = kThreads / BM;  // lanes per row: 4 or 8
   const int tid = threadIdx.x;
-  const int row = tid >> 2, part = tid & 3;
+  const int row = tid / LPR, part = tid % LPR;
   const int K = L.k;  // a multiple of 128
   const int N = L.n;
   const int act = L.act;
   const float alpha = L.alpha, beta = L.bias ? L.beta : 0.f;
-  const int kq = K / 4;
+  const int kq = K / LPR;
   const char* ap = hin + row * hin_pitch + part * kq * 2;
   const char* wp = wl + part * kq * 2;
 #pragma unroll 1
@@ -348,13 +374,13 @@ __device__ __forceinline__ void skinny_layer(const MlpP& P, const LayerP& L, int
         dot += from_bits<DT>((uint16_t)(ar[e] >> 16)) * from_bits<DT>((uint16_t)(wr[e] >> 16));
       }
     }
-    dot += __shfl_xor(dot, 1, 64);
-    dot += __shfl_xor(dot, 2, 64);
+#pragma unroll
+    for (int d = 1; d < LPR; d <<= 1) dot += __shfl_xor(dot, d, 64);
     // hp: [bias | p0 | p1 | p2] x 8, staged in LDS at kernel start (zero where a parameter does not apply)
     if (part == 0) logits[row * BZ_MLP_MAX_HEAD + j] = alpha * dot + beta * hp[j];
   }
   __syncthreads();
-  if (tid >= kBM) return;
+  if (tid >= BM) return;
   float* lr = logits + tid * BZ_MLP_MAX_HEAD;
   const int m = m0 + tid;
   float mx = -INFINITY;
@@ -387,10 +413,10 @@ __device__ __forceinline__ void skinny_layer(const MlpP& P, const LayerP& L, int
   }
 }
 
-template <int DT>
+template <int DT, int BM>
 __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  const int m0 = blockIdx.x * kBM;
+  const int m0 = blockIdx.x * BM;
   const int n_wide = P.n_layers - P.skinny_last;
   const char* hin = nullptr;
   int hin_pitch = 0;
@@ -419,7 +445,7 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
   for (int li = 0; li < n_wide; ++li) {
     char* hout = lds + P.h_off[li & 1];
     if (li == 0) {
-      wide_layer_any<DT, true>(P, P.l[0], m0, lds, nullptr, 0, hout);
+      wide_layer_any<DT, BM, true>(P, P.l[0], m0, lds, nullptr, 0, hout);
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int q = threadIdx.x + i * kThreads;
@@ -427,20 +453,20 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
       }
       if (P.skinny_last && threadIdx.x < 32) *(float*)(lds + P.head_off + head_chunks * 16 + threadIdx.x * 4) = hp;
     } else {
-      wide_layer_any<DT, false>(P, P.l[li], m0, lds, hin, hin_pitch, hout);
+      wide_layer_any<DT, BM, false>(P, P.l[li], m0, lds, hin, hin_pitch, hout);
     }
     __syncthreads();
     hin = hout;
     hin_pitch = P.l[li].n * 2 + 16;
   }
   if (P.skinny_last) {
-    skinny_layer<DT>(P, P.l[P.n_layers - 1], m0, hin, hin_pitch, lds + P.head_off,
+    skinny_layer<DT, BM>(P, P.l[P.n_layers - 1], m0, hin, hin_pitch, lds + P.head_off,
                      (const float*)(lds + P.head_off + head_chunks * 16), (float*)lds);
   } else {
     // the last wide layer's tile: LDS -> global, 16 bytes per lane along rows
     const int n = P.l[n_wide - 1].n;
     const int cpr = n / 8;
-    for (int q = threadIdx.x; q < kBM * cpr; q += kThreads) {
+    for (int q = threadIdx.x; q < BM * cpr; q += kThreads) {
       const int r = q / cpr, ch = q - r * cpr;
       const int m = m0 + r;
       if (m < P.m) *(uint4*)(P.y + ((int64_t)m * P.ldy + ch * 8) * 2) = *(const uint4*)(hin + r * hin_pitch + ch * 16);
@@ -448,8 +474,8 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
   }
 }
 
-// [N, ldw] K-contiguous -> fragment major: element (((wave*KT2 + s)*NB + j)*4 + kk)*512 + lane*8 + e holds
-// W[n = wave*NB*32 + j*32 + lane%32][k = s*64 + kk*16 + (lane/32)*8 + e], zero beyond K.
+// [N, ldw] K-contiguous -> fragment major: element (((wave*KTP + s)*NB + j)*4 + kk)*512 + lane*8 + e holds
+// W[n = wave*NB*32 + j*32 + lane%32][k = s*64 + kk*16 + (lane/32)*8 + e], zero beyond K (KTP = ktp_of(K) steps).
 __global__ __launch_bounds__(256) void bz_mlp_pack_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst, int K, int N,
                                                           int64_t ldw, int KT2) {
   const int NB = N / 128;
@@ -477,13 +503,11 @@ __global__ __launch_bounds__(256) void bz_mlp_pack_kernel(const uint16_t* __rest
   }
 }
 
-int kt2_of(int k) { return (k + 2 * kBK - 1) / (2 * kBK) * 2; }
-
 }  // namespace
 
 extern "C" int64_t bz_mlp_packed_elems(int k, int n) {
   if (k <= 0 || n <= 0 || n % 128 != 0) return 0;
-  return (int64_t)kt2_of(k) * kBK * n;
+  return (int64_t)ktp_of(k) * kBK * n;
 }
 
 extern "C" int bz_mlp_pack_weight(const void* w_nk, int dtype, int k, int n, int64_t ldw, void* dst, bz_stream_t stream) {
@@ -493,7 +517,7 @@ extern "C" int bz_mlp_pack_weight(const void* w_nk, int dtype, int k, int n, int
              BZ_MLP_MAX_WIDTH);
   BZ_REQUIRE(ldw >= k, "bz_mlp_pack_weight: ldw=%lld < k=%d", (long long)ldw, k);
   BZ_REQUIRE((uintptr_t)dst % 16 == 0, "bz_mlp_pack_weight: dst must be 16-byte aligned");
-  const int KT2 = kt2_of(k);
+  const int KT2 = ktp_of(k);
   const int64_t groups = (int64_t)KT2 * kBK * n / 8;
   const int grid = (int)((groups + 255) / 256 < 4096 ? (groups + 255) / 256 : 4096);
   hipLaunchKernelGGL(bz_mlp_pack_kernel, dim3(grid), dim3(256), 0, bz::as_stream(stream), (const uint16_t*)w_nk, (uint16_t*)dst, k, n,
@@ -513,6 +537,9 @@ extern "C" int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream) {
   const int skinny_last = last.n <= BZ_MLP_MAX_HEAD ? 1 : 0;
   BZ_REQUIRE(d.n_layers - skinny_last >= 1, "bz_mlp_fused: needs at least one wide layer");
   MlpP P = {};
+  // 64 rows per workgroup amortise the weight stream over twice the MFMA work; below 64 such workgroups the chip is
+  // better used by twice as many of 32 rows (a batch of 2048: 64 workgroups instead of 32)
+  const int bm = (d.m + kBM - 1) / kBM >= 64 ? kBM : 32;
   int k_in = d.layer[0].k;
   BZ_REQUIRE(k_in > 0 && k_in % 8 == 0 && d.ldx >= k_in, "bz_mlp_fused: input width %d (multiple of 8, <= ldx)", k_in);
   int h_size[2] = {0, 0};
@@ -530,7 +557,7 @@ extern "C" int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream) {
       BZ_REQUIRE(s.n % 128 == 0 && s.n >= 128 && s.n <= BZ_MLP_MAX_WIDTH, "bz_mlp_fused: layer %d: n=%d (multiple of 128, <= %d)", i,
                  s.n, BZ_MLP_MAX_WIDTH);
       BZ_REQUIRE(s.act != BZ_ACT_SOFTMAX, "bz_mlp_fused: layer %d: softmax only on a head of at most %d outputs", i, BZ_MLP_MAX_HEAD);
-      const int bytes = kBM * (s.n * 2 + 16);
+      const int bytes = bm * (s.n * 2 + 16);
       h_size[i & 1] = bytes > h_size[i & 1] ? bytes : h_size[i & 1];
     }
     if (s.act == BZ_ACT_PRELU) BZ_REQUIRE(s.p0 != nullptr && (s.act_size == 1 || s.act_size == s.n), "bz_mlp_fused: layer %d: PReLU slope", i);
@@ -564,29 +591,36 @@ extern "C" int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream) {
   P.n_layers = d.n_layers;
   P.out_dtype = d.out_dtype;
   P.skinny_last = skinny_last;
-  const int a_bytes = 2 * kBM * kAPitch;
+  const int a_bytes = 2 * bm * kAPitch;
   P.h_off[0] = a_bytes;
   P.h_off[1] = a_bytes + h_size[0];
   P.head_off = a_bytes + h_size[0] + h_size[1];
   const int lds_bytes = P.head_off + (skinny_last ? last.n * last.k * 2 + 128 : 0);
   BZ_REQUIRE(lds_bytes <= 160 * 1024, "bz_mlp_fused: the stack needs %d bytes of LDS (limit 163840)", lds_bytes);
   hipStream_t st = bz::as_stream(stream);
-  const int grid = (d.m + kBM - 1) / kBM;
+  const int grid = (d.m + bm - 1) / bm;
+  // (the opt-in to more than 64 KB of dynamic LDS is per kernel function and per device)
+#define BZ_MLP_LAUNCH(DT, BM)                                                                                              \
+  do {                                                                                                                     \
+    static thread_local int set = 0;                                                                                       \
+    if (set < lds_bytes) {                                                                                                 \
+      BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_mlp_kernel<DT, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); \
+      set = 160 * 1024;                                                                                                    \
+    }                                                                                                                      \
+    hipLaunchKernelGGL((bz_mlp_kernel<DT, BM>), dim3(grid), dim3(kThreads), lds_bytes, st, P);                             \
+  } while (0)
   if (d.dtype == BZ_F16) {
-    static thread_local int set16 = 0;
-    if (set16 < lds_bytes) {
-      BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_mlp_kernel<BZ_F16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      set16 = 160 * 1024;
-    }
-    hipLaunchKernelGGL(bz_mlp_kernel<BZ_F16>, dim3(grid), dim3(kThreads), lds_bytes, st, P);
+    if (bm == kBM)
+      BZ_MLP_LAUNCH(BZ_F16, kBM);
+    else
+      BZ_MLP_LAUNCH(BZ_F16, 32);
   } else {
-    static thread_local int setb = 0;
-    if (setb < lds_bytes) {
-      BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_mlp_kernel<BZ_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      setb = 160 * 1024;
-    }
-    hipLaunchKernelGGL(bz_mlp_kernel<BZ_BF16>, dim3(grid), dim3(kThreads), lds_bytes, st, P);
+    if (bm == kBM)
+      BZ_MLP_LAUNCH(BZ_BF16, kBM);
+    else
+      BZ_MLP_LAUNCH(BZ_BF16, 32);
   }
+#undef BZ_MLP_LAUNCH
   BZ_LAUNCH_OK("bz_mlp_kernel");
   return BZ_OK;
 }
