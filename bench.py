@@ -173,13 +173,21 @@ def main():
         n_feed = max(fT, min(K, 400) // fT * fT)
         fbar = threading.Barrier(fT + 1)
 
+        # one Blaze_PredictorFeedMany call per step (79 inputs); the argument arrays are built once per batch
+        feeds = []
+        for b in range(fwd.n_batches):
+            items = []
+            for (fg, _, _), (ids, vals, seg) in zip(fgs, sparse[b]):
+                items += [(fg + ".ids", ids), (fg + ".values", vals), (fg + ".segments", seg)]
+            items.append(("dense", dense[b].astype(np.float16)))
+            feeds.append(predictors[b].feed_batch(items))
+
         def feed_worker(t):
-            from ctr_model import feed_inputs
             for i in range(t, n_feed + 2 * fT, fT):
                 if i == t + 2 * fT:
                     fbar.wait()
                 b = i % fwd.n_batches
-                feed_inputs(predictors[b], fgs, sparse[b], dense[b], np.float16)
+                predictors[b].feed_many(feeds[b])
                 predictors[b].forward()
                 predictors[b].output_asnumpy("prob")
 

@@ -111,6 +111,12 @@ BLAZE_API int Blaze_ConvertNetDef(const char* in, size_t len, int in_is_text, in
 BLAZE_API int Blaze_PredictorInputDevicePtr(PredictorHandle handle, const char* name, void** ptr);
 BLAZE_API int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char* name, void** ptr);
 
+/* Blaze_PredictorFeed for `count` inputs in one call (a sparse model has three inputs per feature group).  The shapes
+ * must have been set (ReshapeInput).  Inputs that are plain device tensors are staged side by side and travel in one
+ * transfer; the predictor's input tensors then view slices of that one device buffer. */
+BLAZE_API int Blaze_PredictorFeedMany(PredictorHandle handle, int count, const char* const* names, const void* const* data,
+                                      const size_t* lens);
+
 /* run Forward `count` times on the calling thread (benchmark loops without per-call host overhead) */
 BLAZE_API int Blaze_PredictorForwardN(PredictorHandle handle, int count);
 

@@ -459,3 +459,49 @@ def test_embedding_operator_scans_first_when_the_batch_is_large(pb):
     assert got.shape == (cfg.batch, cfg.slots * cfg.dim) and got.any()
     assert np.array_equal(got.view(np.uint16), out.cpu().numpy().view(np.uint16))
     assert p.output_asnumpy("prob").shape == (cfg.batch, 2)
+
+
+def test_feed_many_equals_feeding_one_by_one(pb):
+    """Blaze_PredictorFeedMany: all inputs in one call, the plain device inputs in one transfer through an arena the
+    input tensors then view.  Same probabilities as feeding one by one -- after the first call, after the batch grows
+    (the arena is outgrown), after it shrinks, and when single Feed calls follow on the re-viewed tensors; a wrong
+    length is refused with the reference's message."""
+    from ctr_model import build_manager, feed_inputs
+    from synth import Config2
+
+    def items_of(fgs, sp, dn):
+        items = []
+        for (fg, _, _), (ids, vals, seg) in zip(fgs, sp):
+            items += [(fg + ".ids", ids), (fg + ".values", vals), (fg + ".segments", seg)]
+        return items + [("dense", dn.astype(np.float16))]
+
+    base = Config2(batch=64, rows=3000, slots=26)
+    tables, mlp = base.tables(), base.mlp()
+    pm, fgs = build_manager(base, tables, mlp, np.float16)
+    one, many = pm.create_predictor(1, 0), pm.create_predictor(1, 0)
+    for batch, seed in ((64, 0), (300, 3), (17, 5), (300, 7)):
+        cfg = Config2(batch=batch, rows=3000, slots=26)
+        sparse, dense = cfg.batches(1, seed_offset=seed)
+        feed_inputs(one, fgs, sparse[0], dense[0], np.float16)
+        one.forward()
+        want = one.output_asnumpy("prob").copy()
+        items = items_of(fgs, sparse[0], dense[0])
+        for name, a in items:
+            many.reshape_input(name, a.shape)
+        fb = many.feed_batch(items)
+        for _ in range(2):  # the second call finds the tensors already viewing the arena
+            many.feed_many(fb)
+            many.forward()
+            np.testing.assert_array_equal(many.output_asnumpy("prob"), want)
+    # single feeds on tensors that view the arena
+    sparse, dense = Config2(batch=300, rows=3000, slots=26).batches(1, seed_offset=11)
+    feed_inputs(one, fgs, sparse[0], dense[0], np.float16)
+    one.forward()
+    many.feed("fg00.values", sparse[0][0][1])          # same shape as before: reshape + Feed
+    for name, a in items_of(fgs, sparse[0], dense[0]):
+        many.feed(name, a)
+    many.forward()
+    np.testing.assert_array_equal(many.output_asnumpy("prob"), one.output_asnumpy("prob"))
+    bad = many.feed_batch([("fg00.segments", np.zeros(7, np.int32))])
+    with pytest.raises(pb.BlazeError, match="FeedMany failed"):
+        many.feed_many(bad)

@@ -173,6 +173,14 @@ int Blaze_PredictorFeed(PredictorHandle handle, const char* name, void* data, in
   }
   return 0;
 }
+int Blaze_PredictorFeedMany(PredictorHandle handle, int count, const char* const* names, const void* const* data, const size_t* lens) {
+  auto* p = reinterpret_cast<Predictor*>(handle);
+  if (p == nullptr || count < 0 || (count > 0 && (names == nullptr || data == nullptr || lens == nullptr))) return -1;
+  for (int i = 0; i < count; ++i)
+    if (names[i] == nullptr || (data[i] == nullptr && lens[i] != 0)) return Fail("FeedMany: null name or data");
+  if (!p->FeedMany(count, names, data, lens)) return Fail("FeedMany failed");
+  return 0;
+}
 int Blaze_PredictorForward(PredictorHandle handle) {
   auto* p = reinterpret_cast<Predictor*>(handle);
   if (p == nullptr) return -1;

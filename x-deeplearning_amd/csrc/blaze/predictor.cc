@@ -30,6 +30,10 @@ Predictor::Predictor(std::shared_ptr<Net> net) : net_(net) {
 }
 
 Predictor::~Predictor() {
+  if (feed_done_) (void)hipEventSynchronize(feed_done_);
+  if (arena_host_) (void)hipHostFree(arena_host_);
+  if (arena_dev_) (void)hipFree(arena_dev_);
+  for (void* a : retired_arenas_) (void)hipFree(a);
   if (forward_done_) {
     (void)hipEventSynchronize(forward_done_);
     (void)hipEventDestroy(forward_done_);
@@ -120,6 +124,76 @@ bool Predictor::Feed(size_t idx, const void* data, size_t len) {
     }
   } catch (std::exception& e) {
     LOG_ERROR("feed failed: %s", e.what());
+    return false;
+  }
+  return true;
+}
+
+bool Predictor::FeedMany(int count, const char* const* names, const void* const* data, const size_t* lens) {
+  try {
+    struct Item {
+      int idx;
+      int arg;
+      size_t offset;
+    };
+    std::vector<Item> in_arena;
+    size_t total = 0;
+    const DeviceOption* dev = nullptr;
+    for (int i = 0; i < count; ++i) {
+      const int idx = InputName2Idx(names[i]);
+      if (idx < 0) {
+        LOG_ERROR("The name: %s is not The input of net", names[i]);
+        return false;
+      }
+      Blob* blob = external_input_blob_[idx];
+      const size_t need = blob->size() * DataTypeSize(blob->data_type());
+      if (lens[i] != need) {
+        LOG_ERROR("The len=%zu need size=%zu blob->size()=%zu", lens[i], need, (size_t)blob->size());
+        return false;
+      }
+      if (blob->device_type() != kHIP || blob->pitch() != 0) {
+        if (!Feed((size_t)idx, data[i], lens[i])) return false;
+        continue;
+      }
+      dev = &blob->device_option();
+      in_arena.push_back({idx, i, total});
+      total += (need + 255) / 256 * 256;  // every slice 256-byte aligned
+    }
+    if (in_arena.empty()) return true;
+    HIPContext ctx(*dev);
+    ctx.Activate();
+    hipStream_t st = ctx.hip_stream();
+    if (feed_done_ == nullptr) HIP_CHECK(hipEventCreateWithFlags(&feed_done_, hipEventDisableTiming));
+    if (any_feed_pending_) {  // the staging arena may still be read by the previous transfer
+      HIP_CHECK(hipEventSynchronize(feed_done_));
+      std::fill(feed_pending_.begin(), feed_pending_.end(), false);
+      any_feed_pending_ = false;
+    }
+    if (total > arena_cap_) {
+      if (arena_host_) HIP_CHECK(hipHostFree(arena_host_));
+      if (arena_dev_) retired_arenas_.push_back(arena_dev_);
+      arena_host_ = arena_dev_ = nullptr;
+      arena_cap_ = 0;
+      const size_t cap = total + total / 4;
+      HIP_CHECK(hipHostMalloc((void**)&arena_host_, cap, hipHostMallocDefault));
+      HIP_CHECK(hipMalloc((void**)&arena_dev_, cap));
+      arena_cap_ = cap;
+    }
+    for (const Item& it : in_arena) memcpy(arena_host_ + it.offset, data[it.arg], lens[it.arg]);
+    HIP_CHECK(hipMemcpyAsync(arena_dev_, arena_host_, total, hipMemcpyHostToDevice, st));
+    HIP_CHECK(hipEventRecord(feed_done_, st));
+    for (const Item& it : in_arena) {
+      Blob* blob = external_input_blob_[it.idx];
+      if (blob->data() != arena_dev_ + it.offset) {
+        const std::vector<TIndex> shape = blob->shape();
+        blob->RefReshape(shape, arena_dev_ + it.offset);
+      }
+      feed_pending_[it.idx] = true;
+    }
+    any_feed_pending_ = true;
+  } catch (std::exception& e) {
+    LOG_ERROR("feed failed: %s", e.what());
+    last_error_for_thread() = e.what();
     return false;
   }
   return true;

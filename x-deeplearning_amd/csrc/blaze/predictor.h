@@ -38,6 +38,11 @@ class Predictor {
   // copies len bytes in; len must equal size * sizeof(dtype) (predictor_impl.cc:110-138)
   bool Feed(const char* name, const void* data, size_t len);
   bool Feed(size_t idx, const void* data, size_t len);
+  // extension: feed `count` inputs at once.  Inputs that are plain device tensors travel in ONE transfer: they are
+  // staged side by side in a pinned arena, copied to a device arena of the same layout, and the input blobs become
+  // views of their slices (a model with 26 feature groups has 79 inputs; one queued copy instead of 79).  Other
+  // inputs (host tensors, inputs living inside a Concat's output) are fed one by one.
+  bool FeedMany(int count, const char* const* names, const void* const* data, const size_t* lens);
   size_t InputSize() const { return external_input_blob_.size(); }
   int InputDataType(const char* name) const;
   const std::vector<std::string>& ListInputName() const { return net_->external_input(); }
@@ -85,6 +90,10 @@ class Predictor {
   bool any_feed_pending_ = false;
   hipEvent_t feed_done_ = nullptr;  // recorded behind the last queued transfer; Forward's stream waits for it
                                     // (Feed and Forward may be called from different threads = different streams)
+  char* arena_host_ = nullptr;         // FeedMany's pinned staging arena and its device twin
+  char* arena_dev_ = nullptr;
+  size_t arena_cap_ = 0;
+  std::vector<void*> retired_arenas_;  // device arenas outgrown while blobs may still view them: freed with the predictor
   hipEvent_t forward_done_ = nullptr;  // recorded behind the last operator of a ForwardLaunch
   void* launched_on_ = nullptr;
   bool forward_in_flight_ = false;

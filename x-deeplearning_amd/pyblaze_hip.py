@@ -29,7 +29,7 @@ EXPORTS = [
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
     "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_PredictorForwardLaunch",
-    "Blaze_PredictorForwardWait"
+    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany"
 ]
 
 
@@ -85,6 +85,7 @@ def lib():
         l.Blaze_ServePoolSetDepth.argtypes = [vp, i]
         l.Blaze_PredictorForwardLaunch.argtypes = [vp]
         l.Blaze_PredictorForwardWait.argtypes = [vp]
+        l.Blaze_PredictorFeedMany.argtypes = [vp, i, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_size_t)]
         _lib = l
     return _lib
 
@@ -129,6 +130,21 @@ class Predictor(object):
         """Feed without reshaping (to exercise the length check of the ABI)."""
         data = np.ascontiguousarray(data)
         check_call(lib().Blaze_PredictorFeed(self.handle, name.encode(), data.ctypes.data_as(C.c_void_p), nbytes))
+
+    @staticmethod
+    def feed_batch(items):
+        """items: [(name, contiguous numpy array)] -> an object for feed_many (argument arrays built once; it keeps
+        the arrays alive)."""
+        arrays = [np.ascontiguousarray(a) for _, a in items]
+        n = len(items)
+        names = (C.c_char_p * n)(*[name.encode() for name, _ in items])
+        data = (C.c_void_p * n)(*[a.ctypes.data for a in arrays])
+        lens = (C.c_size_t * n)(*[a.nbytes for a in arrays])
+        return (n, names, data, lens, arrays)
+
+    def feed_many(self, batch):
+        """Feed every input of a feed_batch in one call; the shapes must already be set (a first feed() does)."""
+        check_call(lib().Blaze_PredictorFeedMany(self.handle, batch[0], batch[1], batch[2], batch[3]))
 
     def forward(self):
         check_call(lib().Blaze_PredictorForward(self.handle))
