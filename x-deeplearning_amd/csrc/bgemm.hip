@@ -38,29 +38,59 @@ __device__ __forceinline__ void st<__half>(__half* p, float v) {
   *p = __float2half_rn(v);
 }
 
-template <typename T>
+// One wave per batch item, one lane per output element; K is walked in steps of kUnroll with all loads of a step
+// issued before the first multiply-add (the products are still added in ascending k, so the sum is the plain loop's).
+constexpr int kUnroll = 16;
+
+template <typename T, bool TA, bool TB>
 __global__ __launch_bounds__(256) void bz_bgemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
-                                                       int64_t sa, int64_t sb, int64_t sc, int ta, int tb, int M, int N,
-                                                       int K, int batch, float alpha, float beta) {
+                                                       int64_t sa, int64_t sb, int64_t sc, int M, int N, int K, int batch,
+                                                       float alpha, float beta) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t item = (int64_t)blockIdx.x * 4 + wave;
   if (item >= batch) return;
   const T* a = A + sa * item;
   const T* b = B + sb * item;
   T* c = C + sc * item;
-  const int lda = ta ? M : K, ldb = tb ? K : N;
+  const int lda = TA ? M : K, ldb = TB ? K : N;
   for (int e = lane; e < M * N; e += 64) {
     const int m = e / N, n = e - m * N;
+    const T* ap = TA ? a + m : a + (int64_t)m * lda;  // element k: ap[k * (TA ? lda : 1)]
+    const T* bp = TB ? b + (int64_t)n * ldb : b + n;  // element k: bp[k * (TB ? 1 : ldb)]
+    const int64_t as = TA ? lda : 1, bs = TB ? 1 : ldb;
     float acc = 0.f;
-    for (int k = 0; k < K; ++k) {
-      const float av = ld<T>(ta ? a + (int64_t)k * lda + m : a + (int64_t)m * lda + k);
-      const float bv = ld<T>(tb ? b + (int64_t)n * ldb + k : b + (int64_t)k * ldb + n);
-      acc = fmaf(av, bv, acc);
+    for (int k0 = 0; k0 < K; k0 += kUnroll) {
+      float av[kUnroll], bv[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int k = k0 + u < K ? k0 + u : K - 1;  // clamped address; the product is skipped below
+        av[u] = ld<T>(ap + k * as);
+        bv[u] = ld<T>(bp + k * bs);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        if (k0 + u < K) acc = fmaf(av[u], bv[u], acc);
     }
     float v = alpha * acc;
     if (beta != 0.f) v += beta * ld<T>(c + e);  // beta == 0: C is not read (BLAS rule)
     st<T>(c + e, v);
   }
+}
+
+template <typename T>
+void launch_bgemm(const bz_bgemm_desc& d, int grid, hipStream_t s) {
+#define BZ_BGEMM(TA, TB)                                                                                                     \
+  hipLaunchKernelGGL((bz_bgemm_kernel<T, TA, TB>), dim3(grid), dim3(256), 0, s, (const T*)d.a, (const T*)d.b, (T*)d.c, d.stride_a, \
+                     d.stride_b, d.stride_c, d.m, d.n, d.k, d.batch, d.alpha, d.beta)
+  if (d.trans_a && d.trans_b)
+    BZ_BGEMM(true, true);
+  else if (d.trans_a)
+    BZ_BGEMM(true, false);
+  else if (d.trans_b)
+    BZ_BGEMM(false, true);
+  else
+    BZ_BGEMM(false, false);
+#undef BZ_BGEMM
 }
 
 }  // namespace
@@ -78,13 +108,9 @@ extern "C" int bz_gemm_strided_batched(const bz_bgemm_desc* desc, bz_stream_t st
   const int grid = (d.batch + 3) / 4;
   hipStream_t s = bz::as_stream(stream);
   if (d.dtype == BZ_F32)
-    hipLaunchKernelGGL(bz_bgemm_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)d.a, (const float*)d.b,
-                       (float*)d.c, d.stride_a, d.stride_b, d.stride_c, d.trans_a, d.trans_b, d.m, d.n, d.k, d.batch,
-                       d.alpha, d.beta);
+    launch_bgemm<float>(d, grid, s);
   else if (d.dtype == BZ_F16)
-    hipLaunchKernelGGL(bz_bgemm_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)d.a, (const __half*)d.b,
-                       (__half*)d.c, d.stride_a, d.stride_b, d.stride_c, d.trans_a, d.trans_b, d.m, d.n, d.k, d.batch,
-                       d.alpha, d.beta);
+    launch_bgemm<__half>(d, grid, s);
   else
     return bz::fail(BZ_ENOTSUP, "bz_gemm_strided_batched: unsupported dtype %d", d.dtype);
   BZ_LAUNCH_OK("bz_bgemm_kernel");
