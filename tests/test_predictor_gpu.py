@@ -396,6 +396,14 @@ def test_forward_in_two_halves_and_serve_pool_match_plain_forward(pb):
         del pool
     with pytest.raises(pb.BlazeError, match="multiple of the pool's threads"):
         pb.ServePool(3).run(preds, 4)
+    # the serving threads (and their streams) are gone; destroying predictors whose last passes ran on those streams
+    # must not leave a runtime error behind for the caller's next GPU call
+    import gc
+    preds[0].forward_launch()  # one pass still in flight at destruction, on this thread's stream
+    del preds, p
+    gc.collect()
+    assert float(torch.ones(4, device="cuda").sum()) == 4.0
+    torch.cuda.synchronize()
 
 
 def test_skinny_last_layer_rides_in_the_launch_before_it(pb, oracle):

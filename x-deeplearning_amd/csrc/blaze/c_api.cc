@@ -1,6 +1,8 @@
 // c_api.cc -- the Blaze_* C ABI over Predictor / PredictorManager (include/blaze_c_api.h).
 #include "blaze_c_api.h"
 
+#include <hip/hip_runtime.h>
+
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -86,6 +88,7 @@ int Blaze_PredictorManagerCreate(PredictorManagerHandle* handle) {
 }
 int Blaze_PredictorManagerDelete(PredictorManagerHandle handle) {
   delete reinterpret_cast<PredictorManager*>(handle);
+  (void)hipGetLastError();  // teardown ignores the runtime's return codes; none may surface in the caller's next call
   return 0;
 }
 int Blaze_PredictorManagerSetDataType(PredictorManagerHandle handle, int data_type) {
@@ -150,6 +153,7 @@ int Blaze_PredictorCreate(PredictorManagerHandle mgr, int device_type, int devic
 int Blaze_PredictorDelete(PredictorHandle handle) {
   if (handle == nullptr) return -1;
   delete reinterpret_cast<Predictor*>(handle);
+  (void)hipGetLastError();
   return 0;
 }
 
@@ -323,6 +327,7 @@ int Blaze_PredictorForwardWait(PredictorHandle handle) {
 }
 int Blaze_ServePoolDelete(ServePoolHandle handle) {
   delete reinterpret_cast<ServePool*>(handle);
+  (void)hipGetLastError();
   return 0;
 }
 

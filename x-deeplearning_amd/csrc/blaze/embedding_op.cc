@@ -147,20 +147,30 @@ class EmbeddingOp final : public Operator<Context> {
 
   void RunEmbedding(int key_type, int value_type, int num_type) {
     const size_t n_fg = config_.feature_group_config.size();
-    std::vector<store::SparsePullerInput> inputs(n_fg);
-    std::vector<store::SparsePullerOutput> outputs(n_fg);
+    // the puller structs live in the operator: their names, item lists and input positions are the same every run,
+    // only pointers and sizes change (a request-sized forward pass should not pay 2 allocations per feature group)
+    std::vector<store::SparsePullerInput>& inputs = puller_in_;
+    std::vector<store::SparsePullerOutput>& outputs = puller_out_;
+    if (inputs.size() != n_fg) {
+      inputs.assign(n_fg, store::SparsePullerInput());
+      outputs.assign(n_fg, store::SparsePullerOutput());
+      fg_input_.assign(n_fg, -1);
+      for (size_t i = 0; i < n_fg; ++i) {
+        inputs[i].name = config_.feature_group_config[i].table_name;
+        auto it = input_fg_idx_.find(config_.feature_group_config[i].feature_group);
+        if (it != input_fg_idx_.end()) fg_input_[i] = (int)it->second;
+      }
+    }
     for (size_t i = 0; i < n_fg; ++i) {
       const auto& fgc = config_.feature_group_config[i];
       auto& in = inputs[i];
       auto& out = outputs[i];
-      in.name = fgc.table_name;
-      auto it = input_fg_idx_.find(fgc.feature_group);
-      if (it == input_fg_idx_.end()) {
+      if (fg_input_[i] < 0) {
         // a configured group that is not fed: its items' columns stay zero (embedding_op.h:204-208)
         for (const auto& bi : fg_blocks_[i]) needs_zero_[bi.block_idx] = true;
         continue;
       }
-      const int idx = (int)it->second;
+      const int idx = fg_input_[i];
       Blob* ids = this->Input(idx * 3);
       Blob* values = this->Input(idx * 3 + 1);
       Blob* nums = this->Input(idx * 3 + 2);
@@ -208,6 +218,9 @@ class EmbeddingOp final : public Operator<Context> {
   std::unordered_map<std::string, size_t> input_fg_idx_;    // feature group -> input triple index
   std::unordered_map<std::string, size_t> fg_config_idx_;   // feature group -> config index
   std::vector<bool> needs_zero_;
+  std::vector<store::SparsePullerInput> puller_in_;    // reused every run (RunEmbedding)
+  std::vector<store::SparsePullerOutput> puller_out_;
+  std::vector<int> fg_input_;  // feature group -> position of its triple among the inputs, -1 = not fed
   std::unique_ptr<SparsePuller::DeviceCache> cache_;
   int out_dtype_ = 0;
 };

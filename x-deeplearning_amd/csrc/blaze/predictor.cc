@@ -30,18 +30,16 @@ Predictor::Predictor(std::shared_ptr<Net> net) : net_(net) {
 }
 
 Predictor::~Predictor() {
-  if (feed_done_) (void)hipEventSynchronize(feed_done_);
+  // Wait only for work that is still queued: an event that was already waited for may belong to a stream that died with
+  // its serving thread.  Nothing here may leave an error behind for the caller's next runtime call.
+  if (feed_done_ && any_feed_pending_) (void)hipEventSynchronize(feed_done_);
+  if (forward_done_ && forward_in_flight_) (void)hipEventSynchronize(forward_done_);
   if (arena_host_) (void)hipHostFree(arena_host_);
   if (arena_dev_) (void)hipFree(arena_dev_);
   for (void* a : retired_arenas_) (void)hipFree(a);
-  if (forward_done_) {
-    (void)hipEventSynchronize(forward_done_);
-    (void)hipEventDestroy(forward_done_);
-  }
-  if (feed_done_) {
-    (void)hipEventSynchronize(feed_done_);
-    (void)hipEventDestroy(feed_done_);
-  }
+  if (forward_done_) (void)hipEventDestroy(forward_done_);
+  if (feed_done_) (void)hipEventDestroy(feed_done_);
+  (void)hipGetLastError();
 }
 
 int Predictor::InputName2Idx(const char* name) const {

@@ -109,6 +109,7 @@ bool DenseKeys(const std::vector<uint64_t>& keys, std::vector<int64_t>* pos_of_k
 
 struct SlotCache : SparsePuller::DeviceCache {
   std::vector<bz_embed_slot> host;
+  std::vector<bz_embed_slot> scratch;  // this call's records, rebuilt in place every call
   bz_embed_slot* pinned = nullptr;
   bz_embed_slot* dev = nullptr;
   size_t cap = 0;
@@ -323,7 +324,8 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
   if (input.size() != output.size()) return kFail;
   if (!*cache) cache->reset(new SlotCache());
   SlotCache* sc = static_cast<SlotCache*>(cache->get());
-  std::vector<bz_embed_slot> slots;
+  std::vector<bz_embed_slot>& slots = sc->scratch;
+  slots.clear();
   for (size_t i = 0; i < input.size(); ++i) {
     const SparsePullerInput& in = input[i];
     const SparsePullerOutput& out = output[i];
