@@ -59,6 +59,7 @@ struct MlpP {
   int n_layers;
   int out_dtype;
   int skinny_last;
+  int warm_l2;   // touch the weights ahead of use (see the kernel)
   int h_off[2];  // byte offsets of the two activation buffers in LDS
   int head_off;  // byte offset of the head layer's weights in LDS ([n][k], staged once per workgroup)
   LayerP l[BZ_MLP_MAX_LAYERS];
@@ -420,6 +421,32 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
   const int n_wide = P.n_layers - P.skinny_last;
   const char* hin = nullptr;
   int hin_pitch = 0;
+  // Warm-up of the L2: every workgroup streams ALL the weights, so the workgroups that share an XCD (the hardware
+  // deals workgroup ids round robin over the 8 XCDs) would each miss on the same lines one K step after the other when
+  // the weights are not in that XCD's L2 -- which is the normal case after a pooling kernel.  Instead each of them
+  // first touches its own eighth of every layer's pack, one dword per 128-byte line, so that between them the whole
+  // pack is on its way before the K loop starts.  The values are folded into `warm`, which is consumed (by a store
+  // that never happens) after the first layer.
+  uint32_t warm = 0;
+  if (P.warm_l2) {
+    const int slice = (blockIdx.x / 8) & 7;
+    for (int li = 0; li < n_wide; ++li) {
+      const int64_t bytes = (int64_t)ktp_of(P.l[li].k) * kBK * P.l[li].n * 2;
+      const int64_t lo = bytes * slice / 8 / 128 * 128, hi = bytes * (slice + 1) / 8;
+      // eight loads in flight per thread and trip (one trip covers 256 KB of a slice: every layer up to 512 x 2048)
+#pragma unroll 1
+      for (int64_t base = lo + (int64_t)threadIdx.x * 128; base < hi; base += (int64_t)8 * kThreads * 128) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int64_t off = base + (int64_t)u * kThreads * 128;
+          v[u] = off < hi ? *(const uint32_t*)(P.l[li].w + off) : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) warm ^= v[u];
+      }
+    }
+  }
   // the head's weights (at most 8 x 512 elements) are requested now and parked in LDS after the first layer, so
   // that the head finds them on chip instead of paying a round trip to L2 per chunk
   uint4 hw[2] = {};
@@ -452,6 +479,7 @@ __global__ __launch_bounds__(kThreads, 1) void bz_mlp_kernel(MlpP P) {
         if (q < head_chunks) *(uint4*)(lds + P.head_off + q * 16) = hw[i];
       }
       if (P.skinny_last && threadIdx.x < 32) *(float*)(lds + P.head_off + head_chunks * 16 + threadIdx.x * 4) = hp;
+      if (warm == 0x9e3779b9u && P.m < 0) *(uint32_t*)P.y = warm;  // (m is never negative)
     } else {
       wide_layer_any<DT, BM, false>(P, P.l[li], m0, lds, hin, hin_pitch, hout);
     }
@@ -591,6 +619,8 @@ extern "C" int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream) {
   P.n_layers = d.n_layers;
   P.out_dtype = d.out_dtype;
   P.skinny_last = skinny_last;
+  // with fewer workgroups than two per XCD there is nobody to share the warm-up with
+  P.warm_l2 = (d.m + bm - 1) / bm >= 16 ? 1 : 0;
   const int a_bytes = 2 * bm * kAPitch;
   P.h_off[0] = a_bytes;
   P.h_off[1] = a_bytes + h_size[0];
