@@ -94,7 +94,17 @@ __global__ __launch_bounds__(256) void bz_softmax_kernel(const T* __restrict__ x
   for (int64_t c = lane; c < cols; c += 64) stf<T>(yr + c, expf(ldf<T>(xr + c) - mx) / sum);
 }
 
-// side-by-side concatenation: blockIdx.y picks the piece, threads copy 16 bytes each when every address allows
+// side-by-side concatenation: blockIdx.y picks the piece; a thread copies the widest power-of-two granule (16 ... 1
+// bytes) that the piece's addresses, width and both pitches are all multiples of
+template <typename G>
+__device__ __forceinline__ void concat_piece(const char* src, char* dst, int64_t width, int64_t sp, int64_t dp, int64_t rows) {
+  const int64_t cpr = width / (int64_t)sizeof(G), total = cpr * rows;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / cpr, c = i - r * cpr;
+    *(G*)(dst + r * dp + c * sizeof(G)) = *(const G*)(src + r * sp + c * sizeof(G));
+  }
+}
+
 __global__ __launch_bounds__(256) void bz_concat_kernel(bz_concat_desc d) {
   const int k = blockIdx.y;
   const char* src = (const char*)d.src[k];
@@ -103,21 +113,17 @@ __global__ __launch_bounds__(256) void bz_concat_kernel(bz_concat_desc d) {
   for (int i = 0; i < k; ++i) col += d.width[i];
   char* dst = (char*)d.dst + col;
   const int64_t sp = d.src_pitch[k];
-  const bool vec = ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0) && (width % 16 == 0) && (d.dst_pitch % 16 == 0) &&
-                   (sp % 16 == 0);
-  if (vec) {
-    const int64_t cpr = width / 16, total = cpr * d.rows;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-      const int64_t r = i / cpr, c = i - r * cpr;
-      *(uint4*)(dst + r * d.dst_pitch + c * 16) = *(const uint4*)(src + r * sp + c * 16);
-    }
-  } else {
-    const int64_t total = width * d.rows;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-      const int64_t r = i / width, c = i - r * width;
-      dst[r * d.dst_pitch + c] = src[r * sp + c];
-    }
-  }
+  const uint64_t all = (uint64_t)(uintptr_t)src | (uint64_t)(uintptr_t)dst | (uint64_t)width | (uint64_t)d.dst_pitch | (uint64_t)sp;
+  if (all % 16 == 0)
+    concat_piece<uint4>(src, dst, width, sp, d.dst_pitch, d.rows);
+  else if (all % 8 == 0)
+    concat_piece<uint2>(src, dst, width, sp, d.dst_pitch, d.rows);
+  else if (all % 4 == 0)
+    concat_piece<uint32_t>(src, dst, width, sp, d.dst_pitch, d.rows);
+  else if (all % 2 == 0)
+    concat_piece<uint16_t>(src, dst, width, sp, d.dst_pitch, d.rows);
+  else
+    concat_piece<uint8_t>(src, dst, width, sp, d.dst_pitch, d.rows);
 }
 
 }  // namespace
