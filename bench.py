@@ -270,8 +270,19 @@ def main():
         for t in ths:
             t.join()
         c1 = time.perf_counter()
+        s0 = time.perf_counter()  # ... and the same port on one core alone
+        for j in range(per_thread):
+            oracle_forward(orc, cfg, tabs, mlp_np, sparse[j % len(sparse)], dense[j % len(sparse)])
+        s1 = time.perf_counter()
+        model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), "")
+        except OSError:
+            pass
         cpu = {"value": round(cfg.batch * threads * per_thread / (c1 - c0), 1), "unit": "samples/s", "cores": threads,
-               "kind": "port",
+               "kind": "port", "value_1_core": round(cfg.batch * per_thread / (s1 - s0), 1), "host_cpus": os.cpu_count(),
+               "cpu_model": model,
                "sample": "%d batches of %d (one per thread, one single-threaded predictor per core), fp32 oracle: "
                          "hash-free row lookup, ksum, textbook sgemm + separate PReLU pass, softmax" % (
                              threads * per_thread, cfg.batch)}
