@@ -513,3 +513,52 @@ def test_feed_many_equals_feeding_one_by_one(pb):
     bad = many.feed_batch([("fg00.segments", np.zeros(7, np.int32))])
     with pytest.raises(pb.BlazeError, match="FeedMany failed"):
         many.feed_many(bad)
+
+
+def test_threads_feeding_alternating_requests_get_their_own_results(pb):
+    """Four serving threads, a predictor each, every step another request (two request sizes alternate, so the feed
+    arena's layout, the tensors' addresses and the pooling kernel's slot records change every step) through
+    FeedMany + Forward + Output: every result equals the one computed for that request alone."""
+    import threading
+    from ctr_model import build_manager, feed_inputs
+    from synth import Config2
+    base = Config2(batch=128, rows=3000, slots=26)
+    tables, mlp = base.tables(), base.mlp()
+    pm, fgs = build_manager(base, tables, mlp, np.float16)
+    requests = []
+    ref = pm.create_predictor(1, 0)
+    for batch, seed in ((128, 1), (61, 2), (128, 3), (200, 4)):
+        cfg = Config2(batch=batch, rows=3000, slots=26)
+        sparse, dense = cfg.batches(1, seed_offset=seed)
+        feed_inputs(ref, fgs, sparse[0], dense[0], np.float16)
+        ref.forward()
+        items = []
+        for (fg, _, _), (ids, vals, seg) in zip(fgs, sparse[0]):
+            items += [(fg + ".ids", ids), (fg + ".values", vals), (fg + ".segments", seg)]
+        items.append(("dense", dense[0].astype(np.float16)))
+        requests.append((items, ref.output_asnumpy("prob").copy()))
+    errors = []
+
+    def worker(t):
+        try:
+            p = pm.create_predictor(1, 0)
+            batches = [p.feed_batch(items) for items, _ in requests]
+            for i in range(60):
+                r = (i + t) % len(requests)
+                for name, a in requests[r][0]:
+                    p.reshape_input(name, a.shape)
+                p.feed_many(batches[r])
+                p.forward()
+                got = p.output_asnumpy("prob")
+                if not np.array_equal(got, requests[r][1]):
+                    errors.append("thread %d step %d request %d: max diff %g" % (t, i, r, np.abs(got.astype(np.float32) - requests[r][1].astype(np.float32)).max()))
+                    return
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (t, e))
+
+    threads = [threading.Thread(target=worker, args=(t, )) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
