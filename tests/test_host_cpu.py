@@ -281,3 +281,21 @@ def test_embedding_planner_geometry_and_scan_advice():
     assert launch.fused_scan == 0 and launch.scan_first == 0
     slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 64 positions per workgroup
     assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 64] * 3
+
+
+def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle):
+    """bench.py times the oracle with the products handed to the BLAS numpy links (as the reference hands them to
+    MKL, math/gemm.cc:13-27).  That variant must be the same computation: on a scaled-down config 2 it agrees with
+    the k-ascending sums the parity tests use to fp32 summation-order noise (rel 1e-5)."""
+    from pipeline import oracle_forward
+    from synth import Config2
+    cfg = Config2(batch=96, rows=5000, slots=5)
+    tables = cfg.tables(device="cpu")
+    mlp_np = [(w.numpy(), b.numpy(), s.numpy()) for (w, b, s) in cfg.mlp(device="cpu")]
+    sparse, dense = cfg.batches(1)
+    tabs = [oracle.Table(t.numpy()) for t in tables]
+    pooled, want = oracle_forward(oracle, cfg, tabs, mlp_np, sparse[0], dense[0])
+    pooled_b, got = oracle_forward(oracle, cfg, tabs, mlp_np, sparse[0], dense[0], blas=True)
+    np.testing.assert_array_equal(pooled_b, pooled)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-7)
+    assert got.shape == (96, 2) and np.allclose(got.sum(1), 1.0, atol=1e-6)

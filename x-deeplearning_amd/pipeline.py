@@ -154,9 +154,12 @@ class CtrForward:
         return [2.0 * self.cfg.batch * L[i] * L[i + 1] for i in range(len(L) - 1)]
 
 
-def oracle_forward(oracle, cfg, tables_np, mlp_np, sparse, dense, in_round=None):
+def oracle_forward(oracle, cfg, tables_np, mlp_np, sparse, dense, in_round=None, blas=False):
     """The same forward on the CPU oracle (fp32 path fed the kernel's rounded inputs).  tables_np: list of
-    oracle.Table; mlp_np: [(W [K,N] fp32, b, slope)].  Returns (pooled [B, in_dim] fp32, probs [B, 2])."""
+    oracle.Table; mlp_np: [(W [K,N] fp32, b, slope)].  Returns (pooled [B, in_dim] fp32, probs [B, 2]).
+    blas=True hands the products to the optimised sgemm numpy links (the reference calls MKL's cblas_sgemm there,
+    math/gemm.cc:13-27) for timing a CPU baseline; its summation order is the library's, so parity tests keep the
+    default k-ascending sums."""
     B = cfg.batch
     x = np.zeros((B, cfg.in_dim), np.float32)
     x[:, :cfg.dense] = dense if in_round is None else in_round(dense)
@@ -166,6 +169,11 @@ def oracle_forward(oracle, cfg, tables_np, mlp_np, sparse, dense, in_round=None)
     pooled = h.copy()
     n = len(mlp_np)
     for li, (w, b, slope) in enumerate(mlp_np):
+        if blas:
+            y = np.matmul(h, w)
+            y += b  # the Gemm operator's bias broadcast
+            h = oracle.softmax(y, 1) if li == n - 1 else oracle.prelu(y, slope)
+            continue
         wt = np.ascontiguousarray(w.T)  # [N,K] + transB: same k-ascending sums, contiguous inner loop
         if li == n - 1:
             h = oracle.fc(h, wt, b, act="softmax", transb=True)
