@@ -365,10 +365,10 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
 // ---------------------------------------------------------------------------------------------
 // specialised ksum / kavg kernel: every slot has table dtype DT and LPR lanes per row
 // ---------------------------------------------------------------------------------------------
-constexpr int kBlockIds = 16;  // ids walked per step
+constexpr int kBlockIds = 4;  // ids walked per step (measured at 2, 4, 8, 16: 4 is best or equal on segments of 1-4, 8 and 20 ids)
 // Above this many bytes of repeated count reads a separate scan launch (about 15 us with its gap) is cheaper than the
-// fused one: config 5 (200 slots x 256 workgroups x batch 8192: 840 MB) pools in 262 + 16 us with offsets against
-// 427 us fused; config 4 (26 MB) and config 2 (3 MB) stay fused.
+// fused one: config 5 (200 slots x 256 workgroups x batch 8192: 840 MB) pools in 155 + 16 us with offsets against
+// 261 us fused; config 4 (26 MB) and config 2 (3 MB) stay fused.
 constexpr int64_t kScanFirstBytes = 128ll << 20;
 
 template <int DT, int LPR>
