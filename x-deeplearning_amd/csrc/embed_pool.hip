@@ -35,7 +35,7 @@
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 8;
+constexpr int kUnroll = 4;  // rows in flight per lane group in the generic kernel (8 held 118 VGPRs and was no faster)
 
 // ---------------------------------------------------------------------------------------------
 // segments -> offsets (exclusive scan), one workgroup per array
