@@ -697,7 +697,9 @@ int dispatch_head(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
   }
   if (d.n <= 128) return launch_mfma<DT, OutT, 32, 128, BK, 1, 4, 4, true, true>(d, ep, true, true, st);
   // eight waves: with one workgroup per 32 rows only M / 32 CUs work, and each has 288 KB of operands to pull in
-  return launch_mfma<DT, OutT, 32, 256, BK, 1, 8, 4, true, true>(d, ep, true, true, st);
+  // (two K tiles in flight: with eight waves taking turns that hides the loads, and it is faster than four both alone,
+  // 10.5 against 11.3 us on config 2's 512 -> 256 -> 2, and next to other kernels)
+  return launch_mfma<DT, OutT, 32, 256, BK, 1, 8, 2, true, true>(d, ep, true, true, st);
 }
 
 template <int DT, typename OutT>
@@ -726,11 +728,9 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
   if (d.n > 64 && wg128 >= 512) return launch_mfma<DT, OutT, 128, 128, BK, 2, 2, 3, true>(d, ep, vec_a, vec_w, st);
   if (d.n > 64 && wg64x128 >= 512) return launch_mfma<DT, OutT, 64, 128, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
   if (wg64 >= 256) {
-    // K tiles in flight: the loop exposes one round trip per D tiles, so seven instead of four when that saves a trip
-    // without padding the loop by more than two empty tiles (config 2's 896-deep layer: 14 tiles = 2 x 7, 10.1 -> 9.2 us)
-    const int kt = (d.k + BK - 1) / BK;
-    const int trips4 = (kt + 3) / 4, trips7 = (kt + 6) / 7;
-    if (trips7 < trips4 && trips7 * 7 - kt <= 2) return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 7, true>(d, ep, vec_a, vec_w, st);
+    // Four K tiles in flight (120 VGPRs, three waves per SIMD).  Seven save a round trip on config 2's 896-deep layer
+    // when the kernel runs alone (9.2 against 9.8 us) but hold 182 VGPRs, and next to the kernels of other serving
+    // threads the leaner one wins: 127.5 against 121 M samples/s at the same forward latency.
     return launch_mfma<DT, OutT, 64, 64, BK, 2, 2, 4, true>(d, ep, vec_a, vec_w, st);
   }
   return launch_mfma<DT, OutT, 32, 64, BK, 1, 2, 4, true>(d, ep, vec_a, vec_w, st);
