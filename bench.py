@@ -25,7 +25,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
 # HBM-side bytes per launch of the pooling kernel on this exact workload (default seed, pool of 32 batches), from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, averaged over 1704 dispatches) scaled by what the same
 # counters read for a plain 256 MiB copy (`--calibrate-copy`: FETCH_SIZE reads 0.5 of the bytes, WRITE_SIZE all of them):
-# fetch 11984.89 KiB x 2.0 + write 3329.15 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
+# fetch 11958.20 KiB x 2.0 + write 3328.52 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
 POOL_TRAFFIC_BYTES = int((11958.20 * 2.0 + 3328.52) * 1024)
 
 
@@ -39,6 +39,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
                          "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
+    ap.add_argument("--gather-probe", action="store_true",
+                    help="only measure what the memory system gives random 64-byte row gathers (a kernel that does nothing else, "
+                         "the pooling kernel on uniform ids with 64-id segments, a row copy through the kassign path) and exit")
     ap.add_argument("--threads", type=int, default=8,
                     help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
                          "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
@@ -75,6 +78,63 @@ def main():
         assert bool((dst == 1).all())
         print(json.dumps({"calibration": "bz_concat_kernel", "launches": 5, "bytes_read_per_launch": rows * width,
                           "bytes_written_per_launch": rows * width}))
+        return
+    if args.gather_probe:
+        def ev_time(fn, reps=20):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / reps  # us
+        g = torch.Generator(device="cuda").manual_seed(1)
+        res = {"probe": "random gathers of 64-byte rows", "device": arch}
+        # (o) nothing but the access pattern: four-lane groups read hashed 64-byte rows of a 2 GiB region
+        region = torch.ones(2 << 30, dtype=torch.uint8, device="cuda")
+        sink = torch.empty((1 << 20) * 64, dtype=torch.uint8, device="cuda")
+        pure = {}
+        for groups, per in ((1 << 20, 8), (1 << 20, 16), (425984, 1), (106496, 4), (53248, 8)):
+            seed = [0]
+            def launch():
+                seed[0] += 7919
+                bz.check(bz.lib().bz_probe_gather64(region.data_ptr(), region.numel(), sink.data_ptr(), groups, per, seed[0], None))
+            us = ev_time(launch, 50)
+            pure["%d groups x %d rows" % (groups, per)] = {"us": round(us, 2), "row_read_GB/s": round(groups * per * 64 / us / 1e3, 1)}
+        res["pure_gather_2GiB_region"] = pure
+        del region, sink
+        # (i) the pooling kernel where the dependent chain of a launch is amortised and no row is hot:
+        # config 2's tables (26 x 64 MB), uniform ids, every segment 64 ids long
+        cfg = Config2()
+        tables = [bz.DeviceTable(t) for t in cfg.tables()]
+        L = 64
+        out = torch.zeros((cfg.batch, cfg.slots * cfg.dim), dtype=torch.float16, device="cuda")
+        items = []
+        for s_ in range(cfg.slots):
+            ids = torch.randint(0, cfg.rows, (cfg.batch * L, ), device="cuda", generator=g)
+            items.append(dict(table=tables[s_], ids=ids, values=torch.ones(cfg.batch * L, device="cuda"),
+                              segments=torch.full((cfg.batch, ), L, dtype=torch.int32, device="cuda"), out=out,
+                              col=s_ * cfg.dim, udf=bz.SUM))
+        plan = bz.EmbeddingPlan(items, fused_scan=True)
+        us = ev_time(plan.pool)
+        nnz = cfg.slots * cfg.batch * L
+        alg = nnz * (64 + 12) + cfg.slots * cfg.batch * 4 + out.numel() * 2
+        res["pool_kernel_uniform_ids_64_per_segment"] = {"ids": nnz, "us": round(us, 1),
+                                                         "row_read_GB/s": round(nnz * 64 / us / 1e3, 1),
+                                                         "algorithmic_GB/s": round(alg / us / 1e3, 1)}
+        # (ii) a pure gather through the kassign path: every id's row is copied to its own output position, one lane group
+        # per position, so nothing is summed and nothing waits on a neighbour (row read + row written per id)
+        wide = torch.zeros((cfg.batch, cfg.slots * L * cfg.dim), dtype=torch.float16, device="cuda")
+        for s_, it in enumerate(items):
+            it.update(out=wide, col=s_ * L * cfg.dim, udf=bz.ASSIGN, trunc_num=L, trunc_dir=bz.ORDER)
+        plan = bz.EmbeddingPlan(items, fused_scan=True)
+        us = ev_time(plan.pool)
+        res["kassign_copy_of_the_same_rows"] = {"ids": nnz, "us": round(us, 1), "row_read_GB/s": round(nnz * 64 / us / 1e3, 1),
+                                                "read_plus_written_GB/s": round(nnz * (64 + 12 + 64) / us / 1e3, 1)}
+        print(json.dumps(res))
         return
     cfg = Config2()
     tables = cfg.tables()

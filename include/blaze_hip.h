@@ -158,6 +158,18 @@ BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* 
 /* name of the pooling kernel as profilers report it (for tooling) */
 BZ_API const char* bz_embed_pool_kernel_name(void);
 
+/*
+ * Measurement aid, no counterpart in the reference: a pure random gather of 64-byte rows, the access pattern of
+ * the pooling kernel with everything else taken away.  `groups` four-lane groups each read `rows_per_group`
+ * (1, 4, 8 or 16) rows at hashed positions of `region` (region_bytes >= 64, 16-byte aligned; all loads of a group are
+ * issued before the first is used), fold them and write one 64-byte row to sink[group].  The caller times the launch;
+ * bytes read = groups * rows_per_group * 64.  Row of load r of group g, 32-bit arithmetic: h = (g * rows_per_group + r) *
+ * 2654435761 + seed; h ^= h >> 15; h *= 2246822519; h ^= h >> 13; row = (h * rows) >> 32 with rows = region_bytes / 64.
+ * Fold: of each 16-byte quarter row, words 0 and 2 are summed and words 1 and 3 xor-ed over the group's rows.
+ */
+BZ_API int bz_probe_gather64(const void* region, int64_t region_bytes, void* sink, int64_t groups, int rows_per_group,
+                             uint32_t seed, bz_stream_t stream);
+
 /* ------------------------------------------------------------------------- */
 /* Dense                                                                      */
 /* ------------------------------------------------------------------------- */

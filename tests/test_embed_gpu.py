@@ -295,3 +295,35 @@ def test_config2_full_size(bz, oracle):
     assert np.array_equal(out.cpu().numpy(), got)
     for s in range(slots):
         assert np.array_equal(plan2.offsets[s].cpu().numpy(), oracle.segments_to_offsets(inputs[s][2]))
+
+
+@pytest.mark.parametrize("per", [1, 4, 8, 16])
+def test_gather_probe_reads_the_rows_it_claims(bz, per):
+    """bz_probe_gather64 (the measurement aid behind the gather-ceiling figure) really reads rows_per_group distinct
+    hashed 64-byte rows per group: with row r holding the words 16r .. 16r+15, the folded row a group writes equals
+    the sums / xors over exactly the rows the documented hash picks.  Integer work: bit-exact."""
+    import torch
+    rows, groups, seed = 1000, 777, 12345
+    region = np.arange(rows * 16, dtype=np.uint32).reshape(rows, 16)
+    d_region = _dev(region)
+    sink = torch.zeros((groups, 16), dtype=torch.int32, device="cuda")
+    bz.check(bz.lib().bz_probe_gather64(d_region.data_ptr(), rows * 64, sink.data_ptr(), groups, per, seed, None))
+    torch.cuda.synchronize()
+    got = sink.cpu().numpy().view(np.uint32)
+    gid = np.arange(groups, dtype=np.uint64)[:, None]
+    r = np.arange(per, dtype=np.uint64)[None, :]
+    h = ((gid * per + r) * 2654435761 + seed) & 0xFFFFFFFF
+    h ^= h >> 15
+    h = (h * 2246822519) & 0xFFFFFFFF
+    h ^= h >> 13
+    picked = (h * rows) >> 32  # [groups, per]
+    assert picked.max() < rows and len(np.unique(picked)) > rows // 2
+    words = region[picked.astype(np.int64)]  # [groups, per, 16]
+    want = np.empty((groups, 16), np.uint32)
+    for j in range(16):
+        col = words[:, :, j]
+        want[:, j] = col.sum(1, dtype=np.uint64).astype(np.uint32) if j % 2 == 0 else np.bitwise_xor.reduce(col, axis=1)
+    np.testing.assert_array_equal(got, want)
+    # error convention
+    assert bz.lib().bz_probe_gather64(d_region.data_ptr(), rows * 64, sink.data_ptr(), groups, 3, seed, None) != 0
+    assert b"rows_per_group" in bz.lib().bz_last_error()

@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
+    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew", "bz_probe_gather64"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 MAX_RANK = 6
@@ -127,6 +127,7 @@ def lib():
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
+        l.bz_probe_gather64.argtypes = [vp, i64, vp, i64, C.c_int, C.c_uint32, vp]
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]

@@ -541,6 +541,36 @@ int groups_per_wg(const bz_embed_slot& s) {
   return kThreads / lpr;
 }
 
+// ---------------------------------------------------------------------------------------------
+// measurement aid: the pooling kernel's access pattern alone (random 64-byte rows, four lanes a row)
+// ---------------------------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(kThreads) void bz_probe_gather_kernel(const uint4* __restrict__ region, uint4* __restrict__ sink,
+                                                                   uint32_t rows, int64_t groups, uint32_t seed) {
+  const int64_t gid = ((int64_t)blockIdx.x * kThreads + threadIdx.x) >> 2;
+  const int l = threadIdx.x & 3;
+  if (gid >= groups) return;
+  uint4 v[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    uint32_t h = ((uint32_t)gid * R + r) * 2654435761u + seed;
+    h ^= h >> 15;
+    h *= 2246822519u;
+    h ^= h >> 13;
+    const uint32_t row = (uint32_t)(((uint64_t)h * rows) >> 32);  // uniform over [0, rows)
+    v[r] = region[(size_t)row * 4 + l];
+  }
+  uint4 acc = make_uint4(0, 0, 0, 0);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    acc.x += v[r].x;
+    acc.y ^= v[r].y;
+    acc.z += v[r].z;
+    acc.w ^= v[r].w;
+  }
+  sink[(size_t)gid * 4 + l] = acc;
+}
+
 }  // namespace
 
 extern "C" {
@@ -662,5 +692,28 @@ int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch,
 }
 
 const char* bz_embed_pool_kernel_name(void) { return "bz_embed_pool_kernel"; }
+
+int bz_probe_gather64(const void* region, int64_t region_bytes, void* sink, int64_t groups, int rows_per_group,
+                      uint32_t seed, bz_stream_t stream) {
+  BZ_REQUIRE(region != nullptr && sink != nullptr && region_bytes >= 64 && ((uintptr_t)region & 15) == 0 &&
+                 ((uintptr_t)sink & 15) == 0,
+             "bz_probe_gather64: null or misaligned buffer (region_bytes=%lld)", (long long)region_bytes);
+  BZ_REQUIRE(groups > 0 && groups <= (1ll << 28), "bz_probe_gather64: groups=%lld outside (0, 2^28]", (long long)groups);
+  const int64_t rows = region_bytes / 64;
+  BZ_REQUIRE(rows < (1ll << 32), "bz_probe_gather64: region larger than 2^32 rows");
+  const dim3 grid((unsigned)((groups * 4 + kThreads - 1) / kThreads)), block(kThreads);
+  hipStream_t st = bz::as_stream(stream);
+  const uint4* t = (const uint4*)region;
+  uint4* out = (uint4*)sink;
+  switch (rows_per_group) {
+    case 1: hipLaunchKernelGGL(bz_probe_gather_kernel<1>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
+    case 4: hipLaunchKernelGGL(bz_probe_gather_kernel<4>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
+    case 8: hipLaunchKernelGGL(bz_probe_gather_kernel<8>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
+    case 16: hipLaunchKernelGGL(bz_probe_gather_kernel<16>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
+    default: return bz::fail(BZ_EINVAL, "bz_probe_gather64: rows_per_group=%d is not 1, 4, 8 or 16", rows_per_group);
+  }
+  BZ_LAUNCH_OK("bz_probe_gather_kernel");
+  return BZ_OK;
+}
 
 }  // extern "C"
