@@ -40,8 +40,8 @@ def main():
                     help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
                          "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     ap.add_argument("--gather-probe", action="store_true",
-                    help="only measure what the memory system gives random 64-byte row gathers (a kernel that does nothing else, "
-                         "the pooling kernel on uniform ids with 64-id segments, a row copy through the kassign path) and exit")
+                    help="only measure what the memory system gives random 64-byte row gathers (a kernel that does nothing else, and "
+                         "the pooling kernel on uniform ids with 64-id segments) and exit")
     ap.add_argument("--threads", type=int, default=8,
                     help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
                          "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
@@ -125,15 +125,6 @@ def main():
         res["pool_kernel_uniform_ids_64_per_segment"] = {"ids": nnz, "us": round(us, 1),
                                                          "row_read_GB/s": round(nnz * 64 / us / 1e3, 1),
                                                          "algorithmic_GB/s": round(alg / us / 1e3, 1)}
-        # (ii) a pure gather through the kassign path: every id's row is copied to its own output position, one lane group
-        # per position, so nothing is summed and nothing waits on a neighbour (row read + row written per id)
-        wide = torch.zeros((cfg.batch, cfg.slots * L * cfg.dim), dtype=torch.float16, device="cuda")
-        for s_, it in enumerate(items):
-            it.update(out=wide, col=s_ * L * cfg.dim, udf=bz.ASSIGN, trunc_num=L, trunc_dir=bz.ORDER)
-        plan = bz.EmbeddingPlan(items, fused_scan=True)
-        us = ev_time(plan.pool)
-        res["kassign_copy_of_the_same_rows"] = {"ids": nnz, "us": round(us, 1), "row_read_GB/s": round(nnz * 64 / us / 1e3, 1),
-                                                "read_plus_written_GB/s": round(nnz * (64 + 12 + 64) / us / 1e3, 1)}
         print(json.dumps(res))
         return
     cfg = Config2()

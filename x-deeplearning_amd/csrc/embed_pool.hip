@@ -473,20 +473,29 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
 __device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (dt == BZ_F16 ? 8 : 16); }
 
 __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const bz_embed_slot* __restrict__ slots,
-                                                                         int n_slots, int total_wg, int wg_per_xcd) {
+                                                                         int n_slots, int total_wg, int wg_per_xcd,
+                                                                         int wg_per_slot) {
   __shared__ int64_t s_off[kThreads + 1];
   __shared__ int64_t s_part[2 * kThreads / bz::kWave];
   // XCD-aware order: hardware deals consecutive workgroup ids round robin over the 8 XCDs; give
   // each XCD a contiguous range of the logical workgroup space (= a contiguous range of slots).
   const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
   if (v >= total_wg) return;
-  int lo = 0, hi = n_slots - 1;  // last slot with wg_begin <= v (empty slots share a begin: take the last)
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (slots[mid].wg_begin <= v)
-      lo = mid;
-    else
-      hi = mid - 1;
+  // The slot that owns workgroup v = the last one with wg_begin <= v (empty slots share a begin with their successor).
+  // Begins never decrease, so that is (number of begins <= v) - 1: every wave counts them 64 at a time with one load
+  // and a ballot - one trip to memory where a binary search would make log2(n_slots) dependent ones.
+  int lo;
+  if (wg_per_slot > 0) {
+    lo = v / wg_per_slot;
+  } else {
+    const int lane = threadIdx.x & (bz::kWave - 1);
+    int cnt = 0;
+    for (int base = 0; base < n_slots; base += bz::kWave) {
+      const int i = base + lane;
+      const bool le = i < n_slots && slots[i].wg_begin <= v;
+      cnt += __popcll(__ballot(le));
+    }
+    lo = __builtin_amdgcn_readfirstlane(cnt - 1);
   }
   // slots with wg_count == 0 sharing this begin come before the one that owns the workgroup
   const bz_embed_slot s = slots[lo];
@@ -658,7 +667,8 @@ int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch,
   const dim3 grid(per_xcd * bz::kNumXcd), block(kThreads);
   hipStream_t st = bz::as_stream(stream);
   if (L.variant == 0) {
-    hipLaunchKernelGGL(bz_embed_pool_generic_kernel, grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd);
+    hipLaunchKernelGGL(bz_embed_pool_generic_kernel, grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd,
+                       ((int64_t)L.wg_per_slot * L.n_slots == L.total_wg) ? L.wg_per_slot : 0);
     BZ_LAUNCH_OK("bz_embed_pool_generic_kernel");
     return BZ_OK;
   }
