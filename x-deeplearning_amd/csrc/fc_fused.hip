@@ -193,14 +193,29 @@ __device__ __forceinline__ uint4 load_chunk(const char* base, int64_t row, int64
   return out;
 }
 
-// the same for operands whose rows are 16-byte aligned and K a multiple of the chunk: no branches, so
-// the loads of several K tiles can stay in flight (a chunk is either wholly inside K or zero)
+// The same for operands whose rows are 16-byte aligned and K a multiple of the chunk (a chunk is either wholly inside
+// K or absent): no branches and nothing done to the loaded value, so the loads of several K tiles can stay in
+// flight.  A chunk beyond K is read from 16 bytes of zeros instead of being masked after the load: a mask is an
+// instruction on the loaded register, and the scheduler is free to place it - and the wait for the load it implies -
+// right behind the load (it did so in the 128x256 tile: one exposed trip to memory in every K tile).
+__device__ uint4 kZeroChunk = {0u, 0u, 0u, 0u};  // never written; not const, so that it lives in the global address space like the operands (a select between a global and a constant-space pointer would be loaded through FLAT)
+
 template <int DT>
 __device__ __forceinline__ uint4 load_chunk_aligned(const char* base, int64_t row, int64_t ld, int k, int K) {
   constexpr int ES = In<DT>::kSize;
+  const char* p = k < K ? base + (row * ld + k) * ES : (const char*)&kZeroChunk;
+  return *(const uint4*)p;
+}
+
+// The variant that reads a clamped address and leaves the zeroing of chunks beyond K to the consumer.  The eight-wave
+// tile with the skinny head keeps it: there the address select costs more (11.1 against 10.5 us on config 2's
+// 512 -> 256 -> 2) than the mask, which the scheduler leaves at the LDS store in that kernel.
+template <int DT>
+__device__ __forceinline__ uint4 load_chunk_clamped(const char* base, int64_t row, int64_t ld, int k, int K) {
+  constexpr int ES = In<DT>::kSize;
   constexpr int CH = In<DT>::kChunk;
   const int kc = k < K ? k : K - CH;
-  return *(const uint4*)(base + (row * ld + kc) * ES);  // caller zeroes chunks with k >= K when it consumes them
+  return *(const uint4*)(base + (row * ld + kc) * ES);
 }
 
 constexpr int kSkinnyMaxN = 8;
@@ -283,8 +298,9 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         const int r = q / CPR, ch = q % CPR;
         int m = m0 + r;
         m = m < M ? m : M - 1;
-        ra[set][i] = ALIGNED ? load_chunk_aligned<DT>(A, m, lda, k0 + ch * T::kChunk, K)
-                             : load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a);
+        ra[set][i] = !ALIGNED ? load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a)
+                     : HEAD ? load_chunk_clamped<DT>(A, m, lda, k0 + ch * T::kChunk, K)
+                            : load_chunk_aligned<DT>(A, m, lda, k0 + ch * T::kChunk, K);
       }
     }
 #pragma unroll
@@ -294,15 +310,15 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         const int r = q / CPR, ch = q % CPR;
         int n = n0 + r;
         n = n < N ? n : N - 1;
-        rw[set][i] = ALIGNED ? load_chunk_aligned<DT>(W, n, ldw, k0 + ch * T::kChunk, K)
-                             : load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w);
+        rw[set][i] = !ALIGNED ? load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w)
+                     : HEAD ? load_chunk_clamped<DT>(W, n, ldw, k0 + ch * T::kChunk, K)
+                            : load_chunk_aligned<DT>(W, n, ldw, k0 + ch * T::kChunk, K);
       }
     }
   };
-  // registers -> LDS.  The aligned path masks chunks beyond K here, at the point of use, so that nothing
-  // touches a loaded register (and forces a wait) while later tiles are still being requested.
+  // registers -> LDS (chunks beyond K already arrived as zeros, except from the clamped loader)
   auto masked = [&](uint4 v, int k) {
-    if (ALIGNED) {
+    if (ALIGNED && HEAD) {
       const uint32_t keep = k < K ? 0xffffffffu : 0u;
       v.x &= keep;
       v.y &= keep;
@@ -376,6 +392,52 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   lstore(0, 0, 0);
   __syncthreads();
   const int frag_row = lane & 31, frag_half = lane >> 5;
+  // Large tiles are bound by how well LDS traffic hides behind the MFMAs, and a barrier lines all waves up in the same
+  // phase: a burst of fragment reads right after it (matrix pipes idle), a burst of tile stores right before it.  PIPE
+  // reorders a K tile: the next tile goes to the other LDS buffer first (its registers arrived long ago), fragments
+  // are read one sub-step ahead of the MFMAs that use them, and the barrier sits before the last sub-step's MFMAs,
+  // which then cover the read of the next tile's first fragments.
+  // (not the 256x256 tile: with 128 accumulator registers a wave has no room for a second set of fragments)
+  constexpr bool PIPE = !HEAD && BM * BN >= 128 * 128 && BM * BN < 256 * 256;
+  constexpr int KS = BK / T::kStepK;
+  if constexpr (PIPE) {
+    static_assert(KS % 2 == 0, "fragment double buffer needs an even number of sub-steps");
+    uint4 fa[2][TM], fw[2][TN];
+    auto fread = [&](int slot, int buf, int ks) {
+      const char* la = &lds[buf][(wm * WTM + frag_row) * PITCH + frag_half * 16];
+      const char* lw = &lds[buf][(BM + wn * WTN + frag_row) * PITCH + frag_half * 16];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[slot][i] = *(const uint4*)(la + i * 32 * PITCH + ks * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fw[slot][j] = *(const uint4*)(lw + j * 32 * PITCH + ks * 32);
+    };
+    auto fmma = [&](int slot, int ks) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) T::mma(fa[slot][i], fw[slot][j], acc[ks % KACC][i][j]);
+    };
+    fread(0, 0, 0);
+    for (int kt0 = 0; kt0 < KTR; kt0 += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        const int kt = kt0 + d;
+        const int buf = kt & 1;
+        gload(d, (kt + D) * BK);  // set d held tile kt, which already sits in LDS
+        // the other buffer was last read before the previous barrier: tile kt+1 can go there now
+        lstore((d + 1) % D, buf ^ 1, (kt + 1) * BK);
+#pragma unroll
+        for (int ks = 0; ks + 1 < KS; ++ks) {
+          fread((ks + 1) & 1, buf, ks + 1);
+          fmma(ks & 1, ks);
+        }
+        __syncthreads();           // tile kt+1 is complete; every read of this buffer has returned
+        fread(0, buf ^ 1, 0);      // KS is even: the next tile's first fragments take slot 0 again
+        fmma((KS - 1) & 1, KS - 1);
+      }
+    }
+    __syncthreads();  // the fragments read ahead for a tile that does not exist are dropped; LDS is free for the epilogue
+  } else {
   for (int kt0 = 0; kt0 < KTR; kt0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
@@ -399,6 +461,7 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
       lstore((d + 1) % D, buf ^ 1, (kt + 1) * BK);
       __syncthreads();
     }
+  }
   }
 
   if (KACC == 2) {
