@@ -139,7 +139,10 @@ def test_fc_fp32(bz, oracle, M, N, K, act):
 @pytest.mark.parametrize("M,N,K,act", [(2048, 512, 896, "prelu"), (2048, 256, 512, "prelu"), (300, 80, 216, "dice"),
                                        (300, 40, 80, "dice"), (64, 200, 168, "dice"), (4096, 2048, 256, "relu"),
                                        (4100, 1000, 200, "dice"), (33000, 80, 216, "dice"), (100, 100, 104, "none"),
-                                       (4000, 4104, 72, "prelu")])  # 16 x 17 tiles of 256x256, ragged in M and N
+                                       (4000, 4104, 72, "prelu"),  # 16 x 17 tiles of 256x256, ragged in M and N
+                                       # the software-pipelined K loop: 128x256 tiles (128x128 for fp32 output), ragged
+                                       # in M and N, K ending inside a tile and the loop padded with absent tiles
+                                       (8200, 1000, 520, "prelu"), (33000, 250, 136, "dice")])
 def test_fc_half(bz, oracle, in_name, out_name, M, N, K, act):
     print("case %s->%s M=%d N=%d K=%d act=%s" % (in_name, out_name, M, N, K, act), flush=True)
     _fc_case(bz, oracle, M, N, K, in_name, out_name, act, seed=M + N * 3 + K)
