@@ -289,6 +289,9 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   // D register sets: K tiles kt+1 .. kt+D are in flight from global memory while tile kt is multiplied out of
   // LDS.  The kernel is latency bound at CTR sizes (a tile's MFMAs take ~0.1 us, a round trip ~1 us), so the
   // number of exposed round trips, ceil(KT / D), is what sets its duration.
+  // which aligned loader: the head tile (see load_chunk_clamped) and the 256x256 tile, whose 256 registers have no room
+  // for the zero-chunk select's addresses (it spilled 75 of them)
+  constexpr bool CLAMPED = HEAD || BM * BN >= 256 * 256;
   uint4 ra[D][A_PER], rw[D][W_PER];
   auto gload = [&](int set, int k0) {
 #pragma unroll
@@ -299,7 +302,7 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         int m = m0 + r;
         m = m < M ? m : M - 1;
         ra[set][i] = !ALIGNED ? load_chunk<DT>(A, m, lda, k0 + ch * T::kChunk, K, vec_a)
-                     : HEAD ? load_chunk_clamped<DT>(A, m, lda, k0 + ch * T::kChunk, K)
+                     : CLAMPED ? load_chunk_clamped<DT>(A, m, lda, k0 + ch * T::kChunk, K)
                             : load_chunk_aligned<DT>(A, m, lda, k0 + ch * T::kChunk, K);
       }
     }
@@ -311,14 +314,14 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
         int n = n0 + r;
         n = n < N ? n : N - 1;
         rw[set][i] = !ALIGNED ? load_chunk<DT>(W, n, ldw, k0 + ch * T::kChunk, K, vec_w)
-                     : HEAD ? load_chunk_clamped<DT>(W, n, ldw, k0 + ch * T::kChunk, K)
+                     : CLAMPED ? load_chunk_clamped<DT>(W, n, ldw, k0 + ch * T::kChunk, K)
                             : load_chunk_aligned<DT>(W, n, ldw, k0 + ch * T::kChunk, K);
       }
     }
   };
   // registers -> LDS (chunks beyond K already arrived as zeros, except from the clamped loader)
   auto masked = [&](uint4 v, int k) {
-    if (ALIGNED && HEAD) {
+    if (ALIGNED && CLAMPED) {
       const uint32_t keep = k < K ? 0xffffffffu : 0u;
       v.x &= keep;
       v.y &= keep;
@@ -392,13 +395,14 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   lstore(0, 0, 0);
   __syncthreads();
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  // Large tiles are bound by how well LDS traffic hides behind the MFMAs, and a barrier lines all waves up in the same
+  // Tiles are bound by how well LDS traffic hides behind the MFMAs, and a barrier lines all waves up in the same
   // phase: a burst of fragment reads right after it (matrix pipes idle), a burst of tile stores right before it.  PIPE
   // reorders a K tile: the next tile goes to the other LDS buffer first (its registers arrived long ago), fragments
   // are read one sub-step ahead of the MFMAs that use them, and the barrier sits before the last sub-step's MFMAs,
   // which then cover the read of the next tile's first fragments.
-  // (not the 256x256 tile: with 128 accumulator registers a wave has no room for a second set of fragments)
-  constexpr bool PIPE = !HEAD && BM * BN >= 128 * 128 && BM * BN < 256 * 256;
+  // (not the 256x256 tile: with 128 accumulator registers a wave has no room for a second set of fragments; measured on
+  // the other tiles: 128x256 245 -> 238 us on 8192x12800x1024, 64x64 9.6 -> 9.2 us on config 2's first layer)
+  constexpr bool PIPE = !HEAD && BM * BN >= 64 * 64 && BM * BN < 256 * 256;
   constexpr int KS = BK / T::kStepK;
   if constexpr (PIPE) {
     static_assert(KS % 2 == 0, "fragment double buffer needs an even number of sub-steps");
