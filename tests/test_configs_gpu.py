@@ -148,8 +148,8 @@ def test_config5_fp16_tables_bf16_tower_full_size(bz, oracle):
             keep.append(t)
             items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=out, col=s * D, udf=bz.SUM))
         plan = bz.EmbeddingPlan(items)
-        # 256 workgroups per slot would each re-read up to 8192 counts: the planner asks for the separate scan launch
-        assert plan.launch.fused_scan == 0 and not plan.fused_scan and plan.total_wg == cfg.slots * 256
+        # 128 workgroups per slot would each re-read up to 8192 counts: the planner asks for the separate scan launch
+        assert plan.launch.fused_scan == 0 and not plan.fused_scan and plan.total_wg == cfg.slots * 128
         plan.run()
     torch.cuda.synchronize()
     rng = np.random.default_rng(5)

@@ -271,16 +271,16 @@ def test_embedding_planner_geometry_and_scan_advice():
         assert bz.lib().bz_embed_plan(slots, n_slots, C.byref(launch)) == 0, bz.lib().bz_last_error()
         return slots, launch
 
-    slots, launch = plan(26, 2048, 32)           # config 2: dim 32 fp16 = 4 chunks -> 64 samples per workgroup
-    assert launch.total_wg == 26 * 32 and launch.wg_per_slot == 32 and launch.fused_scan == 1 and launch.scan_first == 0
+    slots, launch = plan(26, 2048, 32)           # config 2: dim 32 fp16 = 4 chunks -> 128 samples per 512-thread workgroup
+    assert launch.total_wg == 26 * 16 and launch.wg_per_slot == 16 and launch.fused_scan == 1 and launch.scan_first == 0
     assert launch.variant == (bz.F16 << 8) | 4
-    assert [s.wg_begin for s in slots][:3] == [0, 32, 64]
-    _, launch = plan(200, 8192, 64)              # config 5: 8 chunks -> 32 samples per workgroup, 256 workgroups a slot
-    assert launch.total_wg == 200 * 256 and launch.fused_scan == 1 and launch.scan_first == 1
+    assert [s.wg_begin for s in slots][:3] == [0, 16, 32]
+    _, launch = plan(200, 8192, 64)              # config 5: 8 chunks -> 64 samples per workgroup, 128 workgroups a slot
+    assert launch.total_wg == 200 * 128 and launch.fused_scan == 1 and launch.scan_first == 1
     _, launch = plan(200, 8192, 64, offsets=True)
     assert launch.fused_scan == 0 and launch.scan_first == 0
-    slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 64 positions per workgroup
-    assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 64] * 3
+    slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 128 positions per workgroup
+    assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 128] * 3
 
 
 def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle):

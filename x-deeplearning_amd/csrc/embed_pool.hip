@@ -9,8 +9,8 @@
 // (36..256 bytes) plus 12 bytes of id/value.  A row is cut into 16-byte chunks
 // (one 128-bit load); a *lane group* of `lpr` = pow2(chunks per row) lanes owns one
 // (sample, slot) segment and walks its ids in order, so every output element is
-// summed in exactly the reference's order (bit-identical fp32).  A 256-thread
-// workgroup holds 256/lpr segments of consecutive samples of one slot.  One launch
+// summed in exactly the reference's order (bit-identical fp32).  A 512-thread
+// workgroup holds 512/lpr segments of consecutive samples of one slot.  One launch
 // covers every slot of the operator; the linear workgroup id is remapped so that
 // each of the 8 XCDs (each with its own L2) serves a contiguous range of slots and
 // therefore caches the hot rows of only those tables.
@@ -34,7 +34,8 @@
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;  // measured at 128 / 256 / 512 / 1024 on config 2: 14.7 / 13.5 / 13.3 / 13.4 us per launch,
+                               // 127 / 131 / 135 / 129 M samples/s with eight serving threads
 constexpr int kUnroll = 4;  // rows in flight per lane group in the generic kernel (8 held 118 VGPRs and was no faster)
 
 // ---------------------------------------------------------------------------------------------
@@ -316,7 +317,7 @@ __device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int
 // offsets of one workgroup's samples, derived from the segment counts
 // ---------------------------------------------------------------------------------------------
 // s_off[0..groups] <- exclusive offsets of samples b0 .. b0+groups (clipped to batch).
-// All 256 threads call it; ends with a barrier.
+// Every thread of the workgroup calls it; ends with a barrier.
 __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0, int groups, int64_t* s_off,
                                               int64_t* s_part) {
   const int tid = threadIdx.x;
