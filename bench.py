@@ -25,8 +25,8 @@ MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
 # HBM-side bytes per launch of the pooling kernel on this exact workload (default seed, pool of 32 batches), from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, averaged over 1704 dispatches) scaled by what the same
 # counters read for a plain 256 MiB copy (`--calibrate-copy`: FETCH_SIZE reads 0.5 of the bytes, WRITE_SIZE all of them):
-# fetch 11960.90 KiB x 2.0 + write 3328.50 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
-POOL_TRAFFIC_BYTES = int((11960.90 * 2.0 + 3328.50) * 1024)
+# fetch 11961.30 KiB x 2.0 + write 3333.59 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
+POOL_TRAFFIC_BYTES = int((11961.30 * 2.0 + 3333.59) * 1024)
 
 
 def main():
