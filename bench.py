@@ -5,13 +5,25 @@
 
 A step is one forward pass (Embedding gather/pool -> FC 896-512-256-2 with PReLU -> softmax) over one
 synthetic batch of 2048 samples (config 2), inputs already resident in HBM.  A pool of pre-generated
-batches is cycled so the id stream is not one cached batch.  By default the step is Predictor.Forward through
-the Blaze_* C ABI (the drop-in path), issued by a few serving threads with one Predictor set and HIP stream
-each, as the reference is deployed.  Prints ONE JSON line.
+batches is cycled so the id stream is not one cached batch.  The step is Predictor.Forward through the Blaze_* C ABI
+(the drop-in path), issued by a few serving threads with one Predictor set and HIP stream each, as the reference is
+deployed (blaze/example/cpp/predictor_example.cc:129-140,189).  Prints ONE JSON line:
+
+  value / ms_per_step     exactly K steps after the warm-up (every predictor has run at least twice before the clock
+                          starts, whatever W says: W is a floor);
+  steady_state            the same loop over a fixed number of steps (>= 2000), so a short K does not hide the rate;
+  p50_ms / p99_ms         one request at a time on one thread, over max(K, 1000) forwards;
+  with_host_feed          every step feeds all inputs from host memory and copies the output back (PCIe inclusive);
+  roofline                the pooling kernel: algorithmic bytes per launch / average launch duration (HIP events
+                          around a replayed graph of back-to-back launches over the pooled batches);
+  per_config              configs 1, 3, 4 and 5 of the benchmark definition, each with its own rate and roofline;
+  cpu_baseline            the CPU restatement of the reference's path on the box's host cores (a bounded sample).
 """
 import argparse
+import ctypes
 import json
 import os
+import re
 import sys
 import threading
 import time
@@ -22,50 +34,73 @@ sys.path.insert(1, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_PEAK_TFLOPS = 2500.0  # dense fp16/bf16
-# HBM-side bytes per launch of the pooling kernel on this exact workload (default seed, pool of 32 batches), from two
-# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, averaged over 1704 dispatches) scaled by what the same
-# counters read for a plain 256 MiB copy (`--calibrate-copy`: FETCH_SIZE reads 0.5 of the bytes, WRITE_SIZE all of them):
-# fetch 11961.30 KiB x 2.0 + write 3333.59 KiB.  Below the algorithmic bytes because Zipf-hot rows hit in L2.
-POOL_TRAFFIC_BYTES = int((11961.30 * 2.0 + 3333.59) * 1024)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "c2_embed_pool_hbm_traffic.md")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--pool", type=int, default=32, help="number of distinct pre-generated batches")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
-                         "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
-    ap.add_argument("--gather-probe", action="store_true",
-                    help="only measure what the memory system gives random 64-byte row gathers (a kernel that does nothing else, and "
-                         "the pooling kernel on uniform ids with 64-id segments) and exit")
-    ap.add_argument("--threads", type=int, default=8,
-                    help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
-                         "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
-    ap.add_argument("--with-feed", action="store_true",
-                    help="also time steps that Feed every input from host memory and copy the output back (the "
-                         "PCIe-inclusive rate; reported as an extra key, never as `value`)")
-    ap.add_argument("--kernel-api", action="store_true",
-                    help="drive the kernel-layer C ABI directly instead of Predictor.Forward (lower host overhead)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (one process, no collectives); --gpus %d is not supported" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
+def pool_traffic_from_profile():
+    """HBM-side bytes per launch of the pooling kernel on the default workload, as the committed counter profile states
+    them (a line `traffic_bytes_per_launch: N` and a line `collected: <date>`); None when the file has no such line."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
+    d = re.search(r"collected:\s*([^\n]+)", text)
+    if not m:
+        return None, None
+    return int(m.group(1)), "profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, collected %s)" % (
+        os.path.basename(TRAFFIC_PROFILE), d.group(1).strip() if d else "?")
 
-    import numpy as np
-    import torch
-    import blaze_hip as bz
-    from pipeline import CtrForward
-    from synth import Config2
 
-    assert torch.cuda.is_available(), "no GPU visible"
-    arch = bz.device_check()
+def graph_timed(torch, fn, n_distinct, reps, rounds=5):
+    """Average duration in us of fn(i): `reps` back-to-back calls recorded into one HIP graph on torch's current stream
+    (so host launch cost is not in it), replayed `rounds` times between two events on that stream."""
+    for i in range(n_distinct):
+        fn(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(reps):
+            fn(i)
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(rounds):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * rounds)
+
+
+def latency_ms(np, step, n):
+    lat = np.empty(n)
+    for i in range(n):
+        a = time.perf_counter()
+        step(i)
+        lat[i] = (time.perf_counter() - a) * 1e3
+    lat.sort()
+    return float(lat[n // 2]), float(lat[min(n - 1, int(n * 0.99))]), n
+
+
+def hbm_roofline(kernel, alg_bytes, us, traffic=None):
+    gbs = alg_bytes / us / 1e3
+    return {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 5), "traffic": traffic, "algorithmic_bytes_per_launch": int(alg_bytes),
+            "avg_launch_us": round(us, 2)}
+
+
+def mfma_roofline(kernel, flops, us):
+    tf = flops / us / 1e6
+    return {"kernel": kernel, "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tf / MFMA_PEAK_TFLOPS, 5), "traffic": None, "flops_per_launch": int(flops), "avg_launch_us": round(us, 2)}
+
+
+# ------------------------------------------------------------------------------------------------ probes
+def run_probes(args, np, torch, bz, arch):
+    """Measurement aids behind the profiles: a plain copy of known size (the reference for scaling counter readings)
+    and the gather probes (what the memory system gives the pooling kernel's access pattern alone)."""
     if args.calibrate_copy:
-        import ctypes
         rows, width = 65536, 4096
         src = torch.ones(rows * width, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
@@ -79,53 +114,320 @@ def main():
         print(json.dumps({"calibration": "bz_concat_kernel", "launches": 5, "bytes_read_per_launch": rows * width,
                           "bytes_written_per_launch": rows * width}))
         return
-    if args.gather_probe:
-        def ev_time(fn, reps=20):
-            for _ in range(5):
-                fn()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(reps):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / reps  # us
-        g = torch.Generator(device="cuda").manual_seed(1)
-        res = {"probe": "random gathers of 64-byte rows", "device": arch}
-        # (o) nothing but the access pattern: four-lane groups read hashed 64-byte rows of a 2 GiB region
-        region = torch.ones(2 << 30, dtype=torch.uint8, device="cuda")
-        sink = torch.empty((1 << 20) * 64, dtype=torch.uint8, device="cuda")
-        pure = {}
-        for groups, per in ((1 << 20, 8), (1 << 20, 16), (425984, 1), (106496, 4), (53248, 8)):
-            seed = [0]
-            def launch():
-                seed[0] += 7919
-                bz.check(bz.lib().bz_probe_gather64(region.data_ptr(), region.numel(), sink.data_ptr(), groups, per, seed[0], None))
-            us = ev_time(launch, 50)
-            pure["%d groups x %d rows" % (groups, per)] = {"us": round(us, 2), "row_read_GB/s": round(groups * per * 64 / us / 1e3, 1)}
-        res["pure_gather_2GiB_region"] = pure
-        del region, sink
-        # (i) the pooling kernel where the dependent chain of a launch is amortised and no row is hot:
-        # config 2's tables (26 x 64 MB), uniform ids, every segment 64 ids long
-        cfg = Config2()
-        tables = [bz.DeviceTable(t) for t in cfg.tables()]
-        L = 64
+
+    def ev_time(fn, reps=20):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps  # us
+
+    res = {"probe": "random gathers of whole rows, nothing else", "device": arch}
+    region = torch.ones(args.probe_region_mib << 20, dtype=torch.uint8, device="cuda")
+    side = torch.ones((args.probe_region_mib << 20) // 64, dtype=torch.float32, device="cuda")
+    sink = torch.empty((1 << 20) * 128, dtype=torch.uint8, device="cuda")
+    cases = [(64, False, 1 << 20, 8), (64, False, 1 << 20, 16), (64, False, 425984, 1), (64, False, 106496, 4),
+             (128, False, 1 << 20, 8), (128, False, 1 << 20, 4), (64, True, 1 << 20, 8), (64, True, 1 << 20, 4)]
+    if args.probe_case is not None:
+        cases = [cases[args.probe_case]]
+    out = {}
+    for row_bytes, with_side, groups, per in cases:
+        seed = [0]
+
+        def launch():
+            seed[0] += 7919
+            bz.check(bz.lib().bz_probe_gather(region.data_ptr(), region.numel(), row_bytes, side.data_ptr() if with_side else None,
+                                              sink.data_ptr(), groups, per, seed[0], None))
+        us = ev_time(launch, 50)
+        nbytes = groups * per * (row_bytes + (4 if with_side else 0))
+        out["%dB rows%s, %d groups x %d" % (row_bytes, " + 4B side word" if with_side else "", groups, per)] = {
+            "us": round(us, 2), "rows": groups * per, "GB/s": round(nbytes / us / 1e3, 1), "Grows/s": round(groups * per / us / 1e3, 2)}
+    res["region_MiB"] = args.probe_region_mib
+    res["cases"] = out
+    print(json.dumps(res))
+
+
+# ------------------------------------------------------------------------------------------------ other configurations
+def bench_predictor_model(np, torch, pb, predictors, batch, threads, steps, lat_steps):
+    """samples/s over `threads` serving threads + single-request latency of a list of fed predictors."""
+    T = threads
+    pool = pb.ServePool(T)
+    pool.run(predictors, 2 * len(predictors))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    pool.run(predictors, steps)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    p50, p99, n = latency_ms(np, lambda i: predictors[i % len(predictors)].forward(), lat_steps)
+    return {"samples/s": round(batch * steps / (t1 - t0), 1), "ms_per_step": round((t1 - t0) * 1e3 / steps, 5), "steps": steps,
+            "serving_threads": T, "p50_ms": round(p50, 4), "p99_ms": round(p99, 4), "latency_samples": n}
+
+
+def count_launches(p):
+    """operators of one Forward that ran (the profile observer's trace), as {op type: count}"""
+    p.register_observers(["profile"])
+    p.forward()
+    ev = json.loads(p.dump_observers()["profile"])["traceEvents"]
+    out = {}
+    for e in ev:
+        if e.get("dur", 0) > 0:
+            k = e["name"].split(":")[0]
+            out[k] = out.get(k, 0) + 1
+    return out
+
+
+def bench_config1(np, torch, bz, pb, threads):
+    from ctr_model import build_manager, make_predictor
+    from synth import Config1, embedding_bytes
+    cfg = Config1()
+    tables, mlp = cfg.tables(), cfg.mlp()
+    n = 2 * threads
+    sparse, dense = cfg.batches(n)
+    pm, fgs = build_manager(cfg, tables, mlp, np.float32)
+    preds = [make_predictor(pm, fgs, sparse[b], dense[b], np.float32) for b in range(n)]
+    res = bench_predictor_model(np, torch, pb, preds, cfg.batch, threads, 4000, 1000)
+    # the pooling kernel alone, through the kernel layer
+    dts = [bz.DeviceTable(t) for t in tables]
+    plans, keep, nnz = [], [], []
+    for b in range(n):
+        out = torch.zeros((cfg.batch, cfg.slots * cfg.dim), dtype=torch.float32, device="cuda")
+        items = []
+        for s, (ids, vals, seg) in enumerate(sparse[b]):
+            t = [torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(), torch.from_numpy(seg).cuda()]
+            keep.append(t)
+            items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=out, col=s * cfg.dim, udf=bz.SUM))
+        plans.append(bz.EmbeddingPlan(items))
+        nnz.append(sum(ids.size for ids, _, _ in sparse[b]))
+    us = graph_timed(torch, lambda i: plans[i % n].run(), n, 8 * n)
+    alg = float(np.mean([embedding_bytes(z, cfg.batch, cfg.slots, cfg.dim * 4, 0, cfg.slots * cfg.dim, 4) for z in nnz]))
+    res["workload"] = cfg.name
+    res["dtype"] = "f32"
+    res["roofline"] = hbm_roofline("bz_embed_pool_kernel", alg, us)
+    return res
+
+
+def bench_config3(np, torch, pb, threads):
+    import din_model
+    cfg = din_model.Config3()
+    tables, weights = cfg.tables(), cfg.weights()
+    n = 2 * threads
+    preds = []
+    pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16)
+    for b in range(n):
+        p = pm.create_predictor(1, 0)
+        din_model.feed(p, inputs, cfg.batch_inputs(seed_offset=b), np.float16)
+        preds.append(p)
+    res = bench_predictor_model(np, torch, pb, preds, cfg.batch, threads, 2000, 1000)
+    probe = pm.create_predictor(1, 0)
+    din_model.feed(probe, inputs, cfg.batch_inputs(seed_offset=0), np.float16)
+    probe.forward()
+    ran = count_launches(probe)
+    B, T = cfg.batch, cfg.T
+    D3 = 3 * cfg.dim
+    att = cfg.att_layers
+    main = cfg.main_layers
+    res["workload"] = cfg.name
+    res["dtype"] = "f16"
+    res["operators_run_per_forward"] = sum(ran.values())
+    res["operators"] = ran
+    res["fc_flops"] = int(2 * B * T * sum(att[i] * att[i + 1] for i in range(3)) + 2 * B * sum(main[i] * main[i + 1] for i in range(3)))
+    res["attention_bgemm_bytes"] = B * T * D3 * 2 + B * T * 4 + B * D3 * 2
+    return res
+
+
+def bench_config4(np, torch, bz):
+    from synth import Config4, embedding_bytes
+    cfg = Config4()
+    free, _ = torch.cuda.mem_get_info()
+    need = cfg.slots * cfg.rows * (cfg.dim + 4)
+    if free < need * 1.15:
+        return {"workload": cfg.name, "skipped": "needs %.0f GB of free HBM, %.0f GB free" % (need * 1.15 / 1e9, free / 1e9)}
+    tables = cfg.tables()
+    dts = [bz.DeviceTable(q, scale=sc) for q, sc in tables]
+    n = 2
+    plans, keep, nnz = [], [], []
+    for b in range(n):
         out = torch.zeros((cfg.batch, cfg.slots * cfg.dim), dtype=torch.float16, device="cuda")
         items = []
-        for s_ in range(cfg.slots):
-            ids = torch.randint(0, cfg.rows, (cfg.batch * L, ), device="cuda", generator=g)
-            items.append(dict(table=tables[s_], ids=ids, values=torch.ones(cfg.batch * L, device="cuda"),
-                              segments=torch.full((cfg.batch, ), L, dtype=torch.int32, device="cuda"), out=out,
-                              col=s_ * cfg.dim, udf=bz.SUM))
-        plan = bz.EmbeddingPlan(items, fused_scan=True)
-        us = ev_time(plan.pool)
-        nnz = cfg.slots * cfg.batch * L
-        alg = nnz * (64 + 12) + cfg.slots * cfg.batch * 4 + out.numel() * 2
-        res["pool_kernel_uniform_ids_64_per_segment"] = {"ids": nnz, "us": round(us, 1),
-                                                         "row_read_GB/s": round(nnz * 64 / us / 1e3, 1),
-                                                         "algorithmic_GB/s": round(alg / us / 1e3, 1)}
-        print(json.dumps(res))
+        sp = cfg.batch_inputs(seed_offset=b)
+        for s, (ids, vals, seg) in enumerate(sp):
+            t = [torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(), torch.from_numpy(seg).cuda()]
+            keep.append(t)
+            items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=out, col=s * cfg.dim, udf=bz.AVG))
+        plans.append(bz.EmbeddingPlan(items))
+        nnz.append(sum(ids.size for ids, _, _ in sp))
+    us = graph_timed(torch, lambda i: plans[i % n].run(), n, 4 * n)
+    alg = float(np.mean([embedding_bytes(z, cfg.batch, cfg.slots, cfg.dim, 4, cfg.slots * cfg.dim, 2) for z in nnz]))
+    res = {"workload": cfg.name, "dtype": "i8 rows x f32 scale -> f32 accumulate -> f16 block", "ids_per_launch": int(np.mean(nnz)),
+           "launches_per_step": 1 if plans[0].fused_scan else 2, "samples/s": round(cfg.batch / us * 1e6, 1),
+           "roofline": hbm_roofline("bz_embed_pool_kernel", alg, us)}
+    del plans, keep, dts, tables
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_config5(np, torch, bz):
+    from synth import Config5, embedding_bytes
+    cfg = Config5()
+    free, _ = torch.cuda.mem_get_info()
+    need = cfg.slots * cfg.rows * cfg.dim * 2
+    if free < need * 1.3:
+        return {"workload": cfg.name, "skipped": "needs %.0f GB of free HBM, %.0f GB free" % (need * 1.3 / 1e9, free / 1e9)}
+    tables = cfg.tables()
+    dts = [bz.DeviceTable(t) for t in tables]
+    mlp = cfg.mlp()
+    B, D = cfg.batch, cfg.dim
+    n = 2
+    plans, keep, nnz, xs = [], [], [], []
+    for b in range(n):
+        x = torch.zeros((B, cfg.slots * D), dtype=torch.bfloat16, device="cuda")
+        xs.append(x)
+        items = []
+        sp = cfg.batch_inputs(seed_offset=b)
+        for s, (ids, vals, seg) in enumerate(sp):
+            t = [torch.from_numpy(ids).cuda(), torch.from_numpy(vals).cuda(), torch.from_numpy(seg).cuda()]
+            keep.append(t)
+            items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=x, col=s * D, udf=bz.SUM))
+        plans.append(bz.EmbeddingPlan(items))
+        nnz.append(sum(ids.size for ids, _, _ in sp))
+    pool_us = graph_timed(torch, lambda i: plans[i % n].run(), n, 4 * n)
+    alg = float(np.mean([embedding_bytes(z, B, cfg.slots, D * 2, 0, cfg.slots * D, 2) for z in nnz]))
+    # the tower: bias + ReLU per layer, sigmoid head riding in the launch of the layer before it
+    packed = [bz.pack_weight(w, False, bz.BF16) for w, _ in mlp]
+    ys = [torch.empty((B, w.shape[1]), dtype=torch.bfloat16, device="cuda") for w, _ in mlp[:-1]]
+    prob = torch.empty((B, 1), dtype=torch.float32, device="cuda")
+    L = cfg.layers
+
+    def layer(i, li):
+        a = xs[i % n] if li == 0 else ys[li - 1]
+        bz.fc_fused(a, packed[li], L[li], bias=mlp[li][1], act=bz.ACT_LEAKY_RELU, act_alpha=0.0, out=ys[li])
+
+    def tail(i):  # layer n-2 with the 1-wide sigmoid layer as its head
+        li = len(mlp) - 2
+        bz.fc_fused(ys[li - 1], packed[li], L[li], bias=mlp[li][1], act=bz.ACT_LEAKY_RELU, act_alpha=0.0, out=ys[li],
+                    head=dict(w=packed[li + 1], bias=mlp[li + 1][1], act=bz.ACT_SIGMOID, out=prob), store_out=False)
+
+    fc_us = [graph_timed(torch, lambda i, li=li: layer(i, li), n, 4 * n) for li in range(len(mlp) - 2)]
+    fc_us.append(graph_timed(torch, tail, n, 4 * n))
+    flops = [2.0 * B * L[i] * L[i + 1] for i in range(len(L) - 1)]
+    step_us = pool_us + sum(fc_us)
+    kern = {"pool": round(pool_us, 2)}
+    for i, u in enumerate(fc_us[:-1]):
+        kern["fc[%d]" % i] = round(u, 2)
+    kern["fc[%d+%d]" % (len(mlp) - 2, len(mlp) - 1)] = round(fc_us[-1], 2)
+    res = {"workload": cfg.name, "dtype": "f16 tables -> bf16 block; bf16 MFMA, f32 accumulate", "ids_per_launch": int(np.mean(nnz)),
+           "pool_launches_per_step": 1 if plans[0].fused_scan else 2, "kernel_us": kern,
+           "samples/s_kernels_back_to_back": round(B / step_us * 1e6, 1),
+           "roofline": hbm_roofline("bz_embed_pool_kernel", alg, pool_us),
+           "roofline_fc": mfma_roofline("bz_fc_mfma_kernel (layer 0: %dx%dx%d)" % (B, L[0], L[1]), flops[0], fc_us[0]),
+           "fc_stack": {"TFLOP/s": round(sum(flops) / sum(fc_us) / 1e6, 2),
+                        "frac_of_mfma_peak": round(sum(flops) / sum(fc_us) / 1e6 / MFMA_PEAK_TFLOPS, 5),
+                        "flops": int(sum(flops)), "us": round(sum(fc_us), 2)}}
+    del plans, keep, dts, tables, xs
+    torch.cuda.empty_cache()
+    return res
+
+
+# ------------------------------------------------------------------------------------------------ CPU baseline
+def cpu_baseline(np, cfg, tables, mlp, sparse, dense):
+    """The oracle (a port of the reference's CPU path), one single-threaded predictor per thread: per id a probe of the
+    reference's hash index (quick_embedding_dict.h:55-71 -> hashtable.cc:45-64), the ksum loop, then per layer sgemm of
+    the BLAS numpy links (as the reference hands the product to MKL's cblas_sgemm, math/gemm.cc:13-27) + a separate
+    PReLU pass, softmax.  A bounded sample of the workload: 8 batches per thread."""
+    import blaze_oracle as orc
+    from model_forward import ctr_forward
+    from threadpoolctl import threadpool_info, threadpool_limits
+    orc.build()
+    rows = tables[0].shape[0]
+    keys = np.arange(rows, dtype=np.uint64)
+    tabs_hash = [orc.Table(t.cpu().numpy(), keys=keys) for t in tables]   # per-id hash probe, the reference's structure
+    tabs_direct = [orc.Table(t.cpu().numpy()) for t in tables]            # id == row, no index
+    mlp_np = [(w.cpu().numpy(), b.cpu().numpy(), s.cpu().numpy()) for (w, b, s) in mlp]
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+    per_thread = 8
+    blas = next(("%s %s (%s)" % (i.get("internal_api"), i.get("version"), i.get("architecture"))
+                 for i in threadpool_info() if i.get("user_api") == "blas"), "numpy's matmul")
+
+    def run_threads(tabs):
+        def worker(t):
+            for j in range(per_thread):
+                b = (t * per_thread + j) % len(sparse)
+                ctr_forward(orc, cfg, tabs, mlp_np, sparse[b], dense[b], blas=True)
+        ctr_forward(orc, cfg, tabs, mlp_np, sparse[0], dense[0], blas=True)  # warm the page cache of the tables
+        c0 = time.perf_counter()
+        ths = [threading.Thread(target=worker, args=(t, )) for t in range(threads)]
+        for t in ths:
+            t.start()
+        for t in ths:
+            t.join()
+        return cfg.batch * threads * per_thread / (time.perf_counter() - c0)
+
+    with threadpool_limits(1, user_api="blas"):
+        rate_hash = run_threads(tabs_hash)
+        rate_direct = run_threads(tabs_direct)
+        s0 = time.perf_counter()  # ... and the hash-probe port on one core alone
+        for j in range(per_thread):
+            ctr_forward(orc, cfg, tabs_hash, mlp_np, sparse[j % len(sparse)], dense[j % len(sparse)], blas=True)
+        s1 = time.perf_counter()
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), "")
+    except OSError:
+        pass
+    return {"value": round(rate_hash, 1), "unit": "samples/s", "cores": threads, "kind": "port",
+            "value_without_hash_index": round(rate_direct, 1), "value_1_core": round(cfg.batch * per_thread / (s1 - s0), 1),
+            "sgemm": blas, "host_cpus": os.cpu_count(), "cpu_model": model,
+            "sample": "%d batches of %d (%d per thread, one single-threaded predictor per core), fp32 oracle: per-id probe of "
+                      "the reference's hash index, ksum, sgemm of the BLAS numpy links on one thread + separate PReLU pass, "
+                      "softmax" % (threads * per_thread, cfg.batch, per_thread)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--pool", type=int, default=32, help="number of distinct pre-generated batches")
+    ap.add_argument("--steady-steps", type=int, default=4000, help="steps of the fixed-length steady-state region (>= 2000)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-config", action="store_true", help="skip configs 1, 3, 4 and 5")
+    ap.add_argument("--no-feed", action="store_true", help="skip the PCIe-inclusive leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
+                         "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
+    ap.add_argument("--gather-probe", action="store_true",
+                    help="only measure what the memory system gives random gathers of 64- and 128-byte rows (a kernel that "
+                         "does nothing else) and exit")
+    ap.add_argument("--probe-region-mib", type=int, default=2048)
+    ap.add_argument("--probe-case", type=int, default=None, help="run one case of --gather-probe only (for counter runs)")
+    ap.add_argument("--threads", type=int, default=8,
+                    help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
+                         "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
+    ap.add_argument("--kernel-api", action="store_true",
+                    help="drive the kernel-layer C ABI directly instead of Predictor.Forward (lower host overhead)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (one process, no collectives); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import blaze_hip as bz
+    import pyblaze_hip as pb
+    from pipeline import CtrForward
+    from synth import Config2
+
+    assert torch.cuda.is_available(), "no GPU visible"
+    arch = bz.device_check()
+    if args.calibrate_copy or args.gather_probe:
+        run_probes(args, np, torch, bz, arch)
         return
     cfg = Config2()
     tables = cfg.tables()
@@ -135,16 +437,20 @@ def main():
     fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16", fused_mlp=bool(int(os.environ.get("BZ_FUSED_MLP", "0"))))
     torch.cuda.synchronize()
     K, W = args.steps, args.warmup
-    T = max(1, min(args.threads, fwd.n_batches))
-    assert fwd.n_batches % T == 0, "--pool must be a multiple of --threads (a pooled batch always runs on one thread)"
+    S = max(2000, args.steady_steps)
+    NB = fwd.n_batches
+    T = max(1, min(args.threads, NB))
+    assert NB % T == 0, "--pool must be a multiple of --threads (a pooled batch always runs on one thread)"
+    warm = max(W, 2 * NB)  # W is a floor: every predictor runs at least twice before the clock starts
 
     predictors = None
+    steady = feed_rate = None
     if not args.kernel_api:
         # the drop-in path: one Predictor per pooled batch (inputs fed once = resident in HBM), Forward through
         # the Blaze_* C ABI; consecutive steps go round robin over T serving threads
         from ctr_model import build_manager, make_predictor
         pm, fgs = build_manager(cfg, tables, mlp, np.float16)
-        predictors = [make_predictor(pm, fgs, sparse[b], dense[b], np.float16) for b in range(fwd.n_batches)]
+        predictors = [make_predictor(pm, fgs, sparse[b], dense[b], np.float16) for b in range(NB)]
         predictors[0].forward()
         ref = fwd.output(0)
         fwd.step(0)
@@ -153,80 +459,76 @@ def main():
         assert np.allclose(predictors[0].output_asnumpy("prob").astype(np.float32), ref.cpu().numpy(), atol=1e-3), \
             "Predictor and kernel-layer harness disagree"
 
-    import ctypes
-    import threading
     streams = [torch.cuda.Stream() for _ in range(T)]
     stream_ptrs = [ctypes.c_void_p(st.cuda_stream) for st in streams]
 
-    def run_step(i, t):
+    def run_step(i, t=0):
         if predictors is not None:
-            predictors[i % fwd.n_batches].forward()  # launches on the calling thread's stream and waits for it
+            predictors[i % NB].forward()  # launches on the calling thread's stream and waits for it
         else:
             fwd.step(i, stream_ptrs[t])
+            streams[t].synchronize()
 
-    # ---- throughput: W warm-up steps, then exactly K steps between two synchronisations.  The Predictor path is
+    # ---- throughput: warm-up, then exactly K steps between two synchronisations.  The Predictor path is
     # driven by the library's own serving threads (Blaze_ServePool*: a C++ loop per thread, as a serving binary
     # would run it); the kernel-layer path by Python threads.
     if predictors is not None:
-        from pyblaze_hip import ServePool
-        pool = ServePool(T)
-        pool.run(predictors, W)
+        pool = pb.ServePool(T)
+        pool.run(predictors, warm)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         pool.run(predictors, K)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-    else:
-        start = threading.Barrier(T + 1)
-        errors = []
-
-        def worker(t):
-            try:
-                for i in range(t, W, T):
-                    run_step(i, t)
-                torch.cuda.synchronize()
-                start.wait()
-                for i in range(t, K, T):
-                    run_step(W - (W % T) + i, t)
-            except Exception as e:  # noqa: BLE001
-                errors.append(e)
-                start.abort()
-
-        threads = [threading.Thread(target=worker, args=(t, )) for t in range(T)]
-        for th in threads:
-            th.start()
-        start.wait()
-        t0 = time.perf_counter()
-        for th in threads:
-            th.join()
+        dt = t1 - t0
+        s0 = time.perf_counter()
+        pool.run(predictors, S)
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        if errors:
-            raise errors[0]
-    ms_per_step = (t1 - t0) * 1e3 / K
-    samples_per_s = cfg.batch * K / (t1 - t0)
+        ds = time.perf_counter() - s0
+    else:
+        def run_region(first, count):
+            start = threading.Barrier(T + 1)
+            errors = []
+
+            def worker(t):
+                try:
+                    start.wait()
+                    for i in range(t, count, T):
+                        fwd.step(first + i, stream_ptrs[t])
+                    streams[t].synchronize()
+                except Exception as e:  # noqa: BLE001
+                    errors.append(e)
+
+            threads = [threading.Thread(target=worker, args=(t, )) for t in range(T)]
+            for th in threads:
+                th.start()
+            start.wait()
+            a = time.perf_counter()
+            for th in threads:
+                th.join()
+            torch.cuda.synchronize()
+            b = time.perf_counter()
+            if errors:
+                raise errors[0]
+            return b - a
+        run_region(0, warm)
+        dt = run_region(warm, K)
+        ds = run_region(warm + K, S)
+    steady = {"steps": S, "ms_per_step": round(ds * 1e3 / S, 5), "samples/s": round(cfg.batch * S / ds, 1)}
+    ms_per_step = dt * 1e3 / K
+    samples_per_s = cfg.batch * K / dt
 
     # ---- latency: one batch at a time on one thread, each step submitted and waited for on its own
-    lat = []
-    for i in range(min(K, 2000)):
-        a = time.perf_counter()
-        run_step(i, 0)
-        if predictors is None:
-            torch.cuda.synchronize()
-        lat.append((time.perf_counter() - a) * 1e3)
-    lat = np.sort(np.array(lat))
-    p50, p99 = float(lat[len(lat) // 2]), float(lat[int(len(lat) * 0.99)])
+    p50, p99, n_lat = latency_ms(np, run_step, max(K, 1000))
 
     # ---- PCIe-inclusive rate: every step feeds all 79 inputs from pageable host memory and copies the output back
-    feed_rate = None
-    if args.with_feed and predictors is not None:
+    if not args.no_feed and predictors is not None:
         fT = T
-        n_feed = max(fT, min(K, 400) // fT * fT)
+        n_feed = max(fT, min(max(K, 400), 800) // fT * fT)
         fbar = threading.Barrier(fT + 1)
-
         # one Blaze_PredictorFeedMany call per step (79 inputs); the argument arrays are built once per batch
         feeds = []
-        for b in range(fwd.n_batches):
+        for b in range(NB):
             items = []
             for (fg, _, _), (ids, vals, seg) in zip(fgs, sparse[b]):
                 items += [(fg + ".ids", ids), (fg + ".values", vals), (fg + ".segments", seg)]
@@ -237,7 +539,7 @@ def main():
             for i in range(t, n_feed + 2 * fT, fT):
                 if i == t + 2 * fT:
                     fbar.wait()
-                b = i % fwd.n_batches
+                b = i % NB
                 predictors[b].feed_many(feeds[b])
                 predictors[b].forward()
                 predictors[b].output_asnumpy("prob")
@@ -250,38 +552,17 @@ def main():
         for th in ths:
             th.join()
         f1 = time.perf_counter()
-        in_bytes = float(np.mean([sum(a.nbytes for trip in sparse[b] for a in trip) + dense[b].size * 2
-                                  for b in range(fwd.n_batches)]))
+        in_bytes = float(np.mean([sum(a.nbytes for trip in sparse[b] for a in trip) + dense[b].size * 2 for b in range(NB)]))
         feed_rate = {"samples/s": round(cfg.batch * n_feed / (f1 - f0), 1), "ms_per_step": round((f1 - f0) * 1e3 / n_feed, 4),
                      "host_bytes_per_step": int(in_bytes), "steps": n_feed, "threads": fT,
                      "note": "Feed of every input from pageable host memory + Forward + Output copy, per step"}
 
-    # ---- per-kernel durations: HIP events on the launch stream around a replayed HIP graph that holds
-    # R back-to-back launches of the one kernel (over the pooled batches), so host launch cost is not in it
-    def timed(fn, reps):
-        for i in range(fwd.n_batches):
-            fn(i)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for i in range(reps):
-                fn(i)
-        g.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        rounds = 5
-        e0.record()
-        for _ in range(rounds):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / (reps * rounds)  # us
-
-    R = 8 * fwd.n_batches
-    kern_us = {"bz_embed_pool_kernel": timed(fwd.pool, R)}
+    # ---- per-kernel durations
+    R = 8 * NB
+    kern_us = {"bz_embed_pool_kernel": graph_timed(torch, fwd.pool, NB, R)}
     for name, launch in fwd.launches():  # the FC launches one step makes (the skinny head rides in the layer before it)
-        kern_us[name] = timed(launch, R)
-    emb_bytes = float(np.mean([fwd.embedding_bytes(i) for i in range(fwd.n_batches)]))
+        kern_us[name] = graph_timed(torch, launch, NB, R)
+    emb_bytes = float(np.mean([fwd.embedding_bytes(i) for i in range(NB)]))
     flops = fwd.fc_flops()
     pool_us = kern_us["bz_embed_pool_kernel"]
     pool_gbs = emb_bytes / pool_us / 1e3
@@ -290,62 +571,25 @@ def main():
     dominant = max(kern_us, key=kern_us.get)
     if dominant != "bz_embed_pool_kernel":
         layers = [int(x) for x in dominant[6:-1].split("+")] if dominant.startswith("bz_fc[") else list(range(len(flops)))
-        ach = sum(flops[li] for li in layers) / kern_us[dominant] / 1e6
-        roofline = {"kernel": "%s (FC layers %s)" % (dominant, layers), "bound": "mfma", "achieved": round(ach, 2),
-                    "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / MFMA_PEAK_TFLOPS, 5), "traffic": None}
+        roofline = mfma_roofline("%s (FC layers %s)" % (dominant, layers), sum(flops[li] for li in layers), kern_us[dominant])
     else:
-        roofline = {"kernel": "bz_embed_pool_kernel", "bound": "hbm", "achieved": round(pool_gbs, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(pool_gbs / HBM_PEAK_GBS, 5),
-                    "traffic": POOL_TRAFFIC_BYTES if args.pool == 32 else None,
-                    "algorithmic_bytes_per_launch": int(emb_bytes), "avg_launch_us": round(pool_us, 2)}
+        traffic, source = pool_traffic_from_profile() if args.pool == 32 else (None, None)
+        roofline = hbm_roofline("bz_embed_pool_kernel", emb_bytes, pool_us, traffic)
+        roofline["traffic_source"] = source
 
-    # ---- CPU baseline: the oracle (a port of the reference's CPU path), one single-threaded predictor per thread.
-    # The products go to the optimised sgemm numpy links, as the reference's go to MKL's cblas_sgemm.
-    cpu = None
-    if not args.no_cpu_baseline:
-        import blaze_oracle as orc
-        from pipeline import oracle_forward
-        from threadpoolctl import threadpool_info, threadpool_limits
-        orc.build()
-        tabs = [orc.Table(t.cpu().numpy()) for t in tables]
-        mlp_np = [(w.cpu().numpy(), b.cpu().numpy(), s.cpu().numpy()) for (w, b, s) in mlp]
-        threads = max(1, min(16, len(os.sched_getaffinity(0))))
-        per_thread = 8
-        blas = next(("%s %s (%s)" % (i.get("internal_api"), i.get("version"), i.get("architecture"))
-                     for i in threadpool_info() if i.get("user_api") == "blas"), "numpy's matmul")
-        def worker(t):
-            for j in range(per_thread):
-                b = (t * per_thread + j) % len(sparse)
-                oracle_forward(orc, cfg, tabs, mlp_np, sparse[b], dense[b], blas=True)
-        with threadpool_limits(1, user_api="blas"):
-            oracle_forward(orc, cfg, tabs, mlp_np, sparse[0], dense[0], blas=True)  # warm the page cache of the tables
-            c0 = time.perf_counter()
-            ths = [threading.Thread(target=worker, args=(t, )) for t in range(threads)]
-            for t in ths:
-                t.start()
-            for t in ths:
-                t.join()
-            c1 = time.perf_counter()
-            s0 = time.perf_counter()  # ... and the same port on one core alone
-            for j in range(per_thread):
-                oracle_forward(orc, cfg, tabs, mlp_np, sparse[j % len(sparse)], dense[j % len(sparse)], blas=True)
-            s1 = time.perf_counter()
-        t0 = time.perf_counter()  # one batch with the oracle's own k-ascending sgemm, for the record
-        oracle_forward(orc, cfg, tabs, mlp_np, sparse[0], dense[0])
-        t1 = time.perf_counter()
-        model = ""
-        try:
-            with open("/proc/cpuinfo") as f:
-                model = next((line.split(":", 1)[1].strip() for line in f if line.startswith("model name")), "")
-        except OSError:
-            pass
-        cpu = {"value": round(cfg.batch * threads * per_thread / (c1 - c0), 1), "unit": "samples/s", "cores": threads,
-               "kind": "port", "value_1_core": round(cfg.batch * per_thread / (s1 - s0), 1),
-               "value_1_core_textbook_sgemm": round(cfg.batch / (t1 - t0), 1), "sgemm": blas,
-               "host_cpus": os.cpu_count(), "cpu_model": model,
-               "sample": "%d batches of %d (%d per thread, one single-threaded predictor per core), fp32 oracle: "
-                         "hash-free row lookup, ksum, sgemm of the BLAS numpy links on one thread + separate PReLU pass, "
-                         "softmax" % (threads * per_thread, cfg.batch, per_thread)}
+    del fwd
+    per_config = None
+    if not args.no_per_config:
+        per_config = {}
+        for key, fn in (("c1", lambda: bench_config1(np, torch, bz, pb, T)), ("c3", lambda: bench_config3(np, torch, pb, T)),
+                        ("c4", lambda: bench_config4(np, torch, bz)), ("c5", lambda: bench_config5(np, torch, bz))):
+            try:
+                per_config[key] = fn()
+            except Exception as e:  # noqa: BLE001  (one configuration failing must not lose the headline line)
+                per_config[key] = {"error": "%s: %s" % (type(e).__name__, e)}
+            torch.cuda.empty_cache()
+
+    cpu = None if args.no_cpu_baseline else cpu_baseline(np, cfg, tables, mlp, sparse, dense)
 
     out = {
         "metric": "samples/sec @batch 2048 fp16 (sparse CTR forward: embedding pool + FC stack)",
@@ -354,16 +598,19 @@ def main():
         "n_gpus": 1,
         "steps": K,
         "warmup": W,
+        "warmup_run": warm,
         "ms_per_step": round(ms_per_step, 5),
+        "steady_state": steady,
         "p50_ms": round(p50, 4),
         "p99_ms": round(p99, 4),
+        "latency_samples": n_lat,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic (seeded; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
         "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
-                   "batch_pool": fwd.n_batches,
+                   "batch_pool": NB,
                    "path": "kernel-layer C ABI (bz_*)" if predictors is None else "Predictor.Forward via Blaze_* C ABI",
                    "serving_threads": T,
                    "device": arch},
@@ -373,10 +620,10 @@ def main():
         "fc_stack": {"TFLOP/s": round(fc_tflops, 2), "frac_of_mfma_peak": round(fc_tflops / MFMA_PEAK_TFLOPS, 5),
                      "flops": int(sum(flops)), "us": round(fc_us, 2)},
         "kernel_us": {k: round(v, 2) for k, v in kern_us.items()},
+        "with_host_feed": feed_rate,
+        "per_config": per_config,
         "cpu_baseline": cpu,
     }
-    if feed_rate is not None:
-        out["with_host_feed"] = feed_rate
     print(json.dumps(out))
 
 

@@ -12,8 +12,8 @@
  * the GPU; -1 = probe; 0 (CPU) fails at operator creation: this build has no CPU execution path.
  *
  * Not provided by this build (they return -1 with a message): the model importers and the offline optimizer
- * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze, Blaze_OptimizeBlaze) and the text-to-QED table
- * builder (Blaze_QuickEmbeddingBuildFp32/Fp16).
+ * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze, Blaze_OptimizeBlaze).  The text-to-QED table
+ * builders of c_api_qed.h (Blaze_QuickEmbeddingBuildFp32/Fp16) are provided.
  */
 #ifndef BLAZE_C_API_H_
 #define BLAZE_C_API_H_
@@ -78,11 +78,13 @@ BLAZE_API int Blaze_PredictorListOutputNames(PredictorHandle handle, size_t* ndi
 BLAZE_API int Blaze_PredictorRegisterObservers(PredictorHandle handle, size_t ndim, const char** names);
 BLAZE_API int Blaze_PredictorDumpObservers(PredictorHandle handle, size_t* ndim, const char*** key, const char*** value);
 
-/* c_api_blaze_converter.h / c_api_blaze_optimizer.h / c_api_quick_embedding.h: not part of this build */
+/* c_api_blaze_converter.h:11-20 / c_api_blaze_optimizer.h: importers and optimizer passes are not part of this
+ * build; both return -1 with a message */
 BLAZE_API int Blaze_ConvertBlaze(const char* model_conf_file, const char* model_data_file, int model_type, int weight_type,
                                  int io_type, int x_type_num, const char** x_type_key, const int* x_type_value,
                                  const char* blaze_model_file, int binary);
 BLAZE_API int Blaze_OptimizeBlaze(const char* raw_model_file, const char* optimized_model_file, int binary);
+/* c_api_qed.h:13-21: text tables (meta file + per-table files under `path`) -> one QED file, fp32 or fp16 rows */
 BLAZE_API int Blaze_QuickEmbeddingBuildFp32(const char* path, const char* meta, const char* output_file, int thread_num);
 BLAZE_API int Blaze_QuickEmbeddingBuildFp16(const char* path, const char* meta, const char* output_file, int thread_num);
 
@@ -116,6 +118,11 @@ BLAZE_API int Blaze_PredictorOutputDevicePtr(PredictorHandle handle, const char*
  * transfer; the predictor's input tensors then view slices of that one device buffer. */
 BLAZE_API int Blaze_PredictorFeedMany(PredictorHandle handle, int count, const char* const* names, const void* const* data,
                                       const size_t* lens);
+
+/* number of device and pinned-host allocations the library has made for blobs, feed arenas and Embedding scratch in
+ * this process so far (no counterpart in the reference): unchanged across a stretch of requests = that stretch
+ * allocated nothing */
+BLAZE_API int Blaze_AllocationCount(int64_t* count);
 
 /* run Forward `count` times on the calling thread (benchmark loops without per-call host overhead) */
 BLAZE_API int Blaze_PredictorForwardN(PredictorHandle handle, int count);

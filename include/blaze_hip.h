@@ -93,6 +93,9 @@ typedef struct bz_embed_slot {
   void* out;                  /* device: block base + this item's column offset */
   int64_t rows;
   int64_t out_stride;         /* elements between consecutive samples of the block */
+  int64_t nnz;                /* elements of ids / values (SparsePullerInput::key_size).  The kernels never read ids or
+                                 values at or beyond nnz: a negative count is taken as 0 and running offsets stop at
+                                 nnz, so counts that disagree with the arrays cannot send a read outside them */
   uint32_t hash_bucket_size;
   int32_t pitch;              /* bytes between table rows */
   int32_t dim;
@@ -121,6 +124,8 @@ typedef struct bz_embed_launch {
   int32_t scan_first;   /* advice, set with fused_scan: 1 when so many workgroups per slot would each re-read the counts
                            before their first sample (batch * workgroups * 2 bytes per slot) that scanning once into
                            slot.offsets (bz_segments_to_offsets_slots) and planning again is the cheaper way */
+  int32_t max_batch;    /* largest slot.batch of the planned slots */
+  int32_t reserved_;
 } bz_embed_launch;
 
 /*
@@ -157,18 +162,6 @@ BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* 
 
 /* name of the pooling kernel as profilers report it (for tooling) */
 BZ_API const char* bz_embed_pool_kernel_name(void);
-
-/*
- * Measurement aid, no counterpart in the reference: a pure random gather of 64-byte rows, the access pattern of
- * the pooling kernel with everything else taken away.  `groups` four-lane groups each read `rows_per_group`
- * (1, 4, 8 or 16) rows at hashed positions of `region` (region_bytes >= 64, 16-byte aligned; all loads of a group are
- * issued before the first is used), fold them and write one 64-byte row to sink[group].  The caller times the launch;
- * bytes read = groups * rows_per_group * 64.  Row of load r of group g, 32-bit arithmetic: h = (g * rows_per_group + r) *
- * 2654435761 + seed; h ^= h >> 15; h *= 2246822519; h ^= h >> 13; row = (h * rows) >> 32 with rows = region_bytes / 64.
- * Fold: of each 16-byte quarter row, words 0 and 2 are summed and words 1 and 3 xor-ed over the group's rows.
- */
-BZ_API int bz_probe_gather64(const void* region, int64_t region_bytes, void* sink, int64_t groups, int rows_per_group,
-                             uint32_t seed, bz_stream_t stream);
 
 /* ------------------------------------------------------------------------- */
 /* Dense                                                                      */

@@ -13,6 +13,11 @@ blaze/blaze/test/operator/operator_test_common.h:20-84).  This script only reads
 those DATA files -- it imports and executes nothing from the reference -- and
 rewrites the numbers as JSON so the tests can run where the reference tree does
 not exist.  Output: tests/golden/reference_kats.json.
+
+It also copies two sets of DATA files the reference holds, byte for byte:
+  blaze/example/tdm_data/model_blaze_optimized (a binary NetDef, 217 ops)          -> model_blaze_optimized.bin
+  blaze/blaze/test/utest_data/store/quick_embedding/{meta,a_01,a_02,a_03}          -> quick_embedding/
+(the text tables of embedding_builder_test.cc:13-23).
 """
 import json
 import os
@@ -160,6 +165,14 @@ def main():
     with open(dst, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)
     print("wrote", dst, "cases:", len(out))
+    import shutil
+    here = os.path.dirname(os.path.abspath(__file__))
+    shutil.copyfile(os.path.join(root, "blaze/example/tdm_data/model_blaze_optimized"), os.path.join(here, "model_blaze_optimized.bin"))
+    os.makedirs(os.path.join(here, "quick_embedding"), exist_ok=True)
+    for name in ("meta", "a_01", "a_02", "a_03"):
+        shutil.copyfile(os.path.join(root, "blaze/blaze/test/utest_data/store/quick_embedding", name),
+                        os.path.join(here, "quick_embedding", name))
+    print("copied model_blaze_optimized.bin and quick_embedding/")
 
 
 if __name__ == "__main__":

@@ -42,7 +42,7 @@ def _bf16_round(x):
 def test_config1_fp32_end_to_end_through_predictor(oracle):
     import torch
     from ctr_model import build_manager, make_predictor
-    from pipeline import oracle_forward
+    from model_forward import ctr_forward as oracle_forward
     from synth import Config1
     cfg = Config1()
     print("config1 full size: batch %d, %d x [%d,%d] fp32" % (cfg.batch, cfg.slots, cfg.rows, cfg.dim), flush=True)
@@ -203,6 +203,7 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     tables, weights and intermediate tensors: 2e-3."""
     import torch
     import din_model
+    import model_forward
     torch.cuda.empty_cache()
     cfg = din_model.Config3()
     print("config3 full size: batch %d, history %d, 3 x [%d,%d] fp16" % (cfg.batch, cfg.T, cfg.rows, cfg.dim), flush=True)
@@ -220,7 +221,7 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
         ids = np.concatenate([batch[k + ".ids"], batch[k + "_his.ids"]])
         tabs[k] = _touched_table(oracle, t, ids)
     rnd = lambda a: np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
-    want = din_model.oracle_forward(oracle, cfg, tabs, weights, batch, rnd)
+    want = model_forward.din_forward(oracle, cfg, tabs, weights, batch, rnd)
     B, T, D3 = cfg.batch, cfg.T, 3 * cfg.dim
     # pooled blocks: exactly the oracle's fp32 result rounded to fp16
     assert np.array_equal(got["q"], want["q"])

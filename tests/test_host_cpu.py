@@ -287,7 +287,7 @@ def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle)
     """bench.py times the oracle with the products handed to the BLAS numpy links (as the reference hands them to
     MKL, math/gemm.cc:13-27).  That variant must be the same computation: on a scaled-down config 2 it agrees with
     the k-ascending sums the parity tests use to fp32 summation-order noise (rel 1e-5)."""
-    from pipeline import oracle_forward
+    from model_forward import ctr_forward as oracle_forward
     from synth import Config2
     cfg = Config2(batch=96, rows=5000, slots=5)
     tables = cfg.tables(device="cpu")
@@ -299,3 +299,106 @@ def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle)
     np.testing.assert_array_equal(pooled_b, pooled)
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-7)
     assert got.shape == (96, 2) and np.allclose(got.sum(1), 1.0, atol=1e-6)
+
+
+# ---------------------------------------------------------------- documents and reference-held data files
+def test_integration_c_snippet_compiles_against_the_header():
+    """The C example of INTEGRATION.md names only entry points include/blaze_c_api.h declares (gcc -fsyntax-only)."""
+    import subprocess
+    import tempfile
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```c\n(.*?)```", text, flags=re.S)
+    assert blocks, "no ```c block in INTEGRATION.md"
+    body = blocks[0].replace("...", "")
+    m = re.match(r"(\s*#include[^\n]*\n)(.*)", body, flags=re.S)
+    src = (m.group(1) + "#include <stdint.h>\nvoid example(const int* shape, void* ids, int nnz, void* out, size_t out_bytes) {\n" +
+           m.group(2) + "\n}\n")
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "snippet.c")
+        open(path, "w").write(src)
+        r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror=implicit-function-declaration", "-fsyntax-only", "-I",
+                            os.path.join(ROOT, "include"), path], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def _arg_value(a):
+    return (a.name, a.f if a.HasField("f") else None, a.i if a.HasField("i") else None, a.s if a.HasField("s") else None,
+            list(a.floats), list(a.ints), list(a.strings))
+
+
+def test_reference_binary_model_decodes_like_protobuf():
+    """tests/golden/model_blaze_optimized.bin is the binary NetDef the reference ships with its TDM example
+    (blaze/example/tdm_data/model_blaze_optimized, 217 operators; what Blaze_PredcitorManagerLoadModel reads,
+    predictor_manager_impl.cc:31-116).  The library's own wire reader must see exactly what protobuf sees: the file is
+    decoded by the C++ codec to text, the text is parsed by protobuf, and the result is compared field by field with
+    protobuf's direct parse of the bytes."""
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    from google.protobuf import text_format
+    wire = open(os.path.join(ROOT, "tests", "golden", "model_blaze_optimized.bin"), "rb").read()
+    ref = NetDef()
+    ref.ParseFromString(wire)
+    assert len(ref.op) == 217
+    text = pb.convert_netdef(wire, False, True).decode("latin-1")
+    got = NetDef()
+    text_format.Parse(text, got)
+    assert got.name == ref.name and got.run_mode == ref.run_mode and got.version == ref.version
+    assert [(v.name, v.dtype, v.level, v.input_type, v.feature_name) for v in got.external_input] == \
+           [(v.name, v.dtype, v.level, v.input_type, v.feature_name) for v in ref.external_input]
+    assert [(v.name, v.dtype) for v in got.external_output] == [(v.name, v.dtype) for v in ref.external_output]
+    assert len(got.op) == len(ref.op)
+    for a, b in zip(got.op, ref.op):
+        assert (a.type, a.name, list(a.input), list(a.output)) == (b.type, b.name, list(b.input), list(b.output))
+        assert [_arg_value(x) for x in a.arg] == [_arg_value(x) for x in b.arg]
+        # the text writer spells scalar fields out with their values whether or not the file set them, so presence
+        # may differ (device_id: 0) while the values may not
+        assert (a.device_option.device_type, a.device_option.device_id, a.device_option.is_pipe) == \
+               (b.device_option.device_type, b.device_option.device_id, b.device_option.is_pipe)
+    assert [_arg_value(x) for x in got.arg] == [_arg_value(x) for x in ref.arg]
+    # wire -> wire through the C++ codec: protobuf parses it to the same message apart from that presence
+    again = NetDef()
+    again.ParseFromString(pb.convert_netdef(wire, False, False))
+    assert len(again.op) == 217 and [o.type for o in again.op] == [o.type for o in ref.op]
+    assert sum(len(o.arg) for o in again.op) == sum(len(o.arg) for o in ref.op)
+    types = {o.type for o in ref.op}
+    assert "ConstantFill" in types and "Gemm" in types
+
+
+def _reference_text_tables():
+    """-> {table: (keys int64 [n], rows fp32 [n, dim])} of tests/golden/quick_embedding (the reference's
+    utest_data/store/quick_embedding: `key,w0,...` lines; the first weight column happens to hold a big integer)."""
+    d = os.path.join(ROOT, "tests", "golden", "quick_embedding")
+    out = {}
+    for name in ("a_01", "a_02", "a_03"):
+        keys, rows = [], []
+        for line in open(os.path.join(d, name)).read().split("\n"):
+            if not line:
+                continue
+            f = line.split(",")
+            keys.append(int(f[0]))
+            rows.append([np.float32(x) for x in f[1:]])
+        out[name] = (np.array(keys, np.int64), np.array(rows, np.float32))
+    return d, out
+
+
+def test_qed_builder_on_the_reference_text_tables(tmp_path, oracle):
+    """embedding_builder_test.cc:13-23 builds utest_data/store/quick_embedding and loads the result.  Same files here:
+    meta names three tables but its last line has no newline, so -- as the reference's ParseMeta -- two are built; the
+    file image holds the hash index the reference's HashTable dumps and the parsed rows."""
+    import pyblaze_hip as pb
+    d, tables = _reference_text_tables()
+    out = str(tmp_path / "ref_tables.qed")
+    pb.build_qed(d, "meta", out)
+    version, trie, parsed = _parse_qed(out)
+    assert version == 2000 and [g for g, _, _ in parsed] == [0, 1]
+    for (gid, himg, bimg), name in zip(parsed, ("a_01", "a_02")):
+        keys, rows = tables[name]
+        assert rows.shape[1] == 9 and len(keys) == {"a_01": 10, "a_02": 51}[name]
+        mine = oracle.HashTable(keys.astype(np.uint64), 1 + 4 * 9 * np.arange(len(keys), dtype=np.uint64))
+        assert bytes(mine.dump()) == himg
+        assert bimg[9:] == rows.tobytes()
+        if oracle.have_ref():
+            ref = oracle.RefStore(keys, rows)
+            assert bytes(ref.hash_dump()) == himg, "differs from the reference's HashTable::Dump"
+    if oracle.have_ref():
+        assert bytes(oracle.RefTrie(["a_01", "a_02"], [0, 1]).dump()) == trie

@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew", "bz_probe_gather64"
+    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 MAX_RANK = 6
@@ -32,14 +32,14 @@ class EmbedSlot(C.Structure):
     _fields_ = [("table", C.c_void_p), ("row_scale", C.c_void_p), ("hash_buckets", C.c_void_p),
                 ("hash_pairs", C.c_void_p), ("ids", C.c_void_p), ("values", C.c_void_p), ("segments", C.c_void_p),
                 ("offsets", C.c_void_p), ("out", C.c_void_p), ("rows", C.c_int64), ("out_stride", C.c_int64),
-                ("hash_bucket_size", C.c_uint32), ("pitch", C.c_int32), ("dim", C.c_int32), ("table_dtype", C.c_int32),
+                ("nnz", C.c_int64), ("hash_bucket_size", C.c_uint32), ("pitch", C.c_int32), ("dim", C.c_int32), ("table_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("udf", C.c_int32), ("trunc_dir", C.c_int32), ("trunc_num", C.c_int32),
                 ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("reserved_", C.c_int32)]
 
 
 class EmbedLaunch(C.Structure):
     _fields_ = [("n_slots", C.c_int32), ("total_wg", C.c_int32), ("wg_per_slot", C.c_int32), ("variant", C.c_int32),
-                ("fused_scan", C.c_int32), ("scan_first", C.c_int32)]
+                ("fused_scan", C.c_int32), ("scan_first", C.c_int32), ("max_batch", C.c_int32), ("reserved_", C.c_int32)]
 
 
 class FcDesc(C.Structure):
@@ -127,7 +127,7 @@ def lib():
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
-        l.bz_probe_gather64.argtypes = [vp, i64, vp, i64, C.c_int, C.c_uint32, vp]
+        l.bz_probe_gather.argtypes = [vp, i64, C.c_int, vp, vp, i64, C.c_int, C.c_uint32, vp]  # csrc/bz_probe.h, not public
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
@@ -285,6 +285,7 @@ class EmbeddingPlan:
                 s.dim = it["dim"]
             s.ids = it["ids"].data_ptr()
             s.values = it["values"].data_ptr()
+            s.nnz = it.get("nnz", min(it["ids"].numel(), it["values"].numel()))
             s.segments = seg.data_ptr()
             s.offsets = off.data_ptr() if off is not None else None
             s.out = out.data_ptr() + it.get("col", 0) * out.element_size()
@@ -311,6 +312,7 @@ class EmbeddingPlan:
         if not self.fused_scan:
             self.scan(stream)
         self.pool(stream)
+
 
 
 def segments_to_offsets(segments, stream=None):

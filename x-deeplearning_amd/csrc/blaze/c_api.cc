@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <mutex>
 #include <thread>
@@ -209,6 +210,8 @@ struct ServePool {
   std::mutex mu;
   std::condition_variable cv_work, cv_done;
   uint64_t generation = 0;
+  std::atomic<uint64_t> generation_hint{0};  // copy of `generation` that idle threads poll without the mutex
+  std::atomic<int> pending_hint{0};          // copy of `pending` that Run polls without the mutex
   int pending = 0;
   bool stop = false;
   // the job of the current generation
@@ -235,6 +238,11 @@ struct ServePool {
     for (;;) {
       int n_threads;
       {
+        // a job that follows the previous one at once (a warm-up run, then the timed one) should not pay a futex
+        // wake-up per thread: poll for a short while before going to sleep
+        const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(2000);
+        while (generation_hint.load(std::memory_order_acquire) == seen && std::chrono::steady_clock::now() < spin_until) {
+        }
         std::unique_lock<std::mutex> lock(mu);
         cv_work.wait(lock, [&] { return stop || generation != seen; });
         if (stop) return;
@@ -270,7 +278,8 @@ struct ServePool {
       }
       {
         std::lock_guard<std::mutex> lock(mu);
-        if (--pending == 0) cv_done.notify_all();
+        pending_hint.store(--pending, std::memory_order_release);
+        if (pending == 0) cv_done.notify_all();
       }
     }
   }
@@ -282,8 +291,16 @@ struct ServePool {
     failed = 0;
     error.clear();
     pending = (int)threads.size();
+    pending_hint.store(pending, std::memory_order_release);
     ++generation;
+    generation_hint.store(generation, std::memory_order_release);
     cv_work.notify_all();
+    lock.unlock();
+    // short jobs end before a sleeping caller could be woken: poll first, sleep only when the job is a long one
+    const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(5000);
+    while (pending_hint.load(std::memory_order_acquire) != 0 && std::chrono::steady_clock::now() < spin_until) {
+    }
+    lock.lock();
     cv_done.wait(lock, [&] { return pending == 0; });
     return failed.load() == 0;
   }
@@ -515,6 +532,11 @@ int Blaze_ConvertNetDef(const char* in, size_t len, int in_is_text, int out_is_t
   return 0;
 }
 
+int Blaze_AllocationCount(int64_t* count) {
+  if (count == nullptr) return Fail("AllocationCount: null argument");
+  *count = blaze::AllocationCount().load();
+  return 0;
+}
 int Blaze_PredictorInputDevicePtr(PredictorHandle handle, const char* name, void** ptr) {
   auto* p = reinterpret_cast<Predictor*>(handle);
   if (p == nullptr || ptr == nullptr) return -1;

@@ -99,6 +99,11 @@ bool Predictor::Feed(size_t idx, const void* data, size_t len) {
       HIPContext ctx(blob->device_option());
       ctx.Activate();
       hipStream_t st = ctx.hip_stream();
+      if (blob->unplaced()) {  // outgrew its slice of the FeedMany arena: back to memory of its own
+        const std::vector<TIndex> shape = blob->shape();
+        blob->DropArenaView();
+        blob->Reshape(shape);
+      }
       // stage in pinned memory and queue the transfer; a second Feed of the same input first waits for the first
       if (feed_done_ == nullptr) HIP_CHECK(hipEventCreateWithFlags(&feed_done_, hipEventDisableTiming));
       if (feed_pending_[idx]) {
@@ -173,6 +178,7 @@ bool Predictor::FeedMany(int count, const char* const* names, const void* const*
       arena_host_ = arena_dev_ = nullptr;
       arena_cap_ = 0;
       const size_t cap = total + total / 4;
+      AllocationCount() += 2;
       HIP_CHECK(hipHostMalloc((void**)&arena_host_, cap, hipHostMallocDefault));
       HIP_CHECK(hipMalloc((void**)&arena_dev_, cap));
       arena_cap_ = cap;
@@ -182,10 +188,9 @@ bool Predictor::FeedMany(int count, const char* const* names, const void* const*
     HIP_CHECK(hipEventRecord(feed_done_, st));
     for (const Item& it : in_arena) {
       Blob* blob = external_input_blob_[it.idx];
-      if (blob->data() != arena_dev_ + it.offset) {
-        const std::vector<TIndex> shape = blob->shape();
-        blob->RefReshape(shape, arena_dev_ + it.offset);
-      }
+      // (also when the slice did not move: this records the slice's new size and clears "unplaced")
+      const std::vector<TIndex> shape = blob->shape();
+      blob->RefReshape(shape, arena_dev_ + it.offset, /*arena_view=*/true);
       feed_pending_[it.idx] = true;
     }
     any_feed_pending_ = true;
@@ -204,6 +209,12 @@ int Predictor::InputDataType(const char* name) const {
 
 bool Predictor::ForwardLaunch() {
   try {
+    for (size_t i = 0; i < external_input_blob_.size(); ++i)
+      if (external_input_blob_[i]->unplaced()) {
+        last_error_for_thread() = "input " + net_->external_input()[i] + " was reshaped beyond its fed size and has not been fed since";
+        LOG_ERROR("%s", last_error_for_thread().c_str());
+        return false;
+      }
     if (any_feed_pending_) {
       // the transfers were queued on the feeding thread's stream: make this thread's stream wait for them
       for (Blob* b : external_input_blob_) {
@@ -253,6 +264,12 @@ bool Predictor::ForwardWait() {
 bool Predictor::Forward(const PredictorCallback&& cb) {
   try {
     if (forward_in_flight_ && !ForwardWait()) return false;  // a launch the caller never waited for
+    for (size_t i = 0; i < external_input_blob_.size(); ++i)
+      if (external_input_blob_[i]->unplaced()) {
+        last_error_for_thread() = "input " + net_->external_input()[i] + " was reshaped beyond its fed size and has not been fed since";
+        LOG_ERROR("%s", last_error_for_thread().c_str());
+        return false;
+      }
     if (any_feed_pending_) {
       // the transfers were queued on the feeding thread's stream: make this thread's stream wait for them
       for (Blob* b : external_input_blob_) {
@@ -381,6 +398,12 @@ void Predictor::DumpObservers(std::unordered_map<std::string, std::string>* dump
 
 void* Predictor::InputDevicePtr(const char* name) {
   const int idx = InputName2Idx(name);
+  if (idx >= 0 && external_input_blob_[idx]->unplaced()) {  // outgrew its feed-arena slice: memory of its own
+    Blob* blob = external_input_blob_[idx];
+    const std::vector<TIndex> shape = blob->shape();
+    blob->DropArenaView();
+    blob->Reshape(shape);
+  }
   // (a strided input -- one that lives inside a Concat's output -- has no plain buffer to hand out)
   return idx < 0 || external_input_blob_[idx]->pitch() != 0 ? nullptr : external_input_blob_[idx]->data();
 }

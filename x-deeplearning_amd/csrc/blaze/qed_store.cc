@@ -116,6 +116,9 @@ struct SlotCache : SparsePuller::DeviceCache {
   bz_embed_launch launch;
   int64_t* offsets = nullptr;  // scratch for the separate scan, when the planner advises it
   size_t offsets_cap = 0;      // in elements
+  // the tables the records point into: held so that a table replaced in the store (AddTable, Load) outlives the
+  // launches that may still read it
+  std::vector<std::shared_ptr<const DeviceTable>> tables;
   ~SlotCache() override {
     if (pinned) (void)hipHostFree(pinned);
     if (dev) (void)hipFree(dev);
@@ -140,6 +143,14 @@ Status QedHipSparsePuller::LoadImpl(const std::string& url) {
     LOG_ERROR("load quick embedding dict failed! url: %s", url.c_str());
     return kFail;
   }
+  is.seekg(0, std::ios::end);
+  const uint64_t file_bytes = (uint64_t)is.tellg();
+  is.seekg(0, std::ios::beg);
+  // sizes read from the file are checked against what is left of it before anything is allocated for them
+  auto left = [&]() -> uint64_t {
+    const std::streamoff at = is.tellg();
+    return at < 0 ? 0 : file_bytes - std::min<uint64_t>(file_bytes, (uint64_t)at);
+  };
   // [1] header
   char magic[31];
   is.read(magic, 31);
@@ -160,7 +171,7 @@ Status QedHipSparsePuller::LoadImpl(const std::string& url) {
   // [2] trie
   uint64_t trie_len = 0;
   is.read((char*)&trie_len, 8);
-  if (!is.good() || trie_len > (1ull << 32)) {
+  if (!is.good() || trie_len > (1ull << 32) || trie_len > left()) {
     LOG_ERROR("load trie failed! url: %s", url.c_str());
     return kFail;
   }
@@ -196,29 +207,29 @@ Status QedHipSparsePuller::LoadImpl(const std::string& url) {
     }
   }
   // [3] tables
-  std::map<uint16_t, std::unique_ptr<DeviceTable>> tables;
+  std::map<uint16_t, std::shared_ptr<DeviceTable>> tables;
   const int esz = ElemSize(file_value_type_);
   uint16_t gid;
   while (is.read((char*)&gid, 2)) {
     uint32_t nbucket = 0;
     is.read((char*)&nbucket, 4);
-    if (!is.good()) { LOG_ERROR("load hashtable failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
+    if (!is.good() || (uint64_t)nbucket * 8 > left()) { LOG_ERROR("load hashtable failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
     std::vector<uint64_t> buckets(nbucket);
     is.read((char*)buckets.data(), (std::streamsize)nbucket * 8);
     uint64_t pair_bytes = 0;
     is.read((char*)&pair_bytes, 8);
-    if (!is.good() || pair_bytes % 16 != 0) { LOG_ERROR("load hashtable failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
+    if (!is.good() || pair_bytes % 16 != 0 || pair_bytes > left()) { LOG_ERROR("load hashtable failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
     std::vector<uint64_t> pairs(pair_bytes / 8);
     is.read((char*)pairs.data(), (std::streamsize)pair_bytes);
     uint64_t blob_bytes = 0;
     is.read((char*)&blob_bytes, 8);
-    if (!is.good() || blob_bytes == 0) { LOG_ERROR("load weight blob failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
+    if (!is.good() || blob_bytes == 0 || blob_bytes > left()) { LOG_ERROR("load weight blob failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
     std::vector<unsigned char> blob(blob_bytes);
     is.read((char*)blob.data(), (std::streamsize)blob_bytes);
     if (!is.good()) { LOG_ERROR("load weight blob failed! url: %s gid: %d", url.c_str(), gid); return kFail; }
 
     const uint64_t n = pair_bytes / 16;
-    std::unique_ptr<DeviceTable> t(new DeviceTable());
+    std::shared_ptr<DeviceTable> t(new DeviceTable());
     t->value_type = file_value_type_;
     t->rows = (int64_t)n;
     if (n == 0) {
@@ -249,7 +260,7 @@ Status QedHipSparsePuller::LoadImpl(const std::string& url) {
     }
     tables[gid] = std::move(t);
   }
-  std::lock_guard<std::mutex> lock(mutex_);
+  std::unique_lock<std::shared_mutex> lock(mutex_);
   trie_paths_ = std::move(paths);
   tables_ = std::move(tables);
   return kOK;
@@ -261,7 +272,7 @@ Status QedHipSparsePuller::AddTable(const std::string& table_name, int value_typ
     BLAZE_CONDITION_THROW(value_type == kFloat || value_type == kFloat16 || value_type == kInt8, "Unsupported value type:", value_type);
     BLAZE_CONDITION_THROW(rows > 0 && dim > 0 && rows_ptr != nullptr, "AddTable: rows=", rows, " dim=", dim);
     BLAZE_CONDITION_THROW(value_type != kInt8 || scale != nullptr, "AddTable: int8 table needs a per-row scale");
-    std::unique_ptr<DeviceTable> t(new DeviceTable());
+    std::shared_ptr<DeviceTable> t(new DeviceTable());
     t->value_type = value_type;
     t->rows = rows;
     t->dim = dim;
@@ -283,7 +294,7 @@ Status QedHipSparsePuller::AddTable(const std::string& table_name, int value_typ
       }
       UploadHash(t.get(), k, r);
     }
-    std::lock_guard<std::mutex> lock(mutex_);
+    std::unique_lock<std::shared_mutex> lock(mutex_);
     uint16_t gid = 0;
     auto it = trie_paths_.find(table_name);
     if (it != trie_paths_.end() && it->second != 0xFF) {
@@ -303,15 +314,17 @@ Status QedHipSparsePuller::AddTable(const std::string& table_name, int value_typ
 }
 
 bool QedHipSparsePuller::LookupGid(const std::string& name, uint16_t* gid) const {
+  std::shared_lock<std::shared_mutex> lock(mutex_);
   auto it = trie_paths_.find(name);
   if (it == trie_paths_.end()) return false;
   *gid = it->second;
   return true;
 }
 
-const DeviceTable* QedHipSparsePuller::table(uint16_t gid) const {
+std::shared_ptr<const DeviceTable> QedHipSparsePuller::table(uint16_t gid) const {
+  std::shared_lock<std::shared_mutex> lock(mutex_);
   auto it = tables_.find(gid);
-  return it == tables_.end() ? nullptr : it->second.get();
+  return it == tables_.end() ? nullptr : it->second;
 }
 
 Status QedHipSparsePuller::Get(const std::vector<SparsePullerInput>&, std::vector<SparsePullerOutput>&) {
@@ -326,6 +339,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
   SlotCache* sc = static_cast<SlotCache*>(cache->get());
   std::vector<bz_embed_slot>& slots = sc->scratch;
   slots.clear();
+  std::vector<std::shared_ptr<const DeviceTable>> held;
   for (size_t i = 0; i < input.size(); ++i) {
     const SparsePullerInput& in = input[i];
     const SparsePullerOutput& out = output[i];
@@ -338,9 +352,10 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
     const int out_type = out.out_type ? out.out_type : in.value_type;
     BLAZE_CONDITION_THROW(out_type == kFloat || out_type == kFloat16, "Unsupported block type:", out_type);
     uint16_t gid = 0;
-    const DeviceTable* t = nullptr;
+    std::shared_ptr<const DeviceTable> t;
     if (LookupGid(in.name, &gid)) t = table(gid);  // table name miss: the block keeps its zeros
     if (t != nullptr && t->rows == 0) t = nullptr;
+    if (t != nullptr) held.push_back(t);
     if (t != nullptr)
       BLAZE_CONDITION_THROW(t->dim == in.dim, "table ", in.name, " has dim ", t->dim, " but the embedding config says ", in.dim);
     for (size_t k = 0; k < in.in_item.size(); ++k) {
@@ -362,6 +377,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
       s.ids = (const int64_t*)in.key;
       s.values = (const float*)in.value;
       s.segments = (const int32_t*)in.key_num;
+      s.nnz = (int64_t)in.key_size;
       s.offsets = nullptr;  // fused scan
       s.out = out.out_item[k].out;
       s.out_stride = (int64_t)out.out_item[k].stride;
@@ -373,6 +389,8 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
       slots.push_back(s);
     }
   }
+  // (the previous call's tables are let go only now: its launch has been waited for before this predictor runs again)
+  sc->tables.swap(held);
   if (slots.empty()) return kOK;
   BZ_CHECK(bz_embed_plan(slots.data(), (int)slots.size(), &sc->launch));
   hipStream_t st = (hipStream_t)stream;
@@ -382,6 +400,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
     for (const auto& s : slots) need += (size_t)s.batch + 1;
     if (sc->offsets_cap < need) {
       if (sc->offsets) HIP_CHECK(hipFree(sc->offsets));  // (its last reader finished: a predictor is waited for before its next pass)
+      ++AllocationCount();
       HIP_CHECK(hipMalloc((void**)&sc->offsets, need * sizeof(int64_t)));
       sc->offsets_cap = need;
     }
@@ -400,6 +419,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
       if (sc->pinned) HIP_CHECK(hipHostFree(sc->pinned));
       if (sc->dev) HIP_CHECK(hipFree(sc->dev));
       sc->cap = slots.size();
+      AllocationCount() += 2;
       HIP_CHECK(hipHostMalloc((void**)&sc->pinned, sc->cap * sizeof(bz_embed_slot), hipHostMallocDefault));
       HIP_CHECK(hipMalloc((void**)&sc->dev, sc->cap * sizeof(bz_embed_slot)));
     }

@@ -15,6 +15,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <shared_mutex>
 #include <string>
 #include <vector>
 
@@ -56,14 +57,16 @@ class QedHipSparsePuller : public SparsePuller {
                   const int64_t* keys, const float* scale);
   // table name -> gid exactly as Trie::Lookup answers (trie.cc:44-68), interior nodes included
   bool LookupGid(const std::string& name, uint16_t* gid) const;
-  const DeviceTable* table(uint16_t gid) const;
+  // (both take the store's lock shared; a table handed out stays alive while the caller holds the pointer, also
+  // when AddTable / Load replace it meanwhile)
+  std::shared_ptr<const DeviceTable> table(uint16_t gid) const;
 
  private:
   Status LoadImpl(const std::string& url);
   std::map<std::string, uint16_t> trie_paths_;  // every node path of the trie -> its value (0xFF on interior nodes)
-  std::map<uint16_t, std::unique_ptr<DeviceTable>> tables_;
+  std::map<uint16_t, std::shared_ptr<DeviceTable>> tables_;
   int file_value_type_ = kFloat;
-  mutable std::mutex mutex_;
+  mutable std::shared_mutex mutex_;  // Get* read the two maps shared, AddTable / Load replace them exclusively
 };
 
 }  // namespace store

@@ -2,6 +2,7 @@
 
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 #include <unordered_set>
 
@@ -16,8 +17,14 @@ std::unordered_set<void*>& PinnedSet() {
 }
 }  // namespace
 
+std::atomic<int64_t>& AllocationCount() {
+  static std::atomic<int64_t> n{0};
+  return n;
+}
+
 void* Alloc(size_t bytes, int device_type, int device_id) {
   if (bytes == 0) bytes = 16;
+  ++AllocationCount();
   void* p = nullptr;
   if (device_type == kCPU) {
     // pinned, so that Feed / Output copies are real DMA transfers instead of the runtime's staged pageable path

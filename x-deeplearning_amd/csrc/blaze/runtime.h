@@ -7,6 +7,7 @@
 // synchronisation inside operators.
 #pragma once
 
+#include <atomic>
 #include <memory>
 #include <vector>
 
@@ -19,6 +20,10 @@ namespace blaze {
 // (hipHostMalloc) whenever a device is usable, so Feed / Output copies run at full PCIe rate; plain malloc otherwise.
 void* Alloc(size_t bytes, int device_type, int device_id);
 void Free(void* ptr, int device_type, int device_id);
+// number of device / pinned-host allocations the host layer has made in this process (Alloc above plus the feed
+// arenas and the Embedding operator's slot and offset buffers): lets a serving loop check that its steady state
+// allocates nothing
+std::atomic<int64_t>& AllocationCount();
 
 class Blob {
  public:
@@ -35,6 +40,15 @@ class Blob {
     if (slices_ && slices_->parent != this && ReshapeAsSlice(dims)) return;
     TIndex n = 1;
     for (auto d : dims) n *= d;
+    if (arena_view_) {
+      // a view of a slice of its predictor's feed arena (Predictor::FeedMany): the next FeedMany places it again, so
+      // a new shape allocates nothing.  A shape that outgrows the slice leaves the blob "unplaced" until it is fed;
+      // Predictor::Forward refuses to run a net with an unplaced input.
+      size_ = n;
+      dims_ = dims;
+      if (size_ > capacity_) unplaced_ = true;
+      return;
+    }
     size_ = n;
     if (size_ > capacity_ || !own_handle_) {
       Destroy();
@@ -56,13 +70,16 @@ class Blob {
     size_ = n;
     dims_ = dims;
   }
-  void RefReshape(const std::vector<TIndex>& dims, void* handle) {
+  // arena_view: `handle` is a slice of the owning predictor's feed arena (see Reshape)
+  void RefReshape(const std::vector<TIndex>& dims, void* handle, bool arena_view = false) {
     if (own_handle_ || data_ != handle) {  // (re-aliasing the same buffer keeps the version)
       Destroy();
       own_handle_ = false;
       data_ = handle;
       ++version_;
     }
+    arena_view_ = arena_view;
+    unplaced_ = false;
     pitch_ = 0;
     slice_view_ = false;
     TIndex n = 1;
@@ -88,6 +105,17 @@ class Blob {
     g->widths = static_widths;
     parent->slices_ = g;
     for (Blob* c : children) c->slices_ = g;
+  }
+  // true after a Reshape beyond the feed-arena slice this blob views, until the next feed gives it memory
+  bool unplaced() const { return unplaced_; }
+  // gives an arena view memory of its own again (a single-input Feed after a FeedMany)
+  void DropArenaView() {
+    if (!arena_view_) return;
+    arena_view_ = unplaced_ = false;
+    data_ = nullptr;
+    capacity_ = 0;
+    own_handle_ = true;
+    ++version_;
   }
   // elements between consecutive rows when this blob is a column slice, else 0 (rows are contiguous)
   TIndex pitch() const { return pitch_; }
@@ -179,6 +207,8 @@ class Blob {
   uint64_t version_ = 0;
   TIndex pitch_ = 0;
   bool slice_view_ = false;
+  bool arena_view_ = false;
+  bool unplaced_ = false;
   std::shared_ptr<SliceGroup> slices_;
 };
 

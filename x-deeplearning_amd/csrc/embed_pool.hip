@@ -31,6 +31,7 @@
 #include <hip/hip_fp16.h>
 
 #include "bz_common.h"
+#include "bz_probe.h"
 
 namespace {
 
@@ -52,7 +53,9 @@ __device__ __forceinline__ int64_t wave_incl_scan(int64_t v, int lane) {
   return v;
 }
 
-__device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restrict__ off, int64_t n) {
+// Counts below zero are taken as zero and the running offset stops at `limit` (the length of the ids / values arrays),
+// so no offset this scan produces points outside them.
+__device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restrict__ off, int64_t n, int64_t limit) {
   __shared__ int64_t wave_tot[kThreads / bz::kWave];
   __shared__ int64_t carry_s;
   const int tid = threadIdx.x;
@@ -64,7 +67,7 @@ __device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restri
     int64_t i0 = base + (int64_t)tid * kScanItems;
     int32_t v[kScanItems];
 #pragma unroll
-    for (int k = 0; k < kScanItems; ++k) v[k] = (i0 + k < n) ? seg[i0 + k] : 0;
+    for (int k = 0; k < kScanItems; ++k) v[k] = (i0 + k < n) ? max(seg[i0 + k], 0) : 0;
     int64_t local = 0;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) local += v[k];
@@ -76,24 +79,32 @@ __device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restri
     int64_t run = before + incl - local;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) {
-      if (i0 + k < n) off[i0 + k] = run;
+      if (i0 + k < n) off[i0 + k] = run < limit ? run : limit;
       run += v[k];
     }
     __syncthreads();
     if (tid == kThreads - 1) carry_s = run;  // last thread's running total = total so far
     __syncthreads();
   }
-  if (tid == 0) off[n] = carry_s;
+  if (tid == 0) off[n] = carry_s < limit ? carry_s : limit;
 }
 
 __global__ __launch_bounds__(kThreads) void bz_scan_segments_kernel(const int32_t* __restrict__ seg,
                                                                     int64_t* __restrict__ off, int64_t n) {
-  scan_segments(seg, off, n);
+  scan_segments(seg, off, n, INT64_MAX);
 }
 
-__global__ __launch_bounds__(kThreads) void bz_scan_segments_slots_kernel(const bz_embed_slot* __restrict__ slots) {
+// ext_off != nullptr: slot i's offsets go to ext_off + i * ext_stride instead of slot.offsets (at most ext_stride - 1
+// samples of a slot are scanned, so a record whose batch disagrees with the plan cannot write past its share)
+__global__ __launch_bounds__(kThreads) void bz_scan_segments_slots_kernel(const bz_embed_slot* __restrict__ slots,
+                                                                          int64_t* __restrict__ ext_off, int64_t ext_stride) {
   const bz_embed_slot* s = &slots[blockIdx.x];
-  scan_segments(s->segments, s->offsets, s->batch);
+  if (ext_off != nullptr) {
+    const int64_t n = s->batch < ext_stride - 1 ? s->batch : ext_stride - 1;
+    scan_segments(s->segments, ext_off + (int64_t)blockIdx.x * ext_stride, n, s->nnz);
+  } else {
+    scan_segments(s->segments, s->offsets, s->batch, s->nnz);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -318,27 +329,32 @@ __device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int
 // ---------------------------------------------------------------------------------------------
 // s_off[0..groups] <- exclusive offsets of samples b0 .. b0+groups (clipped to batch).
 // Every thread of the workgroup calls it; ends with a barrier.
-__device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0, int groups, int64_t* s_off,
-                                              int64_t* s_part) {
+// `offsets`: the slot's precomputed offsets (slot.offsets, or its share of a buffer the launch brings), or nullptr.
+__device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, const int64_t* __restrict__ offsets, int64_t b0,
+                                              int groups, int64_t* s_off, int64_t* s_part) {
   const int tid = threadIdx.x;
   const int lane = tid & (bz::kWave - 1), wave = tid / bz::kWave;
-  if (s.offsets != nullptr) {
+  if (offsets != nullptr) {
     for (int t = tid; t <= groups; t += kThreads)
-      if (b0 + t <= s.batch) s_off[t] = s.offsets[b0 + t];
+      if (b0 + t <= s.batch) {
+        const int64_t o = offsets[b0 + t];
+        s_off[t] = o < 0 ? 0 : (o < s.nnz ? o : s.nnz);  // caller-made offsets get the same bounds as the scan's
+      }
     __syncthreads();
     return;
   }
   // base = sum of the counts before b0 (independent coalesced reads), local = this thread's sample
   // (8 loads in flight per thread: a rolled loop would wait for each load before issuing the next)
   // this thread's own count is requested first so that it travels with the counts summed below
-  const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)s.segments[b0 + tid] : 0;
+  // (a negative count is taken as 0 and the offsets below stop at nnz: see bz_embed_slot.nnz)
+  const int64_t mine = (tid < groups && b0 + tid < s.batch) ? (int64_t)max(s.segments[b0 + tid], 0) : 0;
   int64_t part = 0;
   for (int64_t i0 = 0; i0 < b0; i0 += 8 * kThreads) {
     int32_t c[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int64_t i = i0 + k * kThreads + tid;
-      c[k] = i < b0 ? s.segments[i] : 0;
+      c[k] = i < b0 ? max(s.segments[i], 0) : 0;
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) part += c[k];
@@ -358,8 +374,8 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, int64_t b0
     before += s_part[w];
     if (w < wave) before += s_part[kThreads / bz::kWave + w];
   }
-  if (tid < groups) s_off[tid + 1] = before + incl;
-  if (tid == 0) s_off[0] = before;
+  if (tid < groups) s_off[tid + 1] = (before + incl) < s.nnz ? (before + incl) : s.nnz;
+  if (tid == 0) s_off[0] = before < s.nnz ? before : s.nnz;
   __syncthreads();
 }
 
@@ -374,7 +390,8 @@ constexpr int64_t kScanFirstBytes = 128ll << 20;
 
 template <int DT, int LPR>
 __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
-                                                                 int total_wg, int wg_per_xcd, int wg_per_slot) {
+                                                                 int total_wg, int wg_per_xcd, int wg_per_slot,
+                                                                 const int64_t* __restrict__ ext_off, int64_t ext_stride) {
   constexpr int CE = RowTraits<DT>::kElems;
   constexpr int GROUPS = kThreads / LPR;
   constexpr int SRC = LPR < kBlockIds ? LPR : kBlockIds;  // lanes of a group that fetch ids
@@ -388,7 +405,7 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
   const int tid = threadIdx.x;
   const int g = tid / LPR, l = tid % LPR;
   const int64_t b0 = (int64_t)(v - si * wg_per_slot) * GROUPS;
-  stage_offsets(s, b0, GROUPS, s_off, s_part);
+  stage_offsets(s, ext_off != nullptr ? ext_off + (int64_t)si * ext_stride : s.offsets, b0, GROUPS, s_off, s_part);
   const int64_t b = b0 + g;
   if (b >= s.batch) return;
   const int nchunks = (s.dim + CE - 1) / CE;
@@ -475,7 +492,8 @@ __device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (
 
 __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const bz_embed_slot* __restrict__ slots,
                                                                          int n_slots, int total_wg, int wg_per_xcd,
-                                                                         int wg_per_slot) {
+                                                                         int wg_per_slot, const int64_t* __restrict__ ext_off,
+                                                                         int64_t ext_stride) {
   __shared__ int64_t s_off[kThreads + 1];
   __shared__ int64_t s_part[2 * kThreads / bz::kWave];
   // XCD-aware order: hardware deals consecutive workgroup ids round robin over the 8 XCDs; give
@@ -516,7 +534,7 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   if (i_last >= n_items) i_last = n_items - 1;
   const int64_t b_first = i0 / per;
   const int n_samples = (int)(i_last / per - b_first) + 1;  // <= groups
-  stage_offsets(s, b_first, n_samples, s_off, s_part);
+  stage_offsets(s, ext_off != nullptr ? ext_off + (int64_t)lo * ext_stride : s.offsets, b_first, n_samples, s_off, s_part);
   const int64_t item = i0 + g;
   if (item >= n_items) return;
   const int64_t b = item / per;
@@ -552,15 +570,17 @@ int groups_per_wg(const bz_embed_slot& s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// measurement aid: the pooling kernel's access pattern alone (random 64-byte rows, four lanes a row)
+// measurement aid: the pooling kernel's access pattern alone (random rows of LPR 16-byte chunks, one lane a chunk)
 // ---------------------------------------------------------------------------------------------
-template <int R>
+template <int R, int LPR>
 __global__ __launch_bounds__(kThreads) void bz_probe_gather_kernel(const uint4* __restrict__ region, uint4* __restrict__ sink,
-                                                                   uint32_t rows, int64_t groups, uint32_t seed) {
-  const int64_t gid = ((int64_t)blockIdx.x * kThreads + threadIdx.x) >> 2;
-  const int l = threadIdx.x & 3;
+                                                                   const float* __restrict__ side, uint32_t rows,
+                                                                   int64_t groups, uint32_t seed) {
+  const int64_t gid = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / LPR;
+  const int l = threadIdx.x % LPR;
   if (gid >= groups) return;
   uint4 v[R];
+  float sc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     uint32_t h = ((uint32_t)gid * R + r) * 2654435761u + seed;
@@ -568,17 +588,18 @@ __global__ __launch_bounds__(kThreads) void bz_probe_gather_kernel(const uint4* 
     h *= 2246822519u;
     h ^= h >> 13;
     const uint32_t row = (uint32_t)(((uint64_t)h * rows) >> 32);  // uniform over [0, rows)
-    v[r] = region[(size_t)row * 4 + l];
+    v[r] = region[(size_t)row * LPR + l];
+    sc[r] = side != nullptr ? side[row] : 0.f;  // every lane of the group asks for the same word: one request
   }
   uint4 acc = make_uint4(0, 0, 0, 0);
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    acc.x += v[r].x;
+    acc.x += v[r].x + __float_as_uint(sc[r]);
     acc.y ^= v[r].y;
     acc.z += v[r].z;
     acc.w ^= v[r].w;
   }
-  sink[(size_t)gid * 4 + l] = acc;
+  sink[(size_t)gid * LPR + l] = acc;
 }
 
 }  // namespace
@@ -597,7 +618,7 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
     BZ_REQUIRE(s.out_dtype == BZ_F32 || s.out_dtype == BZ_F16 || s.out_dtype == BZ_BF16, "slot %d: unsupported out dtype %d", i,
                s.out_dtype);
     BZ_REQUIRE(s.udf == BZ_SUM || s.udf == BZ_AVG || s.udf == BZ_ASSIGN, "slot %d: Unsupported udf type: %d", i, s.udf);
-    BZ_REQUIRE(s.dim > 0 && s.batch >= 0, "slot %d: dim=%d batch=%d", i, s.dim, s.batch);
+    BZ_REQUIRE(s.dim > 0 && s.batch >= 0 && s.nnz >= 0, "slot %d: dim=%d batch=%d nnz=%lld", i, s.dim, s.batch, (long long)s.nnz);
     if (s.udf == BZ_ASSIGN)
       BZ_REQUIRE(s.trunc_num > 0 && (s.trunc_dir == BZ_ORDER || s.trunc_dir == BZ_REVERSE),
                  "slot %d: kAssign needs trunc_num > 0 and a trunc direction (trunc_num=%d dir=%d)", i, s.trunc_num,
@@ -640,6 +661,10 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
   int64_t prefix_bytes = 0;
   for (int i = 0; i < n_slots; ++i) prefix_bytes += (int64_t)slots[i].wg_count * slots[i].batch * 2;
   launch->scan_first = (launch->fused_scan && prefix_bytes > kScanFirstBytes) ? 1 : 0;
+  int32_t max_batch = 0;
+  for (int i = 0; i < n_slots; ++i) max_batch = slots[i].batch > max_batch ? slots[i].batch : max_batch;
+  launch->max_batch = max_batch;
+  launch->reserved_ = 0;
   return BZ_OK;
 }
 
@@ -653,23 +678,23 @@ int bz_segments_to_offsets(const int32_t* segments, int64_t* offsets, int64_t n,
 
 int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_slots, bz_stream_t stream) {
   BZ_REQUIRE(slots_dev != nullptr && n_slots > 0, "bz_segments_to_offsets_slots: null argument or n_slots=%d", n_slots);
-  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(n_slots), dim3(kThreads), 0, bz::as_stream(stream), slots_dev);
+  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(n_slots), dim3(kThreads), 0, bz::as_stream(stream), slots_dev,
+                     (int64_t*)nullptr, (int64_t)0);
   BZ_LAUNCH_OK("bz_scan_segments_slots_kernel");
   return BZ_OK;
 }
 
-int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
-  BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool: null argument");
-  const bz_embed_launch& L = *launch;
+// launches the pooling kernel the plan chose; ext_off (may be nullptr) replaces slot.offsets as described at the kernels
+static int launch_pool(const bz_embed_slot* slots_dev, const bz_embed_launch& L, const int64_t* ext_off, int64_t ext_stride,
+                       hipStream_t st) {
   BZ_REQUIRE(L.n_slots > 0 && L.total_wg >= 0 && L.wg_per_slot >= 0, "bz_embed_pool: bad launch record (n_slots=%d total_wg=%d)",
              L.n_slots, L.total_wg);
   if (L.total_wg == 0) return BZ_OK;
   const int per_xcd = (L.total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
   const dim3 grid(per_xcd * bz::kNumXcd), block(kThreads);
-  hipStream_t st = bz::as_stream(stream);
   if (L.variant == 0) {
     hipLaunchKernelGGL(bz_embed_pool_generic_kernel, grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd,
-                       ((int64_t)L.wg_per_slot * L.n_slots == L.total_wg) ? L.wg_per_slot : 0);
+                       ((int64_t)L.wg_per_slot * L.n_slots == L.total_wg) ? L.wg_per_slot : 0, ext_off, ext_stride);
     BZ_LAUNCH_OK("bz_embed_pool_generic_kernel");
     return BZ_OK;
   }
@@ -678,7 +703,7 @@ int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch,
   const int dt = L.variant >> 8, lpr = L.variant & 0xff;
 #define BZ_POOL(DT, LPR)                                                                                             \
   hipLaunchKernelGGL((bz_embed_pool_kernel<DT, LPR>), grid, block, 0, st, slots_dev, L.n_slots, L.total_wg, per_xcd, \
-                     L.wg_per_slot)
+                     L.wg_per_slot, ext_off, ext_stride)
 #define BZ_POOL_LPR(DT)                                                                      \
   switch (lpr) {                                                                             \
     case 1: BZ_POOL(DT, 1); break;                                                           \
@@ -702,27 +727,43 @@ int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch,
   return BZ_OK;
 }
 
+int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
+  BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool: null argument");
+  return launch_pool(slots_dev, *launch, nullptr, 0, bz::as_stream(stream));
+}
+
 const char* bz_embed_pool_kernel_name(void) { return "bz_embed_pool_kernel"; }
 
-int bz_probe_gather64(const void* region, int64_t region_bytes, void* sink, int64_t groups, int rows_per_group,
-                      uint32_t seed, bz_stream_t stream) {
-  BZ_REQUIRE(region != nullptr && sink != nullptr && region_bytes >= 64 && ((uintptr_t)region & 15) == 0 &&
-                 ((uintptr_t)sink & 15) == 0,
-             "bz_probe_gather64: null or misaligned buffer (region_bytes=%lld)", (long long)region_bytes);
-  BZ_REQUIRE(groups > 0 && groups <= (1ll << 28), "bz_probe_gather64: groups=%lld outside (0, 2^28]", (long long)groups);
-  const int64_t rows = region_bytes / 64;
-  BZ_REQUIRE(rows < (1ll << 32), "bz_probe_gather64: region larger than 2^32 rows");
-  const dim3 grid((unsigned)((groups * 4 + kThreads - 1) / kThreads)), block(kThreads);
+int bz_probe_gather(const void* region, int64_t region_bytes, int row_bytes, const float* side, void* sink, int64_t groups,
+                    int rows_per_group, uint32_t seed, bz_stream_t stream) {
+  BZ_REQUIRE(region != nullptr && sink != nullptr && ((uintptr_t)region & 15) == 0 && ((uintptr_t)sink & 15) == 0,
+             "bz_probe_gather: null or misaligned buffer");
+  BZ_REQUIRE(row_bytes == 64 || row_bytes == 128, "bz_probe_gather: row_bytes=%d is not 64 or 128", row_bytes);
+  BZ_REQUIRE(region_bytes >= row_bytes, "bz_probe_gather: region_bytes=%lld", (long long)region_bytes);
+  BZ_REQUIRE(groups > 0 && groups <= (1ll << 28), "bz_probe_gather: groups=%lld outside (0, 2^28]", (long long)groups);
+  const int64_t rows = region_bytes / row_bytes;
+  BZ_REQUIRE(rows < (1ll << 32), "bz_probe_gather: region larger than 2^32 rows");
+  const int lpr = row_bytes / 16;
+  const dim3 grid((unsigned)((groups * lpr + kThreads - 1) / kThreads)), block(kThreads);
   hipStream_t st = bz::as_stream(stream);
   const uint4* t = (const uint4*)region;
   uint4* out = (uint4*)sink;
+#define BZ_PROBE(R, LPR) \
+  hipLaunchKernelGGL((bz_probe_gather_kernel<R, LPR>), grid, block, 0, st, t, out, side, (uint32_t)rows, groups, seed)
+#define BZ_PROBE_R(R)      \
+  if (lpr == 4)            \
+    BZ_PROBE(R, 4);        \
+  else                     \
+    BZ_PROBE(R, 8)
   switch (rows_per_group) {
-    case 1: hipLaunchKernelGGL(bz_probe_gather_kernel<1>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
-    case 4: hipLaunchKernelGGL(bz_probe_gather_kernel<4>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
-    case 8: hipLaunchKernelGGL(bz_probe_gather_kernel<8>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
-    case 16: hipLaunchKernelGGL(bz_probe_gather_kernel<16>, grid, block, 0, st, t, out, (uint32_t)rows, groups, seed); break;
-    default: return bz::fail(BZ_EINVAL, "bz_probe_gather64: rows_per_group=%d is not 1, 4, 8 or 16", rows_per_group);
+    case 1: BZ_PROBE_R(1); break;
+    case 4: BZ_PROBE_R(4); break;
+    case 8: BZ_PROBE_R(8); break;
+    case 16: BZ_PROBE_R(16); break;
+    default: return bz::fail(BZ_EINVAL, "bz_probe_gather: rows_per_group=%d is not 1, 4, 8 or 16", rows_per_group);
   }
+#undef BZ_PROBE_R
+#undef BZ_PROBE
   BZ_LAUNCH_OK("bz_probe_gather_kernel");
   return BZ_OK;
 }

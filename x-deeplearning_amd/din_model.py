@@ -1,5 +1,4 @@
-"""Config 3: a DIN-style model (attention over the behaviour history) as a Blaze NetDef, plus the same forward
-on the CPU oracle (harness for the parity tests).
+"""Config 3: a DIN-style model (attention over the behaviour history) as a Blaze NetDef (harness for the parity tests and the benchmark).
 
 Graph (operator types and arguments as the reference's importer emits them for such a model,
 blaze/model_importer/ulf_importer.cc; structure after tools/example_model/din/model/graph_ulf.txt):
@@ -163,46 +162,3 @@ def feed(p, inputs, batch, dtype=np.float16):
     for name in inputs:
         a = batch[name]
         p.feed(name, a.astype(dtype) if name == "mask" else a)
-
-
-def oracle_forward(oracle, cfg, tables_np, weights, batch, rnd):
-    """The same graph on the CPU oracle.  tables_np: {kind: oracle.Table}; rnd: rounding applied to every operator
-    output (identity for fp32, fp16 round trip for the fp16 model).  -> dict of named fp32 arrays."""
-    B, T, D = cfg.batch, cfg.T, cfg.dim
-    q = np.zeros((B, 3 * D), np.float32)
-    his_k = []
-    for i, k in enumerate(KINDS):
-        oracle.embed_get(tables_np[k], batch[k + ".ids"], batch[k + ".values"], batch[k + ".segments"], [(0, 0, 0, q, i * D)])
-        blk = np.zeros((B, T * D), np.float32)
-        oracle.embed_get(tables_np[k], batch[k + "_his.ids"], batch[k + "_his.values"], batch[k + "_his.segments"],
-                         [(2, 0, T, blk, 0)])
-        his_k.append(oracle.reshape(rnd(blk), [-1, T, D]))
-    q = rnd(q)
-    his = oracle.concat(his_k, 2)
-    q3 = oracle.reshape(q, [-1, 1, 3 * D])
-    sub = rnd(oracle.elementwise("Sub", q3, his))
-    mul = rnd(oracle.elementwise("Mul", q3, his))
-    bq = oracle.broadcast_to(q3, like=sub)
-    x = oracle.concat([bq, his, sub, mul], 2)
-    n_att = len(weights["att"])
-    for li, l in enumerate(weights["att"]):
-        w, b = rnd(l["w"]), rnd(l["b"])
-        x = oracle.gemm_op(x, w, b)
-        if li < n_att - 1:
-            x = oracle.dice(x, rnd(l["gamma"]), rnd(l["mean"]), rnd(l["var"]))
-        x = rnd(x)
-    score = x
-    att_w = rnd(oracle.elementwise("Mul", score, rnd(batch["mask"])))
-    att = oracle.reshape(rnd(oracle.matmul_op(att_w, his, True, False)), [-1, 3 * D])
-    hsum = rnd(oracle.reduce_sum(his, 1, 0))
-    x = oracle.concat([q, hsum, att], 1)
-    main_in = x
-    n_main = len(weights["main"])
-    for li, l in enumerate(weights["main"]):
-        w, b = rnd(l["w"]), rnd(l["b"])
-        x = oracle.gemm_op(x, w, b)
-        if li < n_main - 1:
-            x = rnd(oracle.dice(x, rnd(l["gamma"]), rnd(l["mean"]), rnd(l["var"])))
-    logit = rnd(x)
-    return dict(q=q, his=his, att_in=None, score=score, att=att, hsum=hsum, main_in=main_in, logit=logit,
-                prob=oracle.softmax(logit, 1))

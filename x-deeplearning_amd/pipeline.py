@@ -152,33 +152,3 @@ class CtrForward:
     def fc_flops(self):
         L = self.cfg.layers
         return [2.0 * self.cfg.batch * L[i] * L[i + 1] for i in range(len(L) - 1)]
-
-
-def oracle_forward(oracle, cfg, tables_np, mlp_np, sparse, dense, in_round=None, blas=False):
-    """The same forward on the CPU oracle (fp32 path fed the kernel's rounded inputs).  tables_np: list of
-    oracle.Table; mlp_np: [(W [K,N] fp32, b, slope)].  Returns (pooled [B, in_dim] fp32, probs [B, 2]).
-    blas=True hands the products to the optimised sgemm numpy links (the reference calls MKL's cblas_sgemm there,
-    math/gemm.cc:13-27) for timing a CPU baseline; its summation order is the library's, so parity tests keep the
-    default k-ascending sums."""
-    B = cfg.batch
-    x = np.zeros((B, cfg.in_dim), np.float32)
-    x[:, :cfg.dense] = dense if in_round is None else in_round(dense)
-    for s, (ids, vals, seg) in enumerate(sparse):
-        oracle.embed_get(tables_np[s], ids, vals, seg, [(0, 0, 0, x, cfg.dense + s * cfg.dim)])
-    h = x if in_round is None else in_round(x)
-    pooled = h.copy()
-    n = len(mlp_np)
-    for li, (w, b, slope) in enumerate(mlp_np):
-        if blas:
-            y = np.matmul(h, w)
-            y += b  # the Gemm operator's bias broadcast
-            h = oracle.softmax(y, 1) if li == n - 1 else oracle.prelu(y, slope)
-            continue
-        wt = np.ascontiguousarray(w.T)  # [N,K] + transB: same k-ascending sums, contiguous inner loop
-        if li == n - 1:
-            h = oracle.fc(h, wt, b, act="softmax", transb=True)
-        else:
-            h = oracle.fc(h, wt, b, act="prelu", act_params=(slope, ), transb=True)
-            if in_round is not None:
-                h = in_round(h)
-    return pooled, h

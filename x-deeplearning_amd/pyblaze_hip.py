@@ -29,7 +29,7 @@ EXPORTS = [
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
     "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_PredictorForwardLaunch",
-    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany"
+    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount"
 ]
 
 
@@ -54,6 +54,7 @@ def lib():
         l.Blaze_PredictorManagerSetRunMode.argtypes = [vp, cp]
         l.Blaze_LoadSparseModelWeight.argtypes = [vp, cp]
         l.Blaze_PredcitorManagerLoadModel.argtypes = [vp, cp, i]
+        l.Blaze_PredictorManagerLoadModel.argtypes = [vp, cp, i]
         l.Blaze_PredictorManagerLoadModelFromString.argtypes = [vp, cp, sz, i]
         l.Blaze_PredictorManagerLoadDeepNetModel.argtypes = [vp, cp, cp, i]
         l.Blaze_PredictorCreate.argtypes = [vp, i, i, C.POINTER(vp)]
@@ -86,8 +87,16 @@ def lib():
         l.Blaze_PredictorForwardLaunch.argtypes = [vp]
         l.Blaze_PredictorForwardWait.argtypes = [vp]
         l.Blaze_PredictorFeedMany.argtypes = [vp, i, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_size_t)]
+        l.Blaze_AllocationCount.argtypes = [C.POINTER(C.c_int64)]
         _lib = l
     return _lib
+
+
+def allocation_count():
+    """device / pinned-host allocations the library has made in this process so far"""
+    n = C.c_int64()
+    check_call(lib().Blaze_AllocationCount(C.byref(n)))
+    return n.value
 
 
 def last_error():
