@@ -160,6 +160,21 @@ BZ_API int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_sl
  */
 BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream);
 
+/*
+ * bz_segments_to_offsets_slots + bz_embed_pool for callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The offsets of every slot (the scan
+ * scratch that slot.offsets otherwise brings in; slot.offsets is ignored here) live in a buffer of
+ * BZ_EMBED_STATIC_SCRATCH_BYTES inside the library, one per GPU, held until the process ends.  The call makes two
+ * launches on `stream` (scan of every slot's segments into that buffer, then the pooling kernel the plan chose reading
+ * its offsets from there) and calls no hipMalloc / hipFree or other allocating routine.  Results are those of the
+ * two-call form, bit for bit.
+ * Limit: n_slots * (launch->max_batch + 1) * 8 bytes must fit the buffer, else BZ_EINVAL (config 5, 200 slots x batch
+ * 8192, takes 13.1 MB).  All calls on one GPU share the one buffer: calls whose launches may overlap on the device
+ * (different streams, no ordering between them) race on it; calls on one stream, or ordered by events, do not.
+ */
+#define BZ_EMBED_STATIC_SCRATCH_BYTES (16u << 20)
+BZ_API int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream);
+
 /* name of the pooling kernel as profilers report it (for tooling) */
 BZ_API const char* bz_embed_pool_kernel_name(void);
 

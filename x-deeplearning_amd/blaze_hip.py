@@ -20,7 +20,7 @@ ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 
 
 EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
-    "bz_embed_pool", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
+    "bz_embed_pool", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
     "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
@@ -126,6 +126,7 @@ def lib():
         l.bz_segments_to_offsets.argtypes = [vp, vp, i64, vp]
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
+        l.bz_embed_pool_static_scratch.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
         l.bz_probe_gather.argtypes = [vp, i64, C.c_int, vp, vp, i64, C.c_int, C.c_uint32, vp]  # csrc/bz_probe.h, not public
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
@@ -313,6 +314,9 @@ class EmbeddingPlan:
             self.scan(stream)
         self.pool(stream)
 
+    def run_static_scratch(self, stream=None):
+        """scan + pool with the offsets in the library's own static buffer (the entry point that allocates nothing)"""
+        check(lib().bz_embed_pool_static_scratch(self.slots_dev.data_ptr(), C.byref(self.launch), _stream_ptr(stream)))
 
 
 def segments_to_offsets(segments, stream=None):

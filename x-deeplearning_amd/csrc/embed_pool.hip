@@ -30,6 +30,8 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "bz_common.h"
 #include "bz_probe.h"
 
@@ -602,6 +604,33 @@ __global__ __launch_bounds__(kThreads) void bz_probe_gather_kernel(const uint4* 
   sink[(size_t)gid * LPR + l] = acc;
 }
 
+// ---------------------------------------------------------------------------------------------
+// scratch of the entry point that allocates nothing: every slot's offsets, inside the library's own device image
+// ---------------------------------------------------------------------------------------------
+constexpr int64_t kStaticScratchEntries = BZ_EMBED_STATIC_SCRATCH_BYTES / sizeof(int64_t);
+static __device__ __align__(256) int64_t scratch[kStaticScratchEntries];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle: the address
+// comes from hipGetSymbolAddress, asked once per device with that device current (every GPU holds its own copy of the
+// array at its own address), and only that pointer is ever handed to a kernel.
+constexpr int kMaxDevices = 64;
+int static_scratch_ptr(int64_t** out) {
+  static std::mutex mu;
+  static int64_t* ptr[kMaxDevices] = {};
+  int dev = -1;
+  BZ_HIP_OK(hipGetDevice(&dev));
+  BZ_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptr[dev] == nullptr) {
+    void* p = nullptr;
+    BZ_HIP_OK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    BZ_REQUIRE(p != nullptr, "hipGetSymbolAddress gave no address for the scratch buffer on device %d", dev);
+    ptr[dev] = static_cast<int64_t*>(p);
+  }
+  *out = ptr[dev];
+  return BZ_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -730,6 +759,25 @@ static int launch_pool(const bz_embed_slot* slots_dev, const bz_embed_launch& L,
 int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
   BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool: null argument");
   return launch_pool(slots_dev, *launch, nullptr, 0, bz::as_stream(stream));
+}
+
+int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
+  BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool_static_scratch: null argument");
+  const bz_embed_launch& L = *launch;
+  BZ_REQUIRE(L.n_slots > 0 && L.max_batch >= 0, "bz_embed_pool_static_scratch: bad launch record (n_slots=%d max_batch=%d)",
+             L.n_slots, L.max_batch);
+  const int64_t stride = (int64_t)L.max_batch + 1;  // int64 entries per slot
+  BZ_REQUIRE((int64_t)L.n_slots * stride <= kStaticScratchEntries,
+             "bz_embed_pool_static_scratch: %d slots x (batch %d + 1) offsets = %lld bytes exceed the library's %u-byte buffer",
+             L.n_slots, L.max_batch, (long long)((int64_t)L.n_slots * stride * 8), BZ_EMBED_STATIC_SCRATCH_BYTES);
+  int64_t* off = nullptr;
+  const int rc = static_scratch_ptr(&off);
+  if (rc != BZ_OK) return rc;
+  hipStream_t st = bz::as_stream(stream);
+  // nothing to clear: the scan writes entries [0, batch] of every slot's share, the only ones the pooling kernel reads
+  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(L.n_slots), dim3(kThreads), 0, st, slots_dev, off, stride);
+  BZ_LAUNCH_OK("bz_scan_segments_slots_kernel");
+  return launch_pool(slots_dev, L, off, stride, st);
 }
 
 const char* bz_embed_pool_kernel_name(void) { return "bz_embed_pool_kernel"; }
