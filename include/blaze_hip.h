@@ -73,7 +73,10 @@ BZ_API int bz_device_check(char* name, size_t cap);
  * Table layout (repacked at load time from the QED blob, whose rows start at
  * byte offset 1 and are unaligned, blaze/store/quick_embedding/weight_blob.h:20,42-52):
  * row r starts at table + r*pitch, pitch is a multiple of 16 bytes, the base is
- * 16-byte aligned, bytes between dim*sizeof(elem) and pitch are zero.
+ * 16-byte aligned, bytes between dim*sizeof(elem) and pitch are zero (or hold the
+ * row's scale, see row_scale).  The memory system fetches whole 128-byte lines, so
+ * a table is best laid out with rows that do not straddle lines: bz_table_pitch
+ * gives the pitch this library's own loaders use.
  *
  * ids are row numbers (id outside [0, rows) = not in table) unless hash_buckets is
  * set; then ids are 64-bit keys resolved exactly as HashTable::Lookup does
@@ -82,7 +85,8 @@ BZ_API int bz_device_check(char* name, size_t cap);
  */
 typedef struct bz_embed_slot {
   const void* table;          /* device; NULL = unknown table: the item's columns are zero-filled */
-  const float* row_scale;     /* device [rows]; BZ_I8 tables only */
+  const float* row_scale;     /* device; BZ_I8 tables only: the scale of row r is the float at byte offset
+                                 r * scale_pitch from here (a dense array, or a field inside each table row) */
   const uint64_t* hash_buckets; /* device [hash_bucket_size] records {offset:40 (bytes into pairs), size:24}; or NULL */
   const uint64_t* hash_pairs;   /* device (key,row) pairs */
   const int64_t* ids;         /* device [nnz]   "<fg>.ids"      */
@@ -107,8 +111,16 @@ typedef struct bz_embed_slot {
   int32_t batch;
   int32_t wg_begin;           /* filled by bz_embed_plan: first workgroup of this slot */
   int32_t wg_count;           /* filled by bz_embed_plan */
-  int32_t reserved_;
+  int32_t scale_pitch;        /* bytes between the scales of consecutive rows; 0 = 4 (a dense float array) */
 } bz_embed_slot;
+
+/*
+ * Row pitch in bytes that keeps rows inside 128-byte lines: row_bytes rounded up to 16, then to the next power of two
+ * when that is at most 128, or to a multiple of 128 when that costs at most a third more memory.  scale_bytes (0 or 4)
+ * is room for a per-row scale stored behind the row's elements (int8 tables), at byte offset
+ * round_up(row_bytes, 4) of the row.
+ */
+BZ_API int32_t bz_table_pitch(int64_t row_bytes, int scale_bytes);
 
 /*
  * Launch geometry of one Embedding invocation, produced on the host by bz_embed_plan

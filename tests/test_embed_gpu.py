@@ -334,3 +334,103 @@ def test_gather_probe_reads_the_rows_it_claims(bz, per, row_bytes, with_side):
     # error convention
     assert bz.lib().bz_probe_gather(d_region.data_ptr(), rows * row_bytes, row_bytes, None, sink.data_ptr(), groups, 3, seed, None) != 0
     assert b"rows_per_group" in bz.lib().bz_last_error()
+
+
+def _lengths_case(rng, kind, batch):
+    if kind == "poisson8":
+        return np.clip(rng.poisson(8, batch), 0, 64).astype(np.int32)
+    if kind == "mostly_empty":      # far more owned segments than ids: the reduction runs in rounds
+        return (rng.random(batch) < 0.03).astype(np.int32) * rng.integers(1, 4, batch).astype(np.int32)
+    if kind == "all_empty":
+        return np.zeros(batch, np.int32)
+    if kind == "giants":            # segments far longer than what a workgroup stages behind its range
+        seg = rng.integers(0, 3, batch).astype(np.int32)
+        seg[rng.choice(batch, 6, replace=False)] = rng.integers(700, 2600, 6)
+        return seg
+    if kind == "ones":
+        return np.ones(batch, np.int32)
+    if kind == "empty_ends":
+        seg = rng.integers(1, 20, batch).astype(np.int32)
+        seg[:37] = 0
+        seg[-41:] = 0
+        return seg
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["poisson8", "mostly_empty", "all_empty", "giants", "ones", "empty_ends"])
+@pytest.mark.parametrize("tdtype,dim,batch", [("f16", 32, 2048), ("f16", 64, 8192), ("f32", 16, 131), ("i8", 64, 4096),
+                                              ("f16", 18, 1023), ("f32", 3, 4100), ("f16", 128, 600)])
+def test_pooling_segment_shapes_that_stress_the_bookkeeping(bz, oracle, kind, tdtype, dim, batch):
+    """Segment shapes that stress the offset bookkeeping of the pooling kernels: very long segments among short ones,
+    runs of empty segments (at the ends too), no ids at all, batches that are not multiples of the workgroup's share,
+    hashed keys, absent ids, int8 rows with the scale inside the row.  ksum and kavg in one launch, with the fused scan
+    and with offsets scanned first; fp32 block bit-exact against the oracle."""
+    import torch
+    rng = np.random.default_rng(abs(hash((kind, tdtype, dim, batch))) % (2**31))
+    rows = 3000
+    slots = 3
+    if tdtype == "i8":
+        data = [rng.integers(-127, 128, (rows, dim)).astype(np.int8) for _ in range(slots)]
+        scale = [rng.uniform(1e-3, 1e-2, rows).astype(np.float32) for _ in range(slots)]
+    else:
+        npdt = np.float16 if tdtype == "f16" else np.float32
+        data = [(rng.standard_normal((rows, dim)) * 0.1).astype(npdt) for _ in range(slots)]
+        scale = [None] * slots
+    keys = [None, np.unique(rng.integers(-2**50, 2**50, rows * 2, dtype=np.int64))[:rows], None]
+    out = torch.full((batch, slots * dim), float("nan"), dtype=torch.float32, device="cuda")
+    want = np.full((batch, slots * dim), np.nan, np.float32)
+    items, keep = [], []
+    for s in range(slots):
+        seg = _lengths_case(rng, kind, batch)
+        nnz = int(seg.sum())
+        if keys[s] is None:
+            ids = rng.integers(-2, rows + 2, nnz).astype(np.int64)           # a few ids outside the table
+        else:
+            ids = rng.choice(np.concatenate([keys[s], np.array([7, -7], np.int64)]), nnz).astype(np.int64)
+        vals = rng.uniform(0.5, 1.5, nnz).astype(np.float32)
+        t = bz.DeviceTable(data[s], scale=scale[s], keys=keys[s])
+        d = [_dev(ids), _dev(vals), _dev(seg)]
+        keep.append((t, d))
+        udf = bz.AVG if s == 1 else bz.SUM
+        items.append(dict(table=t, ids=d[0], values=d[1], segments=d[2], out=out, col=s * dim, udf=udf))
+        oracle.embed_get(oracle.Table(data[s], scale=scale[s], keys=keys[s]), ids, vals, seg, [(udf, 0, 0, want, s * dim)])
+    plan = bz.EmbeddingPlan(items, fused_scan=True)
+    print("segment-shape case %s %s dim=%d batch=%d: %d workgroups" % (kind, tdtype, dim, batch, plan.launch.total_wg), flush=True)
+    plan.run()
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # ... and from offsets scanned in a launch of their own
+    out2 = torch.full_like(out, float("nan"))
+    for it in items:
+        it["out"] = out2
+    bz.EmbeddingPlan(items, fused_scan=False).run()
+    torch.cuda.synchronize()
+    assert np.array_equal(out2.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_pooling_unaligned_counts_and_trailing_empty_segments(bz, oracle):
+    """The counts array at an address that is not a multiple of 16, and batches whose ids end long before the samples
+    do (only empty segments behind them)."""
+    import torch
+    rng = np.random.default_rng(99)
+    rows, dim, batch = 2000, 32, 515
+    data = (rng.standard_normal((rows, dim)) * 0.1).astype(np.float16)
+    t = bz.DeviceTable(data)
+    for total in (512, 1024, 1536):
+        seg = np.zeros(batch, np.int32)
+        seg[:total // 4] = 4           # exactly `total` ids, then only empty segments
+        ids = rng.integers(0, rows, total).astype(np.int64)
+        vals = rng.uniform(0.5, 1.5, total).astype(np.float32)
+        holder = torch.zeros(batch + 3, dtype=torch.int32, device="cuda")
+        d_seg = holder[3:]             # 12 bytes past a 16-byte boundary
+        d_seg.copy_(torch.from_numpy(seg))
+        assert d_seg.data_ptr() % 16 == 12
+        out = torch.full((batch, dim), float("nan"), dtype=torch.float32, device="cuda")
+        d_ids, d_vals = _dev(ids), _dev(vals)
+        plan = bz.EmbeddingPlan([dict(table=t, ids=d_ids, values=d_vals, segments=d_seg, out=out, udf=bz.SUM)])
+        plan.run()
+        torch.cuda.synchronize()
+        want = np.full((batch, dim), np.nan, np.float32)
+        oracle.embed_get(oracle.Table(data), ids, vals, seg, [(0, 0, 0, want, 0)])
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))

@@ -258,9 +258,10 @@ def test_embedding_planner_geometry_and_scan_advice():
     import ctypes as C
     import blaze_hip as bz
 
-    def plan(n_slots, batch, dim, udf=bz.SUM, trunc=0, offsets=False, dtype=bz.F16):
+    def plan(n_slots, batch, dim, udf=bz.SUM, trunc=0, offsets=False, dtype=bz.F16, nnz=0):
         slots = (bz.EmbedSlot * n_slots)()
         for s in slots:
+            s.nnz = nnz
             s.table, s.ids, s.values, s.segments, s.out = 0x10000, 0x20000, 0x30000, 0x40000, 0x50000
             s.rows, s.dim, s.pitch = 1000, dim, (dim * 2 + 15) // 16 * 16
             s.table_dtype, s.out_dtype, s.udf, s.batch = dtype, bz.F16, udf, batch
@@ -271,13 +272,14 @@ def test_embedding_planner_geometry_and_scan_advice():
         assert bz.lib().bz_embed_plan(slots, n_slots, C.byref(launch)) == 0, bz.lib().bz_last_error()
         return slots, launch
 
-    slots, launch = plan(26, 2048, 32)           # config 2: dim 32 fp16 = 4 chunks -> 128 samples per 512-thread workgroup
+    slots, launch = plan(26, 2048, 32, nnz=16400)  # config 2: dim 32 fp16 = 4 chunks -> 128 samples per 512-thread workgroup
     assert launch.total_wg == 26 * 16 and launch.wg_per_slot == 16 and launch.fused_scan == 1 and launch.scan_first == 0
     assert launch.variant == (bz.F16 << 8) | 4
     assert [s.wg_begin for s in slots][:3] == [0, 16, 32]
-    _, launch = plan(200, 8192, 64)              # config 5: 8 chunks -> 64 samples per workgroup, 128 workgroups a slot
+    assert launch.max_batch == 2048
+    _, launch = plan(200, 8192, 64, nnz=20480)   # config 5: 8 chunks -> 64 samples per workgroup, 128 workgroups a slot
     assert launch.total_wg == 200 * 128 and launch.fused_scan == 1 and launch.scan_first == 1
-    _, launch = plan(200, 8192, 64, offsets=True)
+    _, launch = plan(200, 8192, 64, offsets=True, nnz=20480)
     assert launch.fused_scan == 0 and launch.scan_first == 0
     slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 128 positions per workgroup
     assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 128] * 3

@@ -19,7 +19,7 @@ ORDER, REVERSE = 0, 1
 ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 2, 3, 4, 5
 
 EXPORTS = [
-    "bz_last_error", "bz_device_check", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
+    "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
     "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
@@ -34,7 +34,7 @@ class EmbedSlot(C.Structure):
                 ("offsets", C.c_void_p), ("out", C.c_void_p), ("rows", C.c_int64), ("out_stride", C.c_int64),
                 ("nnz", C.c_int64), ("hash_bucket_size", C.c_uint32), ("pitch", C.c_int32), ("dim", C.c_int32), ("table_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("udf", C.c_int32), ("trunc_dir", C.c_int32), ("trunc_num", C.c_int32),
-                ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("reserved_", C.c_int32)]
+                ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("scale_pitch", C.c_int32)]
 
 
 class EmbedLaunch(C.Structure):
@@ -122,6 +122,8 @@ def lib():
             raise BlazeHipError("%s does not export %s (stale build?)" % (LIB_PATH, ", ".join(missing)))
         l.bz_last_error.restype = C.c_char_p
         l.bz_device_check.argtypes = [C.c_char_p, C.c_size_t]
+        l.bz_table_pitch.argtypes = [i64, C.c_int]
+        l.bz_table_pitch.restype = i32
         l.bz_embed_plan.argtypes = [C.POINTER(EmbedSlot), C.c_int, C.POINTER(EmbedLaunch)]
         l.bz_segments_to_offsets.argtypes = [vp, vp, i64, vp]
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
@@ -178,13 +180,15 @@ def bz_dtype(t):
 
 # ----------------------------------------------------------------------------------- tables
 class DeviceTable:
-    """An embedding table repacked for the kernels: row pitch padded to 16 bytes, zero padding.
+    """An embedding table repacked for the kernels: rows at the pitch bz_table_pitch gives (rows stay inside 128-byte
+    lines), zero padding; the per-row scale of an int8 table sits behind the row's elements, in the same line.
 
     rows: torch tensor [rows, dim] on cuda (float32 | float16 | int8) or a numpy array (uploaded).
     keys: optional int64/uint64 numpy array -> device hash index with the reference's bucket rule.
+    pitch: "line" (default), "tight" (row bytes rounded up to 16, scale in an array of its own), or a byte count.
     """
 
-    def __init__(self, rows, scale=None, keys=None, device="cuda"):
+    def __init__(self, rows, scale=None, keys=None, device="cuda", pitch="line"):
         import torch
         if isinstance(rows, np.ndarray):
             if rows.dtype == np.uint16:
@@ -195,7 +199,14 @@ class DeviceTable:
         self.rows, self.dim = rows.shape
         esz = rows.element_size()
         row_bytes = self.dim * esz
-        self.pitch = (row_bytes + 15) // 16 * 16
+        in_row_scale = scale is not None and pitch != "tight"
+        if pitch == "line":
+            self.pitch = lib().bz_table_pitch(row_bytes, 4 if in_row_scale else 0)
+        elif pitch == "tight":
+            self.pitch = (row_bytes + 15) // 16 * 16
+        else:
+            self.pitch = int(pitch)
+            assert self.pitch % 16 == 0 and self.pitch >= row_bytes + (4 if in_row_scale else 0)
         if self.pitch == row_bytes:
             self.data = rows.contiguous()
         else:
@@ -204,10 +215,19 @@ class DeviceTable:
             self.data = pad
         assert self.data.data_ptr() % 16 == 0
         self.scale = None
+        self.scale_ptr, self.scale_pitch = None, 0
         if scale is not None:
             if isinstance(scale, np.ndarray):
                 scale = torch.from_numpy(np.ascontiguousarray(scale, dtype=np.float32))
-            self.scale = scale.to(device=device, dtype=torch.float32).contiguous()
+            scale = scale.to(device=device, dtype=torch.float32).contiguous()
+            if in_row_scale:
+                at = (row_bytes + 3) // 4 * 4
+                assert self.data.dtype == torch.int8 and at + 4 <= self.pitch
+                self.data.view(torch.uint8).view(self.rows, self.pitch)[:, at:at + 4] = scale.view(torch.uint8).view(self.rows, 4)
+                self.scale_ptr, self.scale_pitch = self.data.data_ptr() + at, self.pitch
+            else:
+                self.scale = scale
+                self.scale_ptr, self.scale_pitch = scale.data_ptr(), 4
         self.hash_buckets = self.hash_pairs = None
         self.hash_bucket_size = 0
         if keys is not None:
@@ -274,7 +294,8 @@ class EmbeddingPlan:
             s = arr[i]
             if t is not None:
                 s.table = t.data.data_ptr()
-                s.row_scale = t.scale.data_ptr() if t.scale is not None else None
+                s.row_scale = t.scale_ptr
+                s.scale_pitch = t.scale_pitch
                 s.hash_buckets = t.hash_buckets.data_ptr() if t.hash_buckets is not None else None
                 s.hash_pairs = t.hash_pairs.data_ptr() if t.hash_pairs is not None else None
                 s.hash_bucket_size = t.hash_bucket_size

@@ -35,7 +35,7 @@ REGISTER_SPARSE_PULLER_CREATION("qed_sparse_puller", CreateQedHipSparsePuller);
 DeviceTable::~DeviceTable() {
   if (!owns) return;
   if (data) (void)hipFree(data);
-  if (row_scale) (void)hipFree(row_scale);
+  if (row_scale && scale_pitch != pitch) (void)hipFree(row_scale);  // (a scale stored inside the rows is part of `data`)
   if (hash_buckets) (void)hipFree(hash_buckets);
   if (hash_pairs) (void)hipFree(hash_pairs);
 }
@@ -57,7 +57,7 @@ int ElemSize(int value_type) { return value_type == kFloat ? 4 : (value_type == 
 
 // upload rows (host, unpadded, in `order`) to a pitched device table
 void UploadRows(DeviceTable* t, const unsigned char* rows_host, int64_t row_bytes, const std::vector<int64_t>* order) {
-  t->pitch = (int)((row_bytes + 15) / 16 * 16);
+  t->pitch = bz_table_pitch(row_bytes, 0);  // rows never straddle the 128-byte lines the memory system fetches
   std::vector<unsigned char> staged((size_t)t->rows * t->pitch, 0);
   for (int64_t r = 0; r < t->rows; ++r) {
     const int64_t src = order ? (*order)[r] : r;
@@ -277,14 +277,18 @@ Status QedHipSparsePuller::AddTable(const std::string& table_name, int value_typ
     t->rows = rows;
     t->dim = dim;
     const int64_t row_bytes = (int64_t)dim * ElemSize(value_type);
-    t->pitch = (int)((row_bytes + 15) / 16 * 16);
+    t->pitch = bz_table_pitch(row_bytes, scale ? 4 : 0);
+    BLAZE_CONDITION_THROW(t->pitch > 0, "AddTable: row of ", row_bytes, " bytes");
     HIP_CHECK(hipMalloc(&t->data, (size_t)rows * t->pitch));
     if (t->pitch != row_bytes) HIP_CHECK(hipMemset(t->data, 0, (size_t)rows * t->pitch));
     HIP_CHECK(hipMemcpy2D(t->data, t->pitch, rows_ptr, row_bytes, row_bytes, rows,
                           on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice));
     if (scale) {
-      HIP_CHECK(hipMalloc((void**)&t->row_scale, rows * 4));
-      HIP_CHECK(hipMemcpy(t->row_scale, scale, rows * 4, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice));
+      // the scale travels with its row: one line fetch per id instead of two
+      const int64_t at = (row_bytes + 3) / 4 * 4;
+      t->row_scale = (float*)((char*)t->data + at);
+      t->scale_pitch = t->pitch;
+      HIP_CHECK(hipMemcpy2D(t->row_scale, t->pitch, scale, 4, 4, rows, on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice));
     }
     if (keys) {
       std::vector<uint64_t> k(rows), r(rows);
@@ -364,6 +368,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
       if (t) {
         s.table = t->data;
         s.row_scale = t->row_scale;
+        s.scale_pitch = t->scale_pitch;
         s.hash_buckets = t->hash_buckets;
         s.hash_pairs = t->hash_pairs;
         s.hash_bucket_size = t->hash_bucket_size;

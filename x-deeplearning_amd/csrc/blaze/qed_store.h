@@ -31,7 +31,8 @@ struct DeviceTable {
   int64_t rows = 0;
   int pitch = 0;
   void* data = nullptr;       // device
-  float* row_scale = nullptr; // device
+  float* row_scale = nullptr; // device: scale of row r at byte offset r * scale_pitch (inside `data` when scale_pitch == pitch)
+  int scale_pitch = 0;
   uint64_t* hash_buckets = nullptr;
   uint64_t* hash_pairs = nullptr;
   uint32_t hash_bucket_size = 0;

@@ -44,7 +44,7 @@ constexpr int kUnroll = 4;  // rows in flight per lane group in the generic kern
 // ---------------------------------------------------------------------------------------------
 // segments -> offsets (exclusive scan), one workgroup per array
 // ---------------------------------------------------------------------------------------------
-constexpr int kScanItems = 8;  // int32 per thread per tile -> 2048 per workgroup tile
+constexpr int kScanItems = 16;  // int32 per thread per tile -> 8192 per workgroup tile (a batch of 8192 in one pass)
 
 __device__ __forceinline__ int64_t wave_incl_scan(int64_t v, int lane) {
 #pragma unroll
@@ -148,6 +148,40 @@ __device__ __forceinline__ void widen(const uint4& raw, float scale, float (&w)[
         int q = (int)(int8_t)((r[i] >> (8 * b)) & 0xffu);
         w[4 * i + b] = __fmul_rn(scale, (float)q);
       }
+    }
+  }
+}
+
+// scale of row r of an int8 table (a dense float array, or a field inside the table's rows)
+__device__ __forceinline__ float load_scale(const bz_embed_slot& s, int64_t r) {
+  return *(const float*)((const char*)s.row_scale + r * (int64_t)(s.scale_pitch != 0 ? s.scale_pitch : 4));
+}
+
+// acc += value * (the weights of one 16-byte chunk), the product rounded, then the sum rounded (udf_processor.h:66: never
+// one fused operation).  For fp16 rows the widening rides in the multiply: fma(widen(h), value, +0) is the correctly
+// rounded product (a product of -0 comes out as +0, which adds the same).  UNIT: the caller knows value == 1, so the
+// product is the weight itself and acc + w is a single rounding, fma(widen(h), 1, acc) -- one instruction per element
+// where the general form takes three.
+template <int DT, bool UNIT>
+__device__ __forceinline__ void accum_chunk(float (&acc)[RowTraits<DT>::kElems], const uint4& raw, float scale, float value) {
+  const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+  if constexpr (DT == BZ_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float w = __uint_as_float(r[i]);
+      acc[i] = __fadd_rn(acc[i], UNIT ? w : __fmul_rn(value, w));
+    }
+  } else if constexpr (DT == BZ_F16) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float w = __half2float(__ushort_as_half((unsigned short)((r[i / 2] >> (16 * (i & 1))) & 0xffffu)));
+      acc[i] = UNIT ? __builtin_fmaf(w, 1.0f, acc[i]) : __fadd_rn(acc[i], __builtin_fmaf(w, value, 0.0f));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float w = __fmul_rn(scale, (float)(int)(int8_t)((r[i / 4] >> (8 * (i & 3))) & 0xffu));
+      acc[i] = __fadd_rn(acc[i], UNIT ? w : __fmul_rn(value, w));
     }
   }
 }
@@ -257,7 +291,7 @@ __device__ __forceinline__ void pool_sum(const bz_embed_slot& s, int64_t start, 
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t r = row[u] < 0 ? 0 : row[u];
       raw[u] = *(const uint4*)(table + r * (int64_t)s.pitch);
-      sc[u] = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
+      sc[u] = (DT == BZ_I8) ? load_scale(s, r) : 1.f;
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -304,7 +338,7 @@ __device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t star
     if (r >= 0) {
       const float val = s.values[start + j];
       const uint4 raw = *(const uint4*)(table + r * (int64_t)s.pitch);
-      const float sc = (DT == BZ_I8) ? s.row_scale[r] : 1.f;
+      const float sc = (DT == BZ_I8) ? load_scale(s, r) : 1.f;
       float w[CE];
       widen<DT>(raw, sc, w);
 #pragma unroll
@@ -443,9 +477,9 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
 #pragma unroll
     for (int k = 0; k < KPL; ++k) {
       row_own[k] = (l < SRC && k * SRC + l < cnt) ? (int)resolve_row(s, id_next[k]) : -1;
-      // an id without a row contributes value 0 times a zero row: adding +0 leaves the running sum as it is (the
-      // sum starts at +0 and so is never -0), which lets the accumulation below run without the row numbers
-      val_own[k] = row_own[k] >= 0 ? val_next[k] : 0.f;
+      // an id without a row contributes a zero row (times the value 1): adding +0 leaves the running sum as it is
+      // (the sum starts at +0 and so is never -0), which lets the accumulation below run without the row numbers
+      val_own[k] = row_own[k] >= 0 ? val_next[k] : 1.f;
     }
     if (j + kBlockIds < end) fetch_ids(j + kBlockIds);
     int row[kBlockIds];
@@ -463,16 +497,19 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
       sc[u] = 1.f;
       if (has_chunk && row[u] >= 0) {  // row[u] is -1 beyond cnt
         raw[u] = *(const uint4*)(table + (int64_t)row[u] * s.pitch);
-        if (DT == BZ_I8) sc[u] = s.row_scale[row[u]];
+        if (DT == BZ_I8) sc[u] = load_scale(s, row[u]);
       }
     }
+    // ids that carry no weight (value 1, the usual case) take the one-rounding form, when that holds for every lane of the wave
+    bool unit = true;
 #pragma unroll
-    for (int u = 0; u < kBlockIds; ++u) {
-      float w[CE];
-      widen<DT>(raw[u], sc[u], w);
-      // out = out + value * w: two roundings, never an FMA (udf_processor.h:66)
+    for (int u = 0; u < kBlockIds; ++u) unit &= val[u] == 1.f;
+    if (__all(unit)) {
 #pragma unroll
-      for (int i = 0; i < CE; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(val[u], w[i]));
+      for (int u = 0; u < kBlockIds; ++u) accum_chunk<DT, true>(acc, raw[u], sc[u], 1.f);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kBlockIds; ++u) accum_chunk<DT, false>(acc, raw[u], sc[u], val[u]);
     }
   }
   if (s.udf == BZ_AVG) {
@@ -635,6 +672,19 @@ int static_scratch_ptr(int64_t** out) {
 
 extern "C" {
 
+int32_t bz_table_pitch(int64_t row_bytes, int scale_bytes) {
+  if (row_bytes <= 0 || row_bytes > (1 << 24)) return 0;
+  int64_t need = (row_bytes + 3) / 4 * 4 + (scale_bytes > 0 ? 4 : 0);
+  need = (need + 15) / 16 * 16;
+  if (need <= 128) {
+    int64_t p = 16;
+    while (p < need) p <<= 1;
+    return (int32_t)p;
+  }
+  const int64_t lines = (need + 127) / 128 * 128;
+  return (int32_t)(lines * 3 <= need * 4 ? lines : need);
+}
+
 int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
   BZ_REQUIRE(slots != nullptr && launch != nullptr && n_slots > 0, "bz_embed_plan: null argument or n_slots=%d", n_slots);
   int64_t total = 0;
@@ -659,8 +709,10 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
                  "slot %d: row pitch %d must be a multiple of 16 covering dim*elem=%d", i, s.pitch, s.dim * esz);
       BZ_REQUIRE(((uintptr_t)s.table & 15) == 0, "slot %d: table base not 16-byte aligned", i);
       BZ_REQUIRE(s.table_dtype != BZ_I8 || s.row_scale != nullptr, "slot %d: int8 table without row_scale", i);
+      BZ_REQUIRE(s.scale_pitch >= 0 && s.scale_pitch % 4 == 0 && ((uintptr_t)s.row_scale & 3) == 0,
+                 "slot %d: scale_pitch=%d / row_scale must be multiples of 4", i, s.scale_pitch);
       BZ_REQUIRE(s.rows > 0 && s.rows < (1ll << 31), "slot %d: rows=%lld outside (0, 2^31)", i, (long long)s.rows);
-      BZ_REQUIRE(s.ids != nullptr && s.values != nullptr, "slot %d: null ids/values", i);
+      BZ_REQUIRE(s.nnz == 0 || (s.ids != nullptr && s.values != nullptr), "slot %d: null ids/values", i);
       if (s.hash_buckets != nullptr)
         BZ_REQUIRE(s.hash_pairs != nullptr && s.hash_bucket_size > 0, "slot %d: incomplete hash index", i);
     }
