@@ -247,7 +247,15 @@ typedef struct bz_fc_desc {
   int32_t head_n;         /* 0 = no head, else 1..8 */
   int32_t head_act;       /* BZ_ACT_NONE | BZ_ACT_SIGMOID | BZ_ACT_SOFTMAX */
   int32_t head_out_dtype; /* BZ_F32 | BZ_F16 | BZ_BF16 */
-  int32_t reserved2_;
+  /*
+   * P sibling layers that share A in one launch (FusedParallelGemm, blaze/operator/fused_op/fused_parallel_gemm_op.h:
+   * 115-129: GemmStridedBatched with stride_a = 0): W holds the P weights one after the other ([P * n_split, ldw]), n =
+   * P * n_split, bias / activation parameters are [n] (slice after slice), and slice p's output is the matrix
+   * [M, n_split] with row pitch ldy at y + p * y_split_stride (elements).  A full bias (bias_rows == m) is [P, M, n_split].
+   * n_split == 0: a single layer.  No head and no softmax with split outputs.
+   */
+  int32_t n_split;
+  int64_t y_split_stride;
 } bz_fc_desc;
 
 BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);

@@ -356,3 +356,96 @@ def test_activation_random_vs_oracle(bz, oracle):
         got = bz.activation(xd, act, params=tuple(_dev(p) for p in params), **kw)
         torch.cuda.synchronize()
         np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("in_name,P,M,K,N,act,full_bias", [
+    ("f32", 3, 3, 2, 3, "none", False),        # the shape of the reference's fused_parallel_gemm fixtures
+    ("f32", 4, 257, 72, 40, "prelu", False),   # ragged M, slices narrower than a tile
+    ("f16", 3, 2048, 128, 96, "prelu", False), # tiles straddle slice boundaries (96 per slice, 64- or 128-wide tiles)
+    ("f16", 5, 300, 216, 80, "dice", False),
+    ("bf16", 2, 1000, 64, 256, "relu", False),
+    ("f16", 2, 129, 40, 18, "none", False),    # slice width not a whole number of 16-byte chunks: element-wise stores
+    ("f32", 3, 65, 30, 24, "none", True),      # a full [P*M, N] bias (fused_parallel_gemm_op.h:78-94)
+])
+def test_fc_split_outputs_equal_separate_layers(bz, oracle, in_name, P, M, K, N, act, full_bias):
+    """P sibling layers on one input as ONE launch (bz_fc_desc.n_split): weights [P*N, K] stacked, bias and activation
+    parameters [P*N], slice p written as its own [M, N] matrix.  Against the oracle's FusedParallelGemm
+    (fused_parallel_gemm_op.h:43-133) followed by the activation, and bit-equal to P separate launches."""
+    import ctypes as C
+    import torch
+    rng = np.random.default_rng(P * 1000 + M + K + N)
+    tdt = _tdtype(in_name)
+    a = _round_to(rng.standard_normal((M, K)).astype(np.float32), in_name)
+    w = _round_to((rng.standard_normal((P, N, K)) / np.sqrt(K)).astype(np.float32), in_name)   # slice p: [N, K] (transB form)
+    bias = (rng.standard_normal((P, M, N) if full_bias else (P, N)) * 0.1).astype(np.float32)
+    slope = rng.uniform(0.1, 0.4, (P, N)).astype(np.float32)
+    dice = [(rng.standard_normal((P, N)) * 0.1).astype(np.float32), (rng.standard_normal((P, N)) * 0.1).astype(np.float32),
+            rng.uniform(0.5, 1.5, (P, N)).astype(np.float32)]
+    d_a, d_w = _dev(a).to(tdt), _dev(w.reshape(P * N, K)).to(tdt)
+    ldw = (K + 7) // 8 * 8
+    d_wp = torch.zeros((P * N, ldw), dtype=tdt, device="cuda")
+    d_wp[:, :K] = d_w
+    d_bias = _dev(bias.reshape(-1))
+    params = {"none": (), "relu": (), "prelu": (_dev(slope.reshape(-1)), ), "dice": tuple(_dev(x.reshape(-1)) for x in dice)}[act]
+    code = {"none": bz.ACT_NONE, "relu": bz.ACT_LEAKY_RELU, "prelu": bz.ACT_PRELU, "dice": bz.ACT_DICE}[act]
+    y = torch.full((P, M, N), float("nan"), dtype=tdt, device="cuda")
+
+    def desc(a_t, w_t, n, bias_t, ps, y_t):
+        d = bz.FcDesc()
+        d.a, d.w, d.y, d.bias = a_t.data_ptr(), w_t.data_ptr(), y_t.data_ptr(), bias_t.data_ptr()
+        d.lda, d.ldw, d.ldy = K, ldw, N
+        d.m, d.n, d.k = M, n, K
+        d.in_dtype = d.out_dtype = bz.bz_dtype(tdt)
+        d.bias_rows = M if full_bias else 1
+        d.alpha = d.beta = 1.0
+        d.act, d.act_alpha = code, 0.0
+        for name, p_ in zip(("act_p0", "act_p1", "act_p2"), ps):
+            setattr(d, name, p_.data_ptr())
+        d.act_size = n if act == "prelu" else 0
+        return d
+
+    d = desc(d_a, d_wp, P * N, d_bias, params, y)
+    d.n_split, d.y_split_stride = N, M * N
+    print("split case %s P=%d M=%d K=%d N=%d act=%s full_bias=%s" % (in_name, P, M, K, N, act, full_bias), flush=True)
+    bz.check(bz.lib().bz_fc_fused(C.byref(d), None))
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy()
+    # oracle: FusedParallelGemm with B stacked [P*N, K] under transB, then the activation per slice
+    want = oracle.fused_parallel_gemm_op(a, w.reshape(P * N, K), bias.reshape(P * M, N) if full_bias else bias.reshape(-1), P, False, True)
+    want = want.reshape(P, M, N)
+    for p in range(P):
+        if act == "prelu":
+            want[p] = oracle.prelu(want[p], slope[p])
+        elif act == "dice":
+            want[p] = oracle.dice(want[p], dice[0][p], dice[1][p], dice[2][p])
+        elif act == "relu":
+            want[p] = oracle.leaky_relu(want[p], 0.0)
+    tol = 1e-5 if in_name == "f32" else 2e-3
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol * max(1.0, float(np.abs(want).max())))
+    # P separate launches of the same kernel family: the same sums tile by tile is not guaranteed (tile shapes follow N),
+    # so equality is asked at the tolerance of one rounding of the tensor type
+    y2 = torch.full((P, M, N), float("nan"), dtype=tdt, device="cuda")
+    for p in range(P):
+        ps = tuple(x[p * N:(p + 1) * N] for x in params)
+        b_p = d_bias[p * M * N:(p + 1) * M * N] if full_bias else d_bias[p * N:(p + 1) * N]
+        bz.check(bz.lib().bz_fc_fused(C.byref(desc(d_a, d_wp[p * N:(p + 1) * N], N, b_p, ps, y2[p])), None))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(got, y2.float().cpu().numpy(), rtol=tol, atol=tol * max(1.0, float(np.abs(want).max())))
+
+
+def test_fc_split_argument_errors(bz):
+    import ctypes as C
+    import torch
+    a = torch.zeros((8, 16), dtype=torch.float16, device="cuda")
+    w = torch.zeros((32, 16), dtype=torch.float16, device="cuda")
+    y = torch.zeros((2, 8, 16), dtype=torch.float16, device="cuda")
+    d = bz.FcDesc()
+    d.a, d.w, d.y = a.data_ptr(), w.data_ptr(), y.data_ptr()
+    d.lda, d.ldw, d.ldy, d.m, d.n, d.k = 16, 16, 16, 8, 32, 16
+    d.in_dtype = d.out_dtype = bz.F16
+    d.alpha = 1.0
+    d.n_split, d.y_split_stride = 12, 128   # 12 does not divide 32
+    assert bz.lib().bz_fc_fused(C.byref(d), None) == -22 and b"n_split" in bz.lib().bz_last_error()
+    d.n_split = 16
+    d.act = bz.ACT_SOFTMAX
+    assert bz.lib().bz_fc_fused(C.byref(d), None) != 0

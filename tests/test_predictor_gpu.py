@@ -64,11 +64,16 @@ def test_reference_operator_kats_through_predictor(pb, kats, name):
     pm.load_model_from_string(_net_from_kat(pb, case), True)
     p = pm.create_predictor(1, 0)
     print("case", name, flush=True)
+    p.register_observers(["profile"])
     p.forward()
     for out_name, e in case["expected"].items():
         got = p.output_asnumpy(out_name)
         assert list(got.shape) == e["shape"]
         np.testing.assert_allclose(got, np.array(e["values"], np.float32).reshape(e["shape"]), rtol=0, atol=1e-6)
+    if name.startswith("fused_parallel_gemm"):
+        # the parallel_num sibling FCs go out as one launch (the reference: one GemmStridedBatched, fused_parallel_gemm_op.h:115-129)
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["name"].startswith("FusedParallelGemm")]
+        assert len(ev) == 1 and ev[0]["args"]["launches"] == 1, ev
 
 
 def test_reference_embedding_kat_through_predictor(pb, kats):
@@ -562,3 +567,67 @@ def test_threads_feeding_alternating_requests_get_their_own_results(pb):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_sibling_gemms_run_as_one_launch(pb, oracle, dtype):
+    """Three towers read the same input: Gemm + PRelu each with weights of one shape (what the reference's ParallelGemm
+    fusion rewrites into FusedParallelGemm + Split, parallel_gemm_fusion_pattern_impl.cc:20-98), plus a fourth Gemm of
+    another width that must stay on its own.  By default the three run as one launch and their outputs are views of
+    one buffer; with pack_sibling_gemms: 0 each runs by itself.  Both against the oracle; a second request with another
+    batch size reuses the stacked weights."""
+    rng = np.random.default_rng(41)
+    code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
+    K, N, N4 = 48, 24, 40
+    r = (lambda x: np.asarray(x, np.float32).astype(np.float16).astype(np.float32)) if dtype == np.float16 else (lambda x: np.asarray(x, np.float32))
+    ws = [(rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32) for _ in range(3)]
+    bs = [(rng.standard_normal(N) * 0.1).astype(np.float32) for _ in range(3)]
+    slopes = [rng.uniform(0.1, 0.4, N).astype(np.float32) for _ in range(3)]
+    w4 = (rng.standard_normal((K, N4)) / np.sqrt(K)).astype(np.float32)
+    outs = {}
+    for pack in (1, 0):
+        nb = pb.NetBuilder("towers", device_type=1)
+        nb.external_input("x", code)
+        nb.external_output("y", code)
+        nb.arg("pack_sibling_gemms", pack)
+        for t in range(3):
+            nb.constant("w%d" % t, ws[t], dtype=code)
+            nb.constant("b%d" % t, bs[t], dtype=code)
+            nb.constant("s%d" % t, slopes[t], dtype=code)
+        nb.constant("w4", w4, dtype=code)
+        for t in range(3):
+            nb.op("Gemm", ["x", "w%d" % t, "b%d" % t], ["h%d" % t])
+            nb.op("PRelu", ["h%d" % t, "s%d" % t], ["t%d" % t])
+        nb.op("Gemm", ["x", "w4"], ["t3"])
+        nb.op("Concat", ["t0", "t1", "t2", "t3"], ["y"], axis=1)
+        pm = pb.PredictorManager()
+        pm.load_model_from_string(nb.text(), True)
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for batch in (70, 33, 70):
+            x = rng.standard_normal((batch, K)).astype(np.float32) if pack == 1 or True else None
+            x = np.random.default_rng(batch).standard_normal((batch, K)).astype(np.float32)
+            p.reshape_input("x", x.shape)
+            p.feed("x", x.astype(dtype))
+            print("sibling case dtype=%s pack=%d batch=%d" % (dtype.__name__, pack, batch), flush=True)
+            p.forward()
+            got.append((x, p.output_asnumpy("y").astype(np.float32)))
+        ev = json.loads(p.dump_observers()["profile"])["traceEvents"]
+        gemms = [e for e in ev if e["name"].startswith("Gemm") and e["dur"] > 0]
+        if pack:
+            assert len(gemms) == 2 and sorted(e["args"]["launches"] for e in gemms) == [1, 1], gemms
+        else:
+            assert len(gemms) == 4
+        outs[pack] = got
+    tol = 2e-3 if dtype == np.float16 else 1e-5
+    for pack in (1, 0):
+        for x, y in outs[pack]:
+            xr = r(x)
+            want = [oracle.prelu(r(oracle.gemm_op(xr, r(ws[t]), r(bs[t]))), r(slopes[t])) for t in range(3)]
+            want.append(oracle.gemm_op(xr, r(w4), None))
+            want = r(np.concatenate([r(w_) for w_ in want], axis=1))
+            assert y.shape == want.shape
+            np.testing.assert_allclose(y, want, rtol=tol, atol=tol)
+    for (x1, y1), (x0, y0) in zip(outs[1], outs[0]):
+        np.testing.assert_allclose(y1, y0, rtol=tol, atol=tol)

@@ -50,7 +50,7 @@ class FcDesc(C.Structure):
                 ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
                 ("reserved_", C.c_int32), ("head_w", C.c_void_p), ("head_bias", C.c_void_p), ("head_y", C.c_void_p),
                 ("head_ldw", C.c_int64), ("head_ldy", C.c_int64), ("head_n", C.c_int32), ("head_act", C.c_int32),
-                ("head_out_dtype", C.c_int32), ("reserved2_", C.c_int32)]
+                ("head_out_dtype", C.c_int32), ("n_split", C.c_int32), ("y_split_stride", C.c_int64)]
 
 
 class BgemmDesc(C.Structure):

@@ -86,6 +86,11 @@ struct FcCall {
   int act_size = 0;
   bool dice_nosqrt = false;
   float act_alpha = 0.f;
+  // P sibling layers on one input in one launch (bz_fc_desc.n_split): B holds P weights stacked on dim 0 -- [P*N, K]
+  // under trans_b, else [P*K, N] -- bias / activation parameters are [P*N], slice p's output starts p * y_split_stride
+  // elements after y
+  int slices = 1;
+  int64_t y_split_stride = 0;
   // a second, skinny layer in the same launch (bz_fc_desc.head_*); y may then be null
   const void* head_w = nullptr;
   int64_t head_ldw = 0;
@@ -95,9 +100,11 @@ struct FcCall {
 };
 
 void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st) {
+  const int P = c.slices;
   const int M = c.trans_a ? c.a_cols : c.a_rows;
   const int K = c.trans_a ? c.a_rows : c.a_cols;
-  const int N = c.trans_b ? c.b_rows : c.b_cols;
+  const int Ns = c.trans_b ? c.b_rows / P : c.b_cols;  // columns of one slice
+  const int N = Ns * P;
   const int bt = BzType(c.dtype);
   const int es = (int)DataTypeSize(c.dtype);
   const int chunk = 16 / es;
@@ -114,7 +121,8 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
     d.a = c.a;
     d.lda = K;
   }
-  // W: [N,K] with aligned rows is used in place, anything else is packed (once for constants)
+  // W: [N,K] with aligned rows is used in place (stacked slices under trans_b are exactly that), anything else is
+  // packed (once for constants), slice by slice when the slices are stacked [K,N] matrices
   if (c.trans_b && (K % chunk == 0) && ((uintptr_t)c.b % 16 == 0)) {
     d.w = c.b;
     d.ldw = K;
@@ -123,16 +131,26 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
     const bool redo = !c.b_constant || packed_b->Stale(c.b_blob) || packed_b->bytes < (size_t)N * ldw * es;
     if (redo) {
       packed_b->Resize((size_t)N * ldw * es);
-      BZ_CHECK(bz_fc_pack_weight(c.b, bt, c.trans_b ? 1 : 0, K, N, packed_b->ptr, bt, ldw, st));
+      if (c.trans_b) {
+        BZ_CHECK(bz_fc_pack_weight(c.b, bt, 1, K, N, packed_b->ptr, bt, ldw, st));
+      } else {
+        for (int p = 0; p < P; ++p)
+          BZ_CHECK(bz_fc_pack_weight((const char*)c.b + (size_t)p * K * Ns * es, bt, 0, K, Ns,
+                                     (char*)packed_b->ptr + (size_t)p * Ns * ldw * es, bt, ldw, st));
+      }
       packed_b->Mark(c.b_blob);
     }
     d.w = packed_b->ptr;
     d.ldw = ldw;
   }
+  if (P > 1) {
+    d.n_split = Ns;
+    d.y_split_stride = c.y_split_stride;
+  }
   d.bias = c.bias;
   d.bias_rows = c.bias_rows;
   d.y = c.y;
-  d.ldy = N;
+  d.ldy = Ns;
   d.m = M;
   d.n = N;
   d.k = K;
@@ -164,7 +182,7 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
 
 // ------------------------------------------------------------------------------------------ Gemm
 template <class Context>
-class GemmOp : public Operator<Context>, public FusableProducer, public StackableFc {
+class GemmOp : public Operator<Context>, public FusableProducer, public StackableFc, public SiblingFc {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
 
@@ -255,7 +273,41 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   }
   void AbsorbHead(StackableFc* head) override { head_ = static_cast<GemmOp*>(head); }
 
+  // ---- sibling layers (same input, same shape of constant weight, same arguments) in one launch
+  std::string SiblingKey() override {
+    Blob* b = this->Input(1);
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr || !siblings_.empty()) return "";
+    if (this->InputSize() > 2 && (!c_constant_ || this->Input(2)->shape().size() != 1)) return "";
+    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX) return "";
+    const TIndex N = transb_ ? b->shape()[0] : b->shape()[1];
+    if (fused_ && fused_act_ == BZ_ACT_PRELU && (TIndex)fused_->Input(1)->size() != N) return "";  // a scalar slope is per layer
+    Blob* y = fused_ ? fused_->Output(0) : this->Output(0);
+    if (y->pitch() != 0 || y == this->Input(0)) return "";
+    std::stringstream ss;
+    ss << this->def_.input(0) << "|" << b->shape()[0] << "x" << b->shape()[1] << "|" << b->data_type() << "|" << transb_ << "|"
+       << alpha_ << "|" << beta_ << "|" << (this->InputSize() > 2 ? this->Input(2)->data_type() : -1) << "|"
+       << (fused_ ? fused_act_ : -1) << "|" << fused_nosqrt_ << "|" << fused_alpha_ << "|" << y->data_type() << "|"
+       << this->device_option().device_id();
+    return ss.str();
+  }
+  void AbsorbSiblings(const std::vector<SiblingFc*>& others) override {
+    siblings_.clear();
+    for (SiblingFc* o : others) siblings_.push_back(static_cast<GemmOp*>(o));
+  }
+
+  int LaunchesOfLastRun() const override { return launches_; }
+
   bool RunOnDevice() override {
+    launches_ = 1;
+    if (!siblings_.empty()) {
+      if (RunSiblings()) return true;
+      // an input the one-launch form does not take (3-D, few columns): one launch per layer
+      launches_ = 1 + (int)siblings_.size();
+      if (!RunSelf(false)) return false;
+      for (GemmOp* g : siblings_)
+        if (!g->RunSelf(false)) return false;
+      return true;
+    }
     if (head_ != nullptr) {
       if (RunSelf(true)) return true;
       // an input the one-launch form does not take (unaligned rows, mixed types): one launch per layer
@@ -344,6 +396,93 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     FillStackLayer(&d.layer[0], false, st);
     for (size_t i = 0; i < stack_.size(); ++i) stack_[i]->FillStackLayer(&d.layer[1 + i], head && i + 1 == stack_.size(), st);
     BZ_CHECK(bz_mlp_fused(&d, st));
+    return true;
+  }
+
+  // this layer and its absorbed siblings as one launch over the stacked weights; every layer's output blob becomes a
+  // view of its slice of one buffer.  False (nothing launched) when the input is not a plain 2-D matrix.
+  bool RunSiblings() {
+    Blob* a = this->Input(0);
+    Blob* b = this->Input(1);
+    if (a->shape().size() != 2 || a->pitch() != 0) return false;
+    const int P = 1 + (int)siblings_.size();
+    const TIndex M = a->shape()[0], K = a->shape()[1];
+    const TIndex N = transb_ ? b->shape()[0] : b->shape()[1];
+    if ((TIndex)P * N <= 8) return false;
+    CheckValid();
+    std::vector<GemmOp*> all = {this};
+    all.insert(all.end(), siblings_.begin(), siblings_.end());
+    hipStream_t st = context_.hip_stream();
+    const int es = (int)DataTypeSize(b->data_type());
+    const int bt = BzType(b->data_type());
+    const int64_t ldw = (K + 7) / 8 * 8;
+    // stacked constants, built once: weights [P*N, ldw], bias and activation parameters [P*N] fp32
+    bool stale = sib_w_.ptr == nullptr;
+    for (GemmOp* g : all) stale |= g->sib_src_ != g->Input(1) || g->sib_version_ != g->Input(1)->version();
+    if (stale) {
+      sib_w_.Resize((size_t)P * N * ldw * es);
+      const bool has_bias = this->InputSize() > 2;
+      const int n_params = !fused_ ? 0 : (fused_act_ == BZ_ACT_PRELU ? 1 : (fused_act_ == BZ_ACT_DICE ? 3 : 0));
+      sib_f32_.Resize((size_t)(1 + n_params) * P * N * sizeof(float));
+      for (int p = 0; p < P; ++p) {
+        GemmOp* g = all[p];
+        BZ_CHECK(bz_fc_pack_weight(g->Input(1)->data(), bt, transb_ ? 1 : 0, (int)K, (int)N, (char*)sib_w_.ptr + (size_t)p * N * ldw * es,
+                                   bt, ldw, st));
+        if (has_bias)
+          HIP_CHECK(hipMemcpyAsync((float*)sib_f32_.ptr + (size_t)p * N, AsFloatParam(g->Input(2), &g->bias_f32_, true, st),
+                                   N * sizeof(float), hipMemcpyDeviceToDevice, st));
+        for (int q = 0; q < n_params; ++q)
+          HIP_CHECK(hipMemcpyAsync((float*)sib_f32_.ptr + ((size_t)(1 + q) * P + p) * N,
+                                   AsFloatParam(g->fused_->Input(1 + q), &g->p_f32_[q], true, st), N * sizeof(float),
+                                   hipMemcpyDeviceToDevice, st));
+        g->sib_src_ = g->Input(1);
+        g->sib_version_ = g->Input(1)->version();
+      }
+    }
+    Blob* y0 = fused_ ? fused_->Output(0) : this->Output(0);
+    const size_t ys = DataTypeSize(y0->data_type());
+    sib_y_.Resize((size_t)P * M * N * ys);
+    for (int p = 0; p < P; ++p) {
+      Blob* y = all[p]->fused_ ? all[p]->fused_->Output(0) : all[p]->Output(0);
+      y->RefReshape({M, N}, (char*)sib_y_.ptr + (size_t)p * M * N * ys);
+    }
+    bz_fc_desc d;
+    memset(&d, 0, sizeof(d));
+    d.a = a->data();
+    d.lda = K;
+    d.w = sib_w_.ptr;
+    d.ldw = ldw;
+    d.y = sib_y_.ptr;
+    d.ldy = N;
+    d.n_split = (int)N;
+    d.y_split_stride = (int64_t)M * N;
+    d.m = (int)M;
+    d.n = (int)(P * N);
+    d.k = (int)K;
+    d.in_dtype = bt;
+    d.out_dtype = BzType(y0->data_type());
+    d.alpha = alpha_;
+    if (this->InputSize() > 2) {
+      d.bias = sib_f32_.ptr;
+      d.bias_rows = 1;
+      d.beta = beta_;
+    }
+    if (fused_) {
+      d.act = fused_act_;
+      d.dice_nosqrt = fused_nosqrt_ ? 1 : 0;
+      d.act_alpha = fused_alpha_;
+      const float* base = (const float*)sib_f32_.ptr + (size_t)P * N;
+      if (fused_act_ == BZ_ACT_PRELU) {
+        d.act_p0 = base;
+        d.act_size = d.n;
+      } else if (fused_act_ == BZ_ACT_DICE) {
+        d.act_p0 = base;
+        d.act_p1 = base + (size_t)P * N;
+        d.act_p2 = base + (size_t)2 * P * N;
+        d.act_size = d.n;
+      }
+    }
+    BZ_CHECK(bz_fc_fused(&d, st));
     return true;
   }
 
@@ -492,6 +631,11 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   Derived stack_pack_;           // this layer's weight in the fragment-major pack of bz_mlp_fused
   std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
   GemmOp* head_ = nullptr;       // the layer of at most 8 outputs computed in this operator's launch
+  std::vector<GemmOp*> siblings_;  // layers on the same input computed in this operator's launch
+  Derived sib_w_, sib_f32_, sib_y_;  // stacked weights / fp32 parameters / outputs
+  const Blob* sib_src_ = nullptr;    // this layer's weight as it was stacked
+  uint64_t sib_version_ = 0;
+  int launches_ = 1;
   OperatorBase* fused_ = nullptr;
   int fused_act_ = BZ_ACT_NONE;
   bool fused_nosqrt_ = false;
@@ -656,8 +800,14 @@ class FusedParallelGemmOp : public Operator<Context> {
     if (full_bias)
       BLAZE_CONDITION_THROW(a_shape.size() != 3 || a_shape[0] == 1, "3-D FusedParallelGemm with a [P*M,N] bias is not supported on this device");
     const size_t es = DataTypeSize(a->data_type());
-    // the P sibling FCs share the input; slice p owns weights [K,N] (or [N,K]), bias and output slice p
-    for (int p = 0; p < P; ++p) {
+    // The P sibling FCs share the input; slice p owns weights [K,N] (or [N,K]), bias and output slice p.  The reference
+    // hands them to one GemmStridedBatched with stride_a = 0 (fused_parallel_gemm_op.h:115-129); here they are one
+    // launch of the FC kernel over P*N columns whose epilogue scatters each slice to its own [rows, N] matrix.  (A
+    // launch of at most 8 columns would take the skinny kernel, which computes a softmax-sized head: those few cases
+    // run slice by slice.)
+    const bool one_launch = P > 1 && (TIndex)P * N > 8;
+    launches_ = one_launch ? 1 : P;
+    for (int p = 0; p < launches_; ++p) {
       FcCall call;
       call.a = a->data();
       call.a_rows = transa_ ? (int)K : (int)rows;
@@ -677,6 +827,11 @@ class FusedParallelGemmOp : public Operator<Context> {
       if (bias) {
         call.bias = bias + (full_bias ? (size_t)p * rows * N : (size_t)p * N);
         call.bias_rows = full_bias ? (int)rows : 1;
+      }
+      if (one_launch) {
+        call.slices = P;
+        call.y_split_stride = (int64_t)rows * N;
+        call.b_rows = (int)(transb_ ? N : K) * P;
       }
       RunFc(call, &packed_b_[p], &packed_a_, st);
     }
@@ -716,6 +871,10 @@ class FusedParallelGemmOp : public Operator<Context> {
   bool b_constant_ = false, c_constant_ = false;
   std::vector<Derived> packed_b_;
   Derived packed_a_, bias_f32_;
+  int launches_ = 0;  // kernel launches of the last run (1 when the slices went out as one)
+
+ public:
+  int LaunchesOfLastRun() const override { return launches_; }
 };
 
 REGISTER_HIP_OPERATOR(FusedParallelGemm, FusedParallelGemmOp<HIPContext>);

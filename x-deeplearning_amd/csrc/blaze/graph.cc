@@ -165,7 +165,9 @@ std::string Net::DumpProfile() const {
     if (!first) ss << ",";
     first = false;
     ss << "{\"name\":\"" << op->type() << ":" << op->name() << "\",\"ph\":\"X\",\"pid\":0,\"tid\":0,\"ts\":" << t
-       << ",\"dur\":" << op->last_run_us() << "}";
+       << ",\"dur\":" << op->last_run_us();
+    if (op->LaunchesOfLastRun() >= 0) ss << ",\"args\":{\"launches\":" << op->LaunchesOfLastRun() << "}";
+    ss << "}";
     t += op->last_run_us();
   }
   ss << "]}";
@@ -211,6 +213,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     }
     StackFcLayers();
     FuseFcHeads();
+    PackSiblingFcs();
     AliasConcatInputs();
     FuseConcatPieces();
   }
@@ -249,6 +252,34 @@ void SimpleNet::FuseFcHeads() {
 // ConcatPieceSource).  A producer is taken over when its output is read only by the Concat -- or, as a shape
 // reference (second input of BroadcastTo), by another producer the same Concat takes over -- is neither an output of the
 // net nor written in place, and nothing between the producer and the Concat overwrites the producer's inputs.
+void SimpleNet::PackSiblingFcs() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "pack_sibling_gemms");
+  if (arg && arg->has_i && arg->i == 0) return;
+  std::map<std::string, std::vector<size_t>> groups;
+  for (size_t i = 0; i < operators_.size(); ++i) {
+    auto* fc = skipped_[i] ? nullptr : dynamic_cast<SiblingFc*>(operators_[i].get());
+    if (!fc) continue;
+    const std::string key = fc->SiblingKey();
+    if (!key.empty()) groups[key].push_back(i);
+  }
+  for (auto& kv : groups) {
+    std::vector<size_t>& idx = kv.second;
+    if (idx.size() < 2) continue;
+    // the shared input must not be rewritten between the first and the last sibling (an in-place operator in between)
+    const std::string& in = operators_[idx[0]]->operator_def().input(0);
+    bool clean = true;
+    for (size_t k = idx.front() + 1; k < idx.back() && clean; ++k)
+      for (const auto& out : operators_[k]->operator_def().output()) clean &= (out != in);
+    if (!clean) continue;
+    std::vector<SiblingFc*> others;
+    for (size_t m = 1; m < idx.size(); ++m) {
+      others.push_back(dynamic_cast<SiblingFc*>(operators_[idx[m]].get()));
+      skipped_[idx[m]] = true;
+    }
+    dynamic_cast<SiblingFc*>(operators_[idx[0]].get())->AbsorbSiblings(others);
+  }
+}
+
 void SimpleNet::FuseConcatPieces() {
   const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_concat_pieces");
   if (arg && arg->has_i && arg->i == 0) return;

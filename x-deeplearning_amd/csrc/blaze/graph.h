@@ -98,6 +98,7 @@ class SimpleNet : public Net {
   void AliasConcatInputs();
   void FuseConcatPieces();
   void FuseFcHeads();
+  void PackSiblingFcs();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -142,6 +143,21 @@ class StackableFc {
   virtual bool CanHostHead(int* n_out) = 0;   // static eligibility of the first layer; reports its width
   virtual bool CanBeHead(int k_in) = 0;       // static eligibility of the second layer for a first layer of width k_in
   virtual void AbsorbHead(StackableFc* head) = 0;
+};
+
+// Sibling FC operators -- Gemms that read the same input with constant weights of one shape and the same arguments
+// (and the same kind of folded activation) -- run as ONE launch over the stacked weights, each writing its own output
+// matrix: what the reference's ParallelGemm fusion does by rewriting them into FusedParallelGemm + Split
+// (blaze/graph/pattern/in_parallel/parallel_gemm_fusion_pattern_impl.cc:20-98, CanFusion :118-140).  SimpleNet groups
+// operators with equal SiblingKey(); the first of a group absorbs the others, which are skipped.  The outputs become
+// views of one buffer the first operator owns (no Split launch).  Same sums per output element as the separate
+// launches up to the tile shape the wider launch picks: equal within one rounding of the tensor type.
+class SiblingFc {
+ public:
+  virtual ~SiblingFc() {}
+  // empty: not eligible.  Otherwise everything that must agree between siblings, the input blob included.
+  virtual std::string SiblingKey() = 0;
+  virtual void AbsorbSiblings(const std::vector<SiblingFc*>& others) = 0;
 };
 
 // A Concat along the last axis whose inputs are elementwise results (Add / Sub / Mul / Div / BroadcastTo of tensors

@@ -131,6 +131,8 @@ class OperatorBase {
   virtual void* DeviceStream() { return nullptr; }
   // columns of 2-D output `idx` when they are fixed by the operator's arguments (else 0)
   virtual TIndex StaticOutputCols(int idx) const { return 0; }
+  // compute-kernel launches of the operator's last run, when it keeps count (else -1); the profile observer reports it
+  virtual int LaunchesOfLastRun() const { return -1; }
 
   const DeviceOption& device_option() const { return device_option_; }
   void set_net_position(int p) { net_position_ = p; }

@@ -47,7 +47,24 @@ struct Epilogue {
   int act_size;
   int dice_nosqrt;
   float alpha, beta, act_alpha;
+  // the N columns are `split_n`-wide slices (sibling FCs stacked along N): column n belongs to slice n / split_n, whose
+  // output matrix [M, split_n] (row pitch ldy) starts split_stride elements after the previous slice's; a full bias is
+  // laid out the same way, slice after slice.  split_n == 0: one matrix.
+  int split_n;
+  int64_t split_stride;
 };
+
+// element offset of output (m, n) in Y, and of the same element in a full [.., N] bias
+__device__ __forceinline__ int64_t out_index(const Epilogue& ep, int64_t m, int n, int64_t ldy) {
+  if (ep.split_n == 0) return m * ldy + n;
+  const int p = n / ep.split_n;
+  return p * ep.split_stride + m * ldy + (n - p * ep.split_n);
+}
+__device__ __forceinline__ int64_t full_bias_index(const Epilogue& ep, int64_t m, int n, int M, int N) {
+  if (ep.split_n == 0) return m * N + n;
+  const int p = n / ep.split_n;
+  return ((int64_t)p * M + m) * ep.split_n + (n - p * ep.split_n);
+}
 
 __device__ __forceinline__ float apply_act(float v, int n, const Epilogue& e) {
   switch (e.act) {
@@ -502,12 +519,12 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
             if (ep.bias_rows == 1)
               v += ep.beta * cbias[j];
             else if (ep.bias_rows > 1)
-              v += ep.beta * ep.bias[(int64_t)m * N + n];
+              v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
             v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
             if (HEAD || vec_y)
               store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
             else
-              store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+              store_out<OutT>(Y + out_index(ep, m, n, ldy), v);
           }
         }
       }
@@ -544,7 +561,7 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
       for (int q = tid; q < BM * OCPR; q += NT) {
         const int ml = q / OCPR, ch = q % OCPR;
         const int m = m0 + ml, n = n0 + ch * (16 / OS);
-        if (m < M && n < N) *(uint4*)((char*)(Y + (int64_t)m * ldy + n)) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+        if (m < M && n < N) *(uint4*)((char*)(Y + out_index(ep, m, n, ldy))) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
       }
     } else if (Y != nullptr) {  // HEAD with an output that takes no 16-byte stores
       for (int q = tid; q < BM * BN; q += NT) {
@@ -684,7 +701,7 @@ __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restric
           if (ep.bias_rows == 1)
             x += ep.beta * cb[n];
           else if (ep.bias_rows > 1)
-            x += ep.beta * ep.bias[m * N + n];
+            x += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
           v[n] = x;
         }
       }
@@ -710,7 +727,7 @@ __global__ __launch_bounds__(256) void bz_fc_skinny_kernel(const char* __restric
       }
 #pragma unroll
       for (int n = 0; n < kSkinnyMaxN; ++n)
-        if (n < N) store_out<OutT>(Y + m * ldy + n, v[n]);
+        if (n < N) store_out<OutT>(Y + out_index(ep, m, n, ldy), v[n]);
     }
   }
 }
@@ -734,8 +751,10 @@ template <int DT, typename OutT, int BM, int BN, int BK, int WM, int WN, int D, 
 int launch_mfma(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st) {
   const int tiles_m = (d.m + BM - 1) / BM, tiles_n = (d.n + BN - 1) / BN;
   // output rows 16-byte aligned and N a whole number of 16-byte chunks: coalesced stores through LDS
+  // (with split outputs every slice must start on a chunk boundary as well)
   const bool vec_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * (int64_t)sizeof(OutT)) % 16 == 0) &&
-                     (d.n % (16 / (int)sizeof(OutT)) == 0);
+                     (d.n % (16 / (int)sizeof(OutT)) == 0) &&
+                     (d.n_split == 0 || (d.n_split % (16 / (int)sizeof(OutT)) == 0 && (d.y_split_stride * (int64_t)sizeof(OutT)) % 16 == 0));
   HeadArgs head = {};
   if (HEAD) {
     head.w = (const char*)d.head_w;
@@ -843,8 +862,12 @@ int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   const bz_fc_desc& d = *desc;
   BZ_REQUIRE(d.a && d.w && (d.y || d.head_n > 0), "bz_fc_fused: null a/w/y");
   BZ_REQUIRE(d.m >= 0 && d.n > 0 && d.k > 0, "bz_fc_fused: bad shape m=%d n=%d k=%d", d.m, d.n, d.k);
-  BZ_REQUIRE(d.lda >= d.k && d.ldw >= d.k && d.ldy >= d.n, "bz_fc_fused: leading dimension smaller than row (lda=%lld ldw=%lld ldy=%lld)",
-             (long long)d.lda, (long long)d.ldw, (long long)d.ldy);
+  BZ_REQUIRE(d.n_split >= 0 && (d.n_split == 0 || (d.n % d.n_split == 0 && d.y_split_stride >= 0)),
+             "bz_fc_fused: n_split=%d must divide n=%d", d.n_split, d.n);
+  BZ_REQUIRE(d.n_split == 0 || (d.head_n == 0 && d.act != BZ_ACT_SOFTMAX), "bz_fc_fused: split outputs take no head and no softmax");
+  BZ_REQUIRE(d.lda >= d.k && d.ldw >= d.k && d.ldy >= (d.n_split ? d.n_split : d.n),
+             "bz_fc_fused: leading dimension smaller than row (lda=%lld ldw=%lld ldy=%lld)", (long long)d.lda, (long long)d.ldw,
+             (long long)d.ldy);
   BZ_REQUIRE(d.in_dtype == BZ_F16 || d.in_dtype == BZ_BF16 || d.in_dtype == BZ_F32, "bz_fc_fused: unsupported in dtype %d",
              d.in_dtype);
   BZ_REQUIRE(d.bias_rows == 0 || d.bias != nullptr, "bz_fc_fused: bias_rows=%d without bias", d.bias_rows);
@@ -881,6 +904,8 @@ int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   ep.alpha = d.alpha;
   ep.beta = d.beta;
   ep.act_alpha = d.act_alpha;
+  ep.split_n = d.n_split;
+  ep.split_stride = d.y_split_stride;
   const int es = bz::dtype_size(d.in_dtype);
   const bool vec_a = ((uintptr_t)d.a % 16 == 0) && ((d.lda * es) % 16 == 0);
   const bool vec_w = ((uintptr_t)d.w % 16 == 0) && ((d.ldw * es) % 16 == 0);
