@@ -148,6 +148,23 @@ def test_fc_half(bz, oracle, in_name, out_name, M, N, K, act):
     _fc_case(bz, oracle, M, N, K, in_name, out_name, act, seed=M + N * 3 + K)
 
 
+# Large 2-byte layers go to the streaming kernel (256x128 tiles, loader waves, operands straight into LDS) once
+# ceil(M/256) * ceil(N/128) >= 200, K is a multiple of 64 and at least 512, and the output takes 16-byte stores.
+@pytest.mark.parametrize("in_name", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,act,kw", [
+    (7000, 1000, 512, "prelu", {}),                 # ragged in M (88 rows in the last tile) and N (104 columns)
+    (8192, 1024, 576, "dice", {}),                  # whole tiles, an odd number of K tiles
+    (6500, 1032, 640, "none", {"alpha": 0.5, "beta": 2.0}),
+    (6600, 1024, 512, "sigmoid", {"bias": False}),
+    (6400, 1024, 1024, "relu", {"full_bias": True}),
+    (51300, 128, 512, "prelu", {}),                 # one N tile; 201 M tiles: the XCD bands are uneven
+])
+def test_fc_streaming_kernel(bz, oracle, in_name, M, N, K, act, kw):
+    print("case stream %s M=%d N=%d K=%d act=%s %r" % (in_name, M, N, K, act, kw), flush=True)
+    assert -(-M // 256) * -(-N // 128) >= 200 and K % 64 == 0 and K >= 512
+    _fc_case(bz, oracle, M, N, K, in_name, in_name, act, seed=M + N + K, **kw)
+
+
 @pytest.mark.parametrize("in_name", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("M,K,N,N2,act,hact", [
     (2048, 512, 256, 2, "prelu", "softmax"),   # config 2's last two layers: 32x256 tile
@@ -366,6 +383,8 @@ def test_activation_random_vs_oracle(bz, oracle):
     ("bf16", 2, 1000, 64, 256, "relu", False),
     ("f16", 2, 129, 40, 18, "none", False),    # slice width not a whole number of 16-byte chunks: element-wise stores
     ("f32", 3, 65, 30, 24, "none", True),      # a full [P*M, N] bias (fused_parallel_gemm_op.h:78-94)
+    ("bf16", 8, 6400, 512, 136, "prelu", False),  # the streaming kernel (25 x 9 tiles); slices straddle its 128-wide tiles
+    ("f16", 4, 13000, 512, 128, "none", True),    # the streaming kernel with a full bias
 ])
 def test_fc_split_outputs_equal_separate_layers(bz, oracle, in_name, P, M, K, N, act, full_bias):
     """P sibling layers on one input as ONE launch (bz_fc_desc.n_split): weights [P*N, K] stacked, bias and activation

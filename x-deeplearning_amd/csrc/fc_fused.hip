@@ -25,6 +25,7 @@
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "bz_common.h"
@@ -642,6 +643,236 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// streaming kernel: large layers (a 256x128 tile per CU fills the chip, K deep)
+// ---------------------------------------------------------------------------------------------
+// At this size the limit is how fast operands reach a CU, not latency: a 256x128x64 step is 1024 MFMA cycles per SIMD
+// and 48 KB of operands, which the path from L2 into a CU (64 bytes a clock) needs 768 cycles for.  So the tile is the
+// largest one that still gives every CU a workgroup with one wave per SIMD multiplying (128x64 per wave, 128 accumulator
+// registers), and nothing else may stand in the loads' way:
+//  - operands go from global memory straight into LDS (global_load_lds_dwordx4: no registers, no LDS store
+//    instructions), three stages of 48 KB, two tiles in flight;
+//  - four more waves, one per SIMD, do nothing but issue those loads and wait for them; the multiplying waves issue
+//    only LDS reads and MFMAs and meet the loaders at one barrier per K tile (the same wave doing both measured 237 us
+//    on 8192 x 12800 -> 1024 bf16, this split 203 us);
+//  - a tile row is 128 bytes, half of the 64 banks; chunk c of row r is stored at position c ^ ((r >> 1) & 7), so the
+//    16 lanes of a ds_read_b128 phase (16 rows, one logical chunk) hit 16 different bank groups (203 -> 195 us: with
+//    the 32-bank pattern c ^ (r & 7) every other cycle of the LDS was a conflict);
+//  - the scheduler is told to alternate MFMA and fragment read, and not to move either across a phase (195 -> 192 us).
+constexpr int kStreamBM = 256, kStreamBN = 128, kStreamBK = 64, kStreamStages = 3;
+constexpr int kStreamRowB = kStreamBK * 2;
+constexpr int kStreamStageBytes = (kStreamBM + kStreamBN) * kStreamRowB;  // 49152
+constexpr int kStreamLds = kStreamStages * kStreamStageBytes;            // 147456 of the CU's 160 KB
+constexpr int kStreamCompute = 256;                                       // threads that multiply; as many again load
+
+typedef __attribute__((address_space(3))) char lds_char;
+
+// 16 bytes per lane from global memory to LDS at lds_addr + 16 * lane (lds_addr is the same in all lanes)
+__device__ __forceinline__ void load_to_lds(const char* g, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_addr) : "memory", "m0");
+}
+
+// one phase = 6 fragment reads for the phase after next and 8 MFMAs on fragments read a phase ago
+#define BZ_PIN_PHASE()                                     \
+  do {                                                     \
+    _Pragma("unroll") for (int q_ = 0; q_ < 6; ++q_) {     \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   \
+    }                                                      \
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);     \
+    __builtin_amdgcn_sched_barrier(0);                     \
+  } while (0)
+
+template <int DT, typename OutT>
+__global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(const char* __restrict__ A,
+                                                                              const char* __restrict__ W, OutT* __restrict__ Y,
+                                                                              int M, int N, int K, int64_t lda, int64_t ldw,
+                                                                              int64_t ldy, int tiles_m, int tiles_n, Epilogue ep) {
+  using T = In<DT>;
+  static_assert(T::kSize == 2 && sizeof(OutT) == 2, "2-byte operands and outputs");
+  constexpr int BM = kStreamBM, BN = kStreamBN, ROWB = kStreamRowB, STAGES = kStreamStages, NT = kStreamCompute;
+  constexpr int STAGE_BYTES = kStreamStageBytes;
+  constexpr int LOADS = (BM + BN) * (ROWB / 16) / NT;  // 12 chunks per loader thread per stage
+  constexpr int TM = 4, TN = 2;                        // 32x32 blocks per wave tile (128 x 64)
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const bool loader = threadIdx.x >= NT;
+  const int tid = threadIdx.x & (NT - 1), lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  // The 8 XCDs take turns at consecutive workgroup ids.  XCD x walks its own band of M tiles, the N tiles of an M tile
+  // next to each other in time: an A tile is fetched into that XCD's L2 once, the W panel streams through it.
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int per_xcd = (tiles_m + 7) / 8;
+  const int tile_m = xcd * per_xcd + j / tiles_n, tile_n = j % tiles_n;
+  if (tile_m >= tiles_m) return;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_char*)smem;
+  const int KT = K / kStreamBK;
+
+  if (loader) {
+    // chunk p = i*256 + tid of a stage: row p >> 3 (A rows, then W rows), position p & 7
+    const char* src[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int p = i * NT + tid;
+      const int r = p >> 3, c = (p & 7) ^ ((r >> 1) & 7);
+      if (r < BM) {
+        int m = m0 + r;
+        m = m < M ? m : M - 1;
+        src[i] = A + ((int64_t)m * lda) * 2 + c * 16;
+      } else {
+        int n = n0 + (r - BM);
+        n = n < N ? n : N - 1;
+        src[i] = W + ((int64_t)n * ldw) * 2 + c * 16;
+      }
+    }
+    auto issue = [&](int kt) {
+      const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + (kt % STAGES) * STAGE_BYTES + wave * 1024);
+      const int64_t koff = (int64_t)kt * ROWB;
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i) load_to_lds(src[i] + koff, base + i * (NT * 16));
+    };
+    // Barrier kt (counted from 0) says: tile kt has landed, and nobody reads the stage tile kt+2 goes to any more.
+    // The waits are written out because only this code knows how many loads may stay in flight.
+    issue(0);
+    if (KT > 1) issue(1);
+    if (KT > 1)
+      asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt + 2 < KT) {
+        issue(kt + 2);
+        asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      }
+    }
+    __syncthreads();  // the two barriers of the epilogue
+    __syncthreads();
+    return;
+  }
+
+  // per-column epilogue parameters, requested before the K loop
+  float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
+#pragma unroll
+  for (int jn = 0; jn < TN; ++jn) {
+    int n = n0 + wn * 64 + jn * 32 + (lane & 31);
+    n = n < N ? n : N - 1;
+    cbias[jn] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cp0[jn] = cp1[jn] = cp2[jn] = 0.f;
+    if (ep.act == BZ_ACT_PRELU) cp0[jn] = ep.p0[ep.act_size == 1 ? 0 : n];
+    if (ep.act == BZ_ACT_DICE) {
+      cp0[jn] = ep.p0[n];
+      cp1[jn] = ep.p1[n];
+      cp2[jn] = ep.p2[n];
+    }
+  }
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  // lane (row = lane & 31, half = lane >> 5) reads logical chunk 2*ks + half of its row
+  const int frow = lane & 31, fhalf = lane >> 5;
+  int foff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) foff[ks] = frow * ROWB + (((2 * ks + fhalf) ^ ((frow >> 1) & 7)) << 4);
+  const int a_base = (wm * 128) * ROWB, w_base = (BM + wn * 64) * ROWB;
+  uint4 fa[2][TM], fw[2][TN];
+  auto fread = [&](int slot, int stage, int ks) {
+    const char* s = smem + stage * STAGE_BYTES + foff[ks];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[slot][i] = *(const uint4*)(s + a_base + i * 32 * ROWB);
+#pragma unroll
+    for (int jn = 0; jn < TN; ++jn) fw[slot][jn] = *(const uint4*)(s + w_base + jn * 32 * ROWB);
+  };
+  auto fmma = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int jn = 0; jn < TN; ++jn) T::mma(fa[slot][i], fw[slot][jn], acc[i][jn]);
+  };
+
+  asm volatile("s_barrier" ::: "memory");  // tile 0 landed
+  fread(0, 0, 0);
+  for (int kt = 0; kt < KT; ++kt) {
+    const int stage = kt % STAGES;
+    fread(1, stage, 1);
+    fmma(0);
+    BZ_PIN_PHASE();
+    fread(0, stage, 2);
+    fmma(1);
+    BZ_PIN_PHASE();
+    fread(1, stage, 3);
+    fmma(0);
+    BZ_PIN_PHASE();
+    // every read of this stage has returned (the last were issued 8 MFMAs ago); past the barrier tile kt+1 is complete
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (kt + 1 < KT) fread(0, (kt + 1) % STAGES, 0);
+    fmma(1);
+    BZ_PIN_PHASE();
+  }
+
+  // epilogue: lane owns column n of each 32x32 block, rows 8*(r/4) + 4*(lane/32) + r%4; the activated tile goes through
+  // LDS so that global stores are 16 bytes per lane along rows
+  __syncthreads();
+  constexpr int OPITCH = BN * 2 + 16;
+  char* lout = smem;
+  auto epilogue = [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int jn = 0; jn < TN; ++jn) {
+      const int nl = wn * 64 + jn * 32 + (lane & 31);
+      const int n = n0 + nl;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int ml = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const int m = m0 + ml;
+          float v = ep.alpha * acc[i][jn][r];
+          if (ep.bias_rows == 1)
+            v += ep.beta * cbias[jn];
+          else if (ep.bias_rows > 1 && m < M && n < N)
+            v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
+          v = apply_act_t<ACT>(v, ep, cp0[jn], cp1[jn], cp2[jn]);
+          store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
+        }
+      }
+    }
+  };
+  switch (ep.act) {
+    case BZ_ACT_PRELU:
+      epilogue(std::integral_constant<int, BZ_ACT_PRELU>());
+      break;
+    case BZ_ACT_DICE:
+      epilogue(std::integral_constant<int, BZ_ACT_DICE>());
+      break;
+    case BZ_ACT_LEAKY_RELU:
+      epilogue(std::integral_constant<int, BZ_ACT_LEAKY_RELU>());
+      break;
+    case BZ_ACT_SIGMOID:
+      epilogue(std::integral_constant<int, BZ_ACT_SIGMOID>());
+      break;
+    default:
+      epilogue(std::integral_constant<int, BZ_ACT_NONE>());
+      break;
+  }
+  __syncthreads();
+  constexpr int OCPR = BN * 2 / 16;
+  for (int q = tid; q < BM * OCPR; q += NT) {
+    const int ml = q / OCPR, ch = q % OCPR;
+    const int m = m0 + ml, n = n0 + ch * 8;
+    if (m < M && n < N) *(uint4*)((char*)(Y + out_index(ep, m, n, ldy))) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+  }
+}
+#undef BZ_PIN_PHASE
+
 // ---------------------------------------------------------------------------------------------
 // skinny kernel: N <= 8
 // ---------------------------------------------------------------------------------------------
@@ -773,6 +1004,30 @@ int launch_mfma(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec_w,
   return BZ_OK;
 }
 
+
+// 2-byte operands and outputs, 16-byte aligned rows on all three, K a whole number of 64-wide tiles
+template <int DT, typename OutT>
+int launch_stream(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
+  const int tiles_m = (d.m + kStreamBM - 1) / kStreamBM, tiles_n = (d.n + kStreamBN - 1) / kStreamBN;
+  const int grid = (tiles_m + 7) / 8 * 8 * tiles_n;
+  // more dynamic LDS than the default limit: raised once per kernel and device
+  static std::mutex mu;
+  static bool raised[64] = {};
+  int dev = 0;
+  BZ_HIP_OK(hipGetDevice(&dev));
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev >= 0 && dev < 64 && !raised[dev]) {
+      BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_stream_kernel<DT, OutT>, hipFuncAttributeMaxDynamicSharedMemorySize, kStreamLds));
+      raised[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL((bz_fc_stream_kernel<DT, OutT>), dim3(grid), dim3(2 * kStreamCompute), kStreamLds, st, (const char*)d.a,
+                     (const char*)d.w, (OutT*)d.y, d.m, d.n, d.k, d.lda, d.ldw, d.ldy, tiles_m, tiles_n, ep);
+  BZ_LAUNCH_OK("bz_fc_stream_kernel");
+  return BZ_OK;
+}
+
 // Layer + skinny head in one launch: a workgroup owns whole rows of the first layer's output (N <= 256).
 template <int DT, typename OutT>
 int dispatch_head(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
@@ -802,6 +1057,14 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
   // latency-bound small tiles.
   const int64_t wg128x256 = (int64_t)((d.m + 127) / 128) * ((d.n + 255) / 256);
   const int64_t wg64x128 = (int64_t)((d.m + 63) / 64) * ((d.n + 127) / 128);
+  if constexpr (sizeof(OutT) == 2 && In<DT>::kSize == 2) {
+    // the streaming kernel once its 256x128 tiles keep most CUs busy and K is deep enough to pay for filling its ring
+    // (8192 x 12800 -> 1024 bf16: 192 against 238 us; 4096^3: 128 against 139 us)
+    const int64_t wg_stream = (int64_t)((d.m + kStreamBM - 1) / kStreamBM) * ((d.n + kStreamBN - 1) / kStreamBN);
+    const bool vec_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * 2) % 16 == 0) && d.n % 8 == 0 &&
+                       (d.n_split == 0 || (d.n_split % 8 == 0 && (d.y_split_stride * 2) % 16 == 0));
+    if (wg_stream >= 200 && d.k % kStreamBK == 0 && d.k >= 8 * kStreamBK && vec_y) return launch_stream<DT, OutT>(d, ep, st);
+  }
   if constexpr (sizeof(OutT) == 2) {
     // (256x256 once even that fills the chip: 4096^3 bf16 987 against 885 TFLOP/s)
     const int64_t wg256 = (int64_t)((d.m + 255) / 256) * ((d.n + 255) / 256);
