@@ -345,6 +345,30 @@ typedef struct bz_bgemm_desc {
 BZ_API int bz_gemm_strided_batched(const bz_bgemm_desc* desc, bz_stream_t stream);
 
 /*
+ * The tail of a DIN attention block in one launch:
+ *   att[b, c] = sum_t (w[b, t] * mask[b, t]) * x[b, t, c]        sum[b, c] = sum_t x[b, t, c]
+ * i.e. Mul (blaze/operator/op/elementwise_op.h:154-163), MatMul with transA on [B, T, 1] x [B, T, C]
+ * (matmul_op.h:77-89) and ReduceSum over axis 1 (reduce_sum_op.h:18-66) as the reference
+ * runs them one after the other; the product w * mask is rounded to the tensor type
+ * before it is used, as the Mul operator's output would be, and both sums add in
+ * ascending t, so the outputs equal the three operators' bit for bit.
+ * mask null: w is used as it is.  att null or sum null: that output is not computed.
+ */
+typedef struct bz_weighted_pool_desc {
+  const void* w;     /* [batch, t] */
+  const void* mask;  /* [batch, t] or null */
+  const void* x;     /* [batch, t, c] */
+  void* att;         /* [batch, c] or null */
+  void* sum;         /* [batch, c] or null */
+  int64_t batch;
+  int32_t t, c;
+  int32_t dtype;     /* BZ_F32 | BZ_F16 for all five */
+  int32_t reserved_;
+} bz_weighted_pool_desc;
+
+BZ_API int bz_weighted_pool(const bz_weighted_pool_desc* desc, bz_stream_t stream);
+
+/*
  * Standalone activation ops over a [rows, cols] fp32 or fp16 tensor (in place
  * allowed), for graphs where the producer is not a Gemm.  Same formulas and
  * reference citations as bz_act above.

@@ -264,7 +264,7 @@ def test_attention_unit_assembled_by_the_concat_equals_the_separate_operators():
     outs = {}
     for fuse in (1, 0):
         pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("att_in", ),
-                                             net_args={"fuse_concat_pieces": fuse})
+                                             net_args={"fuse_concat_pieces": fuse, "fuse_weighted_pool": 0})
         p = pm.create_predictor(1, 0)
         p.register_observers(["profile"])
         got = []
@@ -285,3 +285,38 @@ def test_attention_unit_assembled_by_the_concat_equals_the_separate_operators():
         q, k = a1[:, :, :D3].astype(np.float32), a1[:, :, D3:2 * D3].astype(np.float32)
         assert np.array_equal(a1[:, :, 2 * D3:3 * D3], (q - k).astype(np.float16))
         assert np.array_equal(a1[:, :, 3 * D3:], (q * k).astype(np.float16))
+
+
+def test_attention_tail_in_one_launch_equals_the_separate_operators():
+    """Mul(score, mask) -> MatMul(transA) and ReduceSum(his, axis 1): by default the MatMul runs all three as one launch
+    (bz_weighted_pool) and the Mul and the ReduceSum never run; with fuse_weighted_pool: 0 each runs.  Same bits in the
+    attention vector, the history sum and the probabilities, also after the batch shrinks and grows again."""
+    import json
+    import torch
+    import din_model
+    cfg = din_model.Config3(batch=96, rows=5000, T=20)
+    small = din_model.Config3(batch=17, rows=5000, T=20)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=5), cfg.batch_inputs(seed_offset=9)]
+    outs = {}
+    for fuse in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("att", "hsum"),
+                                             net_args={"fuse_weighted_pool": fuse})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append(tuple(p.output_asnumpy(n).copy() for n in ("att", "hsum", "prob")))
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        ran = {e["name"].split(":")[0] for e in ev}
+        assert ("ReduceSum" in ran) == (fuse == 0) and ("Mul" in ran) == (fuse == 0), ran
+        assert [e["args"]["launches"] for e in ev if e["name"].startswith("MatMul:")] == [1]
+        outs[fuse] = got
+    torch.cuda.synchronize()
+    for one, sep, b in zip(outs[1], outs[0], (96, 17, 96)):
+        assert one[0].shape == (b, 3 * cfg.dim) and one[0].any() and one[1].any()
+        for x1, x0 in zip(one, sep):
+            assert np.array_equal(x1.view(np.uint16 if x1.dtype == np.float16 else np.uint32),
+                                  x0.view(np.uint16 if x0.dtype == np.float16 else np.uint32))

@@ -468,3 +468,43 @@ def test_fc_split_argument_errors(bz):
     d.n_split = 16
     d.act = bz.ACT_SOFTMAX
     assert bz.lib().bz_fc_fused(C.byref(d), None) != 0
+
+
+@pytest.mark.parametrize("dtype_name", ["f32", "f16"])
+@pytest.mark.parametrize("B,T,Cn", [(1024, 50, 54), (7, 1, 3), (33, 17, 130), (2, 200, 64)])
+def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T, Cn):
+    """bz_weighted_pool against the three launches it replaces (Mul, strided-batched GEMM with transA, ReduceSum), bit
+    for bit, and against the oracle's fp32 sums of the rounded operands."""
+    import torch
+    print("weighted pool %s B=%d T=%d C=%d" % (dtype_name, B, T, Cn), flush=True)
+    tdt = _tdtype(dtype_name)
+    rng = np.random.default_rng(B + T + Cn)
+    x = _round_to(rng.standard_normal((B, T, Cn)), dtype_name)
+    w = _round_to(rng.standard_normal((B, T, 1)), dtype_name)
+    lens = rng.integers(0, T + 1, B)
+    mask = (np.arange(T)[None, :] < lens[:, None]).astype(np.float32).reshape(B, T, 1)
+    dx, dw, dm = _dev(x).to(tdt), _dev(w).to(tdt), _dev(mask).to(tdt)
+    att, tot = bz.weighted_pool(dx, dw, dm)
+    # the separate launches
+    aw = bz.broadcast_op(bz.EW_MUL, dw, dm)
+    c = torch.empty((B, 1, Cn), dtype=tdt, device="cuda")
+    bz.gemm_strided_batched(aw, dx, c, 1, Cn, T, B, T, T * Cn, Cn, trans_a=True)
+    s = bz.reduce_sum(dx, 1, keepdims=False)
+    torch.cuda.synchronize()
+    assert torch.equal(att, c.reshape(B, Cn)) and torch.equal(tot, s)
+    # without a mask, and each output alone
+    att2, none = bz.weighted_pool(dx, dw, None, want_sum=False)
+    bz.gemm_strided_batched(dw, dx, c, 1, Cn, T, B, T, T * Cn, Cn, trans_a=True)
+    none2, tot2 = bz.weighted_pool(dx)
+    torch.cuda.synchronize()
+    assert none is None and none2 is None and torch.equal(att2, c.reshape(B, Cn)) and torch.equal(tot2, s)
+    # oracle: fp32 sums in ascending t of the rounded operands
+    wm = _round_to(w * mask, dtype_name)
+    want_att = np.zeros((B, Cn), np.float32)
+    want_sum = np.zeros((B, Cn), np.float32)
+    for t in range(T):
+        want_att += wm[:, t, :] * x[:, t, :]
+        want_sum += x[:, t, :]
+    tol = 1e-5 if dtype_name == "f32" else 2e-3
+    np.testing.assert_allclose(att.float().cpu().numpy(), want_att, rtol=tol, atol=tol * max(1.0, np.abs(want_att).max()))
+    np.testing.assert_allclose(tot.float().cpu().numpy(), want_sum, rtol=tol, atol=tol * max(1.0, np.abs(want_sum).max()))

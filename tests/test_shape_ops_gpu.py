@@ -179,6 +179,33 @@ def test_concat_of_pieces_computed_on_the_fly_equals_the_separate_operators(bz, 
     assert np.array_equal(got.cpu().numpy().view(view), want.view(view))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("r0,r1,widths", [(40, 50, (54, 18, 8)),    # pieces of different widths: a lane looks its piece up
+                                          (9, 3, (130, 130)),        # one width, but more than 64 lanes' worth of a row
+                                          (300, 7, (64, 64, 64, 64))])
+def test_concat_of_pieces_of_mixed_widths(bz, oracle, dtype, r0, r1, widths):
+    """bz_concat_ew's general kernel (the pieces' widths differ, or a piece is wider than a wave covers): piece i is
+    q_i - k_i for even i and a copy of k_i for odd i, q_i broadcast over the second row coordinate."""
+    import torch
+    rng = np.random.default_rng(r0 + r1 + sum(widths))
+    pieces, want = [], []
+    for i, w in enumerate(widths):
+        q = rng.standard_normal((r0, 1, w)).astype(dtype)
+        k = rng.standard_normal((r0, r1, w)).astype(dtype)
+        if i % 2 == 0:
+            pieces.append((bz.EW_SUB, _dev(q), _dev(k)))
+            want.append(oracle.elementwise("Sub", q.astype(np.float32), k.astype(np.float32)).astype(dtype))
+        else:
+            pieces.append((bz.EW_ASSIGN, _dev(k), None))
+            want.append(k)
+    print("case", dtype.__name__, r0, r1, widths, flush=True)
+    got = bz.concat_ew(pieces)
+    torch.cuda.synchronize()
+    want = np.concatenate(want, axis=2)
+    view = np.uint32 if dtype == np.float32 else np.uint16
+    assert tuple(got.shape) == want.shape and np.array_equal(got.cpu().numpy().view(view), want.view(view))
+
+
 def test_bad_descriptors_are_refused(bz):
     import ctypes as C
     d = bz.BcastDesc()

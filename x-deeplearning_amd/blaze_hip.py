@@ -20,7 +20,7 @@ ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 
 
 EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
-    "bz_embed_pool", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched",
+    "bz_embed_pool", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
     "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
@@ -58,6 +58,11 @@ class BgemmDesc(C.Structure):
                 ("stride_b", C.c_int64), ("stride_c", C.c_int64), ("trans_a", C.c_int32), ("trans_b", C.c_int32),
                 ("m", C.c_int32), ("n", C.c_int32), ("k", C.c_int32), ("batch", C.c_int32), ("dtype", C.c_int32),
                 ("alpha", C.c_float), ("beta", C.c_float)]
+
+
+class WeightedPoolDesc(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("mask", C.c_void_p), ("x", C.c_void_p), ("att", C.c_void_p), ("sum", C.c_void_p),
+                ("batch", C.c_int64), ("t", C.c_int32), ("c", C.c_int32), ("dtype", C.c_int32), ("reserved_", C.c_int32)]
 
 
 class ActDesc(C.Structure):
@@ -134,6 +139,7 @@ def lib():
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]
+        l.bz_weighted_pool.argtypes = [C.POINTER(WeightedPoolDesc), vp]
         l.bz_concat_ew.argtypes = [C.POINTER(ConcatEwDesc), vp]
         l.bz_activation.argtypes = [C.POINTER(ActDesc), vp]
         l.bz_concat_cols.argtypes = [C.POINTER(ConcatDesc), vp]
@@ -416,6 +422,23 @@ def gemm_strided_batched(a, b, c, m, n, k, batch, stride_a, stride_b, stride_c, 
     d.alpha, d.beta = alpha, beta
     check(lib().bz_gemm_strided_batched(C.byref(d), _stream_ptr(stream)))
     return c
+
+
+def weighted_pool(x, w=None, mask=None, want_sum=True, stream=None):
+    """x [B, T, C]; w, mask [B, T] (or [B, T, 1]) -> (att [B, C] or None, sum [B, C] or None), see bz_weighted_pool."""
+    import torch
+    B, T, Cn = x.shape
+    d = WeightedPoolDesc()
+    att = torch.empty((B, Cn), dtype=x.dtype, device=x.device) if w is not None else None
+    tot = torch.empty((B, Cn), dtype=x.dtype, device=x.device) if want_sum else None
+    d.x = x.data_ptr()
+    d.w = w.data_ptr() if w is not None else None
+    d.mask = mask.data_ptr() if mask is not None else None
+    d.att = att.data_ptr() if att is not None else None
+    d.sum = tot.data_ptr() if tot is not None else None
+    d.batch, d.t, d.c, d.dtype = B, T, Cn, bz_dtype(x.dtype)
+    check(lib().bz_weighted_pool(C.byref(d), _stream_ptr(stream)))
+    return att, tot
 
 
 def activation(x, act, params=(), out=None, act_alpha=0.0, dice_nosqrt=False, stream=None):

@@ -93,7 +93,81 @@ void launch_bgemm(const bz_bgemm_desc& d, int grid, hipStream_t s) {
 #undef BZ_BGEMM
 }
 
+// One wave per batch item, lanes over the channels.  Both sums walk t in ascending order, the weighted one with the
+// fused multiply-add bz_bgemm_kernel uses for C = A^T * B, the plain one with separate adds like bz_reduce_sum_kernel,
+// and the weight is rounded to the tensor type first, as the Mul operator would have stored it: the results are the
+// three operators' results bit for bit.
+// (a history of 50 in one round of loads: with one wave per item and four waves per CU the kernel is a chain of
+// round trips to memory, 10 us at 16 steps per round on [1024, 50, 54])
+constexpr int kPoolUnroll = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void bz_weighted_pool_kernel(const T* __restrict__ w, const T* __restrict__ mask,
+                                                               const T* __restrict__ x, T* __restrict__ att, T* __restrict__ sum,
+                                                               int64_t batch, int t_len, int c_len) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+  if (item >= batch) return;
+  const T* wp = w + item * t_len;
+  const T* mp = mask ? mask + item * t_len : nullptr;
+  const T* xp = x + item * (int64_t)t_len * c_len;
+  for (int c = lane; c < c_len; c += 64) {
+    float acc_w = 0.f, acc_s = 0.f;
+    for (int t0 = 0; t0 < t_len; t0 += kPoolUnroll) {
+      // lane l fetches the weight of step t0 + l (every lane needs every weight: they are handed round below), then
+      // its own channel of all the steps; nothing is used before everything has been asked for
+      const int tl = t0 + lane < t_len ? t0 + lane : t_len - 1;
+      const float w_raw = ld<T>(wp + tl);
+      const float m_raw = mp ? ld<T>(mp + tl) : 1.f;
+      float xv[kPoolUnroll];
+#pragma unroll
+      for (int u = 0; u < kPoolUnroll; ++u) {
+        const int t = t0 + u < t_len ? t0 + u : t_len - 1;  // clamped address; the term is skipped below
+        xv[u] = ld<T>(xp + (int64_t)t * c_len + c);
+      }
+      float w_mine = w_raw;
+      if (mp) {
+        T r;
+        st<T>(&r, __fmul_rn(w_raw, m_raw));
+        w_mine = ld<T>(&r);
+      }
+#pragma unroll
+      for (int u = 0; u < kPoolUnroll; ++u)
+        if (t0 + u < t_len) {
+          const float wu = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w_mine), u));
+          acc_w = fmaf(wu, xv[u], acc_w);
+          acc_s = __fadd_rn(acc_s, xv[u]);
+        }
+    }
+    if (att) st<T>(att + item * c_len + c, acc_w);
+    if (sum) st<T>(sum + item * c_len + c, acc_s);
+  }
+}
+
 }  // namespace
+
+extern "C" int bz_weighted_pool(const bz_weighted_pool_desc* desc, bz_stream_t stream) {
+  BZ_REQUIRE(desc != nullptr, "bz_weighted_pool: null descriptor");
+  const bz_weighted_pool_desc& d = *desc;
+  BZ_REQUIRE(d.x != nullptr && (d.att != nullptr || d.sum != nullptr), "bz_weighted_pool: null x, or neither output asked for");
+  BZ_REQUIRE(d.att == nullptr || d.w != nullptr, "bz_weighted_pool: the weighted sum needs w");
+  BZ_REQUIRE(d.batch >= 0 && d.t > 0 && d.c > 0, "bz_weighted_pool: bad shape batch=%lld t=%d c=%d", (long long)d.batch, d.t, d.c);
+  if (d.batch == 0) return BZ_OK;
+  BZ_REQUIRE((d.batch + 3) / 4 < (1ll << 31), "bz_weighted_pool: batch %lld too large", (long long)d.batch);
+  const int grid = (int)((d.batch + 3) / 4);
+  hipStream_t s = bz::as_stream(stream);
+  const void* w = d.att ? d.w : d.x;  // no weighted sum: any readable address of t elements per item will do
+  if (d.dtype == BZ_F32)
+    hipLaunchKernelGGL(bz_weighted_pool_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)w, (const float*)(d.att ? d.mask : nullptr),
+                       (const float*)d.x, (float*)d.att, (float*)d.sum, d.batch, d.t, d.c);
+  else if (d.dtype == BZ_F16)
+    hipLaunchKernelGGL(bz_weighted_pool_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)w,
+                       (const __half*)(d.att ? d.mask : nullptr), (const __half*)d.x, (__half*)d.att, (__half*)d.sum, d.batch, d.t, d.c);
+  else
+    return bz::fail(BZ_ENOTSUP, "bz_weighted_pool: unsupported dtype %d", d.dtype);
+  BZ_LAUNCH_OK("bz_weighted_pool_kernel");
+  return BZ_OK;
+}
 
 extern "C" int bz_gemm_strided_batched(const bz_bgemm_desc* desc, bz_stream_t stream) {
   BZ_REQUIRE(desc != nullptr, "bz_gemm_strided_batched: null descriptor");

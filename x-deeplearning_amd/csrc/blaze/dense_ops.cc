@@ -692,9 +692,16 @@ void UlfCompatibleReshape(Blob* a, Blob* b) {
 
 // ------------------------------------------------------------------------------------------ MatMul
 template <class Context>
-class MatMulOp : public Operator<Context> {
+class MatMulOp : public Operator<Context>, public WeightedPoolHost {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
+  bool WeightedPoolEligible() const override { return transa_ && !transb_ && !from_deepnet_; }
+  void AdoptWeightedPool(OperatorBase* mul, OperatorBase* reduce_sum) override {
+    pool_mul_ = mul;
+    pool_sum_ = reduce_sum;
+  }
+  int LaunchesOfLastRun() const override { return launches_; }
+
   MatMulOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
     transa_ = OperatorBase::GetSingleArgument<bool>("transA", false);
     transb_ = OperatorBase::GetSingleArgument<bool>("transB", false);
@@ -702,6 +709,14 @@ class MatMulOp : public Operator<Context> {
   }
 
   bool RunOnDevice() override {
+    launches_ = 1;
+    if (pool_mul_ || pool_sum_) {
+      if (RunWeightedPool()) return true;
+      // shapes the one-launch form does not take: the adopted operators run after all
+      if (pool_mul_ && !pool_mul_->Run(context_.stream_id())) return false;
+      if (pool_sum_ && !pool_sum_->Run(context_.stream_id())) return false;
+      launches_ += (pool_mul_ != nullptr) + (pool_sum_ != nullptr);
+    }
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
     Blob* c = this->Output(0);
@@ -749,7 +764,46 @@ class MatMulOp : public Operator<Context> {
     shape[shape.size() - 1] = transb_ ? b->shape()[br - 2] : b->shape()[br - 1];
     c->Reshape(shape);
   }
+  // [B, T, 1]^T x [B, T, C] with the weight = product of two [B, T, 1] tensors, and the sum of the history over T:
+  // one launch.  False (nothing launched, no blob touched) when the tensors are not of that form.
+  bool RunWeightedPool() {
+    Blob* x = this->Input(1);
+    Blob* w = pool_mul_ ? pool_mul_->Input(0) : this->Input(0);
+    Blob* mask = pool_mul_ ? pool_mul_->Input(1) : nullptr;
+    const std::vector<TIndex>& xs = x->shape();
+    if (xs.size() != 3 || x->pitch() != 0 || w->pitch() != 0) return false;
+    const std::vector<TIndex> col = {xs[0], xs[1], 1};
+    if (w->shape() != col || w->data_type() != x->data_type()) return false;
+    if (mask && (mask->shape() != col || mask->data_type() != x->data_type() || mask->pitch() != 0)) return false;
+    if (x->data_type() != kFloat && x->data_type() != kFloat16) return false;
+    if (xs[1] <= 0 || xs[2] <= 0 || xs[1] >= (1ll << 31) || xs[2] >= (1ll << 31)) return false;
+    Blob* c = this->Output(0);
+    c->set_data_type((DataType)x->data_type());
+    c->Reshape({xs[0], 1, xs[2]});
+    Blob* s = nullptr;
+    if (pool_sum_) {
+      s = pool_sum_->Output(0);
+      s->set_data_type((DataType)x->data_type());
+      s->Reshape({xs[0], xs[2]});
+    }
+    bz_weighted_pool_desc d;
+    memset(&d, 0, sizeof(d));
+    d.w = w->data();
+    d.mask = mask ? mask->data() : nullptr;
+    d.x = x->data();
+    d.att = c->data();
+    d.sum = s ? s->data() : nullptr;
+    d.batch = (int64_t)xs[0];
+    d.t = (int32_t)xs[1];
+    d.c = (int32_t)xs[2];
+    d.dtype = BzType(x->data_type());
+    BZ_CHECK(bz_weighted_pool(&d, context_.hip_stream()));
+    return true;
+  }
   bool transa_, transb_, from_deepnet_;
+  OperatorBase* pool_mul_ = nullptr;
+  OperatorBase* pool_sum_ = nullptr;
+  int launches_ = 1;
 };
 
 REGISTER_HIP_OPERATOR(MatMul, MatMulOp<HIPContext>);

@@ -216,6 +216,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     PackSiblingFcs();
     AliasConcatInputs();
     FuseConcatPieces();
+    FuseWeightedPools();
   }
 }
 
@@ -248,10 +249,64 @@ void SimpleNet::FuseFcHeads() {
   }
 }
 
-// Concat inputs that are outputs of elementwise operators -> pieces computed by the Concat itself (graph.h,
-// ConcatPieceSource).  A producer is taken over when its output is read only by the Concat -- or, as a shape
-// reference (second input of BroadcastTo), by another producer the same Concat takes over -- is neither an output of the
-// net nor written in place, and nothing between the producer and the Concat overwrites the producer's inputs.
+// Mul -> MatMul(transA) [+ ReduceSum of the MatMul's second input over axis 1] -> the MatMul alone (graph.h,
+// WeightedPoolHost).  The Mul is taken over when its output is read only by the MatMul and is no output of the net; the
+// ReduceSum when it comes after the MatMul and nothing in between writes the tensor both read.  Switch:
+// fuse_weighted_pool: 0.
+void SimpleNet::FuseWeightedPools() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_weighted_pool");
+  if (arg && arg->has_i && arg->i == 0) return;
+  auto readers_of = [&](const std::string& name) {
+    int readers = 0;
+    for (size_t j = 0; j < operators_.size(); ++j)
+      for (const auto& in : operators_[j]->operator_def().input()) readers += (in == name);
+    for (const auto& eo : external_output_) readers += (eo == name);
+    return readers;
+  };
+  for (size_t m = 0; m < operators_.size(); ++m) {
+    auto* host = skipped_[m] ? nullptr : dynamic_cast<WeightedPoolHost*>(operators_[m].get());
+    if (!host || !host->WeightedPoolEligible()) continue;
+    const OperatorDef& md = operators_[m]->operator_def();
+    if (md.input_size() != 2) continue;
+    // the Mul: last writer of Input(0) before the MatMul
+    int mul = -1;
+    for (int j = (int)m - 1; j >= 0 && mul < 0; --j)
+      for (const auto& out : operators_[j]->operator_def().output())
+        if (out == md.input(0)) mul = j;
+    if (mul >= 0) {
+      const OperatorDef& pd = operators_[mul]->operator_def();
+      bool ok = !skipped_[mul] && operators_[mul]->type() == "Mul" && pd.input_size() == 2 && pd.output_size() == 1 &&
+                readers_of(md.input(0)) == 1 && pd.output(0) != pd.input(0) && pd.output(0) != pd.input(1);
+      // nothing between the Mul and the MatMul may overwrite what the Mul reads
+      for (size_t k = mul + 1; k < m && ok; ++k)
+        for (const auto& out : operators_[k]->operator_def().output()) ok &= (out != pd.input(0) && out != pd.input(1));
+      if (!ok) mul = -1;
+    }
+    int red = -1;
+    for (size_t j = m + 1; j < operators_.size() && red < 0; ++j) {
+      const OperatorDef& rd = operators_[j]->operator_def();
+      bool writes = false;
+      for (const auto& out : rd.output()) writes |= (out == md.input(1));
+      if (writes) break;  // the history changes here: a later ReduceSum sums something else
+      if (skipped_[j] || operators_[j]->type() != "ReduceSum" || rd.input_size() != 1 || rd.input(0) != md.input(1)) continue;
+      if (ArgumentHelper::GetSingle<int>(rd.arg(), "axis", 0) != 1 || ArgumentHelper::GetSingle<int>(rd.arg(), "keepdims", 1) != 0) continue;
+      // moved up to the MatMul's position: its output must not be something an operator in between still reads or writes
+      bool ok = rd.output_size() == 1;
+      for (size_t k = m; k < j && ok; ++k) {
+        for (const auto& in : operators_[k]->operator_def().input()) ok &= (in != rd.output(0));
+        for (const auto& out : operators_[k]->operator_def().output()) ok &= (out != rd.output(0));
+      }
+      if (ok) red = (int)j;
+    }
+    if (mul < 0 && red < 0) continue;
+    host->AdoptWeightedPool(mul >= 0 ? operators_[mul].get() : nullptr, red >= 0 ? operators_[red].get() : nullptr);
+    if (mul >= 0) skipped_[mul] = true;
+    if (red >= 0) skipped_[red] = true;
+  }
+}
+
+// Sibling Gemm operators (same input, same attributes, constant weights of one shape) -> one launch over the stacked
+// weights (graph.h, SiblingFc).  Switch: pack_sibling_gemms: 0.
 void SimpleNet::PackSiblingFcs() {
   const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "pack_sibling_gemms");
   if (arg && arg->has_i && arg->i == 0) return;
@@ -280,6 +335,10 @@ void SimpleNet::PackSiblingFcs() {
   }
 }
 
+// Concat inputs that are outputs of elementwise operators -> pieces computed by the Concat itself (graph.h,
+// ConcatPieceSource).  A producer is taken over when its output is read only by the Concat -- or, as a shape
+// reference (second input of BroadcastTo), by another producer the same Concat takes over -- is neither an output of the
+// net nor written in place, and nothing between the producer and the Concat overwrites the producer's inputs.
 void SimpleNet::FuseConcatPieces() {
   const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_concat_pieces");
   if (arg && arg->has_i && arg->i == 0) return;

@@ -99,6 +99,7 @@ class SimpleNet : public Net {
   void FuseConcatPieces();
   void FuseFcHeads();
   void PackSiblingFcs();
+  void FuseWeightedPools();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -182,6 +183,18 @@ class ConcatPieceHost {  // implemented by Concat
   virtual ~ConcatPieceHost() {}
   // input `input_idx` is the output of `producer` (net position `position`), which the net will not run any more
   virtual void AdoptProducer(int input_idx, OperatorBase* producer, int position) = 0;
+};
+
+// MatMul(transA) of a weight column [B, T, 1] with a history [B, T, C] whose weight is the product of two equally
+// shaped tensors (score * mask) read by nothing else, optionally next to a ReduceSum of the same history over T:
+// the MatMul computes all of it in one launch (bz_weighted_pool) and the Mul and the ReduceSum are skipped.  Same
+// bits as the separate operators.
+class WeightedPoolHost {  // implemented by MatMul
+ public:
+  virtual ~WeightedPoolHost() {}
+  virtual bool WeightedPoolEligible() const = 0;  // static part: transA, no transB
+  // mul: producer of Input(0) (may be null); reduce_sum: a ReduceSum(axis 1, keepdims 0) of Input(1) (may be null)
+  virtual void AdoptWeightedPool(OperatorBase* mul, OperatorBase* reduce_sum) = 0;
 };
 
 }  // namespace blaze

@@ -158,8 +158,16 @@ struct CewP {
   int64_t rows, r1, dst_pitch;
 };
 
-// VEC consecutive columns of one output row per thread (the host picks a VEC that divides every width).  IdxT is
-// 32-bit whenever the element count allows: the two divisions per thread are the expensive part of this kernel.
+// VEC consecutive columns of one output row per lane (the host picks a VEC that divides every width, stride and
+// address, so a lane's VEC elements are one aligned load or store).  A wave owns a row at a time: which row, and where
+// its operands start, is worked out once per row for the whole wave; inside the row a lane only has to find its piece.
+// (One flat index per thread cost two integer divisions per VEC elements and element-wise accesses: 24.7 us for the
+// [51200, 216] fp16 attention input of a DIN model, whose 54-wide pieces allow no more than VEC = 2.)
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) CewPack {
+  T e[VEC];
+};
+
 template <typename T, int VEC, typename IdxT>
 __global__ __launch_bounds__(256) void bz_concat_ew_kernel(T* __restrict__ dst, CewP arg) {
   // the piece table is indexed with a run-time piece number: from LDS, not from a per-lane copy of the arguments
@@ -167,37 +175,116 @@ __global__ __launch_bounds__(256) void bz_concat_ew_kernel(T* __restrict__ dst, 
   static_assert(sizeof(CewP) % 4 == 0, "copied in 32-bit words");
   for (int w = threadIdx.x; w < (int)(sizeof(CewP) / 4); w += 256) ((uint32_t*)&p)[w] = ((const uint32_t*)&arg)[w];
   __syncthreads();
-  const IdxT per_row = (IdxT)(p.col0[p.n] / VEC);
-  const IdxT nvec = (IdxT)p.rows * per_row;
-  const IdxT r1 = (IdxT)p.r1;
-  for (IdxT v = (IdxT)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (IdxT)gridDim.x * 256) {
-    const IdxT row = v / per_row;
-    const int col = (int)(v - row * per_row) * VEC;
-    int k = 0;
-#pragma unroll
-    for (int q = 1; q < BZ_CEW_MAX; ++q) k += (q < p.n && col >= p.col0[q]);
-    const int c = col - p.col0[k];
+  using Pack = CewPack<T, VEC>;
+  const int per_row = p.col0[p.n] / VEC;
+  const int lane = threadIdx.x & 63;
+  const IdxT rows = (IdxT)p.rows, r1 = (IdxT)p.r1;
+  const IdxT nwaves = (IdxT)gridDim.x * 4;
+  for (IdxT row = (IdxT)blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += nwaves) {
     const IdxT i0 = row / r1, i1 = row - i0 * r1;
-    const T* x = (const T*)p.x[k] + (int64_t)i0 * p.xs[k][0] + (int64_t)i1 * p.xs[k][1] + c;
-    T* out = dst + (int64_t)row * p.dst_pitch + col;
-    const int op = p.op[k];
-    if (op == BZ_EW_ASSIGN) {
+    T* out_row = dst + (int64_t)row * p.dst_pitch;
+    for (int cv = lane; cv < per_row; cv += 64) {
+      const int col = cv * VEC;
+      int k = 0;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) out[e] = x[e];
-    } else {
-      const T* y = (const T*)p.y[k] + (int64_t)i0 * p.ys[k][0] + (int64_t)i1 * p.ys[k][1] + c;
+      for (int q = 1; q < BZ_CEW_MAX; ++q) k += (q < p.n && col >= p.col0[q]);
+      const int c = col - p.col0[k];
+      const Pack x = *(const Pack*)((const T*)p.x[k] + (int64_t)i0 * p.xs[k][0] + (int64_t)i1 * p.xs[k][1] + c);
+      const int op = p.op[k];
+      Pack o = x;
+      if (op != BZ_EW_ASSIGN) {
+        const Pack y = *(const Pack*)((const T*)p.y[k] + (int64_t)i0 * p.ys[k][0] + (int64_t)i1 * p.ys[k][1] + c);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float a = ldv<T>(&x.e[e]), b = ldv<T>(&y.e[e]);
+          stv<T>(&o.e[e], op == BZ_EW_ADD ? __fadd_rn(a, b) : op == BZ_EW_SUB ? __fsub_rn(a, b) : op == BZ_EW_MUL ? __fmul_rn(a, b) : __fdiv_rn(a, b));
+        }
+      }
+      *(Pack*)(out_row + col) = o;
+    }
+  }
+}
+
+// The same when every piece has the same width W, W / VEC <= 64 and no piece divides (the attention input
+// [q, k, q-k, q*k]): a lane owns VEC columns of a piece and walks the pieces, so it needs no search for its piece, and
+// 64 / (W / VEC) rows share a wave so that no lane idles.  NP >= the number of pieces is a compile-time bound, and
+// there is no branch in the row loop: a branch makes the compiler wait for every load in flight, and selecting among
+// the results of all four operations per element cost some 700 instructions a row (20.9 us on [51200, 216] fp16).
+// Instead every piece is one fused multiply-add whose operands are chosen per piece,
+//   x + y = fma(x, 1, y)    x - y = fma(x, 1, -y)    x * y = fma(x, y, -0)
+// each rounded once like the plain operation (-0 as the addend keeps the sign of a zero product), and a copy keeps the
+// loaded bits.  A piece without a second operand reads its first one twice; an absent piece reads piece 0 again.
+template <typename T, int VEC, int NP>
+__global__ __launch_bounds__(256) void bz_concat_ew_uniform_kernel(T* __restrict__ dst, CewP p) {
+  using Pack = CewPack<T, VEC>;
+  const int per_piece = p.col0[1] / VEC;
+  const int rows_per_wave = 64 / per_piece;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane / per_piece, cv = lane - sub * per_piece;
+  if (sub >= rows_per_wave) return;
+  const uint32_t rows = (uint32_t)p.rows, r1 = (uint32_t)p.r1;
+  const uint32_t step = gridDim.x * 4 * rows_per_wave;
+  for (uint32_t row = (blockIdx.x * 4 + (threadIdx.x >> 6)) * rows_per_wave + sub; row < rows; row += step) {
+    const uint32_t i0 = row / r1, i1 = row - i0 * r1;
+    T* out = dst + (int64_t)row * p.dst_pitch + cv * VEC;
+    Pack xs[NP], ys[NP];
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+      const int kk = k < p.n ? k : 0;
+      const bool two = p.op[kk] != BZ_EW_ASSIGN;
+      const T* yb = two ? (const T*)p.y[kk] : (const T*)p.x[kk];
+      const int64_t ys0 = two ? p.ys[kk][0] : p.xs[kk][0], ys1 = two ? p.ys[kk][1] : p.xs[kk][1];
+      xs[k] = *(const Pack*)((const T*)p.x[kk] + (int64_t)i0 * p.xs[kk][0] + (int64_t)i1 * p.xs[kk][1] + cv * VEC);
+      ys[k] = *(const Pack*)(yb + (int64_t)i0 * ys0 + (int64_t)i1 * ys1 + cv * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+      const int op = p.op[k < p.n ? k : 0];
+      const bool mul = op == BZ_EW_MUL, neg = op == BZ_EW_SUB, copy = op == BZ_EW_ASSIGN;
+      Pack o;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        const float a = ldv<T>(x + e), b = ldv<T>(y + e);
-        stv<T>(out + e, op == BZ_EW_ADD ? __fadd_rn(a, b) : op == BZ_EW_SUB ? __fsub_rn(a, b) : op == BZ_EW_MUL ? __fmul_rn(a, b) : __fdiv_rn(a, b));
+        const float a = ldv<T>(&xs[k].e[e]), b = ldv<T>(&ys[k].e[e]);
+        const float r = __builtin_fmaf(a, mul ? b : 1.f, mul ? -0.f : (neg ? -b : b));
+        stv<T>(&o.e[e], r);
+        if (copy) o.e[e] = xs[k].e[e];
       }
+      if (k < p.n) *(Pack*)(out + p.col0[k]) = o;
     }
   }
 }
 
 template <typename T, typename IdxT>
 int launch_concat_ew_i(void* dst, const CewP& p, int vec, hipStream_t s) {
-  const int grid = grid_for(p.rows * (p.col0[p.n] / vec));
+  bool uniform = p.col0[1] / vec <= 64 && sizeof(IdxT) == 4;
+  for (int k = 0; k < p.n; ++k) uniform &= (p.col0[k + 1] - p.col0[k] == p.col0[1]) && p.op[k] != BZ_EW_DIV;
+  if (uniform) {
+    const int rows_per_wave = 64 / (p.col0[1] / vec);
+    const int64_t blocks = (p.rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave);
+    const int grid = (int)(blocks < 256 * 32 ? blocks : 256 * 32);
+#define BZ_CEW_U(V, NP) hipLaunchKernelGGL((bz_concat_ew_uniform_kernel<T, V, NP>), dim3(grid), dim3(256), 0, s, (T*)dst, p)
+#define BZ_CEW_UV(V)       \
+  do {                     \
+    if (p.n <= 2)          \
+      BZ_CEW_U(V, 2);      \
+    else if (p.n <= 4)     \
+      BZ_CEW_U(V, 4);      \
+    else                   \
+      BZ_CEW_U(V, BZ_CEW_MAX); \
+  } while (0)
+    switch (vec) {
+      case 8: BZ_CEW_UV(8); break;
+      case 4: BZ_CEW_UV(4); break;
+      case 2: BZ_CEW_UV(2); break;
+      default: BZ_CEW_UV(1); break;
+    }
+#undef BZ_CEW_UV
+#undef BZ_CEW_U
+    BZ_LAUNCH_OK("bz_concat_ew_uniform_kernel");
+    return BZ_OK;
+  }
+  const int64_t blocks = (p.rows + 3) / 4;  // a wave per row, four waves per block
+  const int grid = (int)(blocks < 256 * 32 ? blocks : 256 * 32);
   switch (vec) {
     case 8: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 8, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
     case 4: hipLaunchKernelGGL((bz_concat_ew_kernel<T, 4, IdxT>), dim3(grid), dim3(256), 0, s, (T*)dst, p); break;
@@ -210,9 +297,8 @@ int launch_concat_ew_i(void* dst, const CewP& p, int vec, hipStream_t s) {
 
 template <typename T>
 int launch_concat_ew(void* dst, const CewP& p, int vec, hipStream_t s) {
-  const int64_t nvec = p.rows * (p.col0[p.n] / vec);
-  // (the grid-stride loop adds at most 2^21 to an index below nvec)
-  if (nvec < (1ll << 31) - (1ll << 22) && p.r1 < (1ll << 31)) return launch_concat_ew_i<T, uint32_t>(dst, p, vec, s);
+  // (the grid-stride loop adds at most 2^15 to a row index below rows)
+  if (p.rows < (1ll << 31) - (1ll << 16) && p.r1 < (1ll << 31)) return launch_concat_ew_i<T, uint32_t>(dst, p, vec, s);
   return launch_concat_ew_i<T, int64_t>(dst, p, vec, s);
 }
 
