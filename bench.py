@@ -127,6 +127,27 @@ def run_probes(args, np, torch, bz, arch):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / reps  # us
 
+    if args.fc_probe:
+        # config 5's first layer alone (8192 x 12800 -> 1024 bf16, bias + ReLU), inputs alternating between two buffers
+        # so that the activations come from HBM, not from the last-level cache
+        M, K, N = 8192, 12800, 1024
+        g = torch.Generator(device="cuda").manual_seed(5)
+        xs = [(torch.randn((M, K), generator=g, device="cuda") * 0.5).to(torch.bfloat16) for _ in range(2)]
+        w = bz.pack_weight((torch.randn((K, N), generator=g, device="cuda") / K ** 0.5), False, bz.BF16)
+        b = torch.randn(N, generator=g, device="cuda") * 0.1
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        k = [0]
+
+        def launch():
+            k[0] += 1
+            bz.fc_fused(xs[k[0] & 1], w, K, bias=b, act=bz.ACT_LEAKY_RELU, act_alpha=0.0, out=y)
+        us = ev_time(launch, 20)
+        lib_us = ev_time(lambda: torch.nn.functional.linear(xs[0], w[:, :K]), 20)
+        print(json.dumps({"probe": "bz_fc_fused %dx%d -> %d bf16, bias + ReLU" % (M, K, N), "us": round(us, 2),
+                          "TFLOP/s": round(2.0 * M * K * N / us / 1e6, 1), "frac_of_mfma_peak": round(2.0 * M * K * N / us / 1e6 / MFMA_PEAK_TFLOPS, 4),
+                          "library_gemm_us": round(lib_us, 2), "device": arch}))
+        return
+
     res = {"probe": "random gathers of whole rows, nothing else", "device": arch}
     region = torch.ones(args.probe_region_mib << 20, dtype=torch.uint8, device="cuda")
     side = torch.ones((args.probe_region_mib << 20) // 64, dtype=torch.float32, device="cuda")
@@ -408,6 +429,11 @@ def main():
     ap.add_argument("--gather-probe", action="store_true",
                     help="only measure what the memory system gives random gathers of 64- and 128-byte rows (a kernel that "
                          "does nothing else) and exit")
+    ap.add_argument("--counters-run", action="store_true",
+                    help="for runs under rocprofv3 --pmc, where every dispatch is serialised: skip the steady-state region and "
+                         "take the latency from --steps samples only (the line then carries no steady_state)")
+    ap.add_argument("--fc-probe", action="store_true",
+                    help="only run config 5's first FC layer (8192 x 12800 -> 1024 bf16) a few times and exit (for counter runs)")
     ap.add_argument("--probe-region-mib", type=int, default=2048)
     ap.add_argument("--probe-case", type=int, default=None, help="run one case of --gather-probe only (for counter runs)")
     ap.add_argument("--threads", type=int, default=8,
@@ -430,7 +456,7 @@ def main():
 
     assert torch.cuda.is_available(), "no GPU visible"
     arch = bz.device_check()
-    if args.calibrate_copy or args.gather_probe:
+    if args.calibrate_copy or args.gather_probe or args.fc_probe:
         run_probes(args, np, torch, bz, arch)
         return
     cfg = Config2()
@@ -486,7 +512,8 @@ def main():
         t1 = time.perf_counter()
         dt = t1 - t0
         s0 = time.perf_counter()
-        pool.run(predictors, S)
+        if not args.counters_run:
+            pool.run(predictors, S)
         torch.cuda.synchronize()
         ds = time.perf_counter() - s0
     else:
@@ -517,13 +544,14 @@ def main():
             return b - a
         run_region(0, warm)
         dt = run_region(warm, K)
-        ds = run_region(warm + K, S)
-    steady = {"steps": S, "ms_per_step": round(ds * 1e3 / S, 5), "samples/s": round(cfg.batch * S / ds, 1)}
+        ds = 0.0 if args.counters_run else run_region(warm + K, S)
+    if not args.counters_run:
+        steady = {"steps": S, "ms_per_step": round(ds * 1e3 / S, 5), "samples/s": round(cfg.batch * S / ds, 1)}
     ms_per_step = dt * 1e3 / K
     samples_per_s = cfg.batch * K / dt
 
     # ---- latency: one batch at a time on one thread, each step submitted and waited for on its own
-    p50, p99, n_lat = latency_ms(np, run_step, max(K, 1000))
+    p50, p99, n_lat = latency_ms(np, run_step, K if args.counters_run else max(K, 1000))
 
     # ---- PCIe-inclusive rate: every step feeds all 79 inputs from pageable host memory and copies the output back
     if not args.no_feed and predictors is not None:
