@@ -18,15 +18,21 @@
 // The kernel is latency bound before it is bandwidth bound (a batch-2048 launch moves
 // ~36 MB), so the dependent chain is kept at: slot record -> segments -> ids -> rows.
 //   * segments -> offsets is fused: a workgroup sums the counts before its first
-//     sample and scans its own 256/lpr counts in LDS (no separate scan launch, no
+//     sample and scans its own 512/lpr counts in LDS (no separate scan launch, no
 //     offsets round trip);
 //   * with equal work per slot the slot index is a division, not a search;
-//   * the specialised ksum/kavg kernel walks a segment 16 ids at a time: the lanes of
-//     a group load disjoint ids/values (one coalesced read), resolve them to rows,
-//     pass rows and values around with ds_bpermute, then issue up to 16 row loads
-//     before the first add -- that is where the memory-level parallelism comes from.
+//   * the specialised ksum/kavg kernel walks a segment kBlockIds ids at a time: the lanes
+//     of a group load disjoint ids/values (one coalesced read), resolve them to rows,
+//     pass rows and values around with ds_bpermute, then issue the row loads before
+//     the first add.  The block is short on purpose: the memory-level parallelism
+//     comes from eight resident waves per SIMD, not from a deep unroll in each.
 // A generic kernel covers kassign, mixed slot shapes, rows wider than 64 chunks and
 // precomputed offsets.
+//
+// The memory system fetches 128-byte lines: a table whose rows sit inside lines
+// (bz_table_pitch) costs one request per id, and an int8 row's scale lives in the
+// row's own line.  Counts come from the caller and are not trusted: negative counts
+// are zero and offsets stop at the slot's nnz.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
@@ -44,7 +50,11 @@ constexpr int kUnroll = 4;  // rows in flight per lane group in the generic kern
 // ---------------------------------------------------------------------------------------------
 // segments -> offsets (exclusive scan), one workgroup per array
 // ---------------------------------------------------------------------------------------------
-constexpr int kScanItems = 16;  // int32 per thread per tile -> 8192 per workgroup tile (a batch of 8192 in one pass)
+constexpr int kScanItems = 8;  // counts per thread per tile -> 4096 per workgroup tile
+constexpr int kScanTile = kThreads * kScanItems;
+// a thread's kScanItems consecutive entries sit kScanItems + 1 apart from the next thread's: its walk over them does
+// not hit its neighbours' LDS banks
+__device__ __forceinline__ int scan_slot(int i) { return i + i / kScanItems; }
 
 __device__ __forceinline__ int64_t wave_incl_scan(int64_t v, int lane) {
 #pragma unroll
@@ -57,19 +67,47 @@ __device__ __forceinline__ int64_t wave_incl_scan(int64_t v, int lane) {
 
 // Counts below zero are taken as zero and the running offset stops at `limit` (the length of the ids / values arrays),
 // so no offset this scan produces points outside them.
-__device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restrict__ off, int64_t n, int64_t limit) {
+// Global memory is read and written one element per lane, consecutive lanes consecutive elements; the thread-owns-a-run
+// layout the scan wants exists only in LDS.  (With every thread loading and storing its own run directly, a wave's
+// access touched 64 lines for 256 or 512 bytes: 200 slots x 8192 counts took 19.5 us.)
+// Tiles [first_tile, first_tile + n_tiles) of the array (n_tiles < 0: all of them from first_tile on).  A workgroup that
+// does not start at tile 0 first adds up the counts before its first tile - all those loads are independent, so a slot's
+// scan split over several workgroups takes one tile's time, not the array's.
+__device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restrict__ off, int64_t n, int64_t limit,
+                              int64_t first_tile = 0, int64_t n_tiles = -1) {
   __shared__ int64_t wave_tot[kThreads / bz::kWave];
   __shared__ int64_t carry_s;
+  __shared__ int32_t cnt_s[kScanTile + kThreads];
+  __shared__ int64_t off_s[kScanTile + kThreads];
   const int tid = threadIdx.x;
   const int lane = tid & (bz::kWave - 1);
   const int wave = tid / bz::kWave;
-  if (tid == 0) carry_s = 0;
-  __syncthreads();
-  for (int64_t base = 0; base < n; base += (int64_t)kThreads * kScanItems) {
-    int64_t i0 = base + (int64_t)tid * kScanItems;
+  const int64_t begin = first_tile * kScanTile;
+  const int64_t end = (n_tiles < 0 || begin + n_tiles * kScanTile > n) ? n : begin + n_tiles * kScanTile;
+  if (begin > n || (begin == n && n != 0)) return;  // nothing here; whoever scans the last tile writes off[n]
+  {
+    int64_t part = 0;
+    for (int64_t i = tid; i < begin; i += kThreads) part += max(seg[i], 0);
+    part = wave_incl_scan(part, lane);
+    if (lane == bz::kWave - 1) wave_tot[wave] = part;
+    __syncthreads();
+    if (tid == 0) {
+      int64_t c = 0;
+      for (int w = 0; w < kThreads / bz::kWave; ++w) c += wave_tot[w];
+      carry_s = c;
+    }
+    __syncthreads();
+  }
+  for (int64_t base = begin; base < end; base += kScanTile) {
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      const int j = k * kThreads + tid;
+      cnt_s[scan_slot(j)] = (base + j < n) ? max(seg[base + j], 0) : 0;
+    }
+    __syncthreads();
     int32_t v[kScanItems];
 #pragma unroll
-    for (int k = 0; k < kScanItems; ++k) v[k] = (i0 + k < n) ? max(seg[i0 + k], 0) : 0;
+    for (int k = 0; k < kScanItems; ++k) v[k] = cnt_s[tid * (kScanItems + 1) + k];
     int64_t local = 0;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) local += v[k];
@@ -81,14 +119,19 @@ __device__ void scan_segments(const int32_t* __restrict__ seg, int64_t* __restri
     int64_t run = before + incl - local;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) {
-      if (i0 + k < n) off[i0 + k] = run < limit ? run : limit;
+      off_s[tid * (kScanItems + 1) + k] = run < limit ? run : limit;
       run += v[k];
     }
     __syncthreads();
     if (tid == kThreads - 1) carry_s = run;  // last thread's running total = total so far
+#pragma unroll
+    for (int k = 0; k < kScanItems; ++k) {
+      const int j = k * kThreads + tid;
+      if (base + j < n) off[base + j] = off_s[scan_slot(j)];
+    }
     __syncthreads();
   }
-  if (tid == 0) off[n] = carry_s < limit ? carry_s : limit;
+  if (tid == 0 && end == n) off[n] = carry_s < limit ? carry_s : limit;
 }
 
 __global__ __launch_bounds__(kThreads) void bz_scan_segments_kernel(const int32_t* __restrict__ seg,
@@ -98,15 +141,23 @@ __global__ __launch_bounds__(kThreads) void bz_scan_segments_kernel(const int32_
 
 // ext_off != nullptr: slot i's offsets go to ext_off + i * ext_stride instead of slot.offsets (at most ext_stride - 1
 // samples of a slot are scanned, so a record whose batch disagrees with the plan cannot write past its share)
+// Grid (slots, parts): part p of a slot scans tiles p, or, for the last part, every tile from p on.
 __global__ __launch_bounds__(kThreads) void bz_scan_segments_slots_kernel(const bz_embed_slot* __restrict__ slots,
                                                                           int64_t* __restrict__ ext_off, int64_t ext_stride) {
   const bz_embed_slot* s = &slots[blockIdx.x];
+  const int64_t first = blockIdx.y, count = blockIdx.y + 1 == gridDim.y ? -1 : 1;
   if (ext_off != nullptr) {
     const int64_t n = s->batch < ext_stride - 1 ? s->batch : ext_stride - 1;
-    scan_segments(s->segments, ext_off + (int64_t)blockIdx.x * ext_stride, n, s->nnz);
+    scan_segments(s->segments, ext_off + (int64_t)blockIdx.x * ext_stride, n, s->nnz, first, count);
   } else {
-    scan_segments(s->segments, s->offsets, s->batch, s->nnz);
+    scan_segments(s->segments, s->offsets, s->batch, s->nnz, first, count);
   }
+}
+
+// parts a slot's scan is split into: one per tile of the largest batch, at most 8 (a part re-reads the counts before it)
+inline int scan_parts(int64_t max_batch) {
+  const int64_t tiles = (max_batch + kScanTile - 1) / kScanTile;
+  return (int)(tiles < 1 ? 1 : (tiles > 8 ? 8 : tiles));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -759,7 +810,8 @@ int bz_segments_to_offsets(const int32_t* segments, int64_t* offsets, int64_t n,
 
 int bz_segments_to_offsets_slots(const bz_embed_slot* slots_dev, int n_slots, bz_stream_t stream) {
   BZ_REQUIRE(slots_dev != nullptr && n_slots > 0, "bz_segments_to_offsets_slots: null argument or n_slots=%d", n_slots);
-  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(n_slots), dim3(kThreads), 0, bz::as_stream(stream), slots_dev,
+  // the batch sizes are in device memory: always 8 parts a slot; a part beyond its slot's batch returns at once
+  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(n_slots, 8), dim3(kThreads), 0, bz::as_stream(stream), slots_dev,
                      (int64_t*)nullptr, (int64_t)0);
   BZ_LAUNCH_OK("bz_scan_segments_slots_kernel");
   return BZ_OK;
@@ -827,7 +879,8 @@ int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_
   if (rc != BZ_OK) return rc;
   hipStream_t st = bz::as_stream(stream);
   // nothing to clear: the scan writes entries [0, batch] of every slot's share, the only ones the pooling kernel reads
-  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(L.n_slots), dim3(kThreads), 0, st, slots_dev, off, stride);
+  hipLaunchKernelGGL(bz_scan_segments_slots_kernel, dim3(L.n_slots, scan_parts(L.max_batch)), dim3(kThreads), 0, st, slots_dev, off,
+                     stride);
   BZ_LAUNCH_OK("bz_scan_segments_slots_kernel");
   return launch_pool(slots_dev, L, off, stride, st);
 }
