@@ -11,9 +11,11 @@
  * device_type for Blaze_PredictorCreate: 1 = the accelerator (MI355X), the value existing callers pass for
  * the GPU; -1 = probe; 0 (CPU) fails at operator creation: this build has no CPU execution path.
  *
- * Not provided by this build (they return -1 with a message): the model importers and the offline optimizer
- * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze, Blaze_OptimizeBlaze).  The text-to-QED table
- * builders of c_api_qed.h (Blaze_QuickEmbeddingBuildFp32/Fp16) are provided.
+ * Not provided by this build (they return -1 with a message): the model importers
+ * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze).  Blaze_OptimizeBlaze runs the one optimizer pass this
+ * path depends on, the parallel-Gemm fusion (blaze/graph/pattern/in_parallel/parallel_gemm_fusion_pattern_impl.cc), and
+ * writes the model back; the reference's other passes are not part of this build.  The text-to-QED table builders of
+ * c_api_qed.h (Blaze_QuickEmbeddingBuildFp32/Fp16) are provided.
  */
 #ifndef BLAZE_C_API_H_
 #define BLAZE_C_API_H_
@@ -83,6 +85,7 @@ BLAZE_API int Blaze_PredictorDumpObservers(PredictorHandle handle, size_t* ndim,
 BLAZE_API int Blaze_ConvertBlaze(const char* model_conf_file, const char* model_data_file, int model_type, int weight_type,
                                  int io_type, int x_type_num, const char** x_type_key, const int* x_type_value,
                                  const char* blaze_model_file, int binary);
+/* c_api_blaze_optimizer.h:12-14: model file (binary or text NetDef) -> optimized model file (binary != 0: wire format) */
 BLAZE_API int Blaze_OptimizeBlaze(const char* raw_model_file, const char* optimized_model_file, int binary);
 /* c_api_qed.h:13-21: text tables (meta file + per-table files under `path`) -> one QED file, fp32 or fp16 rows */
 BLAZE_API int Blaze_QuickEmbeddingBuildFp32(const char* path, const char* meta, const char* output_file, int thread_num);

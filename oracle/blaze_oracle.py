@@ -474,6 +474,30 @@ def where(cond, x, y):
     return np.ascontiguousarray(np.where(np.broadcast_to(cond, shape) != 0, np.broadcast_to(x, shape), np.broadcast_to(y, shape)))
 
 
+def split(x, n_out, axis=1, splits=None):
+    """Split op (operator/op/split_op.h:33-132, split_op.cc:11-31): `n_out` parts along `axis`, equal unless `splits`
+    gives their sizes; RunSplit's walk: for every outer index, the parts' runs of split_size * inner elements follow
+    each other in x."""
+    x = np.asarray(x)
+    assert axis < x.ndim
+    if splits is None:
+        assert x.shape[axis] % n_out == 0
+        splits = [x.shape[axis] // n_out] * n_out
+    assert len(splits) == n_out and sum(splits) == x.shape[axis]
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    flat = x.reshape(-1)
+    ys = [np.empty(outer * s * inner, x.dtype) for s in splits]
+    at, y_off = 0, [0] * n_out
+    for _ in range(outer):
+        for k, s in enumerate(splits):
+            run = s * inner
+            ys[k][y_off[k]:y_off[k] + run] = flat[at:at + run]
+            at += run
+            y_off[k] += run
+    return [y.reshape(x.shape[:axis] + (s, ) + x.shape[axis + 1:]) for y, s in zip(ys, splits)]
+
+
 def reduce_sum(x, axis=0, keepdims=1):
     """ReduceSum op (operator/op/reduce_sum_op.h:17-58)."""
     x = _f32(x)

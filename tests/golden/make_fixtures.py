@@ -17,7 +17,9 @@ not exist.  Output: tests/golden/reference_kats.json.
 It also copies two sets of DATA files the reference holds, byte for byte:
   blaze/example/tdm_data/model_blaze_optimized (a binary NetDef, 217 ops)          -> model_blaze_optimized.bin
   blaze/blaze/test/utest_data/store/quick_embedding/{meta,a_01,a_02,a_03}          -> quick_embedding/
-(the text tables of embedding_builder_test.cc:13-23).
+(the text tables of embedding_builder_test.cc:13-23), and the input / expected NetDef pair of the optimizer's
+parallel-Gemm fusion test (blaze/blaze/test/graph/pattern/in_parallel/in_parallel_gemm_test.cc):
+  blaze/blaze/test/utest_data/graph/pattern/in_parallel/parallel_gemm_fusion{,_expected}.blaze               -> pattern/
 """
 import json
 import os
@@ -60,6 +62,8 @@ CASES = [
     "op/elementwise/elementwise_broadcast_to_net_v1_cpu.conf",
     "op/elementwise/elementwise_broadcast_to_net_v2_cpu.conf",
     "op/elementwise/elementwise_where_net_v1_cpu.conf",
+    "op/split/split_net_v1_cpu.conf",
+    "op/split/split_net_v2_cpu.conf",
 ]
 
 _TOK = re.compile(r'\s*(?:(#[^\n]*)|("(?:\\.|[^"\\])*")|([{}:])|([^\s{}:"#]+))')
@@ -172,7 +176,11 @@ def main():
     for name in ("meta", "a_01", "a_02", "a_03"):
         shutil.copyfile(os.path.join(root, "blaze/blaze/test/utest_data/store/quick_embedding", name),
                         os.path.join(here, "quick_embedding", name))
-    print("copied model_blaze_optimized.bin and quick_embedding/")
+    os.makedirs(os.path.join(here, "pattern"), exist_ok=True)
+    for name in ("parallel_gemm_fusion.blaze", "parallel_gemm_fusion_expected.blaze"):
+        shutil.copyfile(os.path.join(root, "blaze/blaze/test/utest_data/graph/pattern/in_parallel", name),
+                        os.path.join(here, "pattern", name))
+    print("copied model_blaze_optimized.bin, quick_embedding/ and pattern/")
 
 
 if __name__ == "__main__":

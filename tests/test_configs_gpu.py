@@ -216,6 +216,16 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     din_model.feed(p, inputs, batch, np.float16)
     p.forward()
     got = {name: p.output_asnumpy(name).astype(np.float32) for name in expose + ("prob", )}
+    # ten kernel launches a forward: 2 Embedding, 3 Concat (history, attention input with its pieces, main input),
+    # 4 Gemm (each with its Dice / next skinny layer / softmax folded in), 1 MatMul (with the Mul and the ReduceSum)
+    import json
+    p.register_observers(["profile"])
+    p.forward()
+    ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+    launching = [e for e in ev if e["name"].split(":")[0] not in ("ConstantFill", "Reshape")]
+    kinds = sorted(e["name"].split(":")[0] for e in launching)
+    assert kinds == ["Concat"] * 3 + ["Embedding"] * 2 + ["Gemm"] * 4 + ["MatMul"], kinds
+    assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
     for k, t in zip(din_model.KINDS, tables):
         ids = np.concatenate([batch[k + ".ids"], batch[k + "_his.ids"]])

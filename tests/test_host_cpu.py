@@ -366,6 +366,37 @@ def test_reference_binary_model_decodes_like_protobuf():
     assert "ConstantFill" in types and "Gemm" in types
 
 
+def test_parallel_gemm_fusion_pass_on_the_reference_fixture(tmp_path):
+    """Blaze_OptimizeBlaze on the input of the reference's parallel-Gemm fusion test gives the NetDef that test
+    expects (blaze/blaze/test/graph/pattern/in_parallel/in_parallel_gemm_test.cc; compared as
+    pattern_test_common.h:17-90 compares: operator types, names, inputs, outputs and arguments in order): two Gemms on one
+    input become FusedParallelGemm over the stacked weight + Split(axis 0), and the orphaned constant is gone."""
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    from google.protobuf import text_format
+    src = os.path.join(ROOT, "tests", "golden", "pattern", "parallel_gemm_fusion.blaze")
+    want = NetDef()
+    text_format.Parse(open(os.path.join(ROOT, "tests", "golden", "pattern", "parallel_gemm_fusion_expected.blaze")).read(), want)
+    for binary in (False, True):
+        dst = str(tmp_path / ("opt.%d" % binary))
+        pb.optimize_blaze(src, dst, binary)
+        got = NetDef()
+        if binary:
+            got.ParseFromString(open(dst, "rb").read())
+        else:
+            text_format.Parse(open(dst).read(), got)
+        assert [o.type for o in got.op] == [o.type for o in want.op] == ["ConstantFill", "ConstantFill", "FusedParallelGemm", "Split", "Concat"]
+        for a, b in zip(got.op, want.op):
+            assert (a.type, a.name, list(a.input), list(a.output)) == (b.type, b.name, list(b.input), list(b.output))
+            assert [_arg_value(x) for x in a.arg] == [_arg_value(x) for x in b.arg]
+        assert [(v.name, v.dtype) for v in got.external_output] == [(v.name, v.dtype) for v in want.external_output]
+        assert got.run_mode == want.run_mode
+    # a net without sibling Gemms passes through unchanged; a second run of the pass finds nothing more to fuse
+    again = str(tmp_path / "again")
+    pb.optimize_blaze(str(tmp_path / "opt.1"), again, True)
+    assert open(again, "rb").read() == open(str(tmp_path / "opt.1"), "rb").read()
+
+
 def _reference_text_tables():
     """-> {table: (keys int64 [n], rows fp32 [n, dim])} of tests/golden/quick_embedding (the reference's
     utest_data/store/quick_embedding: `key,w0,...` lines; the first weight column happens to hold a big integer)."""

@@ -90,6 +90,26 @@ def test_reference_dense_kat(oracle, kats, name):
     np.testing.assert_allclose(got, want, rtol=0, atol=ATOL_KAT)
 
 
+@pytest.mark.parametrize("name", ["split_net_v1_cpu", "split_net_v2_cpu"])
+def test_reference_split_kat(oracle, kats, name):
+    case = kats[name]
+    op = case["ops"][0]
+    got = oracle.split(_tensor(case["tensors"][op["inputs"][0]]), len(op["outputs"]), op["args"].get("axis", 1),
+                       op["args"].get("split"))
+    for y, out in zip(got, op["outputs"]):
+        exp = case["expected"][out]
+        assert list(y.shape) == exp["shape"]
+        np.testing.assert_allclose(y, np.array(exp["values"], np.float32).reshape(exp["shape"]), rtol=0, atol=ATOL_KAT)
+    # numpy's own split is the closed form
+    x = np.arange(2 * 6 * 3, dtype=np.float32).reshape(2, 6, 3)
+    for a, b in zip(oracle.split(x, 3, 1), np.split(x, 3, axis=1)):
+        assert np.array_equal(a, b)
+    for a, b in zip(oracle.split(x, 2, 0), np.split(x, 2, axis=0)):
+        assert np.array_equal(a, b)
+    for a, b in zip(oracle.split(x, 2, 2, [1, 2]), np.split(x, [1], axis=2)):
+        assert np.array_equal(a, b)
+
+
 # ---------------------------------------------------------------- embedding op, reference fixture embedding_v1.conf
 EMB_FG = {"101": ("a_01", 4), "102": ("a_02", 8), "104_7": ("a_03", 6)}
 EMB_BLOCKS = [[{"fg": "101", "udf": 0}, {"fg": "102", "udf": 0}],

@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 @pytest.fixture(scope="module")
@@ -54,7 +55,7 @@ DENSE = ["gemm_net_v1_cpu", "prelu_net_v1_cpu", "dice_net_v1_cpu", "leaky_relu_n
          "reshape_net_v1_cpu", "batch_normalization_net_v1_cpu", "elementwise_add_net_v1_cpu", "elementwise_add_net_v2_cpu",
          "elementwise_sub_net_v1_cpu", "elementwise_sub_net_v2_cpu", "elementwise_mul_net_v1_cpu", "elementwise_mul_net_v2_cpu",
          "elementwise_div_net_v1_cpu", "elementwise_div_net_v2_cpu", "elementwise_broadcast_to_net_v1_cpu",
-         "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu"]
+         "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu", "split_net_v1_cpu", "split_net_v2_cpu"]
 
 
 @pytest.mark.parametrize("name", DENSE)
@@ -567,6 +568,67 @@ def test_threads_feeding_alternating_requests_get_their_own_results(pb):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_optimized_model_file_gives_the_same_outputs(pb, oracle, tmp_path):
+    """NetDef -> NetDef: Blaze_OptimizeBlaze rewrites three sibling Gemms (constant weights and biases of one shape)
+    into FusedParallelGemm + Split; the optimized model file, loaded through Blaze_PredcitorManagerLoadModel, gives the
+    outputs of the original one and of the oracle, with one FC launch and a Split that copies nothing.  Also the
+    reference's own fixture (tests/golden/pattern/parallel_gemm_fusion.blaze, moved to the device)."""
+    import json
+    rng = np.random.default_rng(11)
+    M, K, N, P = 37, 24, 16, 3
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    ws = [(rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32) for _ in range(P)]
+    bs = [(rng.standard_normal(N) * 0.1).astype(np.float32) for _ in range(P)]
+    nb = pb.NetBuilder("siblings", device_type=1)
+    nb.external_input("x", pb.K_FLOAT)
+    nb.arg("pack_sibling_gemms", 0)  # keep the in-net packing out of it: this test is about the offline pass
+    for p in range(P):
+        nb.constant("w%d" % p, ws[p])
+        nb.constant("b%d" % p, bs[p])
+    for p in range(P):
+        nb.op("Gemm", ["x", "w%d" % p, "b%d" % p], ["y%d" % p])
+    nb.op("Concat", ["y%d" % p for p in range(P)], ["out"], axis=1)
+    nb.external_output("out", pb.K_FLOAT)
+    raw, opt = str(tmp_path / "raw.blaze"), str(tmp_path / "opt.blaze")
+    open(raw, "wb").write(pb.convert_netdef(nb.text().encode(), True, False))
+    pb.optimize_blaze(raw, opt, True)
+    outs = {}
+    for path in (raw, opt):
+        pm = pb.PredictorManager()
+        pm.load_model(path)
+        p = pm.create_predictor(1, 0)
+        p.reshape_input("x", [M, K])
+        p.feed("x", x)
+        p.register_observers(["profile"])
+        p.forward()
+        outs[path] = p.output_asnumpy("out").copy()
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        kinds = [e["name"].split(":")[0] for e in ev if not e["name"].startswith("ConstantFill")]
+        if path == opt:
+            assert kinds == ["FusedParallelGemm", "Split", "Concat"], kinds
+            assert [e["args"]["launches"] for e in ev if e["name"].split(":")[0] in ("FusedParallelGemm", "Split")] == [1, 0]
+        else:
+            assert kinds == ["Gemm"] * P + ["Concat"], kinds
+    want = np.concatenate([oracle.gemm_op(x, ws[p], bs[p], False, False, 1.0, 1.0) for p in range(P)], axis=1)
+    np.testing.assert_allclose(outs[raw], want, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(outs[opt], want, rtol=1e-5, atol=1e-6)
+    # the reference's fixture: constants only, placed on the device
+    text = open(os.path.join(ROOT, "tests", "golden", "pattern", "parallel_gemm_fusion.blaze")).read().replace("device_type: 0", "device_type: 1")
+    raw2, opt2 = str(tmp_path / "raw2.blaze"), str(tmp_path / "opt2.blaze")
+    open(raw2, "w").write(text)
+    pb.optimize_blaze(raw2, opt2, False)
+    got = []
+    for path in (raw2, opt2):
+        pm = pb.PredictorManager()
+        pm.load_model(path)
+        p = pm.create_predictor(1, 0)
+        p.forward()
+        got.append(p.output_asnumpy("output").copy())
+    a = np.arange(6, dtype=np.float32).reshape(2, 3)
+    w = np.arange(6, dtype=np.float32).reshape(3, 2)
+    assert np.array_equal(got[0], np.concatenate([a @ w, a @ w], axis=1)) and np.array_equal(got[0], got[1])
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])

@@ -13,6 +13,7 @@
 #include <mutex>
 #include <thread>
 
+#include "blaze/optimizer.h"
 #include "blaze/predictor.h"
 #include "blaze/qed_builder.h"
 #include "blaze/qed_store.h"
@@ -468,9 +469,35 @@ int Blaze_ConvertBlaze(const char*, const char*, int, int, int, int, const char*
   Blaze_SetLastErrorString("Blaze_ConvertBlaze: the model importers are not part of this build");
   return -1;
 }
-int Blaze_OptimizeBlaze(const char*, const char*, int) {
-  Blaze_SetLastErrorString("Blaze_OptimizeBlaze: the offline optimizer is not part of this build");
-  return -1;
+// c_api_blaze_optimizer.cc: load the model, run the optimizer, store the result (binary != 0: wire format, else text).
+// Of the reference's passes this build has the parallel-Gemm fusion (blaze/optimizer.h).
+int Blaze_OptimizeBlaze(const char* raw_model_file, const char* optimized_model_file, int binary) {
+  if (raw_model_file == nullptr || optimized_model_file == nullptr) return Fail("OptimizeBlaze: null argument");
+  try {
+    blaze::NetDef def;
+    std::string err;
+    if (!blaze::LoadNetDefFromFile(raw_model_file, &def, &err)) {
+      Blaze_SetLastErrorString("OptimizeBlaze: %s", err.c_str());
+      return -1;
+    }
+    blaze::FuseParallelGemms(&def);
+    std::string s;
+    if (binary)
+      blaze::SerializeNetDefBinary(def, &s);
+    else
+      blaze::SerializeNetDefText(def, &s);
+    FILE* f = fopen(optimized_model_file, "wb");
+    if (f == nullptr || fwrite(s.data(), 1, s.size(), f) != s.size()) {
+      if (f) fclose(f);
+      Blaze_SetLastErrorString("OptimizeBlaze: cannot write %s", optimized_model_file);
+      return -1;
+    }
+    fclose(f);
+  } catch (std::exception& e) {
+    Blaze_SetLastErrorString("OptimizeBlaze: %s", e.what());
+    return -1;
+  }
+  return 0;
 }
 int Blaze_QuickEmbeddingBuildFp32(const char* path, const char* meta, const char* output_file, int thread_num) {
   std::string err;

@@ -14,6 +14,7 @@
 #include "blaze_hip.h"
 
 #include <algorithm>
+#include <climits>
 
 namespace blaze {
 
@@ -319,6 +320,85 @@ class ReduceSumOp final : public Operator<Context> {
 };
 REGISTER_HIP_OPERATOR(ReduceSum, ReduceSumOp<HIPContext>);
 OPERATOR_SCHEMA(ReduceSum).NumInputs(1).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("sum over one axis");
+
+// ------------------------------------------------------------------------------------------ Split
+// blaze/operator/op/split_op.h:33-132, split_op.cc:11-44.  Equal parts along axis 0 are views of the input (the
+// reference's RefReshape: the optimizer's FusedParallelGemm + Split pair costs no copy); any other split copies each
+// part out with one strided copy.
+template <class Context>
+class SplitOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  SplitOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    axis_ = OperatorBase::GetSingleArgument<size_t>("axis", 1);
+    if (OperatorBase::HasArgument("split")) {
+      splits_ = OperatorBase::GetRepeatedArgument<size_t>("split");
+      BLAZE_CONDITION_THROW(splits_.size() == (size_t)this->OutputSize(), "splits_.size()=", splits_.size(),
+                            " this->output_size()=", this->OutputSize());
+    }
+  }
+  int LaunchesOfLastRun() const override { return launches_; }
+  bool RunOnDevice() override {
+    Blob* x = this->Input(0);
+    const int n_out = this->OutputSize();
+    const std::vector<TIndex> shape0 = x->shape();
+    launches_ = 0;
+    BLAZE_CONDITION_THROW(x->pitch() == 0, "Split of a strided view of another tensor");
+    if (splits_.empty() && axis_ == 0) {
+      BLAZE_CONDITION_THROW(!shape0.empty() && shape0[0] % n_out == 0, "shape[0]=", shape0.empty() ? 0 : shape0[0]);
+      std::vector<TIndex> shape = shape0;
+      shape[0] /= n_out;
+      const size_t part = (size_t)(x->size() / n_out) * DataTypeSize(x->data_type());
+      for (int i = 0; i < n_out; ++i) {
+        Blob* y = this->Output(i);
+        y->set_data_type((DataType)x->data_type());
+        y->RefReshape(shape, (char*)x->data() + part * i);
+      }
+      return true;
+    }
+    BLAZE_CONDITION_THROW(axis_ < shape0.size(), "axis_=", axis_, " shape0.size()=", shape0.size());
+    if (splits_.empty()) {
+      BLAZE_CONDITION_THROW(shape0[axis_] % n_out == 0, "shape0[", axis_, "]=", shape0[axis_], " output_size=", n_out,
+                            " op=", this->def_.name());
+    } else {
+      size_t sum_axis = 0;
+      for (auto sp : splits_) sum_axis += sp;
+      BLAZE_CONDITION_THROW(sum_axis == (size_t)shape0[axis_], "sum_axis=", sum_axis, " shape0[", axis_, "]=", shape0[axis_]);
+    }
+    const size_t es = DataTypeSize(x->data_type());
+    const TIndex outer = x->size(0, (int)axis_), inner = x->size((int)axis_ + 1, (int)shape0.size());
+    size_t offset = 0;
+    std::vector<TIndex> shape = shape0;
+    for (int k = 0; k < n_out; ++k) {
+      shape[axis_] = splits_.empty() ? shape0[axis_] / n_out : (TIndex)splits_[k];
+      Blob* y = this->Output(k);
+      y->set_data_type((DataType)x->data_type());
+      y->Reshape(shape);
+      if (y->size() > 0) {
+        bz_concat_desc d;
+        memset(&d, 0, sizeof(d));
+        d.n = 1;
+        d.src[0] = (const char*)x->data() + offset * inner * es;
+        d.width[0] = (int64_t)(shape[axis_] * inner * es);
+        d.src_pitch[0] = (int64_t)(shape0[axis_] * inner * es);
+        d.dst = y->data();
+        d.dst_pitch = d.width[0];
+        d.rows = (int64_t)outer;
+        BZ_CHECK(bz_concat_cols(&d, context_.hip_stream()));
+        ++launches_;
+      }
+      offset += shape[axis_];
+    }
+    return true;
+  }
+
+ private:
+  size_t axis_;
+  std::vector<size_t> splits_;
+  int launches_ = 0;
+};
+REGISTER_HIP_OPERATOR(Split, SplitOp<HIPContext>);
+OPERATOR_SCHEMA(Split).NumInputs(1).NumOutputs(1, INT_MAX).IdenticalTypeOfInput(0).SetDoc("Split a tensor into many tensors.");
 
 // ------------------------------------------------------------------------------------------ Fuse
 template <class Context>

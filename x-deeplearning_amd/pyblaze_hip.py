@@ -78,6 +78,7 @@ def lib():
         l.Blaze_QuickEmbeddingBuildFp16.argtypes = [cp, cp, cp, i]
         l.Blaze_HipStoreAddTable.argtypes = [vp, cp, i, C.c_int64, i, vp, i, vp, vp]
         l.Blaze_ConvertNetDef.argtypes = [cp, sz, i, i, vp, sz, C.POINTER(sz)]
+        l.Blaze_OptimizeBlaze.argtypes = [cp, cp, i]
         l.Blaze_PredictorInputDevicePtr.argtypes = [vp, cp, C.POINTER(vp)]
         l.Blaze_PredictorOutputDevicePtr.argtypes = [vp, cp, C.POINTER(vp)]
         l.Blaze_ServePoolCreate.argtypes = [i, C.POINTER(vp)]
@@ -312,6 +313,11 @@ class PredictorManager(object):
         p = Predictor(h)
         p._manager = self  # the manager owns the workspace (weights and blobs) the predictor points into
         return p
+
+
+def optimize_blaze(raw_model_file, optimized_model_file, binary=True):
+    """Blaze_OptimizeBlaze: model file (binary or text NetDef) -> optimized model file."""
+    check_call(lib().Blaze_OptimizeBlaze(raw_model_file.encode(), optimized_model_file.encode(), int(binary)))
 
 
 def convert_netdef(data, in_is_text, out_is_text):
