@@ -215,6 +215,7 @@ enum bz_act {
  * Gemm with a shared weight (gemm_op.h:52-58,77-91) is the same call with
  * M = batch*M.
  */
+struct bz_concat_ew_desc;
 typedef struct bz_fc_desc {
   const void* a;       /* device [M, lda] */
   const void* w;       /* device [N, ldw] packed */
@@ -256,6 +257,14 @@ typedef struct bz_fc_desc {
    */
   int32_t n_split;
   int64_t y_split_stride;
+  /* A given as pieces computed on the fly instead of as a stored matrix: when non-NULL, `a` and `lda` are ignored and
+   * row r of A is the concatenation bz_concat_ew would write for that row (m = r0 * r1 rows, k = the sum of the widths;
+   * dst / dst_pitch of the descriptor are not used).  The layer then reads the pieces' operands and the tensor is never
+   * stored: DIN's attention input [q, k, q-k, q*k] (tools/example_model/din/model/graph_ulf.txt) costs its 22 MB of
+   * traffic each way otherwise.  Same values as the two-step form: every element of A is rounded to the tensor type
+   * exactly as the concat would store it.  Limits: 2-byte types, pieces of one width that do not divide,
+   * k <= 224, n <= 96, no head, no split outputs, per-column bias only; BZ_ENOTSUP (nothing launched) otherwise. */
+  const struct bz_concat_ew_desc* a_pieces;
 } bz_fc_desc;
 
 BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);

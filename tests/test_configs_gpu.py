@@ -216,15 +216,16 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     din_model.feed(p, inputs, batch, np.float16)
     p.forward()
     got = {name: p.output_asnumpy(name).astype(np.float32) for name in expose + ("prob", )}
-    # ten kernel launches a forward: 2 Embedding, 3 Concat (history, attention input with its pieces, main input),
-    # 4 Gemm (each with its Dice / next skinny layer / softmax folded in), 1 MatMul (with the Mul and the ReduceSum)
+    # nine kernel launches a forward: 2 Embedding, 2 Concat (history, main input), 4 Gemm (each with its Dice / next
+    # skinny layer / softmax folded in; the first also computes the attention input [q, k, q-k, q*k] it reads), 1 MatMul
+    # (with the Mul and the ReduceSum)
     import json
     p.register_observers(["profile"])
     p.forward()
     ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
     launching = [e for e in ev if e["name"].split(":")[0] not in ("ConstantFill", "Reshape")]
     kinds = sorted(e["name"].split(":")[0] for e in launching)
-    assert kinds == ["Concat"] * 3 + ["Embedding"] * 2 + ["Gemm"] * 4 + ["MatMul"], kinds
+    assert kinds == ["Concat"] * 2 + ["Embedding"] * 2 + ["Gemm"] * 4 + ["MatMul"], kinds
     assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
     for k, t in zip(din_model.KINDS, tables):
@@ -330,3 +331,38 @@ def test_attention_tail_in_one_launch_equals_the_separate_operators():
         for x1, x0 in zip(one, sep):
             assert np.array_equal(x1.view(np.uint16 if x1.dtype == np.float16 else np.uint32),
                                   x0.view(np.uint16 if x0.dtype == np.float16 else np.uint32))
+
+
+def test_attention_input_computed_by_its_first_layer_equals_the_separate_operators():
+    """Concat([q, k, q-k, q*k]) -> Gemm + Dice: by default the Gemm computes the Concat's rows while it loads them
+    (bz_fc_desc.a_pieces) and the Concat never runs; with fuse_concat_into_fc: 0 the tensor is stored and read back.  The
+    first attention layer's output agrees to a rounding of the tensor type (another order of the K sum), the
+    probabilities to 2e-3, also after the batch shrinks and grows again."""
+    import json
+    import torch
+    import din_model
+    cfg = din_model.Config3(batch=96, rows=5000, T=20)
+    small = din_model.Config3(batch=17, rows=5000, T=20)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=5), cfg.batch_inputs(seed_offset=9)]
+    outs = {}
+    for fuse in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("att0_y", ),
+                                             net_args={"fuse_concat_into_fc": fuse})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append((p.output_asnumpy("att0_y").astype(np.float32), p.output_asnumpy("prob").copy()))
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        ran = [e["name"] for e in ev]
+        assert ("Concat:concat_att_in" in ran) == (fuse == 0), ran
+        assert [e["args"]["launches"] for e in ev if e["name"] == "Gemm:gemm_att0_g"] == [1]
+        outs[fuse] = got
+    torch.cuda.synchronize()
+    for (y1, p1), (y0, p0), b in zip(outs[1], outs[0], (96, 17, 96)):
+        assert y1.shape == (b, cfg.T, 80) and y1.any()
+        np.testing.assert_allclose(y1, y0, rtol=2e-3, atol=2e-3 * np.abs(y0).max())
+        np.testing.assert_allclose(p1, p0, rtol=2e-3, atol=2e-3)

@@ -508,3 +508,103 @@ def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T,
     tol = 1e-5 if dtype_name == "f32" else 2e-3
     np.testing.assert_allclose(att.float().cpu().numpy(), want_att, rtol=tol, atol=tol * max(1.0, np.abs(want_att).max()))
     np.testing.assert_allclose(tot.float().cpu().numpy(), want_sum, rtol=tol, atol=tol * max(1.0, np.abs(want_sum).max()))
+
+
+def _pieces_desc(bz, pieces, r0, r1, tdt):
+    """bz_concat_ew_desc of (op, x, y) pieces with operands [r0 | 1, r1 | 1, w] (as blaze_hip.concat_ew builds it), without dst"""
+    d = bz.ConcatEwDesc()
+    d.n, d.dtype, d.r0, d.r1 = len(pieces), bz.bz_dtype(tdt), r0, r1
+    for i, (op, x, y) in enumerate(pieces):
+        d.op[i], d.width[i], d.x[i] = op, x.shape[2], x.data_ptr()
+        for name, t in (("x_stride", x), ("y_stride", y)):
+            if t is None:
+                continue
+            getattr(d, name)[i][0] = 0 if t.shape[0] == 1 and r0 > 1 else t.shape[1] * t.shape[2]
+            getattr(d, name)[i][1] = 0 if t.shape[1] == 1 and r1 > 1 else t.shape[2]
+        if y is not None:
+            d.y[i] = y.data_ptr()
+    return d
+
+
+@pytest.mark.parametrize("in_name,out_name", [("f16", "f16"), ("bf16", "bf16"), ("f16", "f32")])
+@pytest.mark.parametrize("r0,r1,w,N,act", [(1024, 50, 54, 80, "dice"),   # DIN's attention input in front of its first layer
+                                           (37, 5, 8, 96, "prelu"),     # 8 columns a lane, ragged last tile, three column blocks
+                                           (300, 1, 40, 24, "none"),    # one column block, K = 160
+                                           (64, 3, 56, 40, "relu")])    # K = 224, the most the kernel holds
+def test_fc_on_pieces_computed_on_the_fly(bz, oracle, in_name, out_name, r0, r1, w, N, act):
+    """bz_fc_fused with a_pieces = [q, k, q-k, q*k] (q broadcast over the second row coordinate) against bz_concat_ew
+    followed by the stored-matrix layer, and against the oracle fed the concat's rounded values."""
+    import ctypes as C
+    import torch
+    print("fc on pieces %s->%s r0=%d r1=%d w=%d N=%d act=%s" % (in_name, out_name, r0, r1, w, N, act), flush=True)
+    tdt, odt = _tdtype(in_name), _tdtype(out_name)
+    rng = np.random.default_rng(r0 + r1 + w + N)
+    M, K = r0 * r1, 4 * w
+    q = _dev(_round_to(rng.standard_normal((r0, 1, w)), in_name)).to(tdt)
+    k = _dev(_round_to(rng.standard_normal((r0, r1, w)), in_name)).to(tdt)
+    Wkn = _round_to(rng.standard_normal((K, N)) / np.sqrt(K), in_name)
+    b = (rng.standard_normal(N) * 0.1).astype(np.float32)
+    params_np = ()
+    if act == "prelu":
+        params_np = (rng.uniform(0.1, 0.4, N).astype(np.float32), )
+    elif act == "dice":
+        params_np = ((rng.standard_normal(N) * 0.1).astype(np.float32), (rng.standard_normal(N) * 0.1).astype(np.float32),
+                     rng.uniform(0.5, 1.5, N).astype(np.float32))
+    params = tuple(_dev(x) for x in params_np)
+    wp = bz.pack_weight(_dev(Wkn).to(tdt), False, bz.bz_dtype(tdt))
+    pieces = [(bz.EW_ASSIGN, q, None), (bz.EW_ASSIGN, k, None), (bz.EW_SUB, q, k), (bz.EW_MUL, q, k)]
+    # two launches
+    a_full = bz.concat_ew(pieces).reshape(M, K)
+    two = bz.fc_fused(a_full, wp, K, bias=_dev(b), act=ACT[act], act_params=params, out_dtype=bz.bz_dtype(odt), act_alpha=0.0)
+    # one launch
+    pd = _pieces_desc(bz, pieces, r0, r1, tdt)
+    one = torch.full((M, N), float("nan"), dtype=odt, device="cuda")
+    d = bz.FcDesc()
+    d.a_pieces = C.cast(C.pointer(pd), C.c_void_p)
+    d.w, d.y, d.bias = wp.data_ptr(), one.data_ptr(), _dev(b).data_ptr()
+    bias_dev = _dev(b)
+    d.bias = bias_dev.data_ptr()
+    d.ldw, d.ldy = wp.stride(0), N
+    d.m, d.n, d.k = M, N, K
+    d.in_dtype, d.out_dtype = bz.bz_dtype(tdt), bz.bz_dtype(odt)
+    d.bias_rows, d.alpha, d.beta = 1, 1.0, 1.0
+    d.act, d.act_alpha = ACT[act], 0.0
+    for name, p_ in zip(("act_p0", "act_p1", "act_p2"), params):
+        setattr(d, name, p_.data_ptr())
+    d.act_size = N if act in ("prelu", "dice") else 0
+    bz.check(bz.lib().bz_fc_fused(C.byref(d), None))
+    torch.cuda.synchronize()
+    got, ref = one.float().cpu().numpy(), two.float().cpu().numpy()
+    assert not np.isnan(got).any()
+    # oracle on the concat's values (each an fp32 operation rounded once to the tensor type)
+    A = a_full.float().cpu().numpy()
+    pre = (A.astype(np.float64) @ Wkn.astype(np.float64) + b).astype(np.float32)
+    scale = np.abs(A).astype(np.float64) @ np.abs(Wkn).astype(np.float64) + np.abs(b)
+    want = {"none": lambda x: x, "relu": lambda x: oracle.leaky_relu(x, 0.0), "prelu": lambda x: oracle.prelu(x, params_np[0]),
+            "dice": lambda x: oracle.dice(x, *params_np)}[act](pre)
+    out_eps = {"f32": 0.0, "f16": 2.0**-11, "bf16": 2.0**-8}[out_name]
+    bound = 2.0 * 2e-3 * scale + out_eps * np.abs(want) + 1e-7
+    assert np.all(np.abs(got - want) <= bound)
+    assert np.all(np.abs(got - ref) <= bound)
+
+
+def test_fc_on_pieces_limits_are_refused(bz):
+    """outside the kernel's model bz_fc_fused answers BZ_ENOTSUP and launches nothing (the caller runs the concat instead)"""
+    import ctypes as C
+    import torch
+    q = torch.zeros((4, 1, 64), dtype=torch.float16, device="cuda")
+    k = torch.zeros((4, 3, 64), dtype=torch.float16, device="cuda")
+    wp = torch.zeros((16, 256), dtype=torch.float16, device="cuda")
+    y = torch.zeros((12, 16), dtype=torch.float16, device="cuda")
+    pieces = [(bz.EW_ASSIGN, q, None), (bz.EW_ASSIGN, k, None), (bz.EW_SUB, q, k), (bz.EW_MUL, q, k)]
+    pd = _pieces_desc(bz, pieces, 4, 3, torch.float16)
+    d = bz.FcDesc()
+    d.a_pieces = C.cast(C.pointer(pd), C.c_void_p)
+    d.w, d.y, d.ldw, d.ldy, d.m, d.n, d.k = wp.data_ptr(), y.data_ptr(), 256, 16, 12, 16, 256
+    d.in_dtype = d.out_dtype = bz.F16
+    d.alpha = 1.0
+    assert bz.lib().bz_fc_fused(C.byref(d), None) == bz.ENOTSUP and b"a_pieces" in bz.lib().bz_last_error()  # k = 256 > 224
+    pd.op[3] = bz.EW_DIV
+    pd.width[0] = pd.width[1] = pd.width[2] = pd.width[3] = 40
+    d.k, d.ldw = 160, 160
+    assert bz.lib().bz_fc_fused(C.byref(d), None) == bz.ENOTSUP  # a piece that divides

@@ -25,6 +25,7 @@ EXPORTS = [
     "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
+OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5  # bz_status
 MAX_RANK = 6
 
 
@@ -50,7 +51,7 @@ class FcDesc(C.Structure):
                 ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
                 ("reserved_", C.c_int32), ("head_w", C.c_void_p), ("head_bias", C.c_void_p), ("head_y", C.c_void_p),
                 ("head_ldw", C.c_int64), ("head_ldy", C.c_int64), ("head_n", C.c_int32), ("head_act", C.c_int32),
-                ("head_out_dtype", C.c_int32), ("n_split", C.c_int32), ("y_split_stride", C.c_int64)]
+                ("head_out_dtype", C.c_int32), ("n_split", C.c_int32), ("y_split_stride", C.c_int64), ("a_pieces", C.c_void_p)]
 
 
 class BgemmDesc(C.Structure):

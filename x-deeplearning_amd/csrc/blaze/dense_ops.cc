@@ -67,6 +67,7 @@ const float* AsFloatParam(Blob* b, Derived* cache, bool constant, hipStream_t st
 struct FcCall {
   // operands
   const void* a = nullptr;
+  const bz_concat_ew_desc* a_pieces = nullptr;  // instead of a: the rows as pieces computed on the fly (bz_fc_desc.a_pieces)
   int a_rows = 0, a_cols = 0;  // as stored
   bool trans_a = false;
   Blob* b_blob = nullptr;
@@ -99,7 +100,8 @@ struct FcCall {
   int head_n = 0, head_act = BZ_ACT_NONE, head_y_dtype = kFloat;
 };
 
-void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st) {
+// false only with a_pieces, when the kernel does not take them (nothing has been launched then)
+bool RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st) {
   const int P = c.slices;
   const int M = c.trans_a ? c.a_cols : c.a_rows;
   const int K = c.trans_a ? c.a_rows : c.a_cols;
@@ -175,14 +177,23 @@ void RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
     d.head_act = c.head_act;
     d.head_out_dtype = BzType(c.head_y_dtype);
   }
+  if (c.a_pieces != nullptr) {
+    d.a_pieces = c.a_pieces;
+    d.a = nullptr;
+    const int rc = bz_fc_fused(&d, st);
+    if (rc == BZ_ENOTSUP) return false;
+    BZ_CHECK(rc);
+    return true;
+  }
   BZ_CHECK(bz_fc_fused(&d, st));
+  return true;
 }
 
 }  // namespace
 
 // ------------------------------------------------------------------------------------------ Gemm
 template <class Context>
-class GemmOp : public Operator<Context>, public FusableProducer, public StackableFc, public SiblingFc {
+class GemmOp : public Operator<Context>, public FusableProducer, public StackableFc, public SiblingFc, public ConcatAdopter {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
 
@@ -295,9 +306,41 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     for (SiblingFc* o : others) siblings_.push_back(static_cast<GemmOp*>(o));
   }
 
+  // ---- the Concat that makes this layer's input, computed while it is loaded
+  // (the static part of what bz_fc_desc.a_pieces takes: a 2-byte layer of 9..96 columns and at most 224 inputs)
+  bool CanAdoptConcat() override {
+    Blob* b = this->Input(1);
+    if (!b_constant_ || transa_ || b->shape().size() != 2) return false;
+    if (b->data_type() != kFloat16) return false;
+    const TIndex K = transb_ ? b->shape()[1] : b->shape()[0], N = transb_ ? b->shape()[0] : b->shape()[1];
+    if (this->InputSize() > 2 && (!c_constant_ || (TIndex)this->Input(2)->size() != N)) return false;
+    return N > 8 && N <= 96 && K <= 224 && !(fused_ && fused_act_ == BZ_ACT_SOFTMAX);
+  }
+  void AdoptConcat(OperatorBase* concat) override { concat_ = concat; }
+
   int LaunchesOfLastRun() const override { return launches_; }
 
   bool RunOnDevice() override {
+    launches_ = 1;
+    if (concat_ != nullptr) {
+      if (siblings_.empty() && head_ == nullptr && stack_.empty()) {
+        bz_concat_ew_desc pieces;
+        auto* c = dynamic_cast<ConcatForFc*>(concat_);
+        if (c != nullptr && c->DescribeAsPieces(&pieces) && RunSelf(false, &pieces)) return true;
+      }
+      // a shape the one-launch form does not take: the Concat runs after all
+      if (!concat_->Run(context_.stream_id())) return false;
+      launches_ = 2;
+      // (the paths below count their own launches from 1)
+    }
+    const int before = launches_ - 1;
+    const bool ok = RunRest();
+    launches_ += before;
+    return ok;
+  }
+
+ protected:
+  bool RunRest() {
     launches_ = 1;
     if (!siblings_.empty()) {
       if (RunSiblings()) return true;
@@ -324,7 +367,6 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     return RunSelf(false);
   }
 
- protected:
   // this layer's entry of the fused stack: packed weight, bias and epilogue parameters
   void FillStackLayer(bz_mlp_layer* L, bool head, hipStream_t st) {
     Blob* b = this->Input(1);
@@ -488,7 +530,8 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
 
   // with_head: also compute head_'s layer in this launch and leave this layer's own output unstored; false when the
   // operands do not allow it (nothing has been launched then)
-  bool RunSelf(bool with_head) {
+  // pieces: the input given as pieces computed on the fly (an adopted Concat); false when the kernel does not take them
+  bool RunSelf(bool with_head, const bz_concat_ew_desc* pieces = nullptr) {
     CheckValid();
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -534,7 +577,8 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     }
     hipStream_t st = context_.hip_stream();
     FcCall call;
-    call.a = a->data();
+    call.a = pieces ? nullptr : a->data();
+    call.a_pieces = pieces;
     call.a_rows = transa_ ? (int)K : (int)rows;
     call.a_cols = transa_ ? (int)rows : (int)K;
     call.trans_a = transa_;
@@ -593,11 +637,9 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
         call.act_size = (int)N;
       }
     }
-    RunFc(call, &packed_b_, &packed_a_, st);
-    return true;
+    return RunFc(call, &packed_b_, &packed_a_, st);
   }
 
- protected:
   void CheckValid() {
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -631,6 +673,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   Derived stack_pack_;           // this layer's weight in the fragment-major pack of bz_mlp_fused
   std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
   GemmOp* head_ = nullptr;       // the layer of at most 8 outputs computed in this operator's launch
+  OperatorBase* concat_ = nullptr;  // the Concat that makes Input(0), computed by this operator's kernel
   std::vector<GemmOp*> siblings_;  // layers on the same input computed in this operator's launch
   Derived sib_w_, sib_f32_, sib_y_;  // stacked weights / fp32 parameters / outputs
   const Blob* sib_src_ = nullptr;    // this layer's weight as it was stacked

@@ -217,6 +217,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     AliasConcatInputs();
     FuseConcatPieces();
     FuseWeightedPools();
+    FuseConcatsIntoFcs();
   }
 }
 
@@ -302,6 +303,43 @@ void SimpleNet::FuseWeightedPools() {
     host->AdoptWeightedPool(mul >= 0 ? operators_[mul].get() : nullptr, red >= 0 ? operators_[red].get() : nullptr);
     if (mul >= 0) skipped_[mul] = true;
     if (red >= 0) skipped_[red] = true;
+  }
+}
+
+// Concat (last axis) -> Gemm, the Concat's output read by nothing else: the Gemm takes the Concat over (graph.h,
+// ConcatForFc) and computes its rows while it loads them.  Nothing between the two may overwrite what the Concat, or an
+// elementwise producer the Concat has taken over, reads.  Switch: fuse_concat_into_fc: 0.
+void SimpleNet::FuseConcatsIntoFcs() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_concat_into_fc");
+  if (arg && arg->has_i && arg->i == 0) return;
+  for (size_t g = 0; g < operators_.size(); ++g) {
+    auto* fc = skipped_[g] ? nullptr : dynamic_cast<ConcatAdopter*>(operators_[g].get());
+    if (!fc || !fc->CanAdoptConcat()) continue;
+    const std::string& in = operators_[g]->operator_def().input(0);
+    int c = -1;
+    for (int j = (int)g - 1; j >= 0 && c < 0; --j)
+      for (const auto& out : operators_[j]->operator_def().output())
+        if (out == in) c = j;
+    if (c < 0 || skipped_[c] || dynamic_cast<ConcatForFc*>(operators_[c].get()) == nullptr) continue;
+    int readers = 0;
+    for (size_t j = 0; j < operators_.size(); ++j)
+      for (const auto& name : operators_[j]->operator_def().input()) readers += (name == in);
+    for (const auto& eo : external_output_) readers += (eo == in);
+    if (readers != 1 || workspace_->HasConstantBlob(in)) continue;
+    // what the Concat reads, directly or through a producer it runs itself
+    std::set<std::string> sources(operators_[c]->operator_def().input().begin(), operators_[c]->operator_def().input().end());
+    for (int j = 0; j < c; ++j) {
+      if (!skipped_[j]) continue;
+      bool feeds = false;
+      for (const auto& out : operators_[j]->operator_def().output()) feeds |= sources.count(out) != 0;
+      if (feeds) sources.insert(operators_[j]->operator_def().input().begin(), operators_[j]->operator_def().input().end());
+    }
+    bool clean = true;
+    for (size_t k = c + 1; k < g && clean; ++k)
+      for (const auto& out : operators_[k]->operator_def().output()) clean &= sources.count(out) == 0;
+    if (!clean) continue;
+    fc->AdoptConcat(operators_[c].get());
+    skipped_[c] = true;
   }
 }
 

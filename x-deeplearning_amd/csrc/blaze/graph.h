@@ -18,6 +18,8 @@
 #include "blaze/operator.h"
 #include "blaze/sparse_puller.h"
 
+struct bz_concat_ew_desc;
+
 namespace blaze {
 
 class Net;
@@ -100,6 +102,7 @@ class SimpleNet : public Net {
   void FuseFcHeads();
   void PackSiblingFcs();
   void FuseWeightedPools();
+  void FuseConcatsIntoFcs();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -183,6 +186,24 @@ class ConcatPieceHost {  // implemented by Concat
   virtual ~ConcatPieceHost() {}
   // input `input_idx` is the output of `producer` (net position `position`), which the net will not run any more
   virtual void AdoptProducer(int input_idx, OperatorBase* producer, int position) = 0;
+};
+
+// A Concat along the last axis -- with or without elementwise producers it has taken over -- whose only reader is an FC
+// operator: the FC computes the Concat's rows itself while it loads them (bz_fc_desc.a_pieces) and the tensor between
+// the two is never stored (the attention unit's [q, k, q-k, q*k] in front of its first layer).  Same values as the
+// separate operators up to the order of the layer's K sum.
+class ConcatForFc {  // implemented by Concat
+ public:
+  virtual ~ConcatForFc() {}
+  // Describes Output(0) as pieces without computing it and gives the output blob its shape (no memory).  False: the
+  // inputs do not fit the piece model; nothing has been touched.
+  virtual bool DescribeAsPieces(bz_concat_ew_desc* desc) = 0;
+};
+class ConcatAdopter {  // implemented by Gemm
+ public:
+  virtual ~ConcatAdopter() {}
+  virtual bool CanAdoptConcat() = 0;  // static part: constant 2-byte weight of a shape the kernel takes, no transposed A
+  virtual void AdoptConcat(OperatorBase* concat) = 0;
 };
 
 // MatMul(transA) of a weight column [B, T, 1] with a history [B, T, C] whose weight is the product of two equally

@@ -236,7 +236,7 @@ OPERATOR_SCHEMA(ConstantFill).NumInputs(0).NumOutputs(1).SetDoc("a constant tens
 
 // ------------------------------------------------------------------------------------------ Concat
 template <class Context>
-class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
+class ConcatOp final : public Operator<Context>, public ConcatPieceHost, public ConcatForFc {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
   ConcatOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
@@ -246,9 +246,10 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
     producers_.push_back({position, input_idx, producer});
     std::sort(producers_.begin(), producers_.end(), [](const Adopted& a, const Adopted& b) { return a.position < b.position; });
   }
+  bool DescribeAsPieces(bz_concat_ew_desc* desc) override { return RunWithPieces(desc); }
   bool RunOnDevice() override {
     if (!producers_.empty()) {
-      if (RunWithPieces()) return true;
+      if (RunWithPieces(nullptr)) return true;
       // shapes the one-launch form does not take: run the adopted operators after all, in net order, then copy
       for (const Adopted& a : producers_)
         if (!a.op->Run(context_.stream_id())) return false;
@@ -311,8 +312,10 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
   // The inputs as pieces of one bz_concat_ew launch.  False when the shapes do not fit that kernel's model (concat
   // along another axis than the last, an operand broadcast along the last axis, or row dims that do not merge into
   // two coordinates); nothing has been launched then.
-  bool RunWithPieces() {
+  // describe != nullptr: only fill *describe (dst stays null) and give the output its shape, no memory, no launch
+  bool RunWithPieces(bz_concat_ew_desc* describe) {
     const int n = this->InputSize();
+    if (n > BZ_CEW_MAX) return false;
     std::vector<ConcatPiece> pieces(n);
     std::vector<bool> described(n, false);
     for (const Adopted& a : producers_) {  // net order: a BroadcastTo may take its shape from an earlier piece
@@ -382,12 +385,15 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
     shape[rank - 1] = total;
     Blob* y = this->Output(0);
     y->set_data_type((DataType)dtype);
-    y->Reshape(shape);
+    if (describe)
+      y->SetShapeOnly(shape);
+    else
+      y->Reshape(shape);
     bz_concat_ew_desc d;
     memset(&d, 0, sizeof(d));
     d.n = n;
     d.dtype = BzType(dtype);
-    d.dst = y->data();
+    d.dst = describe ? nullptr : y->data();
     d.dst_pitch = total;
     d.r0 = group_size[0];
     d.r1 = group_size[1];
@@ -404,6 +410,10 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost {
         st[0] = b0 ? 0 : (b1 ? 1 : d.r1) * w;
         st[1] = b1 ? 0 : w;
       }
+    }
+    if (describe) {
+      *describe = d;
+      return true;
     }
     BZ_CHECK(bz_concat_ew(&d, context_.hip_stream()));
     return true;

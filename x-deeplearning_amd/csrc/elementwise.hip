@@ -14,37 +14,14 @@
 #include <hip/hip_fp16.h>
 
 #include "bz_common.h"
+#include "bz_pieces.h"
 
 namespace {
 
-template <typename T>
-__device__ __forceinline__ float ldv(const T* p);
-template <>
-__device__ __forceinline__ float ldv<float>(const float* p) {
-  return *p;
-}
-template <>
-__device__ __forceinline__ float ldv<__half>(const __half* p) {
-  return __half2float(*p);
-}
-template <>
-__device__ __forceinline__ float ldv<__hip_bfloat16>(const __hip_bfloat16* p) {
-  return __bfloat162float(*p);
-}
-template <typename T>
-__device__ __forceinline__ void stv(T* p, float v);
-template <>
-__device__ __forceinline__ void stv<float>(float* p, float v) {
-  *p = v;
-}
-template <>
-__device__ __forceinline__ void stv<__half>(__half* p, float v) {
-  *p = __float2half_rn(v);
-}
-template <>
-__device__ __forceinline__ void stv<__hip_bfloat16>(__hip_bfloat16* p, float v) {
-  *p = __float2bfloat16(v);
-}
+using bz::ldv;
+using bz::stv;
+using bz::CewP;
+using bz::CewPack;
 
 struct BcastP {
   int64_t dims[BZ_MAX_RANK];  // merged, outermost first; only [0, rank) valid
@@ -148,26 +125,11 @@ int grid_for(int64_t work) {
 }
 
 // ---- concat of pieces computed on the fly -------------------------------------------------------------------
-struct CewP {
-  const void* x[BZ_CEW_MAX];
-  const void* y[BZ_CEW_MAX];
-  int64_t xs[BZ_CEW_MAX][2], ys[BZ_CEW_MAX][2];
-  int32_t op[BZ_CEW_MAX];
-  int32_t col0[BZ_CEW_MAX + 1];  // first output column of each piece; col0[n] = total
-  int n;
-  int64_t rows, r1, dst_pitch;
-};
-
 // VEC consecutive columns of one output row per lane (the host picks a VEC that divides every width, stride and
 // address, so a lane's VEC elements are one aligned load or store).  A wave owns a row at a time: which row, and where
 // its operands start, is worked out once per row for the whole wave; inside the row a lane only has to find its piece.
 // (One flat index per thread cost two integer divisions per VEC elements and element-wise accesses: 24.7 us for the
 // [51200, 216] fp16 attention input of a DIN model, whose 54-wide pieces allow no more than VEC = 2.)
-template <typename T, int VEC>
-struct alignas(sizeof(T) * VEC) CewPack {
-  T e[VEC];
-};
-
 template <typename T, int VEC, typename IdxT>
 __global__ __launch_bounds__(256) void bz_concat_ew_kernel(T* __restrict__ dst, CewP arg) {
   // the piece table is indexed with a run-time piece number: from LDS, not from a per-lane copy of the arguments
@@ -239,16 +201,7 @@ __global__ __launch_bounds__(256) void bz_concat_ew_uniform_kernel(T* __restrict
     }
 #pragma unroll
     for (int k = 0; k < NP; ++k) {
-      const int op = p.op[k < p.n ? k : 0];
-      const bool mul = op == BZ_EW_MUL, neg = op == BZ_EW_SUB, copy = op == BZ_EW_ASSIGN;
-      Pack o;
-#pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float a = ldv<T>(&xs[k].e[e]), b = ldv<T>(&ys[k].e[e]);
-        const float r = __builtin_fmaf(a, mul ? b : 1.f, mul ? -0.f : (neg ? -b : b));
-        stv<T>(&o.e[e], r);
-        if (copy) o.e[e] = xs[k].e[e];
-      }
+      const Pack o = bz::cew_piece<T, VEC>(p.op[k < p.n ? k : 0], xs[k], ys[k]);
       if (k < p.n) *(Pack*)(out + p.col0[k]) = o;
     }
   }
@@ -256,9 +209,7 @@ __global__ __launch_bounds__(256) void bz_concat_ew_uniform_kernel(T* __restrict
 
 template <typename T, typename IdxT>
 int launch_concat_ew_i(void* dst, const CewP& p, int vec, hipStream_t s) {
-  bool uniform = p.col0[1] / vec <= 64 && sizeof(IdxT) == 4;
-  for (int k = 0; k < p.n; ++k) uniform &= (p.col0[k + 1] - p.col0[k] == p.col0[1]) && p.op[k] != BZ_EW_DIV;
-  if (uniform) {
+  if (p.col0[1] / vec <= 64 && sizeof(IdxT) == 4 && bz::cew_uniform(p)) {
     const int rows_per_wave = 64 / (p.col0[1] / vec);
     const int64_t blocks = (p.rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave);
     const int grid = (int)(blocks < 256 * 32 ? blocks : 256 * 32);
@@ -393,50 +344,10 @@ extern "C" int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream) {
 extern "C" int bz_concat_ew(const bz_concat_ew_desc* desc, bz_stream_t stream) {
   BZ_REQUIRE(desc != nullptr, "bz_concat_ew: null descriptor");
   const bz_concat_ew_desc& d = *desc;
-  BZ_REQUIRE(d.n >= 1 && d.n <= BZ_CEW_MAX, "bz_concat_ew: %d pieces outside 1..%d", d.n, BZ_CEW_MAX);
-  BZ_REQUIRE(d.dtype == BZ_F32 || d.dtype == BZ_F16 || d.dtype == BZ_BF16, "bz_concat_ew: unsupported dtype %d", d.dtype);
-  BZ_REQUIRE(d.r0 >= 0 && d.r1 >= 0 && d.dst != nullptr, "bz_concat_ew: r0=%lld r1=%lld or null dst", (long long)d.r0, (long long)d.r1);
-  const int es = bz::dtype_size(d.dtype);
-  CewP p = {};
-  p.n = d.n;
-  p.rows = d.r0 * d.r1;
-  p.r1 = d.r1 > 0 ? d.r1 : 1;
-  p.dst_pitch = d.dst_pitch;
-  int vec = 8;
-  auto fit = [&](int64_t q) {
-    while (vec > 1 && q % vec != 0) vec >>= 1;
-  };
-  int64_t total = 0;
-  for (int i = 0; i < d.n; ++i) {
-    BZ_REQUIRE(d.op[i] >= BZ_EW_ADD && d.op[i] <= BZ_EW_ASSIGN, "bz_concat_ew: piece %d: unknown op %d", i, d.op[i]);
-    BZ_REQUIRE(d.x[i] != nullptr && (d.op[i] == BZ_EW_ASSIGN || d.y[i] != nullptr), "bz_concat_ew: piece %d: null operand", i);
-    BZ_REQUIRE(d.width[i] > 0, "bz_concat_ew: piece %d: width %d", i, d.width[i]);
-    p.x[i] = d.x[i];
-    p.y[i] = d.y[i];
-    p.op[i] = d.op[i];
-    p.col0[i] = (int32_t)total;
-    total += d.width[i];
-    fit(d.width[i]);
-    fit((int64_t)((uintptr_t)d.x[i] / es));
-    BZ_REQUIRE((uintptr_t)d.x[i] % es == 0, "bz_concat_ew: piece %d: misaligned operand", i);
-    for (int k = 0; k < 2; ++k) {
-      BZ_REQUIRE(d.x_stride[i][k] >= 0 && d.y_stride[i][k] >= 0, "bz_concat_ew: piece %d: negative stride", i);
-      p.xs[i][k] = d.x_stride[i][k];
-      p.ys[i][k] = d.y_stride[i][k];
-      fit(d.x_stride[i][k]);
-      if (d.op[i] != BZ_EW_ASSIGN) fit(d.y_stride[i][k]);
-    }
-    if (d.op[i] != BZ_EW_ASSIGN) {
-      BZ_REQUIRE((uintptr_t)d.y[i] % es == 0, "bz_concat_ew: piece %d: misaligned operand", i);
-      fit((int64_t)((uintptr_t)d.y[i] / es));
-    }
-  }
-  BZ_REQUIRE(total <= d.dst_pitch && total < (1ll << 31), "bz_concat_ew: widths sum to %lld, row pitch is %lld", (long long)total,
-             (long long)d.dst_pitch);
-  BZ_REQUIRE((uintptr_t)d.dst % es == 0, "bz_concat_ew: misaligned dst");
-  p.col0[d.n] = (int32_t)total;
-  fit(d.dst_pitch);
-  fit((int64_t)((uintptr_t)d.dst / es));
+  CewP p;
+  int vec = 1;
+  const int rc = bz::cew_build(d, true, &p, &vec, "bz_concat_ew");
+  if (rc != BZ_OK) return rc;
   if (p.rows == 0) return BZ_OK;
   hipStream_t s = bz::as_stream(stream);
   if (d.dtype == BZ_F32) return launch_concat_ew<float>(d.dst, p, vec, s);

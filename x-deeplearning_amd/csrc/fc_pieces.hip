@@ -1,0 +1,296 @@
+// fc_pieces.hip -- an FC layer whose A operand is computed on the fly from pieces (bz_fc_desc.a_pieces), for gfx950.
+// Stands in for the reference's Concat of elementwise results followed by a 3-D Gemm (+ the activation after it) in the
+// attention unit of a DIN model (tools/example_model/din/model/graph_ulf.txt; blaze/operator/op/concat_op.h:46-121,
+// elementwise_op.cc:28-165, gemm_op.h:52-58,77-91) without the tensor between them.
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include <mutex>
+#include <type_traits>
+
+#include "bz_common.h"
+#include "bz_pieces.h"
+#include "fc_common.h"
+
+namespace {
+
+using namespace bz::fc;
+
+// ---------------------------------------------------------------------------------------------
+// pieces kernel: a tall layer of few columns and small K whose A operand is computed on the fly
+// ---------------------------------------------------------------------------------------------
+// A row of A is the concatenation of up to NP pieces x | x op y (bz_concat_ew's model, bz_pieces.h): the attention unit's
+// [q, k, q-k, q*k] with q broadcast over the history.  Stored first and read back, that tensor is 22 MB each way on a
+// batch of 1024 x 50 positions x 216 columns; here a workgroup writes its 128 rows of it into LDS and nowhere else.
+// The rest follows from K being small (<= 224) and N narrow (<= 96):
+//  - all of K is on chip at once, so there is no K loop over memory: one trip for the pieces' operands, one barrier,
+//    then MFMAs only;
+//  - the whole weight is kept in registers as MFMA fragments (N/32 x K/16 fragments of 4 registers: 168 for 96 x 224),
+//    loaded straight from global memory while the pieces are computed; LDS holds only the A tile (59 KB for K = 216), two
+//    workgroups a CU;
+//  - after the barrier a wave touches only its own 32 rows, so it stages its outputs in those rows' LDS without
+//    another barrier.
+// The elements of A are rounded to the tensor type as the concat kernel would have stored them (bz::cew_piece), so the
+// result is the two-launch form's up to the order of the K sum.
+constexpr int kPiecesBM = 128, kPiecesKS = 14, kPiecesMaxN = 96;
+
+// XY4: the pieces are exactly [x, y, x - y, x * y] of two operands (the attention input): a lane loads x and y once and
+// makes all four from them, instead of addressing and loading eight operands.
+template <int DT, typename OutT, int VEC, int NP, int TN, bool XY4>
+__global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const char* __restrict__ W, OutT* __restrict__ Y, int M,
+                                                              int N, int K, int64_t ldw, int64_t ldy, bool stage_y, Epilogue ep) {
+  using T = In<DT>;
+  using ET = typename std::conditional<DT == BZ_F16, __half, __hip_bfloat16>::type;
+  using Pack = bz::CewPack<ET, VEC>;
+  constexpr int BM = kPiecesBM, NT = 256;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int KP = (K + 15) / 16 * 16;   // K as the MFMAs see it; columns K.. are zero
+  const int KS = KP / 16;
+  const int pitch = KP * 2 + 16;       // bytes; the 16 spread the 16 rows of a ds_read_b128 phase over all banks
+  const int m0 = blockIdx.x * BM;
+  const int frow = lane & 31, fhalf = lane >> 5;
+
+  // per-column epilogue parameters
+  float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int n = j * 32 + frow;
+    n = n < N ? n : N - 1;
+    cbias[j] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cp0[j] = cp1[j] = cp2[j] = 0.f;
+    if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
+    if (ep.act == BZ_ACT_DICE) {
+      cp0[j] = ep.p0[n];
+      cp1[j] = ep.p1[n];
+      cp2[j] = dice_inv_den(ep, ep.p2[n]);
+    }
+  }
+
+  // the A tile: a lane owns VEC columns of a piece and walks the pieces; 64 / (W / VEC) rows share a wave.  kGenRows rows
+  // of a lane are in flight at once (no branch round the loads: a row beyond M reads row M-1 and is not stored), so the
+  // tile costs BM / (4 * rows_per_wave * kGenRows) trips to memory, not one per row.
+  {
+    constexpr int kGenRows = 8;
+    const int per_piece = p.col0[1] / VEC;
+    const int rows_per_wave = 64 / per_piece;
+    const int sub = lane / per_piece, cv = lane - sub * per_piece;
+    const uint32_t r1 = (uint32_t)p.r1;
+    if (sub < rows_per_wave) {
+      const int step = 4 * rows_per_wave;
+      for (int base = wave * rows_per_wave + sub; base < BM; base += step * kGenRows) {
+        Pack xs[kGenRows][NP], ys[kGenRows][NP];
+#pragma unroll
+        for (int u = 0; u < kGenRows; ++u) {
+          uint32_t row = (uint32_t)(m0 + base + u * step);
+          row = row < (uint32_t)M ? row : (uint32_t)M - 1;
+          const uint32_t i0 = row / r1, i1 = row - i0 * r1;
+          if constexpr (XY4) {
+            xs[u][0] = *(const Pack*)((const ET*)p.x[0] + (int64_t)i0 * p.xs[0][0] + (int64_t)i1 * p.xs[0][1] + cv * VEC);
+            xs[u][1] = *(const Pack*)((const ET*)p.x[1] + (int64_t)i0 * p.xs[1][0] + (int64_t)i1 * p.xs[1][1] + cv * VEC);
+            continue;
+          }
+#pragma unroll
+          for (int k = 0; k < NP; ++k) {
+            const int kk = k < p.n ? k : 0;
+            const bool two = p.op[kk] != BZ_EW_ASSIGN;
+            const ET* yb = two ? (const ET*)p.y[kk] : (const ET*)p.x[kk];
+            const int64_t ys0 = two ? p.ys[kk][0] : p.xs[kk][0], ys1 = two ? p.ys[kk][1] : p.xs[kk][1];
+            xs[u][k] = *(const Pack*)((const ET*)p.x[kk] + (int64_t)i0 * p.xs[kk][0] + (int64_t)i1 * p.xs[kk][1] + cv * VEC);
+            ys[u][k] = *(const Pack*)(yb + (int64_t)i0 * ys0 + (int64_t)i1 * ys1 + cv * VEC);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kGenRows; ++u) {
+          const int rl = base + u * step;
+          if constexpr (XY4) {
+            if (rl < BM && m0 + rl < M) {
+              char* dst = smem + rl * pitch + cv * VEC * 2;
+              const int wb = p.col0[1] * 2;  // bytes of a piece
+              *(Pack*)dst = xs[u][0];
+              *(Pack*)(dst + wb) = xs[u][1];
+              *(Pack*)(dst + 2 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_SUB, xs[u][0], xs[u][1]);
+              *(Pack*)(dst + 3 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_MUL, xs[u][0], xs[u][1]);
+            }
+            continue;
+          }
+#pragma unroll
+          for (int k = 0; k < NP; ++k) {
+            const Pack o = bz::cew_piece<ET, VEC>(p.op[k < p.n ? k : 0], xs[u][k], ys[u][k]);
+            if (k < p.n && rl < BM && m0 + rl < M) *(Pack*)(smem + rl * pitch + (p.col0[k] + cv * VEC) * 2) = o;
+          }
+        }
+      }
+    }
+    // columns K .. KP-1 of every row
+    for (int q = tid; q < BM * (KP - K); q += NT) {
+      const int rl = q / (KP - K), c = K + q % (KP - K);
+      *(unsigned short*)(smem + rl * pitch + c * 2) = 0;
+    }
+  }
+  // the weight, as fragments: lane (column frow of block j, half fhalf) holds k = 16*ks + 8*fhalf .. +7 of its column
+  uint4 wf[TN][kPiecesKS];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int n = j * 32 + frow;
+    n = n < N ? n : N - 1;
+    const char* wrow = W + (int64_t)n * ldw * 2;
+#pragma unroll
+    for (int ks = 0; ks < kPiecesKS; ++ks) {
+      const int k0 = ks * 16 + fhalf * 8;
+      // (rows are zero from K up to ldw, a multiple of 8: a chunk is wholly inside the row or wholly absent)
+      wf[j][ks] = (ks < KS && k0 < ldw) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
+    }
+  }
+  __syncthreads();
+
+  floatx16 acc[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  const char* arow = smem + (wave * 32 + frow) * pitch + fhalf * 16;
+  uint4 fa = *(const uint4*)arow;
+#pragma unroll
+  for (int ks = 0; ks < kPiecesKS; ++ks) {
+    if (ks < KS) {
+      const uint4 cur = fa;
+      if (ks + 1 < KS) fa = *(const uint4*)(arow + (ks + 1) * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) T::mma(cur, wf[j][ks], acc[j]);
+    }
+  }
+
+  // epilogue: lane owns column n of each block, rows 8*(r/4) + 4*(lane/32) + r%4 of the wave's 32
+  constexpr int OS = (int)sizeof(OutT);
+  constexpr int OPITCH = TN * 32 * OS + 16;
+  char* lout = smem + wave * 32 * pitch;  // this wave's own rows of the A tile (the host checked that the output fits)
+  auto epilogue = [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = j * 32 + frow;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ml = 8 * (r >> 2) + 4 * fhalf + (r & 3);
+        const int m = m0 + wave * 32 + ml;
+        float v = ep.alpha * acc[j][r];
+        if (ep.bias_rows == 1) v += ep.beta * cbias[j];
+        v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
+        if (stage_y)
+          store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, v);
+        else if (m < M && n < N)
+          store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+      }
+    }
+  };
+  switch (ep.act) {
+    case BZ_ACT_PRELU:
+      epilogue(std::integral_constant<int, BZ_ACT_PRELU>());
+      break;
+    case BZ_ACT_DICE:
+      epilogue(std::integral_constant<int, BZ_ACT_DICE>());
+      break;
+    case BZ_ACT_LEAKY_RELU:
+      epilogue(std::integral_constant<int, BZ_ACT_LEAKY_RELU>());
+      break;
+    case BZ_ACT_SIGMOID:
+      epilogue(std::integral_constant<int, BZ_ACT_SIGMOID>());
+      break;
+    default:
+      epilogue(std::integral_constant<int, BZ_ACT_NONE>());
+      break;
+  }
+  if (stage_y) {
+    const int ocpr = N * OS / 16;  // 16-byte chunks per output row (N * OS is a multiple of 16 when stage_y)
+    for (int q = lane; q < 32 * ocpr; q += 64) {
+      const int ml = q / ocpr, ch = q - ml * ocpr;
+      const int m = m0 + wave * 32 + ml;
+      if (m < M) *(uint4*)((char*)(Y + (int64_t)m * ldy) + ch * 16) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+    }
+  }
+}
+
+// A from pieces (bz_fc_desc.a_pieces).  BZ_ENOTSUP, with nothing launched, for anything outside the kernel's model.
+template <int DT, typename OutT, int VEC, int NP, bool XY4>
+int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep, bool stage_y, int smem, hipStream_t st) {
+  const int grid = (d.m + kPiecesBM - 1) / kPiecesBM;
+  const int tn = (d.n + 31) / 32;
+#define BZ_PIECES(TN)                                                                                                          \
+  do {                                                                                                                         \
+    static std::mutex mu;                                                                                                      \
+    static bool raised[64] = {};                                                                                               \
+    int dev = 0;                                                                                                               \
+    BZ_HIP_OK(hipGetDevice(&dev));                                                                                             \
+    {                                                                                                                          \
+      std::lock_guard<std::mutex> lock(mu);                                                                                    \
+      if (dev >= 0 && dev < 64 && !raised[dev]) {                                                                              \
+        BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4>,                                 \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, kPiecesBM * (kPiecesKS * 16 * 2 + 16)));     \
+        raised[dev] = true;                                                                                                    \
+      }                                                                                                                        \
+    }                                                                                                                          \
+    hipLaunchKernelGGL((bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4>), dim3(grid), dim3(256), smem, st, p, (const char*)d.w,     \
+                       (OutT*)d.y, d.m, d.n, d.k, d.ldw, d.ldy, stage_y, ep);                                                  \
+  } while (0)
+  if (tn == 1)
+    BZ_PIECES(1);
+  else if (tn == 2)
+    BZ_PIECES(2);
+  else
+    BZ_PIECES(3);
+#undef BZ_PIECES
+  BZ_LAUNCH_OK("bz_fc_pieces_kernel");
+  return BZ_OK;
+}
+
+template <int DT, typename OutT>
+int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
+  const bz_concat_ew_desc& c = *d.a_pieces;
+  bz::CewP p;
+  int vec = 1;
+  const int rc = bz::cew_build(c, false, &p, &vec, "bz_fc_fused (a_pieces)");
+  if (rc != BZ_OK) return rc;
+  BZ_REQUIRE(c.dtype == d.in_dtype, "bz_fc_fused: a_pieces of dtype %d for a layer of dtype %d", c.dtype, d.in_dtype);
+  BZ_REQUIRE(p.rows == d.m && p.col0[p.n] == d.k, "bz_fc_fused: a_pieces describe [%lld, %d], the layer takes [%d, %d]",
+             (long long)p.rows, p.col0[p.n], d.m, d.k);
+  const int kp = (d.k + 15) / 16 * 16;
+  const int os = (int)sizeof(OutT);
+  if (!bz::cew_uniform(p) || p.col0[1] / (vec == 4 ? 2 : vec) > 64 || p.n > 4 || kp / 16 > kPiecesKS || d.n > kPiecesMaxN || d.n <= kSkinnyMaxN ||
+      d.m >= (1ll << 31) - kPiecesBM)
+    return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces take at most 4 pieces of one width without division, k <= %d, %d < n <= %d",
+                    kPiecesKS * 16, kSkinnyMaxN, kPiecesMaxN);
+  const int pitch = kp * 2 + 16;
+  const int tn = (d.n + 31) / 32;
+  // 16-byte stores of whole output rows through the wave's own rows of the A tile, when they fit there
+  const bool stage_y = ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0) && (tn * 32 * os + 16 <= pitch);
+  const int smem = kPiecesBM * pitch;
+  // (8 or 2 columns a lane; a width that allows 4 takes 2, an odd one is left to the two-launch form)
+  // [x, y, x - y, x * y]: pieces 2 and 3 read exactly what pieces 0 and 1 copy
+  auto same = [&](int k, bool second, int src) {
+    const void* ptr = second ? p.y[k] : p.x[k];
+    const int64_t* s = second ? p.ys[k] : p.xs[k];
+    return ptr == p.x[src] && s[0] == p.xs[src][0] && s[1] == p.xs[src][1];
+  };
+  const bool xy4 = p.n == 4 && p.op[0] == BZ_EW_ASSIGN && p.op[1] == BZ_EW_ASSIGN && p.op[2] == BZ_EW_SUB && p.op[3] == BZ_EW_MUL &&
+                   same(2, false, 0) && same(2, true, 1) && same(3, false, 0) && same(3, true, 1);
+  if (vec == 8) return xy4 ? launch_pieces_tn<DT, OutT, 8, 4, true>(d, p, ep, stage_y, smem, st)
+                           : launch_pieces_tn<DT, OutT, 8, 4, false>(d, p, ep, stage_y, smem, st);
+  if (vec >= 2) return xy4 ? launch_pieces_tn<DT, OutT, 2, 4, true>(d, p, ep, stage_y, smem, st)
+                           : launch_pieces_tn<DT, OutT, 2, 4, false>(d, p, ep, stage_y, smem, st);
+  return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces of odd width");
+}
+
+}  // namespace
+
+int bz::fc_pieces_launch(const bz_fc_desc& d, const bz::fc::Epilogue& ep, hipStream_t st) {
+  if (d.in_dtype == BZ_F16) {
+    if (d.out_dtype == BZ_F32) return launch_pieces<BZ_F16, float>(d, ep, st);
+    if (d.out_dtype == BZ_F16) return launch_pieces<BZ_F16, __half>(d, ep, st);
+  } else if (d.in_dtype == BZ_BF16) {
+    if (d.out_dtype == BZ_F32) return launch_pieces<BZ_BF16, float>(d, ep, st);
+    if (d.out_dtype == BZ_BF16) return launch_pieces<BZ_BF16, __hip_bfloat16>(d, ep, st);
+  }
+  return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces: in dtype %d, out dtype %d", d.in_dtype, d.out_dtype);
+}
