@@ -216,6 +216,29 @@ enum bz_act {
  * M = batch*M.
  */
 struct bz_concat_ew_desc;
+/*
+ * A second full layer in the launch of an a_pieces layer (bz_fc_desc.next): Z = act(alpha * Y * w^T + beta * bias) with
+ * Y the first layer's activated output, rounded to the tensor type as it would have been stored.  With it the
+ * descriptor's head_* fields describe a skinny third layer on Z instead of on Y, and both y pointers may be NULL (that
+ * tensor is then not stored): the three-layer attention MLP of a DIN model (216 -> 80 -> 40 -> 1 in
+ * tools/example_model/din/model/graph_ulf.txt) is one launch that reads q and k and writes the scores.
+ */
+typedef struct bz_fc_next {
+  const void* w;        /* device [n, ldw] packed, K = the first layer's n, dtype in_dtype */
+  const float* bias;    /* device [n] or NULL */
+  void* y;              /* device [M, ldy], dtype in_dtype, or NULL */
+  const float* act_p0;  /* as in bz_fc_desc, for this layer's n columns */
+  const float* act_p1;
+  const float* act_p2;
+  int64_t ldw, ldy;
+  int32_t n;            /* 9..64 */
+  int32_t act;          /* bz_act but BZ_ACT_SOFTMAX */
+  int32_t act_size;
+  int32_t dice_nosqrt;
+  float alpha, beta, act_alpha;
+  int32_t reserved_;
+} bz_fc_next;
+
 typedef struct bz_fc_desc {
   const void* a;       /* device [M, lda] */
   const void* w;       /* device [N, ldw] packed */
@@ -263,8 +286,11 @@ typedef struct bz_fc_desc {
    * stored: DIN's attention input [q, k, q-k, q*k] (tools/example_model/din/model/graph_ulf.txt) costs its 22 MB of
    * traffic each way otherwise.  Same values as the two-step form: every element of A is rounded to the tensor type
    * exactly as the concat would store it.  Limits: 2-byte types, pieces of one width that do not divide,
-   * k <= 224, n <= 96, no head, no split outputs, per-column bias only; BZ_ENOTSUP (nothing launched) otherwise. */
+   * k <= 224, n <= 96, no head (but see next), no split outputs, per-column bias only; BZ_ENOTSUP (nothing launched)
+   * otherwise. */
   const struct bz_concat_ew_desc* a_pieces;
+  /* with a_pieces only: a second layer (and, through head_*, a skinny third) in the same launch; out_dtype == in_dtype */
+  const bz_fc_next* next;
 } bz_fc_desc;
 
 BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);

@@ -216,16 +216,16 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     din_model.feed(p, inputs, batch, np.float16)
     p.forward()
     got = {name: p.output_asnumpy(name).astype(np.float32) for name in expose + ("prob", )}
-    # nine kernel launches a forward: 2 Embedding, 2 Concat (history, main input), 4 Gemm (each with its Dice / next
-    # skinny layer / softmax folded in; the first also computes the attention input [q, k, q-k, q*k] it reads), 1 MatMul
-    # (with the Mul and the ReduceSum)
+    # eight kernel launches a forward: 2 Embedding, 2 Concat (history, main input), 3 Gemm (the whole attention MLP
+    # 216 -> 80 -> 40 -> 1 with its input [q, k, q-k, q*k] computed on the fly; the two launches of the main MLP, each
+    # with its Dice / skinny layer / softmax folded in), 1 MatMul (with the Mul and the ReduceSum)
     import json
     p.register_observers(["profile"])
     p.forward()
     ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
     launching = [e for e in ev if e["name"].split(":")[0] not in ("ConstantFill", "Reshape")]
     kinds = sorted(e["name"].split(":")[0] for e in launching)
-    assert kinds == ["Concat"] * 2 + ["Embedding"] * 2 + ["Gemm"] * 4 + ["MatMul"], kinds
+    assert kinds == ["Concat"] * 2 + ["Embedding"] * 2 + ["Gemm"] * 3 + ["MatMul"], kinds
     assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
     for k, t in zip(din_model.KINDS, tables):
@@ -365,4 +365,37 @@ def test_attention_input_computed_by_its_first_layer_equals_the_separate_operato
     for (y1, p1), (y0, p0), b in zip(outs[1], outs[0], (96, 17, 96)):
         assert y1.shape == (b, cfg.T, 80) and y1.any()
         np.testing.assert_allclose(y1, y0, rtol=2e-3, atol=2e-3 * np.abs(y0).max())
+        np.testing.assert_allclose(p1, p0, rtol=2e-3, atol=2e-3)
+
+
+def test_attention_mlp_in_one_launch_equals_layer_by_layer():
+    """Gemm+Dice (on the Concat it computes itself) -> Gemm+Dice -> Gemm: by default one launch (bz_fc_desc.next + head); with
+    chain_narrow_fcs: 0 the second Gemm runs on its own (hosting the third).  Scores agree to the roundings of the tensor
+    type, probabilities to 2e-3, also after the batch shrinks and grows again."""
+    import json
+    import torch
+    import din_model
+    cfg = din_model.Config3(batch=96, rows=5000, T=20)
+    small = din_model.Config3(batch=17, rows=5000, T=20)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=5), cfg.batch_inputs(seed_offset=9)]
+    outs = {}
+    for chain in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("score", ), net_args={"chain_narrow_fcs": chain})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append((p.output_asnumpy("score").astype(np.float32), p.output_asnumpy("prob").copy()))
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        ran = [e["name"] for e in ev]
+        assert ("Gemm:gemm_att1_g" in ran) == (chain == 0), ran
+        assert [e["args"]["launches"] for e in ev if e["name"] == "Gemm:gemm_att0_g"] == [1]
+        outs[chain] = got
+    torch.cuda.synchronize()
+    for (s1, p1), (s0, p0), b in zip(outs[1], outs[0], (96, 17, 96)):
+        assert s1.shape == (b, cfg.T, 1) and s1.any()
+        np.testing.assert_allclose(s1, s0, rtol=0, atol=4e-3 * max(1.0, float(np.abs(s0).max())))
         np.testing.assert_allclose(p1, p0, rtol=2e-3, atol=2e-3)

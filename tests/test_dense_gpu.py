@@ -608,3 +608,89 @@ def test_fc_on_pieces_limits_are_refused(bz):
     pd.width[0] = pd.width[1] = pd.width[2] = pd.width[3] = 40
     d.k, d.ldw = 160, 160
     assert bz.lib().bz_fc_fused(C.byref(d), None) == bz.ENOTSUP  # a piece that divides
+
+
+@pytest.mark.parametrize("in_name", ["f16", "bf16"])
+@pytest.mark.parametrize("r0,r1,w,N,N2,N3,act2,head_act", [
+    (1024, 50, 54, 80, 40, 1, "dice", "none"),     # DIN's attention MLP 216 -> 80 -> 40 -> 1
+    (37, 5, 24, 96, 64, 2, "prelu", "softmax"),    # widest second layer, a softmax head, ragged last tile
+    (300, 3, 40, 24, 16, 0, "relu", "none"),       # no third layer: the second layer's output is stored
+])
+def test_attention_mlp_as_one_launch(bz, oracle, in_name, r0, r1, w, N, N2, N3, act2, head_act):
+    """bz_fc_fused with a_pieces + next (+ head): the layers after the first run in its launch from rows that never leave
+    the chip.  Against the separate launches (concat, layer, layer with its head), which round and store what this one
+    only rounds."""
+    import ctypes as C
+    import torch
+    print("attention mlp %s r0=%d r1=%d w=%d %d->%d->%d %s %s" % (in_name, r0, r1, w, N, N2, N3, act2, head_act), flush=True)
+    tdt = _tdtype(in_name)
+    dt = bz.bz_dtype(tdt)
+    rng = np.random.default_rng(r0 + w + N + N2)
+    M, K = r0 * r1, 4 * w
+    q = _dev(_round_to(rng.standard_normal((r0, 1, w)), in_name)).to(tdt)
+    k = _dev(_round_to(rng.standard_normal((r0, r1, w)), in_name)).to(tdt)
+    W1 = _dev(_round_to(rng.standard_normal((K, N)) / np.sqrt(K), in_name)).to(tdt)
+    W2 = _dev(_round_to(rng.standard_normal((N, N2)) / np.sqrt(N), in_name)).to(tdt)
+    b1, b2 = _dev((rng.standard_normal(N) * 0.1).astype(np.float32)), _dev((rng.standard_normal(N2) * 0.1).astype(np.float32))
+    dice1 = tuple(_dev(x) for x in ((rng.standard_normal(N) * 0.1).astype(np.float32), (rng.standard_normal(N) * 0.1).astype(np.float32),
+                                    rng.uniform(0.5, 1.5, N).astype(np.float32)))
+    p2 = {"dice": tuple(_dev(x) for x in ((rng.standard_normal(N2) * 0.1).astype(np.float32), (rng.standard_normal(N2) * 0.1).astype(np.float32),
+                                          rng.uniform(0.5, 1.5, N2).astype(np.float32))),
+          "prelu": (_dev(rng.uniform(0.1, 0.4, N2).astype(np.float32)), ), "relu": ()}[act2]
+    wp1, wp2 = bz.pack_weight(W1, False, dt), bz.pack_weight(W2, False, dt)
+    head = None
+    if N3:
+        W3 = _dev(_round_to(rng.standard_normal((N2, N3)) / np.sqrt(N2), in_name)).to(tdt)
+        b3 = _dev((rng.standard_normal(N3) * 0.1).astype(np.float32))
+        wp3 = bz.pack_weight(W3, False, dt)
+    pieces = [(bz.EW_ASSIGN, q, None), (bz.EW_ASSIGN, k, None), (bz.EW_SUB, q, k), (bz.EW_MUL, q, k)]
+    # separate launches
+    a_full = bz.concat_ew(pieces).reshape(M, K)
+    y1 = bz.fc_fused(a_full, wp1, K, bias=b1, act=bz.ACT_DICE, act_params=dice1)
+    if N3:
+        z_ref = torch.empty((M, N3), dtype=torch.float32, device="cuda")
+        bz.fc_fused(y1, wp2, N, bias=b2, act=ACT[act2], act_params=p2, act_alpha=0.0,
+                    head=dict(w=wp3, bias=b3, act=ACT[head_act], out=z_ref), store_out=False)
+    else:
+        y2_ref = bz.fc_fused(y1, wp2, N, bias=b2, act=ACT[act2], act_params=p2, act_alpha=0.0)
+    # one launch
+    pd = _pieces_desc(bz, pieces, r0, r1, tdt)
+    nx = bz.FcNext()
+    nx.w, nx.ldw, nx.n, nx.bias = wp2.data_ptr(), wp2.stride(0), N2, b2.data_ptr()
+    nx.alpha = nx.beta = 1.0
+    nx.act, nx.act_alpha = ACT[act2], 0.0
+    for name, p_ in zip(("act_p0", "act_p1", "act_p2"), p2):
+        setattr(nx, name, p_.data_ptr())
+    nx.act_size = N2 if act2 in ("prelu", "dice") else 0
+    d = bz.FcDesc()
+    d.a_pieces = C.cast(C.pointer(pd), C.c_void_p)
+    d.next = C.cast(C.pointer(nx), C.c_void_p)
+    d.w, d.ldw, d.bias = wp1.data_ptr(), wp1.stride(0), b1.data_ptr()
+    d.m, d.n, d.k, d.ldy = M, N, K, N
+    d.in_dtype = d.out_dtype = dt
+    d.bias_rows, d.alpha, d.beta = 1, 1.0, 1.0
+    d.act, d.act_size = bz.ACT_DICE, N
+    d.act_p0, d.act_p1, d.act_p2 = (t.data_ptr() for t in dice1)
+    if N3:
+        z = torch.full((M, N3), float("nan"), dtype=torch.float32, device="cuda")
+        d.head_w, d.head_ldw, d.head_bias, d.head_y, d.head_ldy = wp3.data_ptr(), wp3.stride(0), b3.data_ptr(), z.data_ptr(), N3
+        d.head_n, d.head_act, d.head_out_dtype = N3, ACT[head_act], bz.F32
+    else:
+        y2 = torch.full((M, N2), float("nan"), dtype=tdt, device="cuda")
+        nx.y, nx.ldy = y2.data_ptr(), N2
+    bz.check(bz.lib().bz_fc_fused(C.byref(d), None))
+    torch.cuda.synchronize()
+    got = (z if N3 else y2).float().cpu().numpy()
+    ref = (z_ref if N3 else y2_ref).float().cpu().numpy()
+    assert not np.isnan(got).any()
+    eps = 2.0**-8 if in_name == "bf16" else 2.0**-11
+    # three roundings of the tensor type on the way, each amplified by at most the next layer's row sums (weights ~ 1/sqrt(K))
+    np.testing.assert_allclose(got, ref, rtol=0, atol=(8 * eps) * max(1.0, float(np.abs(ref).max())) + 2e-3)
+    # also with the first layer's own output stored
+    y1_one = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    d.y = y1_one.data_ptr()
+    bz.check(bz.lib().bz_fc_fused(C.byref(d), None))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(y1_one.float().cpu().numpy(), y1.float().cpu().numpy(), rtol=0,
+                               atol=4 * eps * max(1.0, float(y1.float().abs().max())))
+    np.testing.assert_allclose((z if N3 else y2).float().cpu().numpy(), got, rtol=0, atol=0)

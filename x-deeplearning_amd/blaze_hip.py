@@ -51,7 +51,14 @@ class FcDesc(C.Structure):
                 ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
                 ("reserved_", C.c_int32), ("head_w", C.c_void_p), ("head_bias", C.c_void_p), ("head_y", C.c_void_p),
                 ("head_ldw", C.c_int64), ("head_ldy", C.c_int64), ("head_n", C.c_int32), ("head_act", C.c_int32),
-                ("head_out_dtype", C.c_int32), ("n_split", C.c_int32), ("y_split_stride", C.c_int64), ("a_pieces", C.c_void_p)]
+                ("head_out_dtype", C.c_int32), ("n_split", C.c_int32), ("y_split_stride", C.c_int64), ("a_pieces", C.c_void_p), ("next", C.c_void_p)]
+
+
+class FcNext(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("act_p0", C.c_void_p), ("act_p1", C.c_void_p),
+                ("act_p2", C.c_void_p), ("ldw", C.c_int64), ("ldy", C.c_int64), ("n", C.c_int32), ("act", C.c_int32),
+                ("act_size", C.c_int32), ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float),
+                ("act_alpha", C.c_float), ("reserved_", C.c_int32)]
 
 
 class BgemmDesc(C.Structure):

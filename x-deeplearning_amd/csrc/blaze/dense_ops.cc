@@ -68,6 +68,7 @@ struct FcCall {
   // operands
   const void* a = nullptr;
   const bz_concat_ew_desc* a_pieces = nullptr;  // instead of a: the rows as pieces computed on the fly (bz_fc_desc.a_pieces)
+  const bz_fc_next* next = nullptr;             // with a_pieces: a second layer in the same launch
   int a_rows = 0, a_cols = 0;  // as stored
   bool trans_a = false;
   Blob* b_blob = nullptr;
@@ -179,6 +180,7 @@ bool RunFc(const FcCall& c, Derived* packed_b, Derived* packed_a, hipStream_t st
   }
   if (c.a_pieces != nullptr) {
     d.a_pieces = c.a_pieces;
+    d.next = c.next;
     d.a = nullptr;
     const int rc = bz_fc_fused(&d, st);
     if (rc == BZ_ENOTSUP) return false;
@@ -317,6 +319,23 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     return N > 8 && N <= 96 && K <= 224 && !(fused_ && fused_act_ == BZ_ACT_SOFTMAX);
   }
   void AdoptConcat(OperatorBase* concat) override { concat_ = concat; }
+  bool HasAdoptedConcat() const override { return concat_ != nullptr; }
+  bool CanChainNext(OperatorBase* next_op) override {
+    auto* g = dynamic_cast<GemmOp*>(next_op);
+    if (g == nullptr || concat_ == nullptr || head_ != nullptr || !stack_.empty() || !siblings_.empty() || next_ != nullptr) return false;
+    Blob* b0 = this->Input(1);
+    Blob* b = g->Input(1);
+    if (!g->b_constant_ || g->transa_ || b->shape().size() != 2 || b->data_type() != b0->data_type()) return false;
+    if (!g->stack_.empty() || !g->siblings_.empty() || g->concat_ != nullptr) return false;
+    const TIndex N1 = transb_ ? b0->shape()[0] : b0->shape()[1];
+    const TIndex K2 = g->transb_ ? b->shape()[1] : b->shape()[0], N2 = g->transb_ ? b->shape()[0] : b->shape()[1];
+    if (K2 != N1 || N2 <= 8 || N2 > 64) return false;
+    if (g->InputSize() > 2 && (!g->c_constant_ || (TIndex)g->Input(2)->size() != N2)) return false;
+    if (g->fused_ && g->fused_act_ == BZ_ACT_SOFTMAX) return false;
+    if (g->fused_ && g->fused_act_ == BZ_ACT_PRELU && (TIndex)g->fused_->Input(1)->size() != N2 && g->fused_->Input(1)->size() != 1) return false;
+    return true;
+  }
+  void AdoptNext(OperatorBase* next_op) override { next_ = static_cast<GemmOp*>(next_op); }
 
   int LaunchesOfLastRun() const override { return launches_; }
 
@@ -326,7 +345,10 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
       if (siblings_.empty() && head_ == nullptr && stack_.empty()) {
         bz_concat_ew_desc pieces;
         auto* c = dynamic_cast<ConcatForFc*>(concat_);
-        if (c != nullptr && c->DescribeAsPieces(&pieces) && RunSelf(false, &pieces)) return true;
+        if (c != nullptr && c->DescribeAsPieces(&pieces)) {
+          if (next_ != nullptr && RunSelf(false, &pieces, true)) return true;  // this layer, the next and its head
+          if (RunSelf(false, &pieces)) return RunNextAlone();
+        }
       }
       // a shape the one-launch form does not take: the Concat runs after all
       if (!concat_->Run(context_.stream_id())) return false;
@@ -336,10 +358,17 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     const int before = launches_ - 1;
     const bool ok = RunRest();
     launches_ += before;
-    return ok;
+    return ok && RunNextAlone();
   }
 
  protected:
+  // the adopted next layer as launches of its own
+  bool RunNextAlone() {
+    if (next_ == nullptr) return true;
+    if (!next_->Run(context_.stream_id())) return false;
+    launches_ += next_->LaunchesOfLastRun() > 0 ? next_->LaunchesOfLastRun() : 1;
+    return true;
+  }
   bool RunRest() {
     launches_ = 1;
     if (!siblings_.empty()) {
@@ -531,7 +560,9 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   // with_head: also compute head_'s layer in this launch and leave this layer's own output unstored; false when the
   // operands do not allow it (nothing has been launched then)
   // pieces: the input given as pieces computed on the fly (an adopted Concat); false when the kernel does not take them
-  bool RunSelf(bool with_head, const bz_concat_ew_desc* pieces = nullptr) {
+  // chain: also run next_ (and the skinny layer it hosts) in this launch; this layer's and next_'s own outputs are then
+  // not stored
+  bool RunSelf(bool with_head, const bz_concat_ew_desc* pieces = nullptr, bool chain = false) {
     CheckValid();
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -562,7 +593,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
         hy->Reshape({M, n2});
     }
     if (a_shape.size() == 3) {
-      if (with_head)
+      if (with_head || chain)
         y->SetShapeOnly({a_shape[0], M, N});
       else
         y->Reshape({a_shape[0], M, N});
@@ -570,13 +601,84 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
       // strided-batched case (stride_b = 0, :77-91), which over contiguous slices is again one 2-D product
       BLAZE_CONDITION_THROW(!transa_ || a_shape[0] == 1, "3-D Gemm with transA is not supported on this device");
       rows = a_shape[0] * M;
-    } else if (with_head) {
+    } else if (with_head || chain) {
       y->SetShapeOnly({M, N});
     } else {
       y->Reshape({M, N});
     }
     hipStream_t st = context_.hip_stream();
     FcCall call;
+    bz_fc_next nx;
+    if (chain) {
+      // next_ (with its folded activation) as bz_fc_next, the skinny layer it hosts through the head_* fields
+      GemmOp* g = next_;
+      Blob* b2 = g->Input(1);
+      if (y->data_type() != a->data_type()) return false;
+      const int es2 = (int)DataTypeSize(b2->data_type());
+      const int n2 = (int)(g->transb_ ? b2->shape()[0] : b2->shape()[1]);
+      const int64_t ldw2 = (N + 7) / 8 * 8;
+      if (g->packed_b_.Stale(b2) || g->packed_b_.bytes < (size_t)n2 * ldw2 * es2) {
+        g->packed_b_.Resize((size_t)n2 * ldw2 * es2);
+        BZ_CHECK(bz_fc_pack_weight(b2->data(), BzType(b2->data_type()), g->transb_ ? 1 : 0, (int)N, n2, g->packed_b_.ptr,
+                                   BzType(b2->data_type()), ldw2, st));
+        g->packed_b_.Mark(b2);
+      }
+      memset(&nx, 0, sizeof(nx));
+      nx.w = g->packed_b_.ptr;
+      nx.ldw = ldw2;
+      nx.n = n2;
+      nx.alpha = g->alpha_;
+      nx.beta = g->beta_;
+      if (g->InputSize() > 2) nx.bias = AsFloatParam(g->Input(2), &g->bias_f32_, true, st);
+      if (g->fused_) {
+        nx.act = g->fused_act_;
+        nx.dice_nosqrt = g->fused_nosqrt_ ? 1 : 0;
+        nx.act_alpha = g->fused_alpha_;
+        if (g->fused_act_ == BZ_ACT_PRELU) {
+          nx.act_p0 = AsFloatParam(g->fused_->Input(1), &g->p_f32_[0], true, st);
+          nx.act_size = (int)g->fused_->Input(1)->size();
+        } else if (g->fused_act_ == BZ_ACT_DICE) {
+          nx.act_p0 = AsFloatParam(g->fused_->Input(1), &g->p_f32_[0], true, st);
+          nx.act_p1 = AsFloatParam(g->fused_->Input(2), &g->p_f32_[1], true, st);
+          nx.act_p2 = AsFloatParam(g->fused_->Input(3), &g->p_f32_[2], true, st);
+          nx.act_size = n2;
+        }
+      }
+      Blob* y2 = g->fused_ ? g->fused_->Output(0) : g->Output(0);
+      if (y2->data_type() != a->data_type()) return false;
+      const std::vector<TIndex> shape2 = a_shape.size() == 3 ? std::vector<TIndex>{a_shape[0], M, (TIndex)n2} : std::vector<TIndex>{M, (TIndex)n2};
+      if (g->head_ != nullptr) {
+        GemmOp* h = g->head_;
+        Blob* hb = h->Input(1);
+        const int n3 = (int)(h->transb_ ? hb->shape()[0] : hb->shape()[1]);
+        const int es3 = (int)DataTypeSize(hb->data_type());
+        if (hb->data_type() != a->data_type()) return false;
+        const int64_t ldw3 = (n2 + 7) / 8 * 8;
+        if (h->packed_b_.Stale(hb) || h->packed_b_.bytes < (size_t)n3 * ldw3 * es3) {
+          h->packed_b_.Resize((size_t)n3 * ldw3 * es3);
+          BZ_CHECK(bz_fc_pack_weight(hb->data(), BzType(hb->data_type()), h->transb_ ? 1 : 0, n2, n3, h->packed_b_.ptr,
+                                     BzType(hb->data_type()), ldw3, st));
+          h->packed_b_.Mark(hb);
+        }
+        y2->SetShapeOnly(shape2);
+        Blob* hy3 = h->fused_ ? h->fused_->Output(0) : h->Output(0);
+        std::vector<TIndex> shape3 = shape2;
+        shape3.back() = n3;
+        hy3->Reshape(shape3);
+        call.head_w = h->packed_b_.ptr;
+        call.head_ldw = ldw3;
+        if (h->InputSize() > 2) call.head_bias = AsFloatParam(h->Input(2), &h->bias_f32_, true, st);
+        call.head_y = hy3->data();
+        call.head_y_dtype = hy3->data_type();
+        call.head_n = n3;
+        call.head_act = h->fused_ ? h->fused_act_ : BZ_ACT_NONE;
+      } else {
+        y2->Reshape(shape2);
+        nx.y = y2->data();
+        nx.ldy = n2;
+      }
+      call.next = &nx;
+    }
     call.a = pieces ? nullptr : a->data();
     call.a_pieces = pieces;
     call.a_rows = transa_ ? (int)K : (int)rows;
@@ -589,7 +691,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     call.trans_b = transb_;
     call.b_constant = b_constant_;
     call.dtype = a->data_type();
-    call.y = with_head ? nullptr : y->data();
+    call.y = (with_head || chain) ? nullptr : y->data();
     call.y_dtype = y->data_type();
     call.alpha = alpha_;
     call.beta = beta_;
@@ -674,6 +776,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
   GemmOp* head_ = nullptr;       // the layer of at most 8 outputs computed in this operator's launch
   OperatorBase* concat_ = nullptr;  // the Concat that makes Input(0), computed by this operator's kernel
+  GemmOp* next_ = nullptr;          // the narrow layer after this one, computed in this operator's launch
   std::vector<GemmOp*> siblings_;  // layers on the same input computed in this operator's launch
   Derived sib_w_, sib_f32_, sib_y_;  // stacked weights / fp32 parameters / outputs
   const Blob* sib_src_ = nullptr;    // this layer's weight as it was stacked

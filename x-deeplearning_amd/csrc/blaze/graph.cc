@@ -218,6 +218,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     FuseConcatPieces();
     FuseWeightedPools();
     FuseConcatsIntoFcs();
+    ChainNarrowFcs();
   }
 }
 
@@ -340,6 +341,34 @@ void SimpleNet::FuseConcatsIntoFcs() {
     if (!clean) continue;
     fc->AdoptConcat(operators_[c].get());
     skipped_[c] = true;
+  }
+}
+
+// A Gemm that computes its Concat input itself -> the narrow Gemm that reads only its result: the second (and the skinny
+// layer it may host) runs in the first one's launch (graph.h, ConcatAdopter::CanChainNext).  Switch: chain_narrow_fcs: 0.
+void SimpleNet::ChainNarrowFcs() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "chain_narrow_fcs");
+  if (arg && arg->has_i && arg->i == 0) return;
+  for (size_t i = 0; i < operators_.size(); ++i) {
+    auto* first = skipped_[i] ? nullptr : dynamic_cast<ConcatAdopter*>(operators_[i].get());
+    auto* first_fc = first ? dynamic_cast<StackableFc*>(operators_[i].get()) : nullptr;
+    if (!first || !first_fc || !first->HasAdoptedConcat()) continue;
+    size_t j = i + 1;
+    while (j < operators_.size() && skipped_[j]) ++j;  // (the first layer's folded activation)
+    if (j >= operators_.size()) break;
+    if (!first->CanChainNext(operators_[j].get())) continue;
+    const std::string& mid = first_fc->StackOutputOp()->operator_def().output(0);
+    if (operators_[j]->operator_def().input(0) != mid) continue;
+    int readers = 0;
+    for (size_t k = 0; k < operators_.size(); ++k) {
+      if (skipped_[k]) continue;
+      for (const auto& in : operators_[k]->operator_def().input()) readers += (in == mid);
+    }
+    bool is_output = false;
+    for (const auto& eo : external_output_) is_output |= (eo == mid);
+    if (readers != 1 || is_output) continue;
+    first->AdoptNext(operators_[j].get());
+    skipped_[j] = true;
   }
 }
 

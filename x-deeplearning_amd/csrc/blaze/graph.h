@@ -103,6 +103,7 @@ class SimpleNet : public Net {
   void PackSiblingFcs();
   void FuseWeightedPools();
   void FuseConcatsIntoFcs();
+  void ChainNarrowFcs();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -204,6 +205,12 @@ class ConcatAdopter {  // implemented by Gemm
   virtual ~ConcatAdopter() {}
   virtual bool CanAdoptConcat() = 0;  // static part: constant 2-byte weight of a shape the kernel takes, no transposed A
   virtual void AdoptConcat(OperatorBase* concat) = 0;
+  virtual bool HasAdoptedConcat() const = 0;
+  // The narrow layer after such a layer (with the skinny layer it may already host) in the same launch
+  // (bz_fc_desc.next): the attention MLP 4E -> 80 -> 40 -> 1 as one kernel.  `next` reads only this layer's result, and
+  // nothing else does.
+  virtual bool CanChainNext(OperatorBase* next) = 0;  // static part
+  virtual void AdoptNext(OperatorBase* next) = 0;
 };
 
 // MatMul(transA) of a weight column [B, T, 1] with a history [B, T, C] whose weight is the product of two equally

@@ -973,7 +973,8 @@ extern "C" {
 int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   BZ_REQUIRE(desc != nullptr, "bz_fc_fused: null descriptor");
   const bz_fc_desc& d = *desc;
-  BZ_REQUIRE((d.a || d.a_pieces) && d.w && (d.y || d.head_n > 0), "bz_fc_fused: null a/w/y");
+  BZ_REQUIRE((d.a || d.a_pieces) && d.w && (d.y || d.head_n > 0 || d.next), "bz_fc_fused: null a/w/y");
+  BZ_REQUIRE(d.next == nullptr || d.a_pieces != nullptr, "bz_fc_fused: a second layer (next) only follows a layer on a_pieces");
   BZ_REQUIRE(d.m >= 0 && d.n > 0 && d.k > 0, "bz_fc_fused: bad shape m=%d n=%d k=%d", d.m, d.n, d.k);
   BZ_REQUIRE(d.n_split >= 0 && (d.n_split == 0 || (d.n % d.n_split == 0 && d.y_split_stride >= 0)),
              "bz_fc_fused: n_split=%d must divide n=%d", d.n_split, d.n);
@@ -1024,7 +1025,7 @@ int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream) {
   const bool vec_w = ((uintptr_t)d.w % 16 == 0) && ((d.ldw * es) % 16 == 0);
   hipStream_t st = bz::as_stream(stream);
   if (d.a_pieces != nullptr) {
-    if (d.head_n != 0 || d.n_split != 0 || d.bias_rows > 1 || d.act == BZ_ACT_SOFTMAX || es != 2 || !vec_w)
+    if ((d.head_n != 0 && d.next == nullptr) || d.n_split != 0 || d.bias_rows > 1 || d.act == BZ_ACT_SOFTMAX || es != 2 || !vec_w)
       return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces take a 2-byte layer with aligned weight rows, no head, no split outputs, no softmax and a per-column bias");
     return bz::fc_pieces_launch(d, ep, st);
   }

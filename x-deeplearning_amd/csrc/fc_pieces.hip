@@ -35,11 +35,30 @@ using namespace bz::fc;
 // result is the two-launch form's up to the order of the K sum.
 constexpr int kPiecesBM = 128, kPiecesKS = 14, kPiecesMaxN = 96;
 
+// the layers that follow in the same launch (bz_fc_desc.next, head_*)
+struct ChainArgs {
+  const char* w2;      // [n2, ldw2]
+  void* y2;            // [M, ldy2] or null
+  int64_t ldw2, ldy2;
+  int n2;              // 9..64
+  Epilogue ep2;
+  const char* w3;      // [n3, ldw3] or null
+  const float* bias3;
+  void* y3;            // [M, ldy3]
+  int64_t ldw3, ldy3;
+  int n3, act3, y3_dtype;  // n3 = 0: no third layer
+};
+constexpr int kChainKS = kPiecesMaxN / 16;  // K steps of the second layer (its K is the first layer's N)
+
 // XY4: the pieces are exactly [x, y, x - y, x * y] of two operands (the attention input): a lane loads x and y once and
 // makes all four from them, instead of addressing and loading eight operands.
-template <int DT, typename OutT, int VEC, int NP, int TN, bool XY4>
+// CHAIN: a wave goes on with its 32 rows through a second layer of at most 64 columns and a skinny third one; what the
+// layers hand each other is rounded to the tensor type and staged in the wave's rows of LDS, where the separate launches
+// would have stored it and read it back.
+template <int DT, typename OutT, int VEC, int NP, int TN, bool XY4, bool CHAIN>
 __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const char* __restrict__ W, OutT* __restrict__ Y, int M,
-                                                              int N, int K, int64_t ldw, int64_t ldy, bool stage_y, Epilogue ep) {
+                                                              int N, int K, int64_t ldw, int64_t ldy, bool stage_y, Epilogue ep,
+                                                              ChainArgs ch) {
   using T = In<DT>;
   using ET = typename std::conditional<DT == BZ_F16, __half, __hip_bfloat16>::type;
   using Pack = bz::CewPack<ET, VEC>;
@@ -178,10 +197,14 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
         float v = ep.alpha * acc[j][r];
         if (ep.bias_rows == 1) v += ep.beta * cbias[j];
         v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
-        if (stage_y)
+        if (CHAIN) {
+          store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, n < N ? v : 0.f);  // the next layer's operand: zero beyond N
+          if (!stage_y && Y != nullptr && m < M && n < N) store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+        } else if (stage_y) {
           store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, v);
-        else if (m < M && n < N)
+        } else if (m < M && n < N) {
           store_out<OutT>(Y + (int64_t)m * ldy + n, v);
+        }
       }
     }
   };
@@ -202,19 +225,161 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
       epilogue(std::integral_constant<int, BZ_ACT_NONE>());
       break;
   }
-  if (stage_y) {
+  if (stage_y && Y != nullptr) {
     const int ocpr = N * OS / 16;  // 16-byte chunks per output row (N * OS is a multiple of 16 when stage_y)
     for (int q = lane; q < 32 * ocpr; q += 64) {
-      const int ml = q / ocpr, ch = q - ml * ocpr;
+      const int ml = q / ocpr, c16 = q - ml * ocpr;
       const int m = m0 + wave * 32 + ml;
-      if (m < M) *(uint4*)((char*)(Y + (int64_t)m * ldy) + ch * 16) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+      if (m < M) *(uint4*)((char*)(Y + (int64_t)m * ldy) + c16 * 16) = *(const uint4*)(lout + ml * OPITCH + c16 * 16);
+    }
+  }
+  if constexpr (CHAIN) {
+    static_assert(!CHAIN || sizeof(OutT) == 2, "the layers hand each other the operand type");
+    // ---- second layer: A = the staged rows [32, N] (K2 = N), W2 as fragments, at most two column blocks
+    const int KS2 = (N + 15) / 16;
+    uint4 wf2[2][kChainKS];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      int n2 = j * 32 + frow;
+      n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
+      const char* wrow = ch.w2 + (int64_t)n2 * ch.ldw2 * 2;
+#pragma unroll
+      for (int ks = 0; ks < kChainKS; ++ks) {
+        const int k0 = ks * 16 + fhalf * 8;
+        wf2[j][ks] = (ks < KS2 && k0 < ch.ldw2) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
+      }
+    }
+    float b2[2], q0[2], q1[2], q2[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      int n2 = j * 32 + frow;
+      n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
+      b2[j] = ch.ep2.bias_rows == 1 ? ch.ep2.bias[n2] : 0.f;
+      q0[j] = q1[j] = q2[j] = 0.f;
+      if (ch.ep2.act == BZ_ACT_PRELU) q0[j] = ch.ep2.p0[ch.ep2.act_size == 1 ? 0 : n2];
+      if (ch.ep2.act == BZ_ACT_DICE) {
+        q0[j] = ch.ep2.p0[n2];
+        q1[j] = ch.ep2.p1[n2];
+        q2[j] = dice_inv_den(ch.ep2, ch.ep2.p2[n2]);
+      }
+    }
+    floatx16 acc2[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[j][r] = 0.f;
+    const char* a2 = lout + frow * OPITCH + fhalf * 16;
+#pragma unroll
+    for (int ks = 0; ks < kChainKS; ++ks) {
+      if (ks < KS2) {
+        const uint4 cur = *(const uint4*)(a2 + ks * 32);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) T::mma(cur, wf2[j][ks], acc2[j]);
+      }
+    }
+    // its activated output, staged over the first layer's (every read of that has been consumed by the MFMAs above)
+    constexpr int OPITCH2 = 64 * 2 + 16;
+    auto epilogue2 = [&](auto act_c) {
+      constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int n2 = j * 32 + frow;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int ml = 8 * (r >> 2) + 4 * fhalf + (r & 3);
+          float v = ch.ep2.alpha * acc2[j][r];
+          if (ch.ep2.bias_rows == 1) v += ch.ep2.beta * b2[j];
+          v = apply_act_t<ACT>(v, ch.ep2, q0[j], q1[j], q2[j]);
+          store_out<OutT>((OutT*)(lout + ml * OPITCH2) + n2, n2 < ch.n2 ? v : 0.f);
+        }
+      }
+    };
+    switch (ch.ep2.act) {
+      case BZ_ACT_PRELU:
+        epilogue2(std::integral_constant<int, BZ_ACT_PRELU>());
+        break;
+      case BZ_ACT_DICE:
+        epilogue2(std::integral_constant<int, BZ_ACT_DICE>());
+        break;
+      case BZ_ACT_LEAKY_RELU:
+        epilogue2(std::integral_constant<int, BZ_ACT_LEAKY_RELU>());
+        break;
+      case BZ_ACT_SIGMOID:
+        epilogue2(std::integral_constant<int, BZ_ACT_SIGMOID>());
+        break;
+      default:
+        epilogue2(std::integral_constant<int, BZ_ACT_NONE>());
+        break;
+    }
+    if (ch.y2 != nullptr) {
+      for (int q = lane; q < 32 * ch.n2; q += 64) {
+        const int ml = q / ch.n2, n2 = q - ml * ch.n2;
+        const int m = m0 + wave * 32 + ml;
+        if (m < M) ((OutT*)ch.y2)[(int64_t)m * ch.ldy2 + n2] = ((const OutT*)(lout + ml * OPITCH2))[n2];
+      }
+    }
+    // ---- skinny third layer: two lanes a row, 32 columns each, from the rounded staged tile
+    if (ch.n3 > 0) {
+      const int ml = lane >> 1, hx = lane & 1;
+      const int m = m0 + wave * 32 + ml;
+      float hacc[kSkinnyMaxN];
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] = 0.f;
+      for (int c = hx * 32; c < hx * 32 + 32 && c < ch.n2; ++c) {
+        const float yv = bz::ldv<ET>((const ET*)(lout + ml * OPITCH2) + c);
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j)
+          if (j < ch.n3) hacc[j] = fmaf(yv, bz::ldv<ET>((const ET*)ch.w3 + (int64_t)j * ch.ldw3 + c), hacc[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] += __shfl_xor(hacc[j], 1, 64);
+      if (hx == 0 && m < M) {
+        float v[kSkinnyMaxN];
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j) v[j] = (j < ch.n3) ? hacc[j] + (ch.bias3 ? ch.bias3[j] : 0.f) : 0.f;
+        if (ch.act3 == BZ_ACT_SOFTMAX) {  // softmax_op.cc:21-78: subtract max, exp, sum in order, divide
+          float mx = v[0];
+#pragma unroll
+          for (int j = 1; j < kSkinnyMaxN; ++j)
+            if (j < ch.n3) mx = v[j] > mx ? v[j] : mx;
+          float sum = 0.f;
+#pragma unroll
+          for (int j = 0; j < kSkinnyMaxN; ++j)
+            if (j < ch.n3) {
+              v[j] = expf(v[j] - mx);
+              sum += v[j];
+            }
+#pragma unroll
+          for (int j = 0; j < kSkinnyMaxN; ++j)
+            if (j < ch.n3) v[j] = v[j] / sum;
+        } else if (ch.act3 == BZ_ACT_SIGMOID) {
+#pragma unroll
+          for (int j = 0; j < kSkinnyMaxN; ++j) {
+            const float t = expf(v[j]);
+            v[j] = t / (1.f + t);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < kSkinnyMaxN; ++j) {
+          if (j < ch.n3) {
+            const int64_t at = (int64_t)m * ch.ldy3 + j;
+            if (ch.y3_dtype == BZ_F32)
+              store_out<float>((float*)ch.y3 + at, v[j]);
+            else if (ch.y3_dtype == BZ_F16)
+              store_out<__half>((__half*)ch.y3 + at, v[j]);
+            else
+              store_out<__hip_bfloat16>((__hip_bfloat16*)ch.y3 + at, v[j]);
+          }
+        }
+      }
     }
   }
 }
 
 // A from pieces (bz_fc_desc.a_pieces).  BZ_ENOTSUP, with nothing launched, for anything outside the kernel's model.
-template <int DT, typename OutT, int VEC, int NP, bool XY4>
-int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep, bool stage_y, int smem, hipStream_t st) {
+template <int DT, typename OutT, int VEC, int NP, bool XY4, bool CHAIN>
+int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep, bool stage_y, int smem, const ChainArgs& ch,
+                     hipStream_t st) {
   const int grid = (d.m + kPiecesBM - 1) / kPiecesBM;
   const int tn = (d.n + 31) / 32;
 #define BZ_PIECES(TN)                                                                                                          \
@@ -226,13 +391,13 @@ int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep,
     {                                                                                                                          \
       std::lock_guard<std::mutex> lock(mu);                                                                                    \
       if (dev >= 0 && dev < 64 && !raised[dev]) {                                                                              \
-        BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4>,                                 \
+        BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4, CHAIN>,                                 \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, kPiecesBM * (kPiecesKS * 16 * 2 + 16)));     \
         raised[dev] = true;                                                                                                    \
       }                                                                                                                        \
     }                                                                                                                          \
-    hipLaunchKernelGGL((bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4>), dim3(grid), dim3(256), smem, st, p, (const char*)d.w,     \
-                       (OutT*)d.y, d.m, d.n, d.k, d.ldw, d.ldy, stage_y, ep);                                                  \
+    hipLaunchKernelGGL((bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4, CHAIN>), dim3(grid), dim3(256), smem, st, p, (const char*)d.w,     \
+                       (OutT*)d.y, d.m, d.n, d.k, d.ldw, d.ldy, stage_y, ep, ch);                                              \
   } while (0)
   if (tn == 1)
     BZ_PIECES(1);
@@ -264,8 +429,57 @@ int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
   const int pitch = kp * 2 + 16;
   const int tn = (d.n + 31) / 32;
   // 16-byte stores of whole output rows through the wave's own rows of the A tile, when they fit there
-  const bool stage_y = ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0) && (tn * 32 * os + 16 <= pitch);
+  const bool fits = tn * 32 * os + 16 <= pitch;
+  const bool stage_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0) && fits;
   const int smem = kPiecesBM * pitch;
+  ChainArgs ch = {};
+  const bool chain = d.next != nullptr;
+  if (chain) {
+    const bz_fc_next& x = *d.next;
+    BZ_REQUIRE(x.w != nullptr && (uintptr_t)x.w % 16 == 0 && x.ldw >= d.n && (x.ldw * 2) % 16 == 0,
+               "bz_fc_fused: next.w null or misaligned, or next.ldw=%lld below n=%d", (long long)x.ldw, d.n);
+    BZ_REQUIRE(x.y == nullptr || x.ldy >= x.n, "bz_fc_fused: next.ldy=%lld below next.n=%d", (long long)x.ldy, x.n);
+    BZ_REQUIRE(x.act != BZ_ACT_PRELU || (x.act_p0 && (x.act_size == 1 || x.act_size == x.n)), "bz_fc_fused: next: PRelu slope size %d", x.act_size);
+    BZ_REQUIRE(x.act != BZ_ACT_DICE || (x.act_p0 && x.act_p1 && x.act_p2), "bz_fc_fused: next: Dice needs gamma, mean and var");
+    BZ_REQUIRE(d.y != nullptr || x.y != nullptr || d.head_n > 0, "bz_fc_fused: a chain that stores nothing");
+    if (sizeof(OutT) != 2 || x.n <= kSkinnyMaxN || x.n > 64 || x.act == BZ_ACT_SOFTMAX || x.act < BZ_ACT_NONE || !fits ||
+        32 * (64 * 2 + 16) > 32 * pitch)
+      return bz::fail(BZ_ENOTSUP, "bz_fc_fused: next takes a 2-byte layer of %d < n <= 64 columns without softmax behind a first layer whose tile leaves room for it", kSkinnyMaxN);
+    ch.w2 = (const char*)x.w;
+    ch.y2 = x.y;
+    ch.ldw2 = x.ldw;
+    ch.ldy2 = x.ldy;
+    ch.n2 = x.n;
+    ch.ep2.bias = x.bias;
+    ch.ep2.bias_rows = x.bias ? 1 : 0;
+    ch.ep2.p0 = x.act_p0;
+    ch.ep2.p1 = x.act_p1;
+    ch.ep2.p2 = x.act_p2;
+    ch.ep2.act = x.act;
+    ch.ep2.act_size = x.act_size;
+    ch.ep2.dice_nosqrt = x.dice_nosqrt;
+    ch.ep2.alpha = x.alpha;
+    ch.ep2.beta = x.beta;
+    ch.ep2.act_alpha = x.act_alpha;
+    ch.ep2.split_n = 0;
+    ch.ep2.split_stride = 0;
+    if (d.head_n > 0) {
+      BZ_REQUIRE(d.head_n <= kSkinnyMaxN && d.head_w && d.head_y && d.head_ldw >= x.n && d.head_ldy >= d.head_n,
+                 "bz_fc_fused: head of %d outputs (1..%d), null head_w / head_y, or a leading dimension below its row", d.head_n, kSkinnyMaxN);
+      BZ_REQUIRE(d.head_act == BZ_ACT_NONE || d.head_act == BZ_ACT_SIGMOID || d.head_act == BZ_ACT_SOFTMAX, "bz_fc_fused: head activation %d", d.head_act);
+      BZ_REQUIRE(d.head_out_dtype == BZ_F32 || d.head_out_dtype == BZ_F16 || d.head_out_dtype == BZ_BF16, "bz_fc_fused: head out dtype %d", d.head_out_dtype);
+      ch.w3 = (const char*)d.head_w;
+      ch.bias3 = d.head_bias;
+      ch.y3 = d.head_y;
+      ch.ldw3 = d.head_ldw;
+      ch.ldy3 = d.head_ldy;
+      ch.n3 = d.head_n;
+      ch.act3 = d.head_act;
+      ch.y3_dtype = d.head_out_dtype;
+    }
+  } else if (d.y == nullptr) {
+    return bz::fail(BZ_EINVAL, "bz_fc_fused: null y");
+  }
   // (8 or 2 columns a lane; a width that allows 4 takes 2, an odd one is left to the two-launch form)
   // [x, y, x - y, x * y]: pieces 2 and 3 read exactly what pieces 0 and 1 copy
   auto same = [&](int k, bool second, int src) {
@@ -275,10 +489,19 @@ int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
   };
   const bool xy4 = p.n == 4 && p.op[0] == BZ_EW_ASSIGN && p.op[1] == BZ_EW_ASSIGN && p.op[2] == BZ_EW_SUB && p.op[3] == BZ_EW_MUL &&
                    same(2, false, 0) && same(2, true, 1) && same(3, false, 0) && same(3, true, 1);
-  if (vec == 8) return xy4 ? launch_pieces_tn<DT, OutT, 8, 4, true>(d, p, ep, stage_y, smem, st)
-                           : launch_pieces_tn<DT, OutT, 8, 4, false>(d, p, ep, stage_y, smem, st);
-  if (vec >= 2) return xy4 ? launch_pieces_tn<DT, OutT, 2, 4, true>(d, p, ep, stage_y, smem, st)
-                           : launch_pieces_tn<DT, OutT, 2, 4, false>(d, p, ep, stage_y, smem, st);
+#define BZ_PIECES_V(V)                                                                                         \
+  do {                                                                                                         \
+    if constexpr (sizeof(OutT) == 2) {                                                                         \
+      if (chain)                                                                                               \
+        return xy4 ? launch_pieces_tn<DT, OutT, V, 4, true, true>(d, p, ep, stage_y, smem, ch, st)             \
+                   : launch_pieces_tn<DT, OutT, V, 4, false, true>(d, p, ep, stage_y, smem, ch, st);           \
+    }                                                                                                          \
+    return xy4 ? launch_pieces_tn<DT, OutT, V, 4, true, false>(d, p, ep, stage_y, smem, ch, st)                \
+               : launch_pieces_tn<DT, OutT, V, 4, false, false>(d, p, ep, stage_y, smem, ch, st);              \
+  } while (0)
+  if (vec == 8) BZ_PIECES_V(8);
+  if (vec >= 2) BZ_PIECES_V(2);
+#undef BZ_PIECES_V
   return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces of odd width");
 }
 
