@@ -112,6 +112,11 @@ typedef struct bz_embed_slot {
   int32_t wg_begin;           /* filled by bz_embed_plan: first workgroup of this slot */
   int32_t wg_count;           /* filled by bz_embed_plan */
   int32_t scale_pitch;        /* bytes between the scales of consecutive rows; 0 = 4 (a dense float array) */
+  int32_t assign_pitch;       /* BZ_ASSIGN only: elements between consecutive positions of a sample; 0 = dim (the
+                                 positions of a sample are contiguous, udf_processor.h:103-131).  A larger pitch lets
+                                 several items share the rows of one [batch, trunc_num, sum of dims] tensor, each
+                                 writing its own columns */
+  int32_t reserved_;
 } bz_embed_slot;
 
 /*

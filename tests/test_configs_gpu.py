@@ -216,16 +216,17 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     din_model.feed(p, inputs, batch, np.float16)
     p.forward()
     got = {name: p.output_asnumpy(name).astype(np.float32) for name in expose + ("prob", )}
-    # eight kernel launches a forward: 2 Embedding, 2 Concat (history, main input), 3 Gemm (the whole attention MLP
-    # 216 -> 80 -> 40 -> 1 with its input [q, k, q-k, q*k] computed on the fly; the two launches of the main MLP, each
-    # with its Dice / skinny layer / softmax folded in), 1 MatMul (with the Mul and the ReduceSum)
+    # seven kernel launches a forward: 2 Embedding (the history one writes its three blocks straight into the history
+    # Concat's output; that Concat does not run), 1 Concat (main input), 3 Gemm (the whole attention MLP 216 -> 80 -> 40 -> 1
+    # with its input [q, k, q-k, q*k] computed on the fly; the two launches of the main MLP, each with its Dice / skinny
+    # layer / softmax folded in), 1 MatMul (with the Mul and the ReduceSum)
     import json
     p.register_observers(["profile"])
     p.forward()
     ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
     launching = [e for e in ev if e["name"].split(":")[0] not in ("ConstantFill", "Reshape")]
     kinds = sorted(e["name"].split(":")[0] for e in launching)
-    assert kinds == ["Concat"] * 2 + ["Embedding"] * 2 + ["Gemm"] * 3 + ["MatMul"], kinds
+    assert kinds == ["Concat"] + ["Embedding"] * 2 + ["Gemm"] * 3 + ["MatMul"], kinds
     assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
     for k, t in zip(din_model.KINDS, tables):
@@ -399,3 +400,33 @@ def test_attention_mlp_in_one_launch_equals_layer_by_layer():
         assert s1.shape == (b, cfg.T, 1) and s1.any()
         np.testing.assert_allclose(s1, s0, rtol=0, atol=4e-3 * max(1.0, float(np.abs(s0).max())))
         np.testing.assert_allclose(p1, p0, rtol=2e-3, atol=2e-3)
+
+
+def test_history_blocks_written_into_their_concat_equal_the_copy():
+    """Embedding kAssign blocks [batch, T * D] -> Reshape [batch, T, D] -> Concat(axis 2): the Embedding writes each block at
+    its columns of the Concat's output (interleave_assign_blocks, on by default) and neither the Reshapes nor the Concat
+    run; with the switch off the Concat copies.  Same bits either way, also when the batch changes between forwards."""
+    import json
+    import din_model
+    cfg = din_model.Config3(batch=64, rows=3000, T=12)
+    small = din_model.Config3(batch=9, rows=3000, T=12)
+    big = din_model.Config3(batch=130, rows=3000, T=12)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=1), big.batch_inputs(seed_offset=2), cfg.batch_inputs(seed_offset=3)]
+    outs = {}
+    for alias in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("his", "hsum", "att"), net_args={"interleave_assign_blocks": alias})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append({k: p.output_asnumpy(k).copy() for k in ("his", "hsum", "att", "prob")})
+        ran = [e["name"] for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        assert ("Concat:concat_his" in ran) == (alias == 0), ran
+        outs[alias] = got
+    for g1, g0, b in zip(outs[1], outs[0], (64, 9, 130, 64)):
+        assert g1["his"].shape == (b, cfg.T, 3 * cfg.dim) and g1["his"].any()
+        for k in g1:
+            np.testing.assert_array_equal(g1[k], g0[k], err_msg=k)

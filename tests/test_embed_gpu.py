@@ -189,6 +189,57 @@ def test_pooling_random_bit_exact(bz, oracle, kind, out_dtype, with_keys, fused_
         assert np.array_equal(_bits(got)[written], _bits(want16)[written])
 
 
+@pytest.mark.parametrize("kind,out_dtype", [("f16", np.float16), ("f32", np.float32), ("i8", np.float16)])
+@pytest.mark.parametrize("tdir", [0, 1])
+def test_assign_items_share_the_rows_of_one_history_tensor(bz, oracle, kind, out_dtype, tdir):
+    """bz_embed_slot.assign_pitch: three kAssign items of dims 18, 7 and 32 write their positions at columns 0, 18 and 25
+    of one [batch, T, 57 + 2] tensor (out_stride = T * pitch, assign_pitch = pitch).  Bit-equal to the oracle's contiguous
+    [batch, T * dim] blocks moved there; the two spare columns of every position stay untouched."""
+    import torch
+    rng = np.random.default_rng(77 + tdir + len(kind))
+    batch, T = 201, 9
+    dims = [18, 7, 32]
+    pitch = sum(dims) + 2
+    tdt = torch.float32 if out_dtype == np.float32 else torch.float16
+    out = torch.full((batch, T * pitch), float("nan"), dtype=tdt, device="cuda")
+    want = np.full((batch, T, pitch), np.nan, np.float32)
+    items, col = [], 0
+    keep = []
+    for dim in dims:
+        rows = int(rng.integers(30, 200))
+        t = _make_table(rng, kind, rows, dim, False)
+        seg = rng.integers(0, 2 * T, batch).astype(np.int32)
+        seg[rng.integers(0, batch, 15)] = 0
+        nnz = int(seg.sum())
+        ids = rng.integers(-3, rows + 3, nnz).astype(np.int64)
+        vals = rng.standard_normal(nnz).astype(np.float32)
+        dt = bz.DeviceTable(t["data"], scale=t.get("scale"))
+        keep.append(dt)
+        items.append(dict(table=dt, ids=_dev(ids), values=_dev(vals), segments=_dev(seg), out=out, col=col, udf=2,
+                          trunc_dir=tdir, trunc_num=T, assign_pitch=pitch))
+        block = np.full((batch, T * dim), np.nan, np.float32)
+        oracle.embed_get(oracle.Table(t["data"], scale=t.get("scale")), ids, vals, seg, [(2, tdir, T, block, 0)])
+        want[:, :, col:col + dim] = block.reshape(batch, T, dim)
+        col += dim
+    print("assign_pitch kind=%s out=%s dir=%d" % (kind, out_dtype.__name__, tdir), flush=True)
+    for fused in (True, False):
+        out.fill_(float("nan"))
+        bz.EmbeddingPlan(items, fused_scan=fused).run()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy().reshape(batch, T, pitch)
+        assert np.isnan(got[:, :, col:].astype(np.float32)).all(), "wrote outside the items' columns"
+        w = want[:, :, :col]
+        assert not np.isnan(w).any()
+        assert np.array_equal(_bits(got[:, :, :col]), _bits(w.astype(out_dtype)))
+    # a pitch below the item's dim, or on a pooled item, is refused
+    bad = dict(items[0], assign_pitch=dims[0] - 1)
+    with pytest.raises(RuntimeError, match="assign_pitch"):
+        bz.EmbeddingPlan([bad])
+    bad = dict(items[0], udf=0, assign_pitch=pitch)
+    with pytest.raises(RuntimeError, match="assign_pitch"):
+        bz.EmbeddingPlan([bad])
+
+
 SPECIALISED = [("f32", 4, 1), ("f32", 16, 4), ("f32", 30, 8), ("f32", 64, 16), ("f32", 128, 32), ("f32", 250, 64),
                ("f16", 8, 1), ("f16", 16, 2), ("f16", 18, 4), ("f16", 32, 4), ("f16", 64, 8), ("f16", 100, 16),
                ("f16", 200, 32), ("f16", 512, 64), ("i8", 16, 1), ("i8", 64, 4), ("i8", 100, 8), ("i8", 1000, 64)]

@@ -35,7 +35,8 @@ class EmbedSlot(C.Structure):
                 ("offsets", C.c_void_p), ("out", C.c_void_p), ("rows", C.c_int64), ("out_stride", C.c_int64),
                 ("nnz", C.c_int64), ("hash_bucket_size", C.c_uint32), ("pitch", C.c_int32), ("dim", C.c_int32), ("table_dtype", C.c_int32),
                 ("out_dtype", C.c_int32), ("udf", C.c_int32), ("trunc_dir", C.c_int32), ("trunc_num", C.c_int32),
-                ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("scale_pitch", C.c_int32)]
+                ("batch", C.c_int32), ("wg_begin", C.c_int32), ("wg_count", C.c_int32), ("scale_pitch", C.c_int32),
+                ("assign_pitch", C.c_int32), ("reserved_", C.c_int32)]
 
 
 class EmbedLaunch(C.Structure):
@@ -330,6 +331,7 @@ class EmbeddingPlan:
             s.udf = it.get("udf", SUM)
             s.trunc_dir = it.get("trunc_dir", REVERSE)
             s.trunc_num = it.get("trunc_num", 0)
+            s.assign_pitch = it.get("assign_pitch", 0)
             s.batch = batch
         self.launch = EmbedLaunch()
         check(lib().bz_embed_plan(arr, n, C.byref(self.launch)))

@@ -15,9 +15,33 @@ namespace blaze {
 using store::SparsePuller;
 
 template <class Context>
-class EmbeddingOp final : public Operator<Context> {
+class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
+
+  bool AssignBlock(int idx, int* trunc_num, int* dim) const override {
+    if (idx < 0 || (size_t)idx >= config_.block_config.size()) return false;
+    const auto& items = config_.block_config[idx].embedding_block_config_item;
+    if (items.size() != 1 || items[0].udf_type != kAssign || items[0].trunc_num <= 0) return false;
+    auto it = fg_config_idx_.find(items[0].feature_group);
+    if (it == fg_config_idx_.end()) return false;
+    *trunc_num = items[0].trunc_num;
+    *dim = config_.feature_group_config[it->second].dim;
+    return *dim > 0;
+  }
+  void InterleaveInto(const std::vector<int>& blocks, Blob* target) override {
+    Interleaved g;
+    g.target = target;
+    g.blocks = blocks;
+    int t = 0, d = 0;
+    for (int b : blocks) {
+      BLAZE_CONDITION_THROW(AssignBlock(b, &t, &d) && (g.trunc_num == 0 || g.trunc_num == t), "block ", b, " is no kAssign item of ", g.trunc_num, " positions");
+      g.trunc_num = t;
+      g.col.push_back(g.total);
+      g.total += d;
+    }
+    interleaved_.push_back(g);
+  }
 
   EmbeddingOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
     sparse_puller_ = workspace->GetSparsePuller();
@@ -125,6 +149,7 @@ class EmbeddingOp final : public Operator<Context> {
   // output blocks: [batch, stride]; all groups of a block must agree on the batch (embedding_op.h:155-184)
   void Setup() {
     needs_zero_.assign(config_.block_config.size(), false);
+    for (auto& g : interleaved_) g.shaped = false;
     for (size_t i = 0; i < config_.block_config.size(); ++i) {
       size_t batch = 0;
       bool first = true;
@@ -137,8 +162,40 @@ class EmbeddingOp final : public Operator<Context> {
         first = false;
       }
       Blob* out = this->Output((int)i);
+      int slot = 0;
+      if (Interleaved* g = GroupOf((int)i, &slot)) {
+        // lives in the group's tensor: the block keeps its shape for whoever asks, and no memory
+        out->SetShapeOnly({(TIndex)batch, (TIndex)config_.block_config[i].stride});
+        BLAZE_CONDITION_THROW(!g->shaped || (TIndex)batch == g->batch, "blocks of one history tensor with ", batch, " and ", g->batch,
+                              " samples");
+        if (!g->shaped) {
+          g->shaped = true;
+          g->batch = (TIndex)batch;
+          g->target->set_data_type((DataType)out->data_type());
+          g->target->Reshape({(TIndex)batch, (TIndex)g->trunc_num, (TIndex)g->total});
+        }
+        continue;
+      }
       out->Reshape({(TIndex)batch, (TIndex)config_.block_config[i].stride});
     }
+  }
+  struct Interleaved {
+    Blob* target = nullptr;
+    std::vector<int> blocks;   // in column order
+    std::vector<TIndex> col;   // first column of each
+    TIndex total = 0;          // columns of a position
+    int trunc_num = 0;
+    TIndex batch = 0;          // samples of the run being set up, once `shaped`
+    bool shaped = false;
+  };
+  Interleaved* GroupOf(int block, int* slot) {
+    for (auto& g : interleaved_)
+      for (size_t k = 0; k < g.blocks.size(); ++k)
+        if (g.blocks[k] == block) {
+          *slot = (int)k;
+          return &g;
+        }
+    return nullptr;
   }
 
   TIndex StaticOutputCols(int idx) const override {
@@ -193,9 +250,18 @@ class EmbeddingOp final : public Operator<Context> {
         in.in_item[j].trunc_num = item.trunc_num;
         Blob* block = this->Output(bi.block_idx);
         out.out_type = block->data_type();
+        int slot = 0;
+        if (Interleaved* g = GroupOf(bi.block_idx, &slot)) {
+          // position p of sample b at row b * T + p of the group's tensor, columns col .. col + dim
+          out.out_item[j].out = (char*)g->target->data() + g->col[slot] * DataTypeSize(block->data_type());
+          out.out_item[j].stride = (size_t)(g->trunc_num * g->total);
+          out.out_item[j].assign_pitch = (size_t)g->total;
+          continue;
+        }
         out.out_item[j].out = (char*)block->data() + item.offset * DataTypeSize(block->data_type());
         // a block that lives inside a Concat's output has that tensor's row pitch
         out.out_item[j].stride = block->pitch() ? (int)block->pitch() : config_.block_config[bi.block_idx].stride;
+        out.out_item[j].assign_pitch = 0;
       }
     }
     hipStream_t st = context_.hip_stream();
@@ -203,7 +269,13 @@ class EmbeddingOp final : public Operator<Context> {
       if (needs_zero_[b]) {
         Blob* block = this->Output((int)b);
         const size_t es = DataTypeSize(block->data_type());
-        if (block->pitch())
+        int slot = 0;
+        if (Interleaved* g = GroupOf((int)b, &slot)) {
+          int t = 0, d = 0;
+          AssignBlock((int)b, &t, &d);
+          HIP_CHECK(hipMemset2DAsync((char*)g->target->data() + g->col[slot] * es, g->total * es, 0, d * es,
+                                     (size_t)(g->batch * g->trunc_num), st));
+        } else if (block->pitch())
           HIP_CHECK(hipMemset2DAsync(block->data(), block->pitch() * es, 0, block->shape()[1] * es, block->shape()[0], st));
         else
           HIP_CHECK(hipMemsetAsync(block->data(), 0, block->size() * es, st));
@@ -218,6 +290,7 @@ class EmbeddingOp final : public Operator<Context> {
   std::unordered_map<std::string, size_t> input_fg_idx_;    // feature group -> input triple index
   std::unordered_map<std::string, size_t> fg_config_idx_;   // feature group -> config index
   std::vector<bool> needs_zero_;
+  std::vector<Interleaved> interleaved_;
   std::vector<store::SparsePullerInput> puller_in_;    // reused every run (RunEmbedding)
   std::vector<store::SparsePullerOutput> puller_out_;
   std::vector<int> fg_input_;  // feature group -> position of its triple among the inputs, -1 = not fed

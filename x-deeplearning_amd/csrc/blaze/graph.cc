@@ -215,6 +215,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     FuseFcHeads();
     PackSiblingFcs();
     AliasConcatInputs();
+    InterleaveAssignBlocks();
     FuseConcatPieces();
     FuseWeightedPools();
     FuseConcatsIntoFcs();
@@ -471,6 +472,77 @@ void SimpleNet::FuseConcatPieces() {
       host->AdoptProducer(i, operators_[producer[i]].get(), producer[i]);
       skipped_[producer[i]] = true;
     }
+  }
+}
+
+// Embedding kAssign blocks -> Reshape [batch, T, D] -> Concat(axis 2): the Embedding writes into the Concat's output
+// (graph.h, AssignInterleaver).  Every tensor on the way is read by nothing else and is no output of the net; each
+// Reshape's target is a constant [-1 | 0, T, D_i] with the block's own T and D_i.  Switch: interleave_assign_blocks: 0.
+void SimpleNet::InterleaveAssignBlocks() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "interleave_assign_blocks");
+  if (arg && arg->has_i && arg->i == 0) return;
+  auto readers_of = [&](const std::string& name) {
+    int readers = 0;
+    for (size_t j = 0; j < operators_.size(); ++j)
+      for (const auto& in : operators_[j]->operator_def().input()) readers += (in == name);
+    for (const auto& eo : external_output_) readers += (eo == name);
+    return readers;
+  };
+  auto producer_of = [&](const std::string& name, size_t before, int* out_idx) {
+    for (size_t j = before; j-- > 0;) {
+      const OperatorDef& pd = operators_[j]->operator_def();
+      for (int o = 0; o < pd.output_size(); ++o)
+        if (pd.output(o) == name) {
+          *out_idx = o;
+          return (int)j;
+        }
+    }
+    return -1;
+  };
+  for (size_t c = 0; c < operators_.size(); ++c) {
+    if (skipped_[c] || operators_[c]->type() != "Concat") continue;
+    const OperatorDef& cd = operators_[c]->operator_def();
+    if (ArgumentHelper::GetSingle<int>(cd.arg(), "axis", 1) != 2 || cd.input_size() < 2 || cd.output_size() != 1) continue;
+    int emb = -1, T = 0;
+    std::vector<int> blocks, reshapes;
+    bool ok = true;
+    for (int i = 0; i < cd.input_size() && ok; ++i) {
+      int o = 0, eo = 0, fo = 0;
+      const int r = readers_of(cd.input(i)) == 1 ? producer_of(cd.input(i), c, &o) : -1;
+      if (r < 0 || skipped_[r] || operators_[r]->type() != "Reshape") {
+        ok = false;
+        break;
+      }
+      const OperatorDef& rd = operators_[r]->operator_def();
+      const int e = rd.input_size() == 2 && readers_of(rd.input(0)) == 1 && rd.output(0) != rd.input(0) ? producer_of(rd.input(0), r, &eo) : -1;
+      const int f = rd.input_size() == 2 ? producer_of(rd.input(1), operators_.size(), &fo) : -1;
+      auto* host = e >= 0 && !skipped_[e] ? dynamic_cast<AssignInterleaver*>(operators_[e].get()) : nullptr;
+      int t = 0, d = 0;
+      std::vector<int> target;
+      if (f >= 0 && operators_[f]->type() == "ConstantFill" && workspace_->HasConstantBlob(rd.input(1)))
+        target = ArgumentHelper::GetRepeated<int>(operators_[f]->operator_def().arg(), "value");
+      if (!host || (emb >= 0 && e != emb) || !host->AssignBlock(eo, &t, &d) || (T != 0 && t != T) || target.size() != 3 ||
+          target[0] > 0 || target[1] != t || target[2] != d || std::find(blocks.begin(), blocks.end(), eo) != blocks.end()) {
+        ok = false;
+        break;
+      }
+      emb = e;
+      T = t;
+      blocks.push_back(eo);
+      reshapes.push_back(r);
+    }
+    if (!ok) continue;
+    // the Concat's output appears earlier than before: nothing up to the Concat may touch that name
+    const std::string& out = cd.output(0);
+    for (size_t j = 0; j < c && ok; ++j) {
+      for (const auto& in : operators_[j]->operator_def().input()) ok &= (in != out);
+      for (const auto& o2 : operators_[j]->operator_def().output()) ok &= (o2 != out);
+    }
+    for (const auto& ei : external_input_) ok &= (ei != out);
+    if (!ok) continue;
+    dynamic_cast<AssignInterleaver*>(operators_[emb].get())->InterleaveInto(blocks, operators_[c]->Output(0));
+    for (int r : reshapes) skipped_[r] = true;
+    skipped_[c] = true;
   }
 }
 

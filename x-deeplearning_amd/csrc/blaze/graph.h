@@ -104,6 +104,7 @@ class SimpleNet : public Net {
   void FuseWeightedPools();
   void FuseConcatsIntoFcs();
   void ChainNarrowFcs();
+  void InterleaveAssignBlocks();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };
 
@@ -211,6 +212,19 @@ class ConcatAdopter {  // implemented by Gemm
   // nothing else does.
   virtual bool CanChainNext(OperatorBase* next) = 0;  // static part
   virtual void AdoptNext(OperatorBase* next) = 0;
+};
+
+// Embedding blocks that are each one kAssign item [batch, T * D_i] -> Reshape [batch, T, D_i] (read by nothing else) ->
+// Concat(axis 2) of exactly these, in any block order: the Embedding writes every item at its columns of the Concat's
+// output [batch, T, sum D_i] (bz_embed_slot.assign_pitch) and the Reshapes and the Concat are skipped.  Same bits: the
+// rows only land somewhere else.  DIN's history of (item, category, shop) embeddings.
+class AssignInterleaver {  // implemented by Embedding
+ public:
+  virtual ~AssignInterleaver() {}
+  // whether output block idx is a single kAssign item; its positions a sample and columns a position
+  virtual bool AssignBlock(int idx, int* trunc_num, int* dim) const = 0;
+  // blocks (in the Concat's input order) go to `target` from now on; the blocks themselves only keep their shape
+  virtual void InterleaveInto(const std::vector<int>& blocks, Blob* target) = 0;
 };
 
 // MatMul(transA) of a weight column [B, T, 1] with a history [B, T, C] whose weight is the product of two equally

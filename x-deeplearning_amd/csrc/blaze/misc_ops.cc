@@ -247,7 +247,10 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost, public 
     std::sort(producers_.begin(), producers_.end(), [](const Adopted& a, const Adopted& b) { return a.position < b.position; });
   }
   bool DescribeAsPieces(bz_concat_ew_desc* desc) override { return RunWithPieces(desc); }
+  // (0 when every input already lives in the output)
+  int LaunchesOfLastRun() const override { return launches_; }
   bool RunOnDevice() override {
+    launches_ = 0;
     if (!producers_.empty()) {
       if (RunWithPieces(nullptr)) return true;
       // shapes the one-launch form does not take: run the adopted operators after all, in net order, then copy
@@ -282,6 +285,7 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost, public 
       d.dst_pitch = (int64_t)(total * inner * es);
       d.rows = (int64_t)outer;
       BZ_CHECK(bz_concat_cols(&d, st));
+      ++launches_;
       memset(&d, 0, sizeof(d));
     };
     for (int i = 0; i < this->InputSize(); ++i) {
@@ -309,6 +313,7 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost, public 
     int input_idx;
     OperatorBase* op;
   };
+  int launches_ = 0;
   // The inputs as pieces of one bz_concat_ew launch.  False when the shapes do not fit that kernel's model (concat
   // along another axis than the last, an operand broadcast along the last axis, or row dims that do not merge into
   // two coordinates); nothing has been launched then.
@@ -416,6 +421,7 @@ class ConcatOp final : public Operator<Context>, public ConcatPieceHost, public 
       return true;
     }
     BZ_CHECK(bz_concat_ew(&d, context_.hip_stream()));
+    launches_ = 1;
     return true;
   }
 

@@ -386,6 +386,7 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
       s.offsets = nullptr;  // fused scan
       s.out = out.out_item[k].out;
       s.out_stride = (int64_t)out.out_item[k].stride;
+      s.assign_pitch = (int32_t)out.out_item[k].assign_pitch;
       s.out_dtype = out_type == kFloat ? BZ_F32 : BZ_F16;
       s.udf = (int)in.in_item[k].udf_type;
       s.trunc_dir = (int)in.in_item[k].trunc_direction;

@@ -42,6 +42,8 @@ struct SparsePullerOutput {
   struct OutItem {
     void* out = nullptr;  // block base + item offset; element type = out_type
     size_t stride = 0;    // elements between samples
+    // extension: elements between consecutive positions of a kAssign item; 0 = the group's dim (positions contiguous)
+    size_t assign_pitch = 0;
   };
   std::vector<OutItem> out_item;
   int out_type = 0;       // extension: blaze DataType of the block (kFloat or kFloat16); 0 = same as value_type

@@ -317,6 +317,9 @@ __device__ __forceinline__ void store_elems(void* dst_base, int64_t elem_off, co
   }
 }
 
+// elements between the output positions of a kassign sample
+__device__ __forceinline__ int assign_pitch(const bz_embed_slot& s) { return s.assign_pitch != 0 ? s.assign_pitch : s.dim; }
+
 // ksum / kavg for one lane: chunk `c` of the segment [start, end) of sample b.
 template <int DT>
 __device__ __forceinline__ void pool_sum(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b) {
@@ -396,13 +399,13 @@ __device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t star
       for (int i = 0; i < CE; ++i) out[i] = __fmul_rn(val, w[i]);
     }
   }
-  store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * s.dim + e0, out, nvalid, s.out_dtype);
+  store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * assign_pitch(s) + e0, out, nvalid, s.out_dtype);
 }
 
 // zero fill of one item's columns (unknown table name: quick_embedding_dict.cc:95 leaves the
 // memset block untouched)
 __device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int p, int l, int lpr) {
-  const int64_t base = b * s.out_stride + (int64_t)p * s.dim;  // p = 0 unless kassign
+  const int64_t base = b * s.out_stride + (int64_t)p * assign_pitch(s);  // p = 0 unless kassign
   for (int e = l; e < s.dim; e += lpr) {
     if (s.out_dtype == BZ_F32)
       ((float*)s.out)[base + e] = 0.f;
@@ -753,6 +756,8 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
       BZ_REQUIRE(s.trunc_num > 0 && (s.trunc_dir == BZ_ORDER || s.trunc_dir == BZ_REVERSE),
                  "slot %d: kAssign needs trunc_num > 0 and a trunc direction (trunc_num=%d dir=%d)", i, s.trunc_num,
                  s.trunc_dir);
+    BZ_REQUIRE(s.assign_pitch == 0 || (s.udf == BZ_ASSIGN && s.assign_pitch >= s.dim),
+               "slot %d: assign_pitch=%d is for kAssign items and at least dim=%d", i, s.assign_pitch, s.dim);
     BZ_REQUIRE(s.out != nullptr && (s.batch == 0 || s.segments != nullptr), "slot %d: null out/segments", i);
     if (s.table != nullptr) {
       const int esz = bz::dtype_size(s.table_dtype);
