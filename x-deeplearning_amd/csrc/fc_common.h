@@ -92,13 +92,15 @@ __device__ __forceinline__ float apply_act_regs(float v, const Epilogue& e, floa
   }
 }
 
-// 1 / (the Dice denominator of a column): computed once per column, before the K loop
+// log2(e) / (the Dice denominator of a column): computed once per column, before the K loop
 __device__ __forceinline__ float dice_inv_den(const Epilogue& e, float var) {
-  return 1.f / (e.dice_nosqrt ? var : sqrtf(var + kDiceEps));
+  return 1.44269504088896341f / (e.dice_nosqrt ? var : sqrtf(var + kDiceEps));
 }
 
 // The tile kernels' epilogue, activation fixed at compile time.  For Dice p2 is dice_inv_den() of the column, not its
-// variance: a lane applies the activation to 32..128 outputs one after the other with one or two waves on its SIMD, so
+// variance, and the element costs five plain instructions, one v_exp_f32 and one v_rcp_f32 (the attention MLP applies
+// Dice to 120 outputs a history position: at 51200 x 50 positions the activation arithmetic alone is microseconds of
+// every SIMD): a lane applies the activation to 32..128 outputs one after the other with one or two waves on its SIMD, so
 // the exact expf and the two divisions per element (some 80 dependent instructions) were a third to a half of the run
 // time of the attention layers (51200 x 216 -> 80: 23.6 us with Dice, 13.2 without).  v_exp_f32 and v_rcp_f32 are
 // good to about 1 ulp of fp32 each; what they change in the result is far below the rounding of a 2-byte output and
@@ -108,9 +110,9 @@ __device__ __forceinline__ float apply_act_t(float v, const Epilogue& e, float p
   if constexpr (ACT == BZ_ACT_PRELU) {
     return v * ((float)(v > 0.f) + (float)(v < 0.f) * p0);
   } else if constexpr (ACT == BZ_ACT_DICE) {
-    const float t = __expf((p1 - v) * p2);
+    const float t = __builtin_amdgcn_exp2f((p1 - v) * p2);  // e^((mean - v) / den)
     const float p = __builtin_amdgcn_rcpf(1.f + t);
-    return (1.f - p) * p0 * v + p * v;
+    return fmaf(p, 1.f - p0, p0) * v;  // ((1 - p) gamma + p) v; 1 - gamma is the column's, hoisted out of the rows
   } else if constexpr (ACT == BZ_ACT_LEAKY_RELU) {
     return v >= 0.f ? v : e.act_alpha * v;
   } else if constexpr (ACT == BZ_ACT_SIGMOID) {

@@ -45,6 +45,19 @@ __device__ __forceinline__ uint4 load_chunk(const char* base, int64_t row, int64
   const char* p = base + (row * ld + k) * ES;
   if (vec_ok && k + CH <= K) return *(const uint4*)p;
   if constexpr (ES == 2) {
+    if (((uintptr_t)p & 3) == 0) {
+      // rows that start on 4 bytes (an even row length, e.g. a Concat of 3 x 54 columns): pairs of elements
+      uint32_t d[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        d[i] = 0u;
+        if (k + 2 * i + 1 < K)
+          d[i] = *(const uint32_t*)(p + 4 * i);
+        else if (k + 2 * i < K)
+          d[i] = *(const unsigned short*)(p + 4 * i);
+      }
+      return make_uint4(d[0], d[1], d[2], d[3]);
+    }
     unsigned short e[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) e[i] = (k + i < K) ? *(const unsigned short*)(p + 2 * i) : (unsigned short)0;
@@ -242,7 +255,7 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   for (int j = 0; j < TN; ++j) {
     int n = n0 + wn * WTN + j * 32 + (lane & 31);
     n = n < N ? n : N - 1;
-    cbias[j] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cbias[j] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
     cp0[j] = cp1[j] = cp2[j] = 0.f;
     if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
     if (ep.act == BZ_ACT_DICE) {
@@ -365,10 +378,8 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
           const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           const int m = m0 + ml;
           if (m < M && n_ok) {
-            float v = ep.alpha * acc[0][i][j][r];
-            if (ep.bias_rows == 1)
-              v += ep.beta * cbias[j];
-            else if (ep.bias_rows > 1)
+            float v = fmaf(ep.alpha, acc[0][i][j][r], cbias[j]);  // (cbias: beta * bias of the column, or 0)
+            if (ep.bias_rows > 1)
               v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
             v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
             if (HEAD || vec_y)
@@ -608,7 +619,7 @@ __global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(con
   for (int jn = 0; jn < TN; ++jn) {
     int n = n0 + wn * 64 + jn * 32 + (lane & 31);
     n = n < N ? n : N - 1;
-    cbias[jn] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cbias[jn] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
     cp0[jn] = cp1[jn] = cp2[jn] = 0.f;
     if (ep.act == BZ_ACT_PRELU) cp0[jn] = ep.p0[ep.act_size == 1 ? 0 : n];
     if (ep.act == BZ_ACT_DICE) {
@@ -684,10 +695,8 @@ __global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(con
         for (int r = 0; r < 16; ++r) {
           const int ml = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           const int m = m0 + ml;
-          float v = ep.alpha * acc[i][jn][r];
-          if (ep.bias_rows == 1)
-            v += ep.beta * cbias[jn];
-          else if (ep.bias_rows > 1 && m < M && n < N)
+          float v = fmaf(ep.alpha, acc[i][jn][r], cbias[jn]);  // (cbias: beta * bias of the column, or 0)
+          if (ep.bias_rows > 1 && m < M && n < N)
             v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
           v = apply_act_t<ACT>(v, ep, cp0[jn], cp1[jn], cp2[jn]);
           store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);

@@ -50,6 +50,15 @@ struct ChainArgs {
 };
 constexpr int kChainKS = kPiecesMaxN / 16;  // K steps of the second layer (its K is the first layer's N)
 
+// Row pitch of the A tile in LDS.  A wave stages its outputs in its own 32 rows of the tile once the MFMAs have read
+// them: a row of tn column blocks of the first layer, and of 64 two-byte columns of a chained second layer, must fit.
+__host__ __device__ inline int pieces_pitch(int k, int tn, int out_size, bool chain) {
+  int pitch = (k + 15) / 16 * 16 * 2 + 16;
+  const int o1 = tn * 32 * out_size + 16, o2 = chain ? 64 * 2 + 16 : 0;
+  pitch = pitch > o1 ? pitch : o1;
+  return pitch > o2 ? pitch : o2;
+}
+
 // XY4: the pieces are exactly [x, y, x - y, x * y] of two operands (the attention input): a lane loads x and y once and
 // makes all four from them, instead of addressing and loading eight operands.
 // CHAIN: a wave goes on with its 32 rows through a second layer of at most 64 columns and a skinny third one; what the
@@ -67,7 +76,9 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int KP = (K + 15) / 16 * 16;   // K as the MFMAs see it; columns K.. are zero
   const int KS = KP / 16;
-  const int pitch = KP * 2 + 16;       // bytes; the 16 spread the 16 rows of a ds_read_b128 phase over all banks
+  // bytes between the tile's rows: the 16 spread the 16 rows of a ds_read_b128 phase over all banks; at least what a row
+  // of the outputs staged there takes (pieces_pitch() on the host)
+  const int pitch = pieces_pitch(K, TN, (int)sizeof(OutT), CHAIN);
   const int m0 = blockIdx.x * BM;
   const int frow = lane & 31, fhalf = lane >> 5;
 
@@ -77,7 +88,7 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
   for (int j = 0; j < TN; ++j) {
     int n = j * 32 + frow;
     n = n < N ? n : N - 1;
-    cbias[j] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
+    cbias[j] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
     cp0[j] = cp1[j] = cp2[j] = 0.f;
     if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
     if (ep.act == BZ_ACT_DICE) {
@@ -87,29 +98,60 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
     }
   }
 
+  // a third layer's weight as floats [8][64] behind the tile, zero beyond its n3 rows and n2 columns
+  float* w3s = (float*)(smem + BM * pitch);
+  if constexpr (CHAIN) {
+    for (int q = tid; q < kSkinnyMaxN * 64; q += NT) {
+      const int j = q >> 6, c = q & 63;
+      w3s[q] = (j < ch.n3 && c < ch.n2) ? bz::ldv<ET>((const ET*)ch.w3 + (int64_t)j * ch.ldw3 + c) : 0.f;
+    }
+  }
+
+  // the weight, as fragments: lane (column frow of block j, half fhalf) holds k = 16*ks + 8*fhalf .. +7 of its column.
+  // Asked for right behind the first rows of the A tile's operands, before anything waits for those: the weight (from
+  // L2) and the operands (from HBM) are then one trip to memory and not one after the other.
+  uint4 wf[TN][kPiecesKS];
+  auto load_w = [&]() {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int n = j * 32 + frow;
+      n = n < N ? n : N - 1;
+      const char* wrow = W + (int64_t)n * ldw * 2;
+#pragma unroll
+      for (int ks = 0; ks < kPiecesKS; ++ks) {
+        const int k0 = ks * 16 + fhalf * 8;
+        // (rows are zero from K up to ldw, a multiple of 8: a chunk is wholly inside the row or wholly absent)
+        wf[j][ks] = (ks < KS && k0 < ldw) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+
   // the A tile: a lane owns VEC columns of a piece and walks the pieces; 64 / (W / VEC) rows share a wave.  kGenRows rows
-  // of a lane are in flight at once (no branch round the loads: a row beyond M reads row M-1 and is not stored), so the
-  // tile costs BM / (4 * rows_per_wave * kGenRows) trips to memory, not one per row.
+  // of a lane are in flight at once (no branch round the loads: a row beyond M reads row M-1 and is not stored; one
+  // beyond the tile reads the lane's first row again, a cache hit), so the tile costs BM / (4 * rows_per_wave * kGenRows)
+  // trips to memory, not one per row: one for the attention input of 4 x 54 columns.  kGenRows keeps the rows in flight
+  // within 64 registers.
   {
-    constexpr int kGenRows = 8;
+    constexpr int kGenRows = XY4 ? (VEC == 8 ? 8 : 16) : (VEC == 8 ? 2 : 8);
+    constexpr int NL = XY4 ? 2 : NP;  // operands loaded a row: x and y once, or x and y of every piece
     const int per_piece = p.col0[1] / VEC;
     const int rows_per_wave = 64 / per_piece;
     const int sub = lane / per_piece, cv = lane - sub * per_piece;
     const uint32_t r1 = (uint32_t)p.r1;
-    if (sub < rows_per_wave) {
-      const int step = 4 * rows_per_wave;
-      for (int base = wave * rows_per_wave + sub; base < BM; base += step * kGenRows) {
-        Pack xs[kGenRows][NP], ys[kGenRows][NP];
+    const int step = 4 * rows_per_wave;
+    const int base0 = wave * rows_per_wave + sub;
+    Pack xs[kGenRows][NL], ys[kGenRows][XY4 ? 1 : NP];
+    auto gen_load = [&](int base) {
 #pragma unroll
-        for (int u = 0; u < kGenRows; ++u) {
-          uint32_t row = (uint32_t)(m0 + base + u * step);
-          row = row < (uint32_t)M ? row : (uint32_t)M - 1;
-          const uint32_t i0 = row / r1, i1 = row - i0 * r1;
-          if constexpr (XY4) {
-            xs[u][0] = *(const Pack*)((const ET*)p.x[0] + (int64_t)i0 * p.xs[0][0] + (int64_t)i1 * p.xs[0][1] + cv * VEC);
-            xs[u][1] = *(const Pack*)((const ET*)p.x[1] + (int64_t)i0 * p.xs[1][0] + (int64_t)i1 * p.xs[1][1] + cv * VEC);
-            continue;
-          }
+      for (int u = 0; u < kGenRows; ++u) {
+        const int rl = base + u * step;
+        uint32_t row = (uint32_t)(m0 + (rl < BM ? rl : base));
+        row = row < (uint32_t)M ? row : (uint32_t)M - 1;
+        const uint32_t i0 = row / r1, i1 = row - i0 * r1;
+        if constexpr (XY4) {
+          xs[u][0] = *(const Pack*)((const ET*)p.x[0] + (int64_t)i0 * p.xs[0][0] + (int64_t)i1 * p.xs[0][1] + cv * VEC);
+          xs[u][1] = *(const Pack*)((const ET*)p.x[1] + (int64_t)i0 * p.xs[1][0] + (int64_t)i1 * p.xs[1][1] + cv * VEC);
+        } else {
 #pragma unroll
           for (int k = 0; k < NP; ++k) {
             const int kk = k < p.n ? k : 0;
@@ -120,20 +162,25 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
             ys[u][k] = *(const Pack*)(yb + (int64_t)i0 * ys0 + (int64_t)i1 * ys1 + cv * VEC);
           }
         }
+      }
+    };
+    auto gen_store = [&](int base) {
+      // (an opaque copy: what the loads computed per row - offsets, predicates - is worked out again here instead of
+      // being kept in registers across the weight's loads, where there are none to spare)
+      asm volatile("" : "+v"(base));
 #pragma unroll
-        for (int u = 0; u < kGenRows; ++u) {
-          const int rl = base + u * step;
-          if constexpr (XY4) {
-            if (rl < BM && m0 + rl < M) {
-              char* dst = smem + rl * pitch + cv * VEC * 2;
-              const int wb = p.col0[1] * 2;  // bytes of a piece
-              *(Pack*)dst = xs[u][0];
-              *(Pack*)(dst + wb) = xs[u][1];
-              *(Pack*)(dst + 2 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_SUB, xs[u][0], xs[u][1]);
-              *(Pack*)(dst + 3 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_MUL, xs[u][0], xs[u][1]);
-            }
-            continue;
+      for (int u = 0; u < kGenRows; ++u) {
+        const int rl = base + u * step;
+        if constexpr (XY4) {
+          if (rl < BM && m0 + rl < M) {
+            char* dst = smem + rl * pitch + cv * VEC * 2;
+            const int wb = p.col0[1] * 2;  // bytes of a piece
+            *(Pack*)dst = xs[u][0];
+            *(Pack*)(dst + wb) = xs[u][1];
+            *(Pack*)(dst + 2 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_SUB, xs[u][0], xs[u][1]);
+            *(Pack*)(dst + 3 * wb) = bz::cew_piece<ET, VEC>(BZ_EW_MUL, xs[u][0], xs[u][1]);
           }
+        } else {
 #pragma unroll
           for (int k = 0; k < NP; ++k) {
             const Pack o = bz::cew_piece<ET, VEC>(p.op[k < p.n ? k : 0], xs[u][k], ys[u][k]);
@@ -141,25 +188,21 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
           }
         }
       }
+    };
+    // (the lanes left over when the piece's width does not divide 64 load what their neighbours load and store nothing:
+    // no branch round the loads)
+    const bool mine = sub < rows_per_wave;
+    gen_load(base0);
+    load_w();
+    if (mine) gen_store(base0);
+    for (int base = base0 + step * kGenRows; base < BM; base += step * kGenRows) {
+      gen_load(base);
+      if (mine) gen_store(base);
     }
     // columns K .. KP-1 of every row
     for (int q = tid; q < BM * (KP - K); q += NT) {
       const int rl = q / (KP - K), c = K + q % (KP - K);
       *(unsigned short*)(smem + rl * pitch + c * 2) = 0;
-    }
-  }
-  // the weight, as fragments: lane (column frow of block j, half fhalf) holds k = 16*ks + 8*fhalf .. +7 of its column
-  uint4 wf[TN][kPiecesKS];
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int n = j * 32 + frow;
-    n = n < N ? n : N - 1;
-    const char* wrow = W + (int64_t)n * ldw * 2;
-#pragma unroll
-    for (int ks = 0; ks < kPiecesKS; ++ks) {
-      const int k0 = ks * 16 + fhalf * 8;
-      // (rows are zero from K up to ldw, a multiple of 8: a chunk is wholly inside the row or wholly absent)
-      wf[j][ks] = (ks < KS && k0 < ldw) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
     }
   }
   __syncthreads();
@@ -181,10 +224,35 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
     }
   }
 
+  // the second layer's weight fragments and column parameters: asked for here, so that they arrive during the first
+  // layer's epilogue (the first layer's fragments are dead from here on)
+  constexpr int TN2 = CHAIN ? 2 : 0, KS2MAX = CHAIN ? kChainKS : 0;
+  const int KS2 = (N + 15) / 16;
+  uint4 wf2[TN2 + 1][KS2MAX + 1];
+  float b2[TN2 + 1], q0[TN2 + 1], q1[TN2 + 1], q2[TN2 + 1];
+#pragma unroll
+  for (int j = 0; j < TN2; ++j) {
+    int n2 = j * 32 + frow;
+    n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
+    const char* wrow = ch.w2 + (int64_t)n2 * ch.ldw2 * 2;
+#pragma unroll
+    for (int ks = 0; ks < KS2MAX; ++ks) {
+      const int k0 = ks * 16 + fhalf * 8;
+      wf2[j][ks] = (ks < KS2 && k0 < ch.ldw2) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
+    }
+    b2[j] = ch.ep2.bias_rows == 1 ? ch.ep2.beta * ch.ep2.bias[n2] : 0.f;
+    q0[j] = q1[j] = q2[j] = 0.f;
+    if (ch.ep2.act == BZ_ACT_PRELU) q0[j] = ch.ep2.p0[ch.ep2.act_size == 1 ? 0 : n2];
+    if (ch.ep2.act == BZ_ACT_DICE) {
+      q0[j] = ch.ep2.p0[n2];
+      q1[j] = ch.ep2.p1[n2];
+      q2[j] = dice_inv_den(ch.ep2, ch.ep2.p2[n2]);
+    }
+  }
   // epilogue: lane owns column n of each block, rows 8*(r/4) + 4*(lane/32) + r%4 of the wave's 32
   constexpr int OS = (int)sizeof(OutT);
   constexpr int OPITCH = TN * 32 * OS + 16;
-  char* lout = smem + wave * 32 * pitch;  // this wave's own rows of the A tile (the host checked that the output fits)
+  char* lout = smem + wave * 32 * pitch;  // this wave's own rows of the A tile
   auto epilogue = [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
@@ -194,17 +262,10 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
       for (int r = 0; r < 16; ++r) {
         const int ml = 8 * (r >> 2) + 4 * fhalf + (r & 3);
         const int m = m0 + wave * 32 + ml;
-        float v = ep.alpha * acc[j][r];
-        if (ep.bias_rows == 1) v += ep.beta * cbias[j];
+        float v = fmaf(ep.alpha, acc[j][r], cbias[j]);  // (cbias: beta * bias of the column, or 0)
         v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
-        if (CHAIN) {
-          store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, n < N ? v : 0.f);  // the next layer's operand: zero beyond N
-          if (!stage_y && Y != nullptr && m < M && n < N) store_out<OutT>(Y + (int64_t)m * ldy + n, v);
-        } else if (stage_y) {
-          store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, v);
-        } else if (m < M && n < N) {
-          store_out<OutT>(Y + (int64_t)m * ldy + n, v);
-        }
+        // always through LDS: an address and a bounds check per element here cost more than the whole activation
+        store_out<OutT>((OutT*)(lout + ml * OPITCH) + n, (!CHAIN || n < N) ? v : 0.f);  // (a next layer's operand: zero beyond N)
       }
     }
   };
@@ -232,37 +293,16 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
       const int m = m0 + wave * 32 + ml;
       if (m < M) *(uint4*)((char*)(Y + (int64_t)m * ldy) + c16 * 16) = *(const uint4*)(lout + ml * OPITCH + c16 * 16);
     }
+  } else if (Y != nullptr) {  // rows that do not start on 16 bytes: element by element
+    for (int q = lane; q < 32 * N; q += 64) {
+      const int ml = q / N, n = q - ml * N;
+      const int m = m0 + wave * 32 + ml;
+      if (m < M) Y[(int64_t)m * ldy + n] = ((const OutT*)(lout + ml * OPITCH))[n];
+    }
   }
   if constexpr (CHAIN) {
     static_assert(!CHAIN || sizeof(OutT) == 2, "the layers hand each other the operand type");
-    // ---- second layer: A = the staged rows [32, N] (K2 = N), W2 as fragments, at most two column blocks
-    const int KS2 = (N + 15) / 16;
-    uint4 wf2[2][kChainKS];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      int n2 = j * 32 + frow;
-      n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
-      const char* wrow = ch.w2 + (int64_t)n2 * ch.ldw2 * 2;
-#pragma unroll
-      for (int ks = 0; ks < kChainKS; ++ks) {
-        const int k0 = ks * 16 + fhalf * 8;
-        wf2[j][ks] = (ks < KS2 && k0 < ch.ldw2) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
-      }
-    }
-    float b2[2], q0[2], q1[2], q2[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      int n2 = j * 32 + frow;
-      n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
-      b2[j] = ch.ep2.bias_rows == 1 ? ch.ep2.bias[n2] : 0.f;
-      q0[j] = q1[j] = q2[j] = 0.f;
-      if (ch.ep2.act == BZ_ACT_PRELU) q0[j] = ch.ep2.p0[ch.ep2.act_size == 1 ? 0 : n2];
-      if (ch.ep2.act == BZ_ACT_DICE) {
-        q0[j] = ch.ep2.p0[n2];
-        q1[j] = ch.ep2.p1[n2];
-        q2[j] = dice_inv_den(ch.ep2, ch.ep2.p2[n2]);
-      }
-    }
+    // ---- second layer: A = the staged rows [32, N] (K2 = N), at most two column blocks
     floatx16 acc2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -287,8 +327,7 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int ml = 8 * (r >> 2) + 4 * fhalf + (r & 3);
-          float v = ch.ep2.alpha * acc2[j][r];
-          if (ch.ep2.bias_rows == 1) v += ch.ep2.beta * b2[j];
+          float v = fmaf(ch.ep2.alpha, acc2[j][r], b2[j]);
           v = apply_act_t<ACT>(v, ch.ep2, q0[j], q1[j], q2[j]);
           store_out<OutT>((OutT*)(lout + ml * OPITCH2) + n2, n2 < ch.n2 ? v : 0.f);
         }
@@ -325,11 +364,39 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
       float hacc[kSkinnyMaxN];
 #pragma unroll
       for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] = 0.f;
-      for (int c = hx * 32; c < hx * 32 + 32 && c < ch.n2; ++c) {
-        const float yv = bz::ldv<ET>((const ET*)(lout + ml * OPITCH2) + c);
+      // the lane's 32 columns of its row in four 16-byte reads (columns from n2 up are zero, in the tile and in w3s);
+      // the weights come from LDS, where the workgroup put them at the start: a load from memory per column here made
+      // every wave wait 32 times
+      float yv[32];
+      const uint4* yrow = (const uint4*)(lout + ml * OPITCH2 + hx * 64);
 #pragma unroll
-        for (int j = 0; j < kSkinnyMaxN; ++j)
-          if (j < ch.n3) hacc[j] = fmaf(yv, bz::ldv<ET>((const ET*)ch.w3 + (int64_t)j * ch.ldw3 + c), hacc[j]);
+      for (int q = 0; q < 4; ++q) {
+        const uint4 raw = yrow[q];
+        const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (DT == BZ_F16) {
+            yv[8 * q + 2 * e] = __half2float(__ushort_as_half((unsigned short)(r[e] & 0xffffu)));
+            yv[8 * q + 2 * e + 1] = __half2float(__ushort_as_half((unsigned short)(r[e] >> 16)));
+          } else {  // bf16: the upper 16 bits of the fp32 pattern
+            yv[8 * q + 2 * e] = __uint_as_float(r[e] << 16);
+            yv[8 * q + 2 * e + 1] = __uint_as_float(r[e] & 0xffff0000u);
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kSkinnyMaxN; ++j) {
+        if (j < ch.n3) {
+          const float4* wj = (const float4*)(w3s + j * 64 + hx * 32);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const float4 w = wj[q];
+            hacc[j] = fmaf(yv[4 * q], w.x, hacc[j]);
+            hacc[j] = fmaf(yv[4 * q + 1], w.y, hacc[j]);
+            hacc[j] = fmaf(yv[4 * q + 2], w.z, hacc[j]);
+            hacc[j] = fmaf(yv[4 * q + 3], w.w, hacc[j]);
+          }
+        }
       }
 #pragma unroll
       for (int j = 0; j < kSkinnyMaxN; ++j) hacc[j] += __shfl_xor(hacc[j], 1, 64);
@@ -392,7 +459,8 @@ int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep,
       std::lock_guard<std::mutex> lock(mu);                                                                                    \
       if (dev >= 0 && dev < 64 && !raised[dev]) {                                                                              \
         BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4, CHAIN>,                                 \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, kPiecesBM * (kPiecesKS * 16 * 2 + 16)));     \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,                                                  \
+                                      kPiecesBM * pieces_pitch(kPiecesKS * 16, 3, 4, true) + kSkinnyMaxN * 64 * 4));     \
         raised[dev] = true;                                                                                                    \
       }                                                                                                                        \
     }                                                                                                                          \
@@ -426,12 +494,11 @@ int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
       d.m >= (1ll << 31) - kPiecesBM)
     return bz::fail(BZ_ENOTSUP, "bz_fc_fused: a_pieces take at most 4 pieces of one width without division, k <= %d, %d < n <= %d",
                     kPiecesKS * 16, kSkinnyMaxN, kPiecesMaxN);
-  const int pitch = kp * 2 + 16;
   const int tn = (d.n + 31) / 32;
-  // 16-byte stores of whole output rows through the wave's own rows of the A tile, when they fit there
-  const bool fits = tn * 32 * os + 16 <= pitch;
-  const bool stage_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0) && fits;
-  const int smem = kPiecesBM * pitch;
+  const int pitch = pieces_pitch(d.k, tn, os, d.next != nullptr);
+  // 16-byte stores of whole output rows when they are aligned for them (the outputs always go through LDS)
+  const bool stage_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0);
+  const int smem = kPiecesBM * pitch + (d.next != nullptr ? kSkinnyMaxN * 64 * 4 : 0);
   ChainArgs ch = {};
   const bool chain = d.next != nullptr;
   if (chain) {
@@ -442,9 +509,8 @@ int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
     BZ_REQUIRE(x.act != BZ_ACT_PRELU || (x.act_p0 && (x.act_size == 1 || x.act_size == x.n)), "bz_fc_fused: next: PRelu slope size %d", x.act_size);
     BZ_REQUIRE(x.act != BZ_ACT_DICE || (x.act_p0 && x.act_p1 && x.act_p2), "bz_fc_fused: next: Dice needs gamma, mean and var");
     BZ_REQUIRE(d.y != nullptr || x.y != nullptr || d.head_n > 0, "bz_fc_fused: a chain that stores nothing");
-    if (sizeof(OutT) != 2 || x.n <= kSkinnyMaxN || x.n > 64 || x.act == BZ_ACT_SOFTMAX || x.act < BZ_ACT_NONE || !fits ||
-        32 * (64 * 2 + 16) > 32 * pitch)
-      return bz::fail(BZ_ENOTSUP, "bz_fc_fused: next takes a 2-byte layer of %d < n <= 64 columns without softmax behind a first layer whose tile leaves room for it", kSkinnyMaxN);
+    if (sizeof(OutT) != 2 || x.n <= kSkinnyMaxN || x.n > 64 || x.act == BZ_ACT_SOFTMAX || x.act < BZ_ACT_NONE)
+      return bz::fail(BZ_ENOTSUP, "bz_fc_fused: next takes a 2-byte layer of %d < n <= 64 columns without softmax", kSkinnyMaxN);
     ch.w2 = (const char*)x.w;
     ch.y2 = x.y;
     ch.ldw2 = x.ldw;
