@@ -373,44 +373,76 @@ __device__ __forceinline__ void pool_sum(const bz_embed_slot& s, int64_t start, 
 
 // kassign: position p of the output holds id j = p (in order) or num - trunc + p (reverse);
 // positions without an id, and ids absent from the table, are zero (udf_processor.h:103-131).
-// One call fills chunk c of position p of sample b: the positions of a sample are independent of each other,
-// so the kernel spreads them over lane groups instead of walking them one dependent load after the other.
+// One call fills chunk c of positions p0 .. p0 + kAssignRun - 1 of sample b: the positions of a sample are independent
+// of each other, so the kernel spreads them over lane groups instead of walking them one dependent load after the
+// other, and a group keeps kAssignRun of them in flight (their ids are neighbours in memory): with one position a
+// group, DIN's 50-position histories were bounded by the four dependent trips to memory each group makes for a
+// single 36-byte row.
+constexpr int kAssignRun = 4;
+__host__ __device__ inline int64_t items_per_sample(const bz_embed_slot& s) {
+  return s.udf == BZ_ASSIGN ? (s.trunc_num + kAssignRun - 1) / kAssignRun : 1;
+}
+
 template <int DT>
-__device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b, int p) {
+__device__ __forceinline__ void pool_assign(const bz_embed_slot& s, int64_t start, int64_t end, int c, int64_t b, int p0) {
   constexpr int CE = RowTraits<DT>::kElems;
+  constexpr int R = kAssignRun;
   const int64_t num = end - start;
   const int e0 = c * CE;
   const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
   const char* table = (const char*)s.table + (int64_t)c * 16;
   const int64_t shift = (s.trunc_dir == BZ_ORDER) ? 0 : num - (int64_t)s.trunc_num;
-  const int64_t j = shift + p;
-  float out[CE];
+  // no branch round the loads: a position without an id reads id 0 of the slot (there is one whenever any position
+  // has an id) and row 0 of the table, and the result is dropped
+  bool live[R];
+  int64_t row[R];
+  float val[R];
+  uint4 raw[R];
+  float sc[R];
 #pragma unroll
-  for (int i = 0; i < CE; ++i) out[i] = 0.f;
-  if (j >= 0 && j < num) {
-    const int64_t r = resolve_row(s, s.ids[start + j]);
-    if (r >= 0) {
-      const float val = s.values[start + j];
-      const uint4 raw = *(const uint4*)(table + r * (int64_t)s.pitch);
-      const float sc = (DT == BZ_I8) ? load_scale(s, r) : 1.f;
-      float w[CE];
-      widen<DT>(raw, sc, w);
-#pragma unroll
-      for (int i = 0; i < CE; ++i) out[i] = __fmul_rn(val, w[i]);
+  for (int r = 0; r < R; ++r) {
+    const int64_t j = shift + p0 + r;
+    live[r] = p0 + r < s.trunc_num && j >= 0 && j < num;
+    const int64_t at = live[r] ? start + j : 0;
+    row[r] = -1;
+    val[r] = 0.f;
+    if (num > 0) {  // (uniform over the group's positions: they belong to one sample)
+      row[r] = resolve_row(s, s.ids[at]);
+      val[r] = s.values[at];
     }
   }
-  store_elems<CE>(s.out, b * s.out_stride + (int64_t)p * assign_pitch(s) + e0, out, nvalid, s.out_dtype);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    live[r] = live[r] && row[r] >= 0;
+    const int64_t rr = live[r] ? row[r] : 0;
+    raw[r] = *(const uint4*)(table + rr * (int64_t)s.pitch);
+    sc[r] = (DT == BZ_I8) ? load_scale(s, rr) : 1.f;
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (p0 + r < s.trunc_num) {
+      float out[CE];
+      float w[CE];
+      widen<DT>(raw[r], sc[r], w);
+#pragma unroll
+      for (int i = 0; i < CE; ++i) out[i] = live[r] ? __fmul_rn(val[r], w[i]) : 0.f;
+      store_elems<CE>(s.out, b * s.out_stride + (int64_t)(p0 + r) * assign_pitch(s) + e0, out, nvalid, s.out_dtype);
+    }
+  }
 }
 
 // zero fill of one item's columns (unknown table name: quick_embedding_dict.cc:95 leaves the
 // memset block untouched)
-__device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int p, int l, int lpr) {
-  const int64_t base = b * s.out_stride + (int64_t)p * assign_pitch(s);  // p = 0 unless kassign
-  for (int e = l; e < s.dim; e += lpr) {
-    if (s.out_dtype == BZ_F32)
-      ((float*)s.out)[base + e] = 0.f;
-    else
-      ((__half*)s.out)[base + e] = __ushort_as_half(0);
+__device__ __forceinline__ void pool_zero(const bz_embed_slot& s, int64_t b, int p0, int l, int lpr) {
+  const int run = s.udf == BZ_ASSIGN ? kAssignRun : 1;  // p0 = 0 unless kassign
+  for (int p = p0; p < p0 + run && (p == 0 || p < s.trunc_num); ++p) {
+    const int64_t base = b * s.out_stride + (int64_t)p * assign_pitch(s);
+    for (int e = l; e < s.dim; e += lpr) {
+      if (s.out_dtype == BZ_F32)
+        ((float*)s.out)[base + e] = 0.f;
+      else
+        ((__half*)s.out)[base + e] = __ushort_as_half(0);
+    }
   }
 }
 
@@ -619,8 +651,8 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   const int tid = threadIdx.x;
   const int g = tid / lpr;
   const int l = tid - g * lpr;
-  // a lane group owns one item: a sample (ksum / kavg) or one output position of a sample (kassign)
-  const int64_t per = s.udf == BZ_ASSIGN ? s.trunc_num : 1;
+  // a lane group owns one item: a sample (ksum / kavg) or kAssignRun output positions of a sample (kassign)
+  const int64_t per = items_per_sample(s);
   const int64_t n_items = (int64_t)s.batch * per;
   const int64_t i0 = (int64_t)(v - s.wg_begin) * groups;
   int64_t i_last = i0 + groups - 1;
@@ -631,7 +663,7 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   const int64_t item = i0 + g;
   if (item >= n_items) return;
   const int64_t b = item / per;
-  const int p = (int)(item - b * per);
+  const int p = (int)(item - b * per) * (s.udf == BZ_ASSIGN ? kAssignRun : 1);
   if (s.table == nullptr) {
     pool_zero(s, b, p, l, lpr);
     return;
@@ -778,7 +810,7 @@ int bz_embed_plan(bz_embed_slot* slots, int n_slots, bz_embed_launch* launch) {
     const int lpr = kThreads / g;
     const int ce = s.table_dtype == BZ_F32 ? 4 : (s.table_dtype == BZ_F16 ? 8 : 16);
     s.wg_begin = (int32_t)total;
-    const int64_t items = (int64_t)s.batch * (s.udf == BZ_ASSIGN ? s.trunc_num : 1);  // lane groups needed
+    const int64_t items = (int64_t)s.batch * items_per_sample(s);  // lane groups needed
     BZ_REQUIRE((items + g - 1) / g < (1ll << 30), "slot %d: too many workgroups", i);
     s.wg_count = (int32_t)((items + g - 1) / g);
     total += s.wg_count;
