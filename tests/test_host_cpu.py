@@ -281,8 +281,9 @@ def test_embedding_planner_geometry_and_scan_advice():
     assert launch.total_wg == 200 * 128 and launch.fused_scan == 1 and launch.scan_first == 1
     _, launch = plan(200, 8192, 64, offsets=True, nnz=20480)
     assert launch.fused_scan == 0 and launch.scan_first == 0
-    slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)   # config 3's history: 3 chunks -> 4 lanes, 128 positions per workgroup
-    assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 50 // 128] * 3
+    # config 3's history: 3 chunks -> 4 lanes a group, 128 groups a workgroup, a group takes 4 of a sample's 50 positions
+    slots, launch = plan(3, 1024, 18, udf=bz.ASSIGN, trunc=50)
+    assert launch.variant == 0 and [s.wg_count for s in slots] == [1024 * 13 // 128] * 3
 
 
 def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle):

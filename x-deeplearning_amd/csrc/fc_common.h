@@ -184,5 +184,10 @@ constexpr int kSkinnyMaxN = 8;
 // fc_pieces.hip: the layer whose A operand is given as pieces (bz_fc_desc.a_pieces); called by bz_fc_fused after its
 // argument checks
 int fc_pieces_launch(const bz_fc_desc& d, const fc::Epilogue& ep, hipStream_t st);
+// The layer on a stored A, one function per operand type (fc_fused_f16.hip, fc_fused_bf16.hip, fc_fused_f32.hip): with a
+// head when d.head_n != 0, else the skinny, tile or streaming kernel.  bz_fc_fused has checked the descriptor.
+int fc_run_f16(const bz_fc_desc& d, const fc::Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st);
+int fc_run_bf16(const bz_fc_desc& d, const fc::Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st);
+int fc_run_f32(const bz_fc_desc& d, const fc::Epilogue& ep, bool vec_a, bool vec_w, hipStream_t st);
 
 }  // namespace bz
