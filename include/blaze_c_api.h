@@ -12,9 +12,11 @@
  * the GPU; -1 = probe; 0 (CPU) fails at operator creation: this build has no CPU execution path.
  *
  * Not provided by this build (they return -1 with a message): the model importers
- * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze).  Blaze_OptimizeBlaze runs the one optimizer pass this
- * path depends on, the parallel-Gemm fusion (blaze/graph/pattern/in_parallel/parallel_gemm_fusion_pattern_impl.cc), and
- * writes the model back; the reference's other passes are not part of this build.  The text-to-QED table builders of
+ * (Blaze_PredictorManagerLoadDeepNetModel, Blaze_ConvertBlaze).  Blaze_OptimizeBlaze runs the two optimizer passes that
+ * concern this path's FC layers, the in-order Gemm -> Gemm folding
+ * (blaze/graph/pattern/in_order/gemm_gemm_fusion_pattern_impl.cc) and the parallel-Gemm fusion
+ * (blaze/graph/pattern/in_parallel/parallel_gemm_fusion_pattern_impl.cc), and writes the model back; the reference's
+ * other passes are not part of this build.  The text-to-QED table builders of
  * c_api_qed.h (Blaze_QuickEmbeddingBuildFp32/Fp16) are provided.
  */
 #ifndef BLAZE_C_API_H_

@@ -20,6 +20,8 @@ It also copies two sets of DATA files the reference holds, byte for byte:
 (the text tables of embedding_builder_test.cc:13-23), and the input / expected NetDef pair of the optimizer's
 parallel-Gemm fusion test (blaze/blaze/test/graph/pattern/in_parallel/in_parallel_gemm_test.cc):
   blaze/blaze/test/utest_data/graph/pattern/in_parallel/parallel_gemm_fusion{,_expected}.blaze               -> pattern/
+and the four pairs of its in-order Gemm -> Gemm fusion test (.../test/graph/pattern/in_order/in_order_gemm_gemm_test.cc):
+  blaze/blaze/test/utest_data/graph/pattern/in_order/in_order_gemm_gemm_fusion{,2,3,4}{,_expected}.blaze   -> pattern/
 """
 import json
 import os
@@ -180,6 +182,10 @@ def main():
     for name in ("parallel_gemm_fusion.blaze", "parallel_gemm_fusion_expected.blaze"):
         shutil.copyfile(os.path.join(root, "blaze/blaze/test/utest_data/graph/pattern/in_parallel", name),
                         os.path.join(here, "pattern", name))
+    for case in ("", "2", "3", "4"):
+        for name in ("in_order_gemm_gemm_fusion%s.blaze" % case, "in_order_gemm_gemm_fusion%s_expected.blaze" % case):
+            shutil.copyfile(os.path.join(root, "blaze/blaze/test/utest_data/graph/pattern/in_order", name),
+                            os.path.join(here, "pattern", name))
     print("copied model_blaze_optimized.bin, quick_embedding/ and pattern/")
 
 

@@ -398,6 +398,39 @@ def test_parallel_gemm_fusion_pass_on_the_reference_fixture(tmp_path):
     assert open(again, "rb").read() == open(str(tmp_path / "opt.1"), "rb").read()
 
 
+@pytest.mark.parametrize("case", ["", "2", "3", "4"])
+def test_gemm_gemm_folding_pass_on_the_reference_fixtures(tmp_path, case):
+    """Blaze_OptimizeBlaze on the four inputs of the reference's in-order Gemm -> Gemm fusion test (no bias, a bias on the
+    first, on the second, on both; blaze/blaze/test/graph/pattern/in_order/in_order_gemm_gemm_test.cc) gives the NetDefs
+    that test expects: one Gemm on the product of the weights, alpha and beta as its only arguments, the folded bias in the
+    surviving bias constant, the first Gemm and its orphaned constants gone.  Compared operator by operator in order
+    (types, names, inputs, outputs, argument names, ints exactly, floats to fp32 rounding)."""
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    from google.protobuf import text_format
+    d = os.path.join(ROOT, "tests", "golden", "pattern")
+    want = NetDef()
+    text_format.Parse(open(os.path.join(d, "in_order_gemm_gemm_fusion%s_expected.blaze" % case)).read(), want)
+    dst = str(tmp_path / "opt")
+    pb.optimize_blaze(os.path.join(d, "in_order_gemm_gemm_fusion%s.blaze" % case), dst, False)
+    got = NetDef()
+    text_format.Parse(open(dst).read(), got)
+    assert [o.type for o in got.op] == [o.type for o in want.op]
+    assert got.op[-1].type == "Gemm" and sum(o.type == "Gemm" for o in got.op) == 1
+    for a, b in zip(got.op, want.op):
+        assert (a.type, a.name, list(a.input), list(a.output)) == (b.type, b.name, list(b.input), list(b.output))
+        assert [x.name for x in a.arg] == [x.name for x in b.arg]
+        for x, y in zip(a.arg, b.arg):
+            assert (list(x.ints), x.i if x.HasField("i") else None) == (list(y.ints), y.i if y.HasField("i") else None), x.name
+            np.testing.assert_allclose(list(x.floats), list(y.floats), rtol=2e-7, atol=0, err_msg=a.name + "." + x.name)
+            assert x.HasField("f") == y.HasField("f") and (not x.HasField("f") or x.f == y.f)
+    assert [(v.name, v.dtype) for v in got.external_output] == [(v.name, v.dtype) for v in want.external_output]
+    # nothing left to fold on a second run
+    again = str(tmp_path / "again")
+    pb.optimize_blaze(dst, again, False)
+    assert open(again).read() == open(dst).read()
+
+
 def _reference_text_tables():
     """-> {table: (keys int64 [n], rows fp32 [n, dim])} of tests/golden/quick_embedding (the reference's
     utest_data/store/quick_embedding: `key,w0,...` lines; the first weight column happens to hold a big integer)."""

@@ -693,3 +693,57 @@ def test_sibling_gemms_run_as_one_launch(pb, oracle, dtype):
             np.testing.assert_allclose(y, want, rtol=tol, atol=tol)
     for (x1, y1), (x0, y0) in zip(outs[1], outs[0]):
         np.testing.assert_allclose(y1, y0, rtol=tol, atol=tol)
+
+
+def test_folded_gemm_chain_gives_the_same_outputs(pb, oracle, tmp_path):
+    """Blaze_OptimizeBlaze folds Gemm(transB, alpha, beta, bias) -> Gemm(bias) with nothing between them into one Gemm on
+    the product of the weights; the folded model gives the original's outputs (to the reassociation of fp32 sums) with one
+    FC launch instead of two.  Also the reference's four fixtures (tests/golden/pattern/in_order_gemm_gemm_fusion*.blaze,
+    constants only, moved to the device): the folded nets' outputs are those of the unfolded ones."""
+    import json
+    rng = np.random.default_rng(12)
+    M, K, H, N = 41, 24, 32, 16
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w0 = (rng.standard_normal((H, K)) / np.sqrt(K)).astype(np.float32)   # used transposed
+    w1 = (rng.standard_normal((H, N)) / np.sqrt(H)).astype(np.float32)
+    b0, b1 = (rng.standard_normal(H) * 0.1).astype(np.float32), (rng.standard_normal(N) * 0.1).astype(np.float32)
+    nb = pb.NetBuilder("chain", device_type=1)
+    nb.external_input("x", pb.K_FLOAT)
+    for name, v in (("w0", w0), ("b0", b0), ("w1", w1), ("b1", b1)):
+        nb.constant(name, v)
+    nb.op("Gemm", ["x", "w0", "b0"], ["h"], transB=1, alpha=0.5, beta=2.0)
+    nb.op("Gemm", ["h", "w1", "b1"], ["out"])
+    nb.external_output("out", pb.K_FLOAT)
+    raw, opt = str(tmp_path / "raw.blaze"), str(tmp_path / "opt.blaze")
+    open(raw, "wb").write(pb.convert_netdef(nb.text().encode(), True, False))
+    pb.optimize_blaze(raw, opt, True)
+    outs = {}
+    for path in (raw, opt):
+        pm = pb.PredictorManager()
+        pm.load_model(path)
+        p = pm.create_predictor(1, 0)
+        p.reshape_input("x", [M, K])
+        p.feed("x", x)
+        p.register_observers(["profile"])
+        p.forward()
+        outs[path] = p.output_asnumpy("out").copy()
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        kinds = [e["name"].split(":")[0] for e in ev if not e["name"].startswith("ConstantFill")]
+        assert kinds == (["Gemm"] if path == opt else ["Gemm", "Gemm"]), kinds
+    want = oracle.gemm_op(oracle.gemm_op(x, w0, b0, False, True, 0.5, 2.0), w1, b1, False, False, 1.0, 1.0)
+    np.testing.assert_allclose(outs[raw], want, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(outs[opt], want, rtol=1e-5, atol=1e-5)
+    for case in ("", "2", "3", "4"):
+        text = open(os.path.join(ROOT, "tests", "golden", "pattern", "in_order_gemm_gemm_fusion%s.blaze" % case)).read()
+        raw2, opt2 = str(tmp_path / ("raw%s.blaze" % case)), str(tmp_path / ("opt%s.blaze" % case))
+        open(raw2, "w").write(text.replace("device_type: 0", "device_type: 1"))
+        pb.optimize_blaze(raw2, opt2, False)
+        got = []
+        for path in (raw2, opt2):
+            pm = pb.PredictorManager()
+            pm.load_model(path)
+            p = pm.create_predictor(1, 0)
+            p.forward()
+            got.append(p.output_asnumpy("output").copy())
+        assert got[0].shape == (2, 3) and got[0].any()
+        np.testing.assert_allclose(got[1], got[0], rtol=1e-6, atol=0)

@@ -480,6 +480,7 @@ int Blaze_OptimizeBlaze(const char* raw_model_file, const char* optimized_model_
       Blaze_SetLastErrorString("OptimizeBlaze: %s", err.c_str());
       return -1;
     }
+    blaze::FuseGemmChains(&def);
     blaze::FuseParallelGemms(&def);
     std::string s;
     if (binary)
