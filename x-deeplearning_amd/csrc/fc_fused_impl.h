@@ -367,31 +367,42 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   constexpr int OPITCH = BN * OS + 16;
   static_assert(BM * OPITCH <= (int)sizeof(lds), "output tile must fit the operand buffers");
   char* lout = &lds[0][0];
+  // A bias of one row per sample, the rare form, is folded into the accumulators first, so that the element loop below
+  // has no index to compute and nothing to decide per element.
+  float alpha_e = ep.alpha;
+  if (ep.bias_rows > 1) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          const float b = (m < M && n < N) ? ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)] : 0.f;
+          acc[0][i][j][r] = fmaf(ep.alpha, acc[0][i][j][r], b);
+        }
+      }
+    }
+    alpha_e = 1.f;
+  }
   // The activation is a compile-time parameter of the element loop: a run-time switch per element would turn the
-  // unrolled epilogue into a string of taken branches over far more code than the loop needs.
+  // unrolled epilogue into a string of taken branches over far more code than the loop needs.  Every output goes
+  // into the LDS tile, rows and columns beyond the matrix included (they are not copied out): a bounds check and a
+  // 64-bit address per element cost several times the activation.
   auto epilogue = [&](auto act_c) {
     constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int nl = wn * WTN + j * 32 + (lane & 31);
-      const int n = n0 + nl;
-      const bool n_ok = n < N;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int ml = wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          const int m = m0 + ml;
-          if (m < M && n_ok) {
-            float v = fmaf(ep.alpha, acc[0][i][j][r], cbias[j]);  // (cbias: beta * bias of the column, or 0)
-            if (ep.bias_rows > 1)
-              v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
-            v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
-            if (HEAD || vec_y)
-              store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
-            else
-              store_out<OutT>(Y + out_index(ep, m, n, ldy), v);
-          }
+          float v = fmaf(alpha_e, acc[0][i][j][r], cbias[j]);  // (cbias: beta * bias of the column, or 0)
+          v = apply_act_t<ACT>(v, ep, cp0[j], cp1[j], cp2[j]);
+          store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
         }
       }
     }
@@ -420,20 +431,18 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
       if (q < HW_CHUNKS) *(uint4*)&lds_hw[q * 16] = rhw[i];
     }
   }
-  if (HEAD || vec_y) {
-    __syncthreads();
-    if (vec_y) {
-      constexpr int OCPR = BN * OS / 16;  // 16-byte chunks per tile row
-      for (int q = tid; q < BM * OCPR; q += NT) {
-        const int ml = q / OCPR, ch = q % OCPR;
-        const int m = m0 + ml, n = n0 + ch * (16 / OS);
-        if (m < M && n < N) *(uint4*)((char*)(Y + out_index(ep, m, n, ldy))) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
-      }
-    } else if (Y != nullptr) {  // HEAD with an output that takes no 16-byte stores
-      for (int q = tid; q < BM * BN; q += NT) {
-        const int ml = q / BN, nl = q % BN;
-        if (m0 + ml < M && n0 + nl < N) Y[(int64_t)(m0 + ml) * ldy + n0 + nl] = ((const OutT*)(lout + ml * OPITCH))[nl];
-      }
+  __syncthreads();
+  if (vec_y) {
+    constexpr int OCPR = BN * OS / 16;  // 16-byte chunks per tile row
+    for (int q = tid; q < BM * OCPR; q += NT) {
+      const int ml = q / OCPR, ch = q % OCPR;
+      const int m = m0 + ml, n = n0 + ch * (16 / OS);
+      if (m < M && n < N) *(uint4*)((char*)(Y + out_index(ep, m, n, ldy))) = *(const uint4*)(lout + ml * OPITCH + ch * 16);
+    }
+  } else if (Y != nullptr) {  // an output that takes no 16-byte stores: element by element, along rows
+    for (int q = tid; q < BM * BN; q += NT) {
+      const int ml = q / BN, nl = q % BN;
+      if (m0 + ml < M && n0 + nl < N) Y[out_index(ep, m0 + ml, n0 + nl, ldy)] = ((const OutT*)(lout + ml * OPITCH))[nl];
     }
   }
   if constexpr (HEAD) {
@@ -693,16 +702,12 @@ __global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(con
 #pragma unroll
     for (int jn = 0; jn < TN; ++jn) {
       const int nl = wn * 64 + jn * 32 + (lane & 31);
-      const int n = n0 + nl;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int ml = wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          const int m = m0 + ml;
           float v = fmaf(ep.alpha, acc[i][jn][r], cbias[jn]);  // (cbias: beta * bias of the column, or 0)
-          if (ep.bias_rows > 1 && m < M && n < N)
-            v += ep.beta * ep.bias[full_bias_index(ep, m, n, M, N)];
           v = apply_act_t<ACT>(v, ep, cp0[jn], cp1[jn], cp2[jn]);
           store_out<OutT>((OutT*)(lout + ml * OPITCH) + nl, v);
         }
@@ -913,7 +918,10 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
     const int64_t wg_stream = (int64_t)((d.m + kStreamBM - 1) / kStreamBM) * ((d.n + kStreamBN - 1) / kStreamBN);
     const bool vec_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * 2) % 16 == 0) && d.n % 8 == 0 &&
                        (d.n_split == 0 || (d.n_split % 8 == 0 && (d.y_split_stride * 2) % 16 == 0));
-    if (wg_stream >= 200 && d.k % kStreamBK == 0 && d.k >= 8 * kStreamBK && vec_y) return launch_stream<DT, OutT>(d, ep, st);
+    // (a bias of one row per sample stays with the tile kernels: the streaming kernel's epilogue handles 128 outputs a
+    // lane, and an index and a bounds check per output for that rare form cost every layer ten times the activation)
+    if (wg_stream >= 200 && d.k % kStreamBK == 0 && d.k >= 8 * kStreamBK && vec_y && d.bias_rows <= 1)
+      return launch_stream<DT, OutT>(d, ep, st);
   }
   if constexpr (sizeof(OutT) == 2) {
     // (256x256 once even that fills the chip: 4096^3 bf16 987 against 885 TFLOP/s)

@@ -49,6 +49,7 @@ struct ChainArgs {
   int n3, act3, y3_dtype;  // n3 = 0: no third layer
 };
 constexpr int kChainKS = kPiecesMaxN / 16;  // K steps of the second layer (its K is the first layer's N)
+constexpr int kChainPitch = kPiecesMaxN * 2 + 16;  // bytes between the rows of the second layer's weight in LDS
 
 // Row pitch of the A tile in LDS.  A wave stages its outputs in its own 32 rows of the tile once the MFMAs have read
 // them: a row of tn column blocks of the first layer, and of 64 two-byte columns of a chained second layer, must fit.
@@ -57,6 +58,12 @@ __host__ __device__ inline int pieces_pitch(int k, int tn, int out_size, bool ch
   const int o1 = tn * 32 * out_size + 16, o2 = chain ? 64 * 2 + 16 : 0;
   pitch = pitch > o1 ? pitch : o1;
   return pitch > o2 ? pitch : o2;
+}
+// dynamic LDS of a workgroup: the tile, the first layer's column parameters and, for a chain, the third layer's weight,
+// the second layer's column parameters and its weight
+__host__ __device__ inline int pieces_lds(int k, int tn, int out_size, bool chain) {
+  return kPiecesBM * pieces_pitch(k, tn, out_size, chain) + 4 * kPiecesMaxN * 4 +
+         (chain ? kSkinnyMaxN * 64 * 4 + 4 * 64 * 4 + 64 * kChainPitch : 0);
 }
 
 // XY4: the pieces are exactly [x, y, x - y, x * y] of two operands (the attention input): a lane loads x and y once and
@@ -82,62 +89,140 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
   const int m0 = blockIdx.x * BM;
   const int frow = lane & 31, fhalf = lane >> 5;
 
-  // per-column epilogue parameters
-  float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int n = j * 32 + frow;
-    n = n < N ? n : N - 1;
-    cbias[j] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
-    cp0[j] = cp1[j] = cp2[j] = 0.f;
-    if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
-    if (ep.act == BZ_ACT_DICE) {
-      cp0[j] = ep.p0[n];
-      cp1[j] = ep.p1[n];
-      cp2[j] = dice_inv_den(ep, ep.p2[n]);
-    }
-  }
+  // LDS behind the A tile: the layers' per-column epilogue parameters as finished floats ([4][96]: beta * bias, slope or
+  // gamma, mean, log2(e) / den; [4][64] for a second layer), a third layer's weight as floats [8][64] (zero beyond its n3
+  // rows and n2 columns) and a second layer's weight as the tile the fragment reads expect ([64] rows of kChainPitch
+  // bytes).  pieces_lds() on the host.
+  float* ps1 = (float*)(smem + BM * pitch);
+  float* w3s = ps1 + 4 * kPiecesMaxN;
+  float* ps2 = w3s + kSkinnyMaxN * 64;
+  char* w2s = (char*)(ps2 + 4 * 64);
 
-  // a third layer's weight as floats [8][64] behind the tile, zero beyond its n3 rows and n2 columns
-  float* w3s = (float*)(smem + BM * pitch);
-  if constexpr (CHAIN) {
-    for (int q = tid; q < kSkinnyMaxN * 64; q += NT) {
-      const int j = q >> 6, c = q & 63;
-      w3s[q] = (j < ch.n3 && c < ch.n2) ? bz::ldv<ET>((const ET*)ch.w3 + (int64_t)j * ch.ldw3 + c) : 0.f;
-    }
-  }
-
-  // the weight, as fragments: lane (column frow of block j, half fhalf) holds k = 16*ks + 8*fhalf .. +7 of its column.
-  // Asked for right behind the first rows of the A tile's operands, before anything waits for those: the weight (from
-  // L2) and the operands (from HBM) are then one trip to memory and not one after the other.
-  uint4 wf[TN][kPiecesKS];
-  auto load_w = [&]() {
+  // Everything the workgroup needs from memory is asked for here, at once, and nothing waits before all of it is in
+  // flight: first what comes from L2 and is needed first (the weights, the parameters), then the A tile's operands from
+  // HBM.  Loads return in the order they were issued, so the weights can be put into LDS while the operands travel.
+  //
+  // The first layer's weight goes through LDS: row n of the tile = column n of the layer, coalesced 16-byte loads, and
+  // every wave then reads its fragments (lane: column frow of block j, k = 16*ks + 8*fhalf .. +7) from there.  Loaded
+  // straight from memory as fragments, a load instruction touched 32 different 128-byte lines, and a workgroup's four
+  // waves asked L1 for the same 43 KB four times: 10 000 cycles of a workgroup's 40 000.
+  constexpr int kWPasses = TN * 4;  // 32 lanes a row (28 chunks of 16 bytes at most), 8 rows a pass
+  const int wc = tid & 31, wr = tid >> 5;
+  uint4 wreg[kWPasses];
+  {
+    const bool have = wc * 8 < KP && wc * 8 < ldw;  // (rows are zero from K up to ldw, a multiple of 8)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      int n = j * 32 + frow;
+    for (int i = 0; i < kWPasses; ++i) {
+      int n = wr + 8 * i;
       n = n < N ? n : N - 1;
-      const char* wrow = W + (int64_t)n * ldw * 2;
-#pragma unroll
-      for (int ks = 0; ks < kPiecesKS; ++ks) {
-        const int k0 = ks * 16 + fhalf * 8;
-        // (rows are zero from K up to ldw, a multiple of 8: a chunk is wholly inside the row or wholly absent)
-        wf[j][ks] = (ks < KS && k0 < ldw) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
-      }
+      wreg[i] = *(const uint4*)(W + ((int64_t)n * ldw + (have ? wc * 8 : 0)) * 2);
+      if (!have) wreg[i] = make_uint4(0, 0, 0, 0);
     }
+  }
+  // a second layer's weight the same way: 16 lanes a row (12 chunks at most), 16 rows a pass
+  constexpr int kW2Passes = CHAIN ? 4 : 0;
+  uint4 w2reg[kW2Passes + 1];
+  if constexpr (CHAIN) {
+    const int c2 = tid & 15;
+    const bool have = c2 * 8 < kPiecesMaxN && c2 * 8 < ch.ldw2;
+#pragma unroll
+    for (int i = 0; i < kW2Passes; ++i) {
+      int n2 = (tid >> 4) + 16 * i;
+      n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
+      w2reg[i] = *(const uint4*)(ch.w2 + ((int64_t)n2 * ch.ldw2 + (have ? c2 * 8 : 0)) * 2);
+      if (!have) w2reg[i] = make_uint4(0, 0, 0, 0);
+    }
+  }
+  // the parameters: thread t makes entries t and t + 256 of ps1 and entry t of ps2.  Here only the loads, with no branch
+  // round them (the compiler would wait there for everything asked so far; an entry that does not exist reads the
+  // weight's first word instead) and nothing computed from them yet (that would be a wait for memory as well).
+  auto param_use = [&](const Epilogue& e, int which) {
+    const bool dice = e.act == BZ_ACT_DICE, prelu = e.act == BZ_ACT_PRELU;
+    return which == 0 ? e.bias_rows == 1 : (which == 1 ? (dice || prelu) : dice);
+  };
+  auto param_load = [&](const Epilogue& e, int which, int n) -> float {
+    const float* src = which == 0 ? e.bias : (which == 1 ? e.p0 : (which == 2 ? e.p1 : e.p2));
+    const int at = (which == 1 && e.act == BZ_ACT_PRELU && e.act_size == 1) ? 0 : n;
+    return *(param_use(e, which) ? src + at : (const float*)W);
+  };
+  auto param_finish = [&](const Epilogue& e, int which, float v) -> float {
+    const float r = which == 0 ? e.beta * v : (which == 3 ? dice_inv_den(e, v) : v);
+    return param_use(e, which) ? r : 0.f;
+  };
+  int which1[2];
+  float pv1[2], pv2 = 0.f, w3v[2] = {0.f, 0.f};
+  bool w3use[2] = {false, false};
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int q = tid + h * NT;
+    q = q < 4 * kPiecesMaxN ? q : 0;
+    which1[h] = q / kPiecesMaxN;
+    const int n = q - which1[h] * kPiecesMaxN;
+    pv1[h] = param_load(ep, which1[h], n < N ? n : N - 1);
+  }
+  if constexpr (CHAIN) {
+    const int n2 = tid & 63;
+    pv2 = param_load(ch.ep2, tid >> 6, n2 < ch.n2 ? n2 : ch.n2 - 1);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int q = tid + h * NT, j = q >> 6, c = q & 63;
+      w3use[h] = j < ch.n3 && c < ch.n2;
+      w3v[h] = bz::ldv<ET>(w3use[h] ? (const ET*)ch.w3 + (int64_t)j * ch.ldw3 + c : (const ET*)W);
+    }
+  }
+  // into LDS: the first layer's weight into the A tile's own rows (it is gone from there before the tile is written)
+  uint4 wf[TN][kPiecesKS];
+  auto stage_and_read_w = [&]() {
+    if (wc * 8 < KP) {
+#pragma unroll
+      for (int i = 0; i < kWPasses; ++i) *(uint4*)(smem + (wr + 8 * i) * pitch + wc * 16) = wreg[i];
+    }
+    if constexpr (CHAIN) {
+      const int c2 = tid & 15;
+      if (c2 * 8 < kPiecesMaxN) {
+#pragma unroll
+        for (int i = 0; i < kW2Passes; ++i) *(uint4*)(w2s + ((tid >> 4) + 16 * i) * kChainPitch + c2 * 16) = w2reg[i];
+      }
+      ps2[tid] = param_finish(ch.ep2, tid >> 6, pv2);
+      w3s[tid] = w3use[0] ? w3v[0] : 0.f;
+      w3s[tid + NT] = w3use[1] ? w3v[1] : 0.f;
+    }
+    ps1[tid] = param_finish(ep, which1[0], pv1[0]);
+    if (tid + NT < 4 * kPiecesMaxN) ps1[tid + NT] = param_finish(ep, which1[1], pv1[1]);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int ks = 0; ks < kPiecesKS; ++ks)
+        wf[j][ks] = ks < KS ? *(const uint4*)(smem + (j * 32 + frow) * pitch + ks * 32 + fhalf * 16) : make_uint4(0, 0, 0, 0);
+    __syncthreads();  // every wave has its fragments: the rows are free for the A tile
   };
 
   // the A tile: a lane owns VEC columns of a piece and walks the pieces; 64 / (W / VEC) rows share a wave.  kGenRows rows
   // of a lane are in flight at once (no branch round the loads: a row beyond M reads row M-1 and is not stored; one
   // beyond the tile reads the lane's first row again, a cache hit), so the tile costs BM / (4 * rows_per_wave * kGenRows)
   // trips to memory, not one per row: one for the attention input of 4 x 54 columns.  kGenRows keeps the rows in flight
-  // within 64 registers.
+  // within 32 registers where x and y are loaded once and within 64 otherwise (8 columns a lane mean at most 8 lanes a row,
+  // so 4 rows in flight already cover the tile); the weight's 168 registers are live at the same time.
   {
-    constexpr int kGenRows = XY4 ? (VEC == 8 ? 8 : 16) : (VEC == 8 ? 2 : 8);
+    constexpr int kGenRows = XY4 ? (VEC == 8 ? 4 : 16) : (TN == 3 ? (VEC == 8 ? 1 : 4) : (VEC == 8 ? 2 : 8));
     constexpr int NL = XY4 ? 2 : NP;  // operands loaded a row: x and y once, or x and y of every piece
     const int per_piece = p.col0[1] / VEC;
     const int rows_per_wave = 64 / per_piece;
     const int sub = lane / per_piece, cv = lane - sub * per_piece;
     const uint32_t r1 = (uint32_t)p.r1;
+    // row -> (row / r1, row % r1): one division for the tile's first row (the same for every lane); a row of the tile is
+    // less than BM rows further, and a quotient that small is exact in fp32 up to a correction by one
+    const uint32_t q0_ = (uint32_t)m0 / r1, rem0 = (uint32_t)m0 - q0_ * r1;
+    const float inv_r1 = 1.f / (float)r1;
+    auto split_row = [&](uint32_t row, uint32_t* i0, uint32_t* i1) {
+      const uint32_t t = row - (uint32_t)m0 + rem0;  // < r1 + BM; (a row clamped to M - 1 is not before m0)
+      uint32_t q = (uint32_t)((float)t * inv_r1);
+      q -= (q * r1 > t);
+      q += ((q + 1) * r1 <= t);
+      *i0 = q0_ + q;
+      *i1 = t - q * r1;
+    };
     const int step = 4 * rows_per_wave;
     const int base0 = wave * rows_per_wave + sub;
     Pack xs[kGenRows][NL], ys[kGenRows][XY4 ? 1 : NP];
@@ -147,7 +232,12 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
         const int rl = base + u * step;
         uint32_t row = (uint32_t)(m0 + (rl < BM ? rl : base));
         row = row < (uint32_t)M ? row : (uint32_t)M - 1;
+#ifdef BZ_OLD_DIV
         const uint32_t i0 = row / r1, i1 = row - i0 * r1;
+#else
+        uint32_t i0, i1;
+        split_row(row, &i0, &i1);
+#endif
         if constexpr (XY4) {
           xs[u][0] = *(const Pack*)((const ET*)p.x[0] + (int64_t)i0 * p.xs[0][0] + (int64_t)i1 * p.xs[0][1] + cv * VEC);
           xs[u][1] = *(const Pack*)((const ET*)p.x[1] + (int64_t)i0 * p.xs[1][0] + (int64_t)i1 * p.xs[1][1] + cv * VEC);
@@ -193,17 +283,15 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
     // no branch round the loads)
     const bool mine = sub < rows_per_wave;
     gen_load(base0);
-    load_w();
+    stage_and_read_w();
     if (mine) gen_store(base0);
     for (int base = base0 + step * kGenRows; base < BM; base += step * kGenRows) {
       gen_load(base);
       if (mine) gen_store(base);
     }
-    // columns K .. KP-1 of every row
-    for (int q = tid; q < BM * (KP - K); q += NT) {
-      const int rl = q / (KP - K), c = K + q % (KP - K);
-      *(unsigned short*)(smem + rl * pitch + c * 2) = 0;
-    }
+    // columns K .. KP-1 of every row (at most 15)
+    if (tid < BM)
+      for (int c = K; c < KP; ++c) *(unsigned short*)(smem + tid * pitch + c * 2) = 0;
   }
   __syncthreads();
 
@@ -224,30 +312,31 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
     }
   }
 
-  // the second layer's weight fragments and column parameters: asked for here, so that they arrive during the first
-  // layer's epilogue (the first layer's fragments are dead from here on)
+  // the epilogues' column parameters and the second layer's weight fragments, from LDS (the first layer's fragments are
+  // dead from here on)
+  float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = j * 32 + frow;
+    cbias[j] = ps1[n];
+    cp0[j] = ps1[kPiecesMaxN + n];
+    cp1[j] = ps1[2 * kPiecesMaxN + n];
+    cp2[j] = ps1[3 * kPiecesMaxN + n];
+  }
   constexpr int TN2 = CHAIN ? 2 : 0, KS2MAX = CHAIN ? kChainKS : 0;
   const int KS2 = (N + 15) / 16;
   uint4 wf2[TN2 + 1][KS2MAX + 1];
   float b2[TN2 + 1], q0[TN2 + 1], q1[TN2 + 1], q2[TN2 + 1];
 #pragma unroll
   for (int j = 0; j < TN2; ++j) {
-    int n2 = j * 32 + frow;
-    n2 = n2 < ch.n2 ? n2 : ch.n2 - 1;
-    const char* wrow = ch.w2 + (int64_t)n2 * ch.ldw2 * 2;
+    const int n2 = j * 32 + frow;
 #pragma unroll
-    for (int ks = 0; ks < KS2MAX; ++ks) {
-      const int k0 = ks * 16 + fhalf * 8;
-      wf2[j][ks] = (ks < KS2 && k0 < ch.ldw2) ? *(const uint4*)(wrow + k0 * 2) : make_uint4(0, 0, 0, 0);
-    }
-    b2[j] = ch.ep2.bias_rows == 1 ? ch.ep2.beta * ch.ep2.bias[n2] : 0.f;
-    q0[j] = q1[j] = q2[j] = 0.f;
-    if (ch.ep2.act == BZ_ACT_PRELU) q0[j] = ch.ep2.p0[ch.ep2.act_size == 1 ? 0 : n2];
-    if (ch.ep2.act == BZ_ACT_DICE) {
-      q0[j] = ch.ep2.p0[n2];
-      q1[j] = ch.ep2.p1[n2];
-      q2[j] = dice_inv_den(ch.ep2, ch.ep2.p2[n2]);
-    }
+    for (int ks = 0; ks < KS2MAX; ++ks)
+      wf2[j][ks] = ks < KS2 ? *(const uint4*)(w2s + n2 * kChainPitch + ks * 32 + fhalf * 16) : make_uint4(0, 0, 0, 0);
+    b2[j] = ps2[n2];
+    q0[j] = ps2[64 + n2];
+    q1[j] = ps2[128 + n2];
+    q2[j] = ps2[192 + n2];
   }
   // epilogue: lane owns column n of each block, rows 8*(r/4) + 4*(lane/32) + r%4 of the wave's 32
   constexpr int OS = (int)sizeof(OutT);
@@ -460,7 +549,7 @@ int launch_pieces_tn(const bz_fc_desc& d, const bz::CewP& p, const Epilogue& ep,
       if (dev >= 0 && dev < 64 && !raised[dev]) {                                                                              \
         BZ_HIP_OK(hipFuncSetAttribute((const void*)bz_fc_pieces_kernel<DT, OutT, VEC, NP, TN, XY4, CHAIN>,                                 \
                                       hipFuncAttributeMaxDynamicSharedMemorySize,                                                  \
-                                      kPiecesBM * pieces_pitch(kPiecesKS * 16, 3, 4, true) + kSkinnyMaxN * 64 * 4));     \
+                                      pieces_lds(kPiecesKS * 16, 3, 4, true)));     \
         raised[dev] = true;                                                                                                    \
       }                                                                                                                        \
     }                                                                                                                          \
@@ -498,7 +587,7 @@ int launch_pieces(const bz_fc_desc& d, const Epilogue& ep, hipStream_t st) {
   const int pitch = pieces_pitch(d.k, tn, os, d.next != nullptr);
   // 16-byte stores of whole output rows when they are aligned for them (the outputs always go through LDS)
   const bool stage_y = d.y != nullptr && ((uintptr_t)d.y % 16 == 0) && ((d.ldy * os) % 16 == 0) && ((d.n * os) % 16 == 0);
-  const int smem = kPiecesBM * pitch + (d.next != nullptr ? kSkinnyMaxN * 64 * 4 : 0);
+  const int smem = pieces_lds(d.k, tn, os, d.next != nullptr);
   ChainArgs ch = {};
   const bool chain = d.next != nullptr;
   if (chain) {
