@@ -369,8 +369,9 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   char* lout = &lds[0][0];
   // A bias of one row per sample, the rare form, is folded into the accumulators first, so that the element loop below
   // has no index to compute and nothing to decide per element.
+  // (The 256x256 tile has no registers to spare for it and is not chosen for such a layer.)
   float alpha_e = ep.alpha;
-  if (ep.bias_rows > 1) {
+  if (BM * BN < 256 * 256 && ep.bias_rows > 1) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + wn * WTN + j * 32 + (lane & 31);
@@ -923,10 +924,11 @@ int dispatch_tiles(const bz_fc_desc& d, const Epilogue& ep, bool vec_a, bool vec
     if (wg_stream >= 200 && d.k % kStreamBK == 0 && d.k >= 8 * kStreamBK && vec_y && d.bias_rows <= 1)
       return launch_stream<DT, OutT>(d, ep, st);
   }
-  if constexpr (sizeof(OutT) == 2) {
-    // (256x256 once even that fills the chip: 4096^3 bf16 987 against 885 TFLOP/s)
+  if constexpr (sizeof(OutT) == 2 && In<DT>::kSize == 2) {
+    // (256x256 once even that fills the chip: 4096^3 bf16 987 against 885 TFLOP/s; with fp32 operands these two tiles
+    // do not fit the registers)
     const int64_t wg256 = (int64_t)((d.m + 255) / 256) * ((d.n + 255) / 256);
-    if (wg256 >= 256) return launch_mfma<DT, OutT, 256, 256, BK, 4, 2, 2, true>(d, ep, vec_a, vec_w, st);
+    if (wg256 >= 256 && d.bias_rows <= 1) return launch_mfma<DT, OutT, 256, 256, BK, 4, 2, 2, true>(d, ep, vec_a, vec_w, st);
     if (d.n > 128 && wg128x256 >= 256) return launch_mfma<DT, OutT, 128, 256, BK, 2, 4, 3, true>(d, ep, vec_a, vec_w, st);
   }
   // tall and narrow (the attention MLP over batch x history rows): one 96-wide tile reads A once
