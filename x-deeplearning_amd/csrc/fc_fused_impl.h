@@ -254,19 +254,20 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][i][j][r] = 0.f;
 
-  // per-column epilogue parameters, requested before anything else so their latency hides under the K loop
+  // per-column epilogue parameters, requested before anything else so their latency hides under the K loop; nothing
+  // is computed from them before the epilogue (an instruction on a loaded value here is a wait for memory here)
   float cbias[TN], cp0[TN], cp1[TN], cp2[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     int n = n0 + wn * WTN + j * 32 + (lane & 31);
     n = n < N ? n : N - 1;
-    cbias[j] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
+    cbias[j] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
     cp0[j] = cp1[j] = cp2[j] = 0.f;
     if (ep.act == BZ_ACT_PRELU) cp0[j] = ep.p0[ep.act_size == 1 ? 0 : n];
     if (ep.act == BZ_ACT_DICE) {
       cp0[j] = ep.p0[n];
       cp1[j] = ep.p1[n];
-      cp2[j] = dice_inv_den(ep, ep.p2[n]);
+      cp2[j] = ep.p2[n];
     }
   }
 
@@ -367,6 +368,11 @@ __global__ __launch_bounds__(WM* WN * 64) void bz_fc_mfma_kernel(const char* __r
   constexpr int OPITCH = BN * OS + 16;
   static_assert(BM * OPITCH <= (int)sizeof(lds), "output tile must fit the operand buffers");
   char* lout = &lds[0][0];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    cbias[j] *= ep.beta;
+    if (ep.act == BZ_ACT_DICE) cp2[j] = dice_inv_den(ep, cp2[j]);
+  }
   // A bias of one row per sample, the rare form, is folded into the accumulators first, so that the element loop below
   // has no index to compute and nothing to decide per element.
   // (The 256x256 tile has no registers to spare for it and is not chosen for such a layer.)
@@ -634,13 +640,13 @@ __global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(con
   for (int jn = 0; jn < TN; ++jn) {
     int n = n0 + wn * 64 + jn * 32 + (lane & 31);
     n = n < N ? n : N - 1;
-    cbias[jn] = ep.bias_rows == 1 ? ep.beta * ep.bias[n] : 0.f;
+    cbias[jn] = ep.bias_rows == 1 ? ep.bias[n] : 0.f;
     cp0[jn] = cp1[jn] = cp2[jn] = 0.f;
     if (ep.act == BZ_ACT_PRELU) cp0[jn] = ep.p0[ep.act_size == 1 ? 0 : n];
     if (ep.act == BZ_ACT_DICE) {
       cp0[jn] = ep.p0[n];
       cp1[jn] = ep.p1[n];
-      cp2[jn] = dice_inv_den(ep, ep.p2[n]);
+      cp2[jn] = ep.p2[n];  // (finished in the epilogue: an instruction on a loaded value here is a wait for memory here)
     }
   }
 
@@ -696,6 +702,11 @@ __global__ __launch_bounds__(2 * kStreamCompute, 1) void bz_fc_stream_kernel(con
   // epilogue: lane owns column n of each 32x32 block, rows 8*(r/4) + 4*(lane/32) + r%4; the activated tile goes through
   // LDS so that global stores are 16 bytes per lane along rows
   __syncthreads();
+#pragma unroll
+  for (int jn = 0; jn < TN; ++jn) {
+    cbias[jn] *= ep.beta;
+    if (ep.act == BZ_ACT_DICE) cp2[jn] = dice_inv_den(ep, cp2[jn]);
+  }
   constexpr int OPITCH = BN * 2 + 16;
   char* lout = smem;
   auto epilogue = [&](auto act_c) {
