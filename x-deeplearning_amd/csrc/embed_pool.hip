@@ -264,14 +264,16 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
 
-// Store `nvalid` fp32 results as the slot's output dtype at element pointer `dst`
-// using the widest store the address allows.
+// Store `nvalid` fp32 results as the slot's output dtype at element pointer `dst` using the widest store the address
+// allows - the widest every active lane of the wave allows: lanes of one wave that picked different widths would run
+// the paths one after the other (three kassign items sharing 108-byte rows start on 0, 4, 8 and 12 bytes mod 16, and
+// their stores were 40 % of that kernel).
 template <int N>
 __device__ __forceinline__ void store_elems(void* dst_base, int64_t elem_off, const float (&v)[N], int nvalid,
                                             int out_dtype) {
   if (out_dtype == BZ_F32) {
     float* dst = (float*)dst_base + elem_off;
-    if (nvalid == N && (((uintptr_t)dst) & 15) == 0) {
+    if (__all(nvalid == N && (((uintptr_t)dst) & 15) == 0)) {
 #pragma unroll
       for (int i = 0; i < N; i += 4) *(float4*)(dst + i) = make_float4(v[i], v[i + 1], v[i + 2], v[i + 3]);
     } else {
@@ -295,19 +297,25 @@ __device__ __forceinline__ void store_elems(void* dst_base, int64_t elem_off, co
       pk[i] = lo | (hi << 16);
     }
     const uintptr_t a = (uintptr_t)dst;
-    if (nvalid == N && (a & 15) == 0 && N >= 8) {
+    const bool full = nvalid == N;
+    if (N >= 8 && __all(full && (a & 15) == 0)) {
 #pragma unroll
       for (int i = 0; i + 4 <= N / 2; i += 4) *(uint4*)((uint32_t*)dst + i) = make_uint4(pk[i], pk[i + 1], pk[i + 2], pk[i + 3]);
-    } else if (nvalid == N && (a & 7) == 0) {
+    } else if (__all(full && (a & 7) == 0)) {
 #pragma unroll
       for (int i = 0; i < N / 2; i += 2) *(uint2*)((uint32_t*)dst + i) = make_uint2(pk[i], pk[i + 1]);
-    } else if ((a & 3) == 0) {
+    } else if (__all((a & 3) == 0)) {
+      if (__all(full)) {
 #pragma unroll
-      for (int i = 0; i < N / 2; ++i) {
-        if (2 * i + 1 < nvalid)
-          ((uint32_t*)dst)[i] = pk[i];
-        else if (2 * i < nvalid)
-          dst[2 * i] = __ushort_as_half((unsigned short)(pk[i] & 0xffffu));
+        for (int i = 0; i < N / 2; ++i) ((uint32_t*)dst)[i] = pk[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+          if (2 * i + 1 < nvalid)
+            ((uint32_t*)dst)[i] = pk[i];
+          else if (2 * i < nvalid)
+            dst[2 * i] = __ushort_as_half((unsigned short)(pk[i] & 0xffffu));
+        }
       }
     } else {
 #pragma unroll
