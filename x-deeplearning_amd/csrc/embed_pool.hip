@@ -653,24 +653,33 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   const bz_embed_slot s = slots[lo];
   const int ce = chunk_elems(s.table_dtype);
   const int nchunks = (s.dim + ce - 1) / ce;
-  int lpr = 1;
-  while (lpr < nchunks && lpr < bz::kWave) lpr <<= 1;
-  const int groups = kThreads / lpr;
+  // lpr, a power of two: shifts, not divisions (a 64-bit division is some 150 instructions, and this kernel's threads
+  // each do little else than one or four row gathers)
+  int lpr_log = 0;
+  while ((1 << lpr_log) < nchunks && (1 << lpr_log) < bz::kWave) ++lpr_log;
+  const int lpr = 1 << lpr_log;
+  const int groups = kThreads >> lpr_log;
   const int tid = threadIdx.x;
-  const int g = tid / lpr;
-  const int l = tid - g * lpr;
+  const int g = tid >> lpr_log;
+  const int l = tid - (g << lpr_log);
   // a lane group owns one item: a sample (ksum / kavg) or kAssignRun output positions of a sample (kassign)
   const int64_t per = items_per_sample(s);
   const int64_t n_items = (int64_t)s.batch * per;
   const int64_t i0 = (int64_t)(v - s.wg_begin) * groups;
   int64_t i_last = i0 + groups - 1;
   if (i_last >= n_items) i_last = n_items - 1;
-  const int64_t b_first = i0 / per;
-  const int n_samples = (int)(i_last / per - b_first) + 1;  // <= groups
+  // item -> sample: no division for pooled slots (per == 1), a 32-bit one while the item count allows it
+  auto sample_of = [&](int64_t item) -> int64_t {
+    if (per == 1) return item;
+    if (n_items < (1ll << 31)) return (int64_t)((uint32_t)item / (uint32_t)per);
+    return item / per;
+  };
+  const int64_t b_first = sample_of(i0);
+  const int n_samples = (int)(sample_of(i_last) - b_first) + 1;  // <= groups
   stage_offsets(s, ext_off != nullptr ? ext_off + (int64_t)lo * ext_stride : s.offsets, b_first, n_samples, s_off, s_part);
   const int64_t item = i0 + g;
   if (item >= n_items) return;
-  const int64_t b = item / per;
+  const int64_t b = sample_of(item);
   const int p = (int)(item - b * per) * (s.udf == BZ_ASSIGN ? kAssignRun : 1);
   if (s.table == nullptr) {
     pool_zero(s, b, p, l, lpr);
