@@ -231,6 +231,16 @@ def test_assign_items_share_the_rows_of_one_history_tensor(bz, oracle, kind, out
         w = want[:, :, :col]
         assert not np.isnan(w).any()
         assert np.array_equal(_bits(got[:, :, :col]), _bits(w.astype(out_dtype)))
+    # an item whose table is unknown zero-fills its own columns of every position and nothing else
+    out.fill_(float("nan"))
+    unknown = [dict(items[0]), dict(items[1], table=None, dim=dims[1]), dict(items[2])]
+    bz.EmbeddingPlan(unknown).run()
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().reshape(batch, T, pitch)
+    w = want[:, :, :col].copy()
+    w[:, :, dims[0]:dims[0] + dims[1]] = 0
+    assert np.isnan(got[:, :, col:].astype(np.float32)).all()
+    assert np.array_equal(_bits(got[:, :, :col]), _bits(w.astype(out_dtype)))
     # a pitch below the item's dim, or on a pooled item, is refused
     bad = dict(items[0], assign_pitch=dims[0] - 1)
     with pytest.raises(RuntimeError, match="assign_pitch"):
