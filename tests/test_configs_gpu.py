@@ -430,3 +430,14 @@ def test_history_blocks_written_into_their_concat_equal_the_copy():
         assert g1["his"].shape == (b, cfg.T, 3 * cfg.dim) and g1["his"].any()
         for k in g1:
             np.testing.assert_array_equal(g1[k], g0[k], err_msg=k)
+    # a reshaped block that is also an output of the net keeps its own memory: the rewrite does not apply
+    mid = "his3_" + din_model.KINDS[0]
+    pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("his", mid))
+    p = pm.create_predictor(1, 0)
+    p.register_observers(["profile"])
+    din_model.feed(p, inputs, batches[0], np.float16)
+    p.forward()
+    ran = [e["name"] for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+    assert "Concat:concat_his" in ran, ran
+    np.testing.assert_array_equal(p.output_asnumpy("his"), outs[1][0]["his"])
+    np.testing.assert_array_equal(p.output_asnumpy(mid), outs[1][0]["his"][:, :, :cfg.dim])
