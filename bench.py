@@ -103,88 +103,22 @@ def mfma_roofline(kernel, flops, us):
             "frac": round(tf / MFMA_PEAK_TFLOPS, 5), "traffic": None, "flops_per_launch": int(flops), "avg_launch_us": round(us, 2)}
 
 
-# ------------------------------------------------------------------------------------------------ probes
-def run_probes(args, np, torch, bz, arch):
-    """Measurement aids behind the profiles: a plain copy of known size (the reference for scaling counter readings)
-    and the gather probes (what the memory system gives the pooling kernel's access pattern alone)."""
-    if args.calibrate_copy:
-        rows, width = 65536, 4096
-        src = torch.ones(rows * width, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        d = bz.ConcatDesc()
-        d.src[0], d.width[0], d.src_pitch[0] = src.data_ptr(), width, width
-        d.dst, d.dst_pitch, d.rows, d.n = dst.data_ptr(), width, rows, 1
-        for _ in range(5):
-            bz.check(bz.lib().bz_concat_cols(ctypes.byref(d), None))
-        torch.cuda.synchronize()
-        assert bool((dst == 1).all())
-        print(json.dumps({"calibration": "bz_concat_kernel", "launches": 5, "bytes_read_per_launch": rows * width,
-                          "bytes_written_per_launch": rows * width}))
-        return
-
-    def ev_time(fn, reps=20):
-        for _ in range(5):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / reps  # us
-
-    if args.fc_probe:
-        # config 5's first layer alone (8192 x 12800 -> 1024 bf16, bias + ReLU), inputs alternating between two buffers
-        # so that the activations come from HBM, not from the last-level cache
-        M, K, N = 8192, 12800, 1024
-        g = torch.Generator(device="cuda").manual_seed(5)
-        xs = [(torch.randn((M, K), generator=g, device="cuda") * 0.5).to(torch.bfloat16) for _ in range(2)]
-        w = bz.pack_weight((torch.randn((K, N), generator=g, device="cuda") / K ** 0.5), False, bz.BF16)
-        b = torch.randn(N, generator=g, device="cuda") * 0.1
-        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-        k = [0]
-
-        def launch():
-            k[0] += 1
-            bz.fc_fused(xs[k[0] & 1], w, K, bias=b, act=bz.ACT_LEAKY_RELU, act_alpha=0.0, out=y)
-        # alternating rounds; both kernels keep getting faster for some 100 ms of sustained load (see graph_timed): the
-        # first half of the rounds is dropped
-        def lib_launch():
-            k[0] += 1
-            torch.nn.functional.linear(xs[k[0] & 1], w[:, :K])
-        rounds = [(ev_time(launch, 20), ev_time(lib_launch, 20)) for _ in range(8)]
-        us = float(np.median([r[0] for r in rounds[4:]]))
-        lib_us = float(np.median([r[1] for r in rounds[4:]]))
-        print(json.dumps({"probe": "bz_fc_fused %dx%d -> %d bf16, bias + ReLU" % (M, K, N), "us": round(us, 2),
-                          "rounds_us": [[round(a, 1), round(b_, 1)] for a, b_ in rounds],
-                          "TFLOP/s": round(2.0 * M * K * N / us / 1e6, 1), "frac_of_mfma_peak": round(2.0 * M * K * N / us / 1e6 / MFMA_PEAK_TFLOPS, 4),
-                          "library_gemm_us": round(lib_us, 2), "device": arch}))
-        return
-
-    res = {"probe": "random gathers of whole rows, nothing else", "device": arch}
-    region = torch.ones(args.probe_region_mib << 20, dtype=torch.uint8, device="cuda")
-    side = torch.ones((args.probe_region_mib << 20) // 64, dtype=torch.float32, device="cuda")
-    sink = torch.empty((1 << 20) * 128, dtype=torch.uint8, device="cuda")
-    cases = [(64, False, 1 << 20, 8), (64, False, 1 << 20, 16), (64, False, 425984, 1), (64, False, 106496, 4),
-             (128, False, 1 << 20, 8), (128, False, 1 << 20, 4), (64, True, 1 << 20, 8), (64, True, 1 << 20, 4)]
-    if args.probe_case is not None:
-        cases = [cases[args.probe_case]]
-    out = {}
-    for row_bytes, with_side, groups, per in cases:
-        seed = [0]
-
-        def launch():
-            seed[0] += 7919
-            bz.check(bz.lib().bz_probe_gather(region.data_ptr(), region.numel(), row_bytes, side.data_ptr() if with_side else None,
-                                              sink.data_ptr(), groups, per, seed[0], None))
-        us = ev_time(launch, 50)
-        nbytes = groups * per * (row_bytes + (4 if with_side else 0))
-        out["%dB rows%s, %d groups x %d" % (row_bytes, " + 4B side word" if with_side else "", groups, per)] = {
-            "us": round(us, 2), "rows": groups * per, "GB/s": round(nbytes / us / 1e3, 1), "Grows/s": round(groups * per / us / 1e3, 2)}
-    res["region_MiB"] = args.probe_region_mib
-    res["cases"] = out
-    print(json.dumps(res))
+# ------------------------------------------------------------------------------------------------ counter calibration
+def calibration_copy(torch, bz):
+    """A plain copy of known size (bz_concat_kernel, one piece of 256 MiB, 5 launches): what rocprofv3's FETCH_SIZE /
+    WRITE_SIZE read for it is the scale for the same counters on the other kernels of the run.  Part of --counters-run."""
+    rows, width = 65536, 4096
+    src = torch.ones(rows * width, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    d = bz.ConcatDesc()
+    d.src[0], d.width[0], d.src_pitch[0] = src.data_ptr(), width, width
+    d.dst, d.dst_pitch, d.rows, d.n = dst.data_ptr(), width, rows, 1
+    for _ in range(5):
+        bz.check(bz.lib().bz_concat_cols(ctypes.byref(d), None))
+    torch.cuda.synchronize()
+    assert bool((dst == 1).all())
+    return {"kernel": "bz_concat_kernel", "launches": 5, "bytes_read_per_launch": rows * width,
+            "bytes_written_per_launch": rows * width}
 
 
 # ------------------------------------------------------------------------------------------------ other configurations
@@ -437,19 +371,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-per-config", action="store_true", help="skip configs 1, 3, 4 and 5")
     ap.add_argument("--no-feed", action="store_true", help="skip the PCIe-inclusive leg")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="only run a plain 256 MiB copy (bz_concat_kernel, one piece) a few times and exit: the known-size "
-                         "reference for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
-    ap.add_argument("--gather-probe", action="store_true",
-                    help="only measure what the memory system gives random gathers of 64- and 128-byte rows (a kernel that "
-                         "does nothing else) and exit")
     ap.add_argument("--counters-run", action="store_true",
-                    help="for runs under rocprofv3 --pmc, where every dispatch is serialised: skip the steady-state region and "
-                         "take the latency from --steps samples only (the line then carries no steady_state)")
-    ap.add_argument("--fc-probe", action="store_true",
-                    help="only run config 5's first FC layer (8192 x 12800 -> 1024 bf16) a few times and exit (for counter runs)")
-    ap.add_argument("--probe-region-mib", type=int, default=2048)
-    ap.add_argument("--probe-case", type=int, default=None, help="run one case of --gather-probe only (for counter runs)")
+                    help="for runs under rocprofv3 --pmc, where every dispatch is serialised: skip the steady-state region, take "
+                         "the latency from --steps samples only (the line then carries no steady_state), and run a plain "
+                         "256 MiB copy of known size first (the scale for FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--only", choices=["c1", "c3", "c4", "c5", "c5_fc"], default=None,
+                    help="run one of the other configurations alone and print its record (c5_fc: config 5's FC tower without "
+                         "its 102 GB of tables); with --counters-run fewer repetitions, for runs under rocprofv3 --pmc")
     ap.add_argument("--threads", type=int, default=8,
                     help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
                          "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
@@ -470,9 +398,14 @@ def main():
 
     assert torch.cuda.is_available(), "no GPU visible"
     arch = bz.device_check()
-    if args.calibrate_copy or args.gather_probe or args.fc_probe:
-        run_probes(args, np, torch, bz, arch)
+    if args.only is not None:
+        T = max(1, args.threads)
+        fn = {"c1": lambda: bench_config1(np, torch, bz, pb, T), "c3": lambda: bench_config3(np, torch, bz, pb, T),
+              "c4": lambda: bench_config4(np, torch, bz), "c5": lambda: bench_config5(np, torch, bz),
+              "c5_fc": lambda: bench_config5(np, torch, bz, tables=False)}[args.only]
+        print(json.dumps({"only": args.only, "device": arch, "result": fn()}))
         return
+    calibration = calibration_copy(torch, bz) if args.counters_run else None
     cfg = Config2()
     tables = cfg.tables()
     mlp = cfg.mlp()
@@ -670,6 +603,8 @@ def main():
         "per_config": per_config,
         "cpu_baseline": cpu,
     }
+    if calibration is not None:
+        out["counter_calibration"] = calibration
     print(json.dumps(out))
 
 

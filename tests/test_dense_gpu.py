@@ -471,7 +471,10 @@ def test_fc_split_argument_errors(bz):
 
 
 @pytest.mark.parametrize("dtype_name", ["f32", "f16"])
-@pytest.mark.parametrize("B,T,Cn", [(1024, 50, 54), (7, 1, 3), (33, 17, 130), (2, 200, 64)])
+@pytest.mark.parametrize("B,T,Cn", [(1024, 50, 54), (7, 1, 3), (33, 17, 130), (2, 200, 64),
+                                    # fewer channels than steps (first pass or tail pass): the lanes past the last
+                                    # channel still hold the weights the others read
+                                    (64, 50, 16), (64, 50, 24), (19, 70, 8), (19, 40, 70), (5, 130, 1)])
 def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T, Cn):
     """bz_weighted_pool against the three launches it replaces (Mul, strided-batched GEMM with transA, ReduceSum), bit
     for bit, and against the oracle's fp32 sums of the rounded operands."""

@@ -358,45 +358,6 @@ def test_config2_full_size(bz, oracle):
         assert np.array_equal(plan2.offsets[s].cpu().numpy(), oracle.segments_to_offsets(inputs[s][2]))
 
 
-@pytest.mark.parametrize("per", [1, 4, 8, 16])
-@pytest.mark.parametrize("row_bytes,with_side", [(64, False), (128, False), (64, True)])
-def test_gather_probe_reads_the_rows_it_claims(bz, per, row_bytes, with_side):
-    """bz_probe_gather (the measurement aid behind the gather-ceiling figures, csrc/bz_probe.h) really reads
-    rows_per_group hashed rows of row_bytes per group, and with a side array the word side[row] with each: with row r
-    holding the words W*r .. W*r+W-1, the folded row a group writes equals the sums / xors over exactly the rows the
-    documented hash picks.  Integer work: bit-exact."""
-    import torch
-    rows, groups, seed = 1000, 777, 12345
-    W = row_bytes // 4
-    region = np.arange(rows * W, dtype=np.uint32).reshape(rows, W)
-    side = (np.arange(rows, dtype=np.uint32) * 2654435761 & 0x7FFFFF).astype(np.uint32)  # small positive floats' bit patterns
-    d_region, d_side = _dev(region), _dev(side.view(np.float32))
-    sink = torch.zeros((groups, W), dtype=torch.int32, device="cuda")
-    bz.check(bz.lib().bz_probe_gather(d_region.data_ptr(), rows * row_bytes, row_bytes, d_side.data_ptr() if with_side else None,
-                                      sink.data_ptr(), groups, per, seed, None))
-    torch.cuda.synchronize()
-    got = sink.cpu().numpy().view(np.uint32)
-    gid = np.arange(groups, dtype=np.uint64)[:, None]
-    r = np.arange(per, dtype=np.uint64)[None, :]
-    h = ((gid * per + r) * 2654435761 + seed) & 0xFFFFFFFF
-    h ^= h >> 15
-    h = (h * 2246822519) & 0xFFFFFFFF
-    h ^= h >> 13
-    picked = (h * rows) >> 32  # [groups, per]
-    assert picked.max() < rows and len(np.unique(picked)) > rows // 2
-    words = region[picked.astype(np.int64)]  # [groups, per, W]
-    want = np.empty((groups, W), np.uint32)
-    for j in range(W):
-        col = words[:, :, j]
-        want[:, j] = col.sum(1, dtype=np.uint64).astype(np.uint32) if j % 2 == 0 else np.bitwise_xor.reduce(col, axis=1)
-        if with_side and j % 4 == 0:  # every lane adds the side words of its group's rows to word 0 of its chunk
-            want[:, j] += side[picked.astype(np.int64)].sum(1, dtype=np.uint64).astype(np.uint32)
-    np.testing.assert_array_equal(got, want)
-    # error convention
-    assert bz.lib().bz_probe_gather(d_region.data_ptr(), rows * row_bytes, row_bytes, None, sink.data_ptr(), groups, 3, seed, None) != 0
-    assert b"rows_per_group" in bz.lib().bz_last_error()
-
-
 def _lengths_case(rng, kind, batch):
     if kind == "poisson8":
         return np.clip(rng.poisson(8, batch), 0, 64).astype(np.int32)

@@ -431,6 +431,42 @@ def test_gemm_gemm_folding_pass_on_the_reference_fixtures(tmp_path, case):
     assert open(again).read() == open(dst).read()
 
 
+def test_gemm_gemm_folding_carries_the_second_alpha_into_the_first_bias(tmp_path):
+    """alpha1 * (alpha0 * x * W0 + beta0 * b0) * W1 + beta1 * b1: the first layer's bias is scaled by the second layer's
+    alpha as well (the reference's fixtures all have alpha1 = 1 and its CalcNewBias leaves the factor out).  The folded
+    constants are compared with numpy's float64 products."""
+    import pyblaze_hip as pb
+    from blaze_proto import NetDef
+    from google.protobuf import text_format
+    rng = np.random.default_rng(5)
+    K, H, N = 6, 5, 4
+    w0 = rng.standard_normal((K, H)).astype(np.float32)
+    w1 = rng.standard_normal((H, N)).astype(np.float32)
+    b0, b1 = rng.standard_normal(H).astype(np.float32), rng.standard_normal(N).astype(np.float32)
+    a0, be0, a1, be1 = 0.75, 2.0, 0.5, 3.0
+    nb = pb.NetBuilder("chain", device_type=1)
+    nb.external_input("x", pb.K_FLOAT)
+    for name, v in (("w0", w0), ("b0", b0), ("w1", w1), ("b1", b1)):
+        nb.constant(name, v)
+    nb.op("Gemm", ["x", "w0", "b0"], ["h"], alpha=a0, beta=be0)
+    nb.op("Gemm", ["h", "w1", "b1"], ["out"], alpha=a1, beta=be1)
+    nb.external_output("out", pb.K_FLOAT)
+    raw, opt = str(tmp_path / "raw.blaze"), str(tmp_path / "opt.blaze")
+    open(raw, "w").write(nb.text())
+    pb.optimize_blaze(raw, opt, False)
+    got = NetDef()
+    text_format.Parse(open(opt).read(), got)
+    gemms = [o for o in got.op if o.type == "Gemm"]
+    assert len(gemms) == 1 and list(gemms[0].input)[0] == "x"
+    consts = {o.output[0]: np.array([a for a in o.arg if a.name == "value"][0].floats, np.float64) for o in got.op
+              if o.type == "ConstantFill"}
+    args = {a.name: a.f for a in gemms[0].arg}
+    w, b = consts[gemms[0].input[1]].reshape(K, N), consts[gemms[0].input[2]]
+    x = rng.standard_normal((3, K))
+    want = a1 * ((a0 * x @ w0.astype(np.float64) + be0 * b0) @ w1.astype(np.float64)) + be1 * b1
+    np.testing.assert_allclose(args["alpha"] * x @ w + args["beta"] * b, want, rtol=1e-5, atol=1e-6)
+
+
 def _reference_text_tables():
     """-> {table: (keys int64 [n], rows fp32 [n, dim])} of tests/golden/quick_embedding (the reference's
     utest_data/store/quick_embedding: `key,w0,...` lines; the first weight column happens to hold a big integer)."""

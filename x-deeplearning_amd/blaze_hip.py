@@ -144,7 +144,6 @@ def lib():
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_static_scratch.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
-        l.bz_probe_gather.argtypes = [vp, i64, C.c_int, vp, vp, i64, C.c_int, C.c_uint32, vp]  # csrc/bz_probe.h, not public
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
         l.bz_gemm_strided_batched.argtypes = [C.POINTER(BgemmDesc), vp]

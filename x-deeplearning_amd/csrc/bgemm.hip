@@ -111,7 +111,12 @@ __global__ __launch_bounds__(256) void bz_weighted_pool_kernel(const T* __restri
   const T* wp = w + item * t_len;
   const T* mp = mask ? mask + item * t_len : nullptr;
   const T* xp = x + item * (int64_t)t_len * c_len;
-  for (int c = lane; c < c_len; c += 64) {
+  // The channel loop is uniform over the wave: every lane runs every pass, so that lane u holds the weight of step
+  // t0 + u when it is read with v_readlane below, whatever c_len is; a lane past the last channel reads the last
+  // channel's address and stores nothing.
+  for (int c0 = 0; c0 < c_len; c0 += 64) {
+    const bool live = c0 + lane < c_len;
+    const int c = live ? c0 + lane : c_len - 1;
     float acc_w = 0.f, acc_s = 0.f;
     for (int t0 = 0; t0 < t_len; t0 += kPoolUnroll) {
       // lane l fetches the weight of step t0 + l (every lane needs every weight: they are handed round below), then
@@ -139,8 +144,8 @@ __global__ __launch_bounds__(256) void bz_weighted_pool_kernel(const T* __restri
           acc_s = __fadd_rn(acc_s, xv[u]);
         }
     }
-    if (att) st<T>(att + item * c_len + c, acc_w);
-    if (sum) st<T>(sum + item * c_len + c, acc_s);
+    if (live && att) st<T>(att + item * c_len + c, acc_w);
+    if (live && sum) st<T>(sum + item * c_len + c, acc_s);
   }
 }
 

@@ -290,9 +290,10 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   std::string SiblingKey() override {
     Blob* b = this->Input(1);
     if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr || !siblings_.empty()) return "";
-    if (this->InputSize() > 2 && (!c_constant_ || this->Input(2)->shape().size() != 1)) return "";
-    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX) return "";
     const TIndex N = transb_ ? b->shape()[0] : b->shape()[1];
+    // (the stacked parameter vectors take N floats from every sibling: a bias of another length is no sibling's)
+    if (this->InputSize() > 2 && (!c_constant_ || this->Input(2)->shape().size() != 1 || (TIndex)this->Input(2)->size() != N)) return "";
+    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX) return "";
     if (fused_ && fused_act_ == BZ_ACT_PRELU && (TIndex)fused_->Input(1)->size() != N) return "";  // a scalar slope is per layer
     Blob* y = fused_ ? fused_->Output(0) : this->Output(0);
     if (y->pitch() != 0 || y == this->Input(0)) return "";

@@ -223,6 +223,18 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
   }
 }
 
+// Readers of a tensor name among all operators -- skipped ones too: an operator that another one has taken over still
+// runs, through its host, and reads what its definition names -- except `folded`, the activation a layer has folded
+// into its own epilogue (written in place it names the layer's output as its input).
+int SimpleNet::ReadersOf(const std::string& name, const OperatorBase* folded) const {
+  int readers = 0;
+  for (const auto& op : operators_) {
+    if (op.get() == folded) continue;
+    for (const auto& in : op->operator_def().input()) readers += (in == name);
+  }
+  return readers;
+}
+
 // FC layer (with its folded activation) -> FC layer of at most 8 outputs (with its folded Softmax / Sigmoid), the
 // first one's result read by nothing else: one launch (graph.h, StackableFc::CanHostHead).  Switch: fuse_fc_head: 0.
 void SimpleNet::FuseFcHeads() {
@@ -239,11 +251,8 @@ void SimpleNet::FuseFcHeads() {
     if (!second || !second->CanBeHead(n1)) continue;
     const std::string& mid = first->StackOutputOp()->operator_def().output(0);
     if (operators_[j]->operator_def().input(0) != mid) continue;
-    int readers = 0;
-    for (size_t k = 0; k < operators_.size(); ++k) {
-      if (skipped_[k]) continue;
-      for (const auto& in : operators_[k]->operator_def().input()) readers += (in == mid);
-    }
+    OperatorBase* out_op = first->StackOutputOp();
+    const int readers = ReadersOf(mid, out_op != operators_[i].get() ? out_op : nullptr);
     bool is_output = false;
     for (const auto& eo : external_output_) is_output |= (eo == mid);
     if (readers != 1 || is_output) continue;
@@ -330,11 +339,15 @@ void SimpleNet::FuseConcatsIntoFcs() {
     if (readers != 1 || workspace_->HasConstantBlob(in)) continue;
     // what the Concat reads, directly or through a producer it runs itself
     std::set<std::string> sources(operators_[c]->operator_def().input().begin(), operators_[c]->operator_def().input().end());
-    for (int j = 0; j < c; ++j) {
-      if (!skipped_[j]) continue;
-      bool feeds = false;
-      for (const auto& out : operators_[j]->operator_def().output()) feeds |= sources.count(out) != 0;
-      if (feeds) sources.insert(operators_[j]->operator_def().input().begin(), operators_[j]->operator_def().input().end());
+    // (to a fixed point: a taken-over producer may itself read another one's result, BroadcastTo -> Sub -> Concat)
+    for (size_t before = 0; before != sources.size();) {
+      before = sources.size();
+      for (int j = c - 1; j >= 0; --j) {
+        if (!skipped_[j]) continue;
+        bool feeds = false;
+        for (const auto& out : operators_[j]->operator_def().output()) feeds |= sources.count(out) != 0;
+        if (feeds) sources.insert(operators_[j]->operator_def().input().begin(), operators_[j]->operator_def().input().end());
+      }
     }
     bool clean = true;
     for (size_t k = c + 1; k < g && clean; ++k)
@@ -360,11 +373,8 @@ void SimpleNet::ChainNarrowFcs() {
     if (!first->CanChainNext(operators_[j].get())) continue;
     const std::string& mid = first_fc->StackOutputOp()->operator_def().output(0);
     if (operators_[j]->operator_def().input(0) != mid) continue;
-    int readers = 0;
-    for (size_t k = 0; k < operators_.size(); ++k) {
-      if (skipped_[k]) continue;
-      for (const auto& in : operators_[k]->operator_def().input()) readers += (in == mid);
-    }
+    OperatorBase* out_op = first_fc->StackOutputOp();
+    const int readers = ReadersOf(mid, out_op != operators_[i].get() ? out_op : nullptr);
     bool is_output = false;
     for (const auto& eo : external_output_) is_output |= (eo == mid);
     if (readers != 1 || is_output) continue;
@@ -393,6 +403,17 @@ void SimpleNet::PackSiblingFcs() {
     bool clean = true;
     for (size_t k = idx.front() + 1; k < idx.back() && clean; ++k)
       for (const auto& out : operators_[k]->operator_def().output()) clean &= (out != in);
+    // a later sibling's result appears where the first sibling runs: nothing from there up to the sibling's own place may
+    // read or write that name (or the name of the tensor between the sibling and its folded activation)
+    for (size_t m = 1; m < idx.size() && clean; ++m) {
+      std::set<std::string> names(operators_[idx[m]]->operator_def().output().begin(), operators_[idx[m]]->operator_def().output().end());
+      if (auto* st = dynamic_cast<StackableFc*>(operators_[idx[m]].get()))
+        names.insert(st->StackOutputOp()->operator_def().output().begin(), st->StackOutputOp()->operator_def().output().end());
+      for (size_t k = idx.front(); k < idx[m] && clean; ++k) {
+        for (const auto& in : operators_[k]->operator_def().input()) clean &= names.count(in) == 0;
+        for (const auto& out : operators_[k]->operator_def().output()) clean &= names.count(out) == 0;
+      }
+    }
     if (!clean) continue;
     std::vector<SiblingFc*> others;
     for (size_t m = 1; m < idx.size(); ++m) {
@@ -601,14 +622,6 @@ void SimpleNet::StackFcLayers() {
   const char* env = getenv("BLAZE_FC_STACK");
   const bool on = (arg && arg->has_i && arg->i != 0) || (env && atoi(env) != 0);
   if (!on) return;
-  auto readers = [&](const std::string& name) {
-    int n = 0;
-    for (size_t j = 0; j < operators_.size(); ++j) {
-      if (skipped_[j]) continue;
-      for (const auto& in : operators_[j]->operator_def().input()) n += (in == name);
-    }
-    return n;
-  };
   auto is_external_output = [&](const std::string& name) {
     for (const auto& eo : external_output_)
       if (eo == name) return true;
@@ -639,7 +652,8 @@ void SimpleNet::StackFcLayers() {
       if (!next || !next->StackEligible(&k2, &n2)) break;
       const std::string& mid = chain.back()->StackOutputOp()->operator_def().output(0);
       if (operators_[j]->operator_def().input(0) != mid || k2 != widths.back()) break;
-      if (readers(mid) != 1 || is_external_output(mid)) break;
+      OperatorBase* out_op = chain.back()->StackOutputOp();
+      if (ReadersOf(mid, out_op != operators_[last].get() ? out_op : nullptr) != 1 || is_external_output(mid)) break;
       const bool is_head = n2 <= BZ_MLP_MAX_HEAD;
       if (!is_head && !wide(n2)) break;
       int need[2] = {lds[0], lds[1]};

@@ -104,6 +104,7 @@ class SimpleNet : public Net {
   void FuseWeightedPools();
   void FuseConcatsIntoFcs();
   void ChainNarrowFcs();
+  int ReadersOf(const std::string& name, const OperatorBase* folded) const;
   void InterleaveAssignBlocks();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
 };

@@ -280,7 +280,9 @@ int FuseGemmChains(NetDef* net) {
       if (has_b0) {
         const int64_t rows = b0.shape.size() == 1 ? 1 : b0.shape[0];
         if (b0.shape.size() > 2 || b0.shape.back() != k1) continue;
-        bias = MatMul(b0.value, false, w1.value, tb1, rows, n, k1, beta0);
+        // alpha1 * (alpha0 * A * W0 + beta0 * b0) * W1: the first bias passes through the second product and its alpha
+        // (the reference's CalcNewBias leaves alpha1 out, gemm_gemm_fusion_pattern_impl.cc; its fixtures have alpha1 = 1)
+        bias = MatMul(b0.value, false, w1.value, tb1, rows, n, k1, alpha1 * beta0);
         bias_shape = b0.shape.size() == 1 ? std::vector<int64_t>{n} : std::vector<int64_t>{rows, n};
       }
       if (has_b1) {

@@ -39,7 +39,6 @@
 #include <mutex>
 
 #include "bz_common.h"
-#include "bz_probe.h"
 
 namespace {
 
@@ -712,39 +711,6 @@ int groups_per_wg(const bz_embed_slot& s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// measurement aid: the pooling kernel's access pattern alone (random rows of LPR 16-byte chunks, one lane a chunk)
-// ---------------------------------------------------------------------------------------------
-template <int R, int LPR>
-__global__ __launch_bounds__(kThreads) void bz_probe_gather_kernel(const uint4* __restrict__ region, uint4* __restrict__ sink,
-                                                                   const float* __restrict__ side, uint32_t rows,
-                                                                   int64_t groups, uint32_t seed) {
-  const int64_t gid = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / LPR;
-  const int l = threadIdx.x % LPR;
-  if (gid >= groups) return;
-  uint4 v[R];
-  float sc[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    uint32_t h = ((uint32_t)gid * R + r) * 2654435761u + seed;
-    h ^= h >> 15;
-    h *= 2246822519u;
-    h ^= h >> 13;
-    const uint32_t row = (uint32_t)(((uint64_t)h * rows) >> 32);  // uniform over [0, rows)
-    v[r] = region[(size_t)row * LPR + l];
-    sc[r] = side != nullptr ? side[row] : 0.f;  // every lane of the group asks for the same word: one request
-  }
-  uint4 acc = make_uint4(0, 0, 0, 0);
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    acc.x += v[r].x + __float_as_uint(sc[r]);
-    acc.y ^= v[r].y;
-    acc.z += v[r].z;
-    acc.w ^= v[r].w;
-  }
-  sink[(size_t)gid * LPR + l] = acc;
-}
-
-// ---------------------------------------------------------------------------------------------
 // scratch of the entry point that allocates nothing: every slot's offsets, inside the library's own device image
 // ---------------------------------------------------------------------------------------------
 constexpr int64_t kStaticScratchEntries = BZ_EMBED_STATIC_SCRATCH_BYTES / sizeof(int64_t);
@@ -940,39 +906,5 @@ int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_
 }
 
 const char* bz_embed_pool_kernel_name(void) { return "bz_embed_pool_kernel"; }
-
-int bz_probe_gather(const void* region, int64_t region_bytes, int row_bytes, const float* side, void* sink, int64_t groups,
-                    int rows_per_group, uint32_t seed, bz_stream_t stream) {
-  BZ_REQUIRE(region != nullptr && sink != nullptr && ((uintptr_t)region & 15) == 0 && ((uintptr_t)sink & 15) == 0,
-             "bz_probe_gather: null or misaligned buffer");
-  BZ_REQUIRE(row_bytes == 64 || row_bytes == 128, "bz_probe_gather: row_bytes=%d is not 64 or 128", row_bytes);
-  BZ_REQUIRE(region_bytes >= row_bytes, "bz_probe_gather: region_bytes=%lld", (long long)region_bytes);
-  BZ_REQUIRE(groups > 0 && groups <= (1ll << 28), "bz_probe_gather: groups=%lld outside (0, 2^28]", (long long)groups);
-  const int64_t rows = region_bytes / row_bytes;
-  BZ_REQUIRE(rows < (1ll << 32), "bz_probe_gather: region larger than 2^32 rows");
-  const int lpr = row_bytes / 16;
-  const dim3 grid((unsigned)((groups * lpr + kThreads - 1) / kThreads)), block(kThreads);
-  hipStream_t st = bz::as_stream(stream);
-  const uint4* t = (const uint4*)region;
-  uint4* out = (uint4*)sink;
-#define BZ_PROBE(R, LPR) \
-  hipLaunchKernelGGL((bz_probe_gather_kernel<R, LPR>), grid, block, 0, st, t, out, side, (uint32_t)rows, groups, seed)
-#define BZ_PROBE_R(R)      \
-  if (lpr == 4)            \
-    BZ_PROBE(R, 4);        \
-  else                     \
-    BZ_PROBE(R, 8)
-  switch (rows_per_group) {
-    case 1: BZ_PROBE_R(1); break;
-    case 4: BZ_PROBE_R(4); break;
-    case 8: BZ_PROBE_R(8); break;
-    case 16: BZ_PROBE_R(16); break;
-    default: return bz::fail(BZ_EINVAL, "bz_probe_gather: rows_per_group=%d is not 1, 4, 8 or 16", rows_per_group);
-  }
-#undef BZ_PROBE_R
-#undef BZ_PROBE
-  BZ_LAUNCH_OK("bz_probe_gather_kernel");
-  return BZ_OK;
-}
 
 }  // extern "C"

@@ -232,12 +232,8 @@ __global__ __launch_bounds__(256, 2) void bz_fc_pieces_kernel(bz::CewP p, const 
         const int rl = base + u * step;
         uint32_t row = (uint32_t)(m0 + (rl < BM ? rl : base));
         row = row < (uint32_t)M ? row : (uint32_t)M - 1;
-#ifdef BZ_OLD_DIV
-        const uint32_t i0 = row / r1, i1 = row - i0 * r1;
-#else
         uint32_t i0, i1;
         split_row(row, &i0, &i1);
-#endif
         if constexpr (XY4) {
           xs[u][0] = *(const Pack*)((const ET*)p.x[0] + (int64_t)i0 * p.xs[0][0] + (int64_t)i1 * p.xs[0][1] + cv * VEC);
           xs[u][1] = *(const Pack*)((const ET*)p.x[1] + (int64_t)i0 * p.xs[1][0] + (int64_t)i1 * p.xs[1][1] + cv * VEC);
