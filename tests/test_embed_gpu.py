@@ -422,13 +422,26 @@ def test_pooling_segment_shapes_that_stress_the_bookkeeping(bz, oracle, kind, td
     torch.cuda.synchronize()
     got = out.cpu().numpy()
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # ... with the slot records handed over as kernel arguments (bz_embed_pool_args)
+    assert plan.args_eligible()
+    out3 = torch.full_like(out, float("nan"))
+    for it in items:
+        it["out"] = out3
+    bz.EmbeddingPlan(items, fused_scan=True).pool_args()
+    torch.cuda.synchronize()
+    assert np.array_equal(out3.cpu().numpy().view(np.uint32), want.view(np.uint32))
     # ... and from offsets scanned in a launch of their own
     out2 = torch.full_like(out, float("nan"))
     for it in items:
         it["out"] = out2
-    bz.EmbeddingPlan(items, fused_scan=False).run()
+    plan2 = bz.EmbeddingPlan(items, fused_scan=False)
+    plan2.run()
     torch.cuda.synchronize()
     assert np.array_equal(out2.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    # (records with offsets of their own are not for the kernel-argument form: refused, nothing launched)
+    assert not plan2.args_eligible()
+    with pytest.raises(RuntimeError, match="bz_embed_pool_args"):
+        plan2.pool_args()
 
 
 def test_pooling_unaligned_counts_and_trailing_empty_segments(bz, oracle):

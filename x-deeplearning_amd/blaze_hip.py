@@ -20,7 +20,7 @@ ACT_NONE, ACT_PRELU, ACT_DICE, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_SOFTMAX = 0, 1, 
 
 EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
-    "bz_embed_pool", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
+    "bz_embed_pool", "bz_embed_pool_args", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
     "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
 ]
@@ -143,6 +143,7 @@ def lib():
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_static_scratch.argtypes = [vp, C.POINTER(EmbedLaunch), vp]
+        l.bz_embed_pool_args.argtypes = [C.POINTER(EmbedSlot), C.POINTER(EmbedLaunch), vp]
         l.bz_embed_pool_kernel_name.restype = C.c_char_p
         l.bz_fc_fused.argtypes = [C.POINTER(FcDesc), vp]
         l.bz_fc_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, C.c_int, i64, vp]
@@ -344,6 +345,14 @@ class EmbeddingPlan:
 
     def pool(self, stream=None):
         check(lib().bz_embed_pool(self.slots_dev.data_ptr(), C.byref(self.launch), _stream_ptr(stream)))
+
+    def args_eligible(self):
+        """what bz_embed_pool_args takes: one row shape, scan fused in, few slots"""
+        return bool(self.launch.variant != 0 and self.launch.fused_scan and not self.launch.scan_first and self.n <= 26)
+
+    def pool_args(self, stream=None):
+        """the same launch with the slot records handed over as kernel arguments"""
+        check(lib().bz_embed_pool_args(self.host, C.byref(self.launch), _stream_ptr(stream)))
 
     def run(self, stream=None):
         if not self.fused_scan:

@@ -36,6 +36,8 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <string.h>
+
 #include <mutex>
 
 #include "bz_common.h"
@@ -509,6 +511,83 @@ __device__ __forceinline__ void stage_offsets(const bz_embed_slot& s, const int6
 }
 
 // ---------------------------------------------------------------------------------------------
+// the same for the specialised kernel, where lane group g of the workgroup owns sample b0 + g: every lane ends up with
+// its own segment [start, end) in registers
+// ---------------------------------------------------------------------------------------------
+// All sums saturate at cap = nnz (< 2^31 here; larger arrays take stage_offsets): every term is >= 0, so
+// min(a + b, cap) is associative and gives the clamped offsets whatever the order of the additions, in 32 bits.
+__device__ __forceinline__ uint32_t sat_add(uint32_t a, uint32_t b, uint32_t cap) {
+  const uint32_t t = a + b;  // a, b <= cap < 2^31: no wrap
+  return t < cap ? t : cap;
+}
+
+// Inclusive scan over the 64 lanes with data-parallel primitives (row_shr within rows of 16 lanes, then lane 15 and
+// lane 31 handed on to the following rows): a dozen VALU instructions, where the same scan through ds_bpermute
+// (__shfl_up) is six dependent trips to LDS per 32 bits.
+__device__ __forceinline__ uint32_t wave_scan_sat(uint32_t v, uint32_t cap) {
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false), cap);  // row_shr:1
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false), cap);  // row_shr:2
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false), cap);  // row_shr:4
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false), cap);  // row_shr:8
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false), cap);  // row_bcast:15 -> rows 1, 3
+  v = sat_add(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false), cap);  // row_bcast:31 -> rows 2, 3
+  return v;
+}
+
+// start / end of sample b = b0 + g for every lane of lane group g (LPR lanes, g = tid / LPR); lanes of samples beyond
+// the batch get an empty segment.  Every thread of the workgroup calls it; one barrier.
+template <int LPR>
+__device__ __forceinline__ void own_segment(const bz_embed_slot& s, int64_t b0, uint32_t* s_tot, int64_t* start, int64_t* end) {
+  constexpr int WAVES = kThreads / bz::kWave;
+  const int tid = threadIdx.x;
+  const int lane = tid & (bz::kWave - 1), wave = tid / bz::kWave;
+  const int g = tid / LPR, l = tid % LPR;
+  const int64_t b = b0 + g;
+  const uint32_t cap = (uint32_t)s.nnz;
+  // this group's own count first (all its lanes ask for the same word), then the counts before b0, 8 loads in flight a
+  // thread: everything is requested before anything is used
+  const int32_t own = b < s.batch ? s.segments[b] : 0;
+  uint64_t part = 0;
+  for (int64_t i0 = 0; i0 < b0; i0 += 8 * kThreads) {
+    int32_t c[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int64_t i = i0 + k * kThreads + tid;
+      c[k] = i < b0 ? s.segments[i] : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) part += (uint32_t)max(c[k], 0);
+  }
+  const uint32_t mine = min((uint32_t)max(own, 0), cap);
+  // the group's count sits in its last lane: after the scan that lane holds the inclusive sum and the group's other
+  // lanes the exclusive one (they add nothing)
+  const uint32_t scan = wave_scan_sat(l == LPR - 1 ? mine : 0u, cap);
+  const uint32_t before_b0 = wave_scan_sat((uint32_t)(part < cap ? part : cap), cap);
+  if (lane == bz::kWave - 1) {
+    s_tot[wave] = before_b0;
+    s_tot[WAVES + wave] = scan;
+  }
+  __syncthreads();
+  uint32_t before = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    before = sat_add(before, s_tot[w], cap);
+    if (w < wave) before = sat_add(before, s_tot[WAVES + w], cap);
+  }
+  const uint32_t x = sat_add(before, scan, cap);
+  if constexpr (LPR == 1) {
+    uint32_t excl = (uint32_t)__shfl_up((int)scan, 1, bz::kWave);
+    if (lane == 0) excl = 0;
+    *start = (int64_t)sat_add(before, excl, cap);
+    *end = (int64_t)x;
+  } else {
+    const int gbase = lane - l;
+    *start = (int64_t)(uint32_t)__shfl((int)x, gbase, bz::kWave);
+    *end = (int64_t)(uint32_t)__shfl((int)x, gbase + LPR - 1, bz::kWave);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // specialised ksum / kavg kernel: every slot has table dtype DT and LPR lanes per row
 // ---------------------------------------------------------------------------------------------
 constexpr int kBlockIds = 4;  // ids walked per step (measured at 2, 4, 8, 16: 4 is best or equal on segments of 1-4, 8 and 20 ids)
@@ -517,29 +596,36 @@ constexpr int kBlockIds = 4;  // ids walked per step (measured at 2, 4, 8, 16: 4
 // 261 us fused; config 4 (26 MB) and config 2 (3 MB) stay fused.
 constexpr int64_t kScanFirstBytes = 128ll << 20;
 
+// Slot records handed over as kernel arguments: a workgroup then has its record after the one scalar load every
+// kernel starts with, instead of after a second trip to memory for slots[si] (measured on config 2: 1050 cycles from
+// the start of a wave to its kernel arguments, 2200 more to the record).
+struct SlotPack {
+  bz_embed_slot s[BZ_EMBED_ARG_SLOTS];
+};
+static_assert(sizeof(SlotPack) + 64 <= 4096, "the records and the other arguments fit the 4 KB kernel-argument segment");
+
 template <int DT, int LPR>
-__global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
-                                                                 int total_wg, int wg_per_xcd, int wg_per_slot,
-                                                                 const int64_t* __restrict__ ext_off, int64_t ext_stride) {
+__device__ __forceinline__ void pool_samples(const bz_embed_slot& s, int64_t b0, const int64_t* __restrict__ offsets) {
   constexpr int CE = RowTraits<DT>::kElems;
   constexpr int GROUPS = kThreads / LPR;
   constexpr int SRC = LPR < kBlockIds ? LPR : kBlockIds;  // lanes of a group that fetch ids
   constexpr int KPL = kBlockIds / SRC;                    // ids fetched per such lane
   __shared__ int64_t s_off[GROUPS + 1];
   __shared__ int64_t s_part[2 * kThreads / bz::kWave];
-  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
-  if (v >= total_wg) return;
-  const int si = v / wg_per_slot;
-  const bz_embed_slot s = slots[si];
   const int tid = threadIdx.x;
   const int g = tid / LPR, l = tid % LPR;
-  const int64_t b0 = (int64_t)(v - si * wg_per_slot) * GROUPS;
-  stage_offsets(s, ext_off != nullptr ? ext_off + (int64_t)si * ext_stride : s.offsets, b0, GROUPS, s_off, s_part);
+  int64_t start, end;
+  if (offsets == nullptr && s.nnz < (1ll << 31)) {
+    own_segment<LPR>(s, b0, (uint32_t*)s_part, &start, &end);
+  } else {
+    stage_offsets(s, offsets, b0, GROUPS, s_off, s_part);
+    start = s_off[g];
+    end = s_off[g + 1];
+  }
   const int64_t b = b0 + g;
   if (b >= s.batch) return;
   const int nchunks = (s.dim + CE - 1) / CE;
   const bool has_chunk = l < nchunks;
-  const int64_t start = s_off[g], end = s_off[g + 1];
   const int gbase = (tid & (bz::kWave - 1)) - l;  // first lane of this group within the wave
   const char* table = (const char*)s.table + (int64_t)l * 16;
   float acc[CE];
@@ -618,6 +704,31 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_
     const int nvalid = (s.dim - e0) < CE ? (s.dim - e0) : CE;
     store_elems<CE>(s.out, b * s.out_stride + e0, acc, nvalid, s.out_dtype);
   }
+}
+
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_kernel(const bz_embed_slot* __restrict__ slots, int n_slots,
+                                                                 int total_wg, int wg_per_xcd, int wg_per_slot,
+                                                                 const int64_t* __restrict__ ext_off, int64_t ext_stride) {
+  constexpr int GROUPS = kThreads / LPR;
+  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
+  if (v >= total_wg) return;
+  const int si = v / wg_per_slot;
+  const bz_embed_slot s = slots[si];
+  const int64_t b0 = (int64_t)(v - si * wg_per_slot) * GROUPS;
+  pool_samples<DT, LPR>(s, b0, ext_off != nullptr ? ext_off + (int64_t)si * ext_stride : s.offsets);
+}
+
+template <int DT, int LPR>
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_args_kernel(const SlotPack pack, int total_wg, int wg_per_xcd,
+                                                                      int wg_per_slot) {
+  constexpr int GROUPS = kThreads / LPR;
+  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
+  if (v >= total_wg) return;
+  const int si = v / wg_per_slot;
+  const bz_embed_slot s = pack.s[si];
+  const int64_t b0 = (int64_t)(v - si * wg_per_slot) * GROUPS;
+  pool_samples<DT, LPR>(s, b0, s.offsets);
 }
 
 __device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (dt == BZ_F16 ? 8 : 16); }
@@ -883,6 +994,49 @@ static int launch_pool(const bz_embed_slot* slots_dev, const bz_embed_launch& L,
 int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {
   BZ_REQUIRE(slots_dev != nullptr && launch != nullptr, "bz_embed_pool: null argument");
   return launch_pool(slots_dev, *launch, nullptr, 0, bz::as_stream(stream));
+}
+
+int bz_embed_pool_args(const bz_embed_slot* slots_host, const bz_embed_launch* launch, bz_stream_t stream) {
+  BZ_REQUIRE(slots_host != nullptr && launch != nullptr, "bz_embed_pool_args: null argument");
+  const bz_embed_launch& L = *launch;
+  BZ_REQUIRE(L.n_slots > 0 && L.total_wg >= 0 && L.wg_per_slot >= 0, "bz_embed_pool_args: bad launch record (n_slots=%d total_wg=%d)",
+             L.n_slots, L.total_wg);
+  if (L.variant == 0 || L.n_slots > BZ_EMBED_ARG_SLOTS || !L.fused_scan || L.scan_first)
+    return bz::fail(BZ_ENOTSUP, "bz_embed_pool_args: takes ksum / kavg plans of one row shape with at most %d slots and the scan fused in",
+                    BZ_EMBED_ARG_SLOTS);
+  BZ_REQUIRE(L.wg_per_slot > 0 && (int64_t)L.wg_per_slot * L.n_slots == L.total_wg,
+             "bz_embed_pool_args: variant %#x needs equal work per slot", L.variant);
+  if (L.total_wg == 0) return BZ_OK;
+  SlotPack pack;
+  memcpy(pack.s, slots_host, (size_t)L.n_slots * sizeof(bz_embed_slot));
+  memset(pack.s + L.n_slots, 0, (size_t)(BZ_EMBED_ARG_SLOTS - L.n_slots) * sizeof(bz_embed_slot));
+  const int per_xcd = (L.total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
+  const dim3 grid(per_xcd * bz::kNumXcd), block(kThreads);
+  hipStream_t st = bz::as_stream(stream);
+  const int dt = L.variant >> 8, lpr = L.variant & 0xff;
+#define BZ_POOL(DT, LPR) \
+  hipLaunchKernelGGL((bz_embed_pool_args_kernel<DT, LPR>), grid, block, 0, st, pack, L.total_wg, per_xcd, L.wg_per_slot)
+#define BZ_POOL_LPR(DT)                                                                           \
+  switch (lpr) {                                                                                  \
+    case 1: BZ_POOL(DT, 1); break;                                                                \
+    case 2: BZ_POOL(DT, 2); break;                                                                \
+    case 4: BZ_POOL(DT, 4); break;                                                                \
+    case 8: BZ_POOL(DT, 8); break;                                                                \
+    case 16: BZ_POOL(DT, 16); break;                                                              \
+    case 32: BZ_POOL(DT, 32); break;                                                              \
+    case 64: BZ_POOL(DT, 64); break;                                                              \
+    default: return bz::fail(BZ_EINVAL, "bz_embed_pool_args: bad lanes-per-row %d in variant", lpr); \
+  }
+  switch (dt) {
+    case BZ_F32: BZ_POOL_LPR(BZ_F32); break;
+    case BZ_F16: BZ_POOL_LPR(BZ_F16); break;
+    case BZ_I8: BZ_POOL_LPR(BZ_I8); break;
+    default: return bz::fail(BZ_EINVAL, "bz_embed_pool_args: bad table dtype %d in variant", dt);
+  }
+#undef BZ_POOL_LPR
+#undef BZ_POOL
+  BZ_LAUNCH_OK("bz_embed_pool_args_kernel");
+  return BZ_OK;
 }
 
 int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream) {

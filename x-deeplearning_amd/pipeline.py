@@ -96,7 +96,10 @@ class CtrForward:
 
     def pool(self, i, st=None):
         p = self.steps[i % self.n_batches]["plan"]
-        bz.check(self.lib.bz_embed_pool(p.slots_dev.data_ptr(), C.byref(p.launch), st or self._stream()))
+        if p.args_eligible():  # as the Embedding operator launches it: the slot records travel as kernel arguments
+            bz.check(self.lib.bz_embed_pool_args(p.host, C.byref(p.launch), st or self._stream()))
+        else:
+            bz.check(self.lib.bz_embed_pool(p.slots_dev.data_ptr(), C.byref(p.launch), st or self._stream()))
 
     def fc(self, i, layer, st=None):
         d = self.steps[i % self.n_batches]["descs"][layer]
