@@ -12,7 +12,10 @@ deployed (blaze/example/cpp/predictor_example.cc:129-140,189).  Prints ONE JSON 
   value / ms_per_step     exactly K steps after the warm-up (every predictor has run at least twice before the clock
                           starts, whatever W says: W is a floor);
   steady_state            the same loop over a fixed number of steps (>= 2000), so a short K does not hide the rate;
-  p50_ms / p99_ms         one request at a time on one thread, over max(K, 1000) forwards;
+  p50_ms / p99_ms         latency of a request under the load of the steady-state run: every pass of that run, from the
+                          start of its launch to the return of its wait on its serving thread (latency_by_load: the
+                          throughput / latency pairs at one and two passes queued per thread and at fewer threads; latency_unloaded: one
+                          request at a time on one thread, over max(K, 1000) forwards);
   with_host_feed          every step feeds all inputs from host memory and copies the output back (PCIe inclusive);
   roofline                the pooling kernel: algorithmic bytes per launch / average launch duration (HIP events
                           around a replayed graph of back-to-back launches over the pooled batches);
@@ -90,6 +93,16 @@ def latency_ms(np, step, n):
     return float(lat[n // 2]), float(lat[min(n - 1, int(n * 0.99))]), n
 
 
+def latency_stats(np, lat_ms):
+    """p50 / p99 / mean of a set of per-pass latencies (ms)"""
+    lat = np.sort(np.asarray(lat_ms, dtype=np.float64))
+    n = len(lat)
+    if n == 0:
+        return None
+    return {"p50_ms": round(float(lat[n // 2]), 4), "p99_ms": round(float(lat[min(n - 1, int(n * 0.99))]), 4),
+            "mean_ms": round(float(lat.mean()), 4), "samples": n}
+
+
 def hbm_roofline(kernel, alg_bytes, us, traffic=None):
     gbs = alg_bytes / us / 1e3
     return {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -132,9 +145,12 @@ def bench_predictor_model(np, torch, pb, predictors, batch, threads, steps, lat_
     pool.run(predictors, steps)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    loaded = latency_stats(np, pool.latencies_ms())  # every pass of that run, launch to the return of its wait
     p50, p99, n = latency_ms(np, lambda i: predictors[i % len(predictors)].forward(), lat_steps)
     return {"samples/s": round(batch * steps / (t1 - t0), 1), "ms_per_step": round((t1 - t0) * 1e3 / steps, 5), "steps": steps,
-            "serving_threads": T, "p50_ms": round(p50, 4), "p99_ms": round(p99, 4), "latency_samples": n}
+            "serving_threads": T, "p50_ms": loaded["p50_ms"], "p99_ms": loaded["p99_ms"], "latency_samples": loaded["samples"],
+            "unloaded": {"p50_ms": round(p50, 4), "p99_ms": round(p99, 4), "latency_samples": n,
+                         "note": "one request at a time on one thread"}}
 
 
 def count_launches(p):
@@ -180,7 +196,7 @@ def bench_config1(np, torch, bz, pb, threads):
     return res
 
 
-def bench_config3(np, torch, pb, threads):
+def bench_config3(np, torch, bz, pb, threads):
     import din_model
     cfg = din_model.Config3()
     tables, weights = cfg.tables(), cfg.weights()
@@ -206,6 +222,28 @@ def bench_config3(np, torch, pb, threads):
     res["operators"] = ran
     res["fc_flops"] = int(2 * B * T * sum(att[i] * att[i + 1] for i in range(3)) + 2 * B * sum(main[i] * main[i + 1] for i in range(3)))
     res["attention_bgemm_bytes"] = B * T * D3 * 2 + B * T * 4 + B * D3 * 2
+    # the two kernels of the attention block alone, through the kernel layer on operands of the model's shapes (two
+    # sets, alternating): the attention MLP [q, k, q-k, q*k] -> 80 -> 40 -> 1 as one launch, and the attention tail
+    # (score * mask, weighted sum over the history, plain sum) as one launch
+    g = torch.Generator(device="cuda").manual_seed(33)
+    rnd = lambda *shape: torch.randn(shape, generator=g, device="cuda")
+    sets = []
+    for _ in range(2):
+        q, k = rnd(B, 1, D3).half(), rnd(B, T, D3).half()
+        ws = [bz.pack_weight(rnd(att[i], att[i + 1]).half() / att[i] ** 0.5, False, bz.F16) for i in range(3)]
+        bs = [rnd(att[i + 1]) * 0.1 for i in range(3)]
+        dice = [(rnd(att[i + 1]) * 0.1, rnd(att[i + 1]) * 0.1, torch.rand(att[i + 1], generator=g, device="cuda") + 0.5) for i in range(2)]
+        score = torch.empty((B * T, 1), dtype=torch.float32, device="cuda")
+        mlp = bz.AttentionMlp(q, k, ws[0], bs[0], dice[0], ws[1], bs[1], dice[1], ws[2], bs[2], score)
+        w16 = rnd(B, T, 1).half()
+        mask = (torch.rand((B, T, 1), generator=g, device="cuda") < 0.5).half()
+        sets.append((mlp, k, w16, mask))
+    mlp_us = graph_timed(torch, lambda i: sets[i % 2][0].run(), 2, 16, warm_ms=20.0)
+    tail_us = graph_timed(torch, lambda i: bz.weighted_pool(sets[i % 2][1], sets[i % 2][2], sets[i % 2][3]), 2, 16, warm_ms=20.0)
+    res["roofline_attention_mlp"] = mfma_roofline("bz_fc_pieces_kernel (%dx%d: %d->%d->%d->%d)" % (B, T, att[0], att[1], att[2], att[3]),
+                                                  sets[0][0].flops, mlp_us)
+    res["roofline_attention_tail"] = hbm_roofline("bz_weighted_pool_kernel (history read once; scores and mask in, weighted sum and plain sum out)",
+                                                  B * T * D3 * 2 + 2 * B * T * 2 + 2 * B * D3 * 2, tail_us)
     return res
 
 
@@ -381,6 +419,9 @@ def main():
     ap.add_argument("--threads", type=int, default=8,
                     help="serving threads, each with its own Predictors and HIP stream (the reference's model: one "
                          "Predictor per thread, blaze/api/cpp_api/predictor.h:90-92)")
+    ap.add_argument("--depth", type=int, default=1,
+                    help="passes a serving thread keeps queued on its stream (1 = a plain synchronous Forward per request, as "
+                         "the reference's serving loop; with 8 threads 2 gives 1 %% more throughput at twice the latency)")
     ap.add_argument("--kernel-api", action="store_true",
                     help="drive the kernel-layer C ABI directly instead of Predictor.Forward (lower host overhead)")
     args = ap.parse_args()
@@ -421,7 +462,7 @@ def main():
     warm = max(W, 2 * NB)  # W is a floor: every predictor runs at least twice before the clock starts
 
     predictors = None
-    steady = feed_rate = None
+    steady = feed_rate = loaded = by_depth = None
     if not args.kernel_api:
         # the drop-in path: one Predictor per pooled batch (inputs fed once = resident in HBM), Forward through
         # the Blaze_* C ABI; consecutive steps go round robin over T serving threads
@@ -450,7 +491,7 @@ def main():
     # driven by the library's own serving threads (Blaze_ServePool*: a C++ loop per thread, as a serving binary
     # would run it); the kernel-layer path by Python threads.
     if predictors is not None:
-        pool = pb.ServePool(T)
+        pool = pb.ServePool(T, args.depth)
         pool.run(predictors, warm)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -463,6 +504,24 @@ def main():
             pool.run(predictors, S)
         torch.cuda.synchronize()
         ds = time.perf_counter() - s0
+        if not args.counters_run:
+            # latency under load: every pass of the steady-state run, from the start of its launch to the return of its
+            # wait on its serving thread; then the (throughput, latency) pair at one and at two passes queued per thread
+            loaded = latency_stats(np, pool.latencies_ms())
+            by_depth = {}
+            points = [(t, 1) for t in (1, 2, 4) if t < T and NB % t == 0] + [(T, 1), (T, 2)]
+            for threads_, depth in points:
+                dp = pb.ServePool(threads_, depth)
+                dp.run(predictors, 2 * NB)
+                torch.cuda.synchronize()
+                d0 = time.perf_counter()
+                dp.run(predictors, S // 2)
+                torch.cuda.synchronize()
+                d1 = time.perf_counter()
+                st = latency_stats(np, dp.latencies_ms())
+                st["samples/s"] = round(cfg.batch * (S // 2) / (d1 - d0), 1)
+                by_depth["threads_%d_depth_%d" % (threads_, depth)] = st
+                del dp
     else:
         def run_region(first, count):
             start = threading.Barrier(T + 1)
@@ -560,7 +619,7 @@ def main():
     per_config = None
     if not args.no_per_config:
         per_config = {}
-        for key, fn in (("c1", lambda: bench_config1(np, torch, bz, pb, T)), ("c3", lambda: bench_config3(np, torch, pb, T)),
+        for key, fn in (("c1", lambda: bench_config1(np, torch, bz, pb, T)), ("c3", lambda: bench_config3(np, torch, bz, pb, T)),
                         ("c4", lambda: bench_config4(np, torch, bz)), ("c5", lambda: bench_config5(np, torch, bz))):
             try:
                 per_config[key] = fn()
@@ -580,9 +639,15 @@ def main():
         "warmup_run": warm,
         "ms_per_step": round(ms_per_step, 5),
         "steady_state": steady,
-        "p50_ms": round(p50, 4),
-        "p99_ms": round(p99, 4),
-        "latency_samples": n_lat,
+        # latency of a request under the load that `steady_state` is measured at (every pass of that run); without that
+        # run (--counters-run, --kernel-api) the unloaded figure
+        "p50_ms": loaded["p50_ms"] if loaded else round(p50, 4),
+        "p99_ms": loaded["p99_ms"] if loaded else round(p99, 4),
+        "latency_samples": loaded["samples"] if loaded else n_lat,
+        "latency_at": ("steady_state: %d serving threads, %d pass(es) queued per thread" % (T, args.depth)) if loaded else "one request at a time",
+        "latency_by_load": by_depth,
+        "latency_unloaded": {"p50_ms": round(p50, 4), "p99_ms": round(p99, 4), "samples": n_lat,
+                             "note": "one request at a time on one thread"},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -591,7 +656,7 @@ def main():
         "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
                    "batch_pool": NB,
                    "path": "kernel-layer C ABI (bz_*)" if predictors is None else "Predictor.Forward via Blaze_* C ABI",
-                   "serving_threads": T,
+                   "serving_threads": T, "passes_queued_per_thread": args.depth,
                    "device": arch},
         "roofline": roofline,
         "embedding_pool": {"GB/s": round(pool_gbs, 1), "frac_of_hbm_peak": round(pool_gbs / HBM_PEAK_GBS, 5),

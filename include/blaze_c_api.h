@@ -153,6 +153,13 @@ typedef void* ServePoolHandle;
 BLAZE_API int Blaze_ServePoolCreate(int n_threads, ServePoolHandle* handle);
 BLAZE_API int Blaze_ServePoolRun(ServePoolHandle handle, PredictorHandle* predictors, int n_predictors, int64_t steps);
 BLAZE_API int Blaze_ServePoolSetDepth(ServePoolHandle handle, int depth);
+/*
+ * What every pass of the last Blaze_ServePoolRun took on its thread, from the start of its launch to the return of its
+ * wait, in milliseconds: the latency of a request under that job's load (the reference's example times each Forward
+ * inside its serving loop, blaze/example/cpp/predictor_example.cc:129-140).  Writes at most `capacity` values, thread
+ * after thread, and the number there are to *count.
+ */
+BLAZE_API int Blaze_ServePoolLatencies(ServePoolHandle handle, float* out_ms, int64_t capacity, int64_t* count);
 BLAZE_API int Blaze_ServePoolDelete(ServePoolHandle handle);
 
 #ifdef __cplusplus

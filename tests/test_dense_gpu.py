@@ -514,19 +514,7 @@ def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T,
 
 
 def _pieces_desc(bz, pieces, r0, r1, tdt):
-    """bz_concat_ew_desc of (op, x, y) pieces with operands [r0 | 1, r1 | 1, w] (as blaze_hip.concat_ew builds it), without dst"""
-    d = bz.ConcatEwDesc()
-    d.n, d.dtype, d.r0, d.r1 = len(pieces), bz.bz_dtype(tdt), r0, r1
-    for i, (op, x, y) in enumerate(pieces):
-        d.op[i], d.width[i], d.x[i] = op, x.shape[2], x.data_ptr()
-        for name, t in (("x_stride", x), ("y_stride", y)):
-            if t is None:
-                continue
-            getattr(d, name)[i][0] = 0 if t.shape[0] == 1 and r0 > 1 else t.shape[1] * t.shape[2]
-            getattr(d, name)[i][1] = 0 if t.shape[1] == 1 and r1 > 1 else t.shape[2]
-        if y is not None:
-            d.y[i] = y.data_ptr()
-    return d
+    return bz.pieces_desc(pieces, r0, r1, bz.bz_dtype(tdt))
 
 
 @pytest.mark.parametrize("in_name,out_name", [("f16", "f16"), ("bf16", "bf16"), ("f16", "f32")])

@@ -399,6 +399,9 @@ def test_forward_in_two_halves_and_serve_pool_match_plain_forward(pb):
         torch.cuda.synchronize()
         for b in range(4):
             np.testing.assert_array_equal(preds[b].output_asnumpy("prob"), want[b])
+        # one latency per pass of the job (launch to the return of its wait), positive and well under a second
+        lat = pool.latencies_ms()
+        assert lat.shape == (steps, ) and (steps == 0 or (lat.min() > 0 and lat.max() < 1000.0)), lat
         del pool
     with pytest.raises(pb.BlazeError, match="multiple of the pool's threads"):
         pb.ServePool(3).run(preds, 4)

@@ -540,6 +540,56 @@ def concat_ew(pieces, stream=None):
     return out
 
 
+def pieces_desc(pieces, r0, r1, dtype):
+    """bz_concat_ew_desc (without a destination) of (op, x, y) pieces with operands [r0 | 1, r1 | 1, w]: what
+    bz_fc_desc.a_pieces takes"""
+    d = ConcatEwDesc()
+    d.n, d.dtype, d.r0, d.r1 = len(pieces), dtype, r0, r1
+    for i, (op, x, y) in enumerate(pieces):
+        d.op[i], d.width[i], d.x[i] = op, x.shape[2], x.data_ptr()
+        for name, t in (("x_stride", x), ("y_stride", y)):
+            if t is None:
+                continue
+            getattr(d, name)[i][0] = 0 if t.shape[0] == 1 and r0 > 1 else t.shape[1] * t.shape[2]
+            getattr(d, name)[i][1] = 0 if t.shape[1] == 1 and r1 > 1 else t.shape[2]
+        if y is not None:
+            d.y[i] = y.data_ptr()
+    return d
+
+
+class AttentionMlp:
+    """DIN's attention MLP as ONE bz_fc_fused launch (a_pieces + next + head): rows [q, k, q - k, q * k] of a history
+    k [r0, r1, w] against a target q [r0, 1, w] -> layer 1 + Dice -> layer 2 + Dice -> a skinny head into `out`
+    [r0 * r1, n3] (fp32).  Weights are packed [n, ld] tensors (pack_weight), biases and Dice triples fp32."""
+
+    def __init__(self, q, k, w1, b1, dice1, w2, b2, dice2, w3, b3, out, head_act=ACT_NONE):
+        r0, r1, w = k.shape
+        self.keep = (q, k, w1, b1, dice1, w2, b2, dice2, w3, b3, out)
+        dt = bz_dtype(k.dtype)
+        self.pieces = pieces_desc([(EW_ASSIGN, q, None), (EW_ASSIGN, k, None), (EW_SUB, q, k), (EW_MUL, q, k)], r0, r1, dt)
+        nx = self.next = FcNext()
+        nx.w, nx.ldw, nx.n, nx.bias = w2.data_ptr(), w2.stride(0), w2.shape[0], b2.data_ptr()
+        nx.alpha = nx.beta = 1.0
+        nx.act, nx.act_size = ACT_DICE, w2.shape[0]
+        nx.act_p0, nx.act_p1, nx.act_p2 = (t.data_ptr() for t in dice2)
+        d = self.desc = FcDesc()
+        d.a_pieces = C.cast(C.pointer(self.pieces), C.c_void_p)
+        d.next = C.cast(C.pointer(nx), C.c_void_p)
+        d.w, d.ldw, d.bias = w1.data_ptr(), w1.stride(0), b1.data_ptr()
+        d.m, d.n, d.k, d.ldy = r0 * r1, w1.shape[0], 4 * w, w1.shape[0]
+        d.in_dtype = d.out_dtype = dt
+        d.bias_rows, d.alpha, d.beta = 1, 1.0, 1.0
+        d.act, d.act_size = ACT_DICE, w1.shape[0]
+        d.act_p0, d.act_p1, d.act_p2 = (t.data_ptr() for t in dice1)
+        d.head_w, d.head_ldw, d.head_bias = w3.data_ptr(), w3.stride(0), b3.data_ptr()
+        d.head_y, d.head_ldy, d.head_n = out.data_ptr(), out.stride(0), w3.shape[0]
+        d.head_act, d.head_out_dtype = head_act, bz_dtype(out.dtype)
+        self.flops = 2.0 * r0 * r1 * (4 * w * w1.shape[0] + w1.shape[0] * w2.shape[0] + w2.shape[0] * w3.shape[0])
+
+    def run(self, stream=None):
+        check(lib().bz_fc_fused(C.byref(self.desc), _stream_ptr(stream)))
+
+
 def reduce_sum(x, axis, keepdims=True, stream=None):
     import torch
     outer = int(np.prod(x.shape[:axis], dtype=np.int64))

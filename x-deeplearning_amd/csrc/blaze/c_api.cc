@@ -222,8 +222,12 @@ struct ServePool {
   int depth = 2;  // passes a thread keeps queued on its stream
   std::atomic<int> failed{0};
   std::string error;
+  // what every pass of the last job took on its thread, launch to "the wait has returned" (milliseconds): the latency a
+  // request sees under the load of that job, as the reference's example times each Forward inside its serving loop
+  // (example/cpp/predictor_example.cc:129-140)
+  std::vector<std::vector<float>> latency_ms;
 
-  explicit ServePool(int n) {
+  explicit ServePool(int n) : latency_ms(n) {
     for (int t = 0; t < n; ++t) threads.emplace_back([this, t] { Loop(t); });
   }
   ~ServePool() {
@@ -262,18 +266,31 @@ struct ServePool {
           error = blaze::last_error_for_thread();
         }
       };
+      using Clock = std::chrono::steady_clock;
+      std::vector<float>& lat = latency_ms[t];
+      lat.clear();
+      lat.reserve((size_t)std::min<int64_t>(steps / n_threads + 1, 1 << 22));
+      auto record = [&](Clock::time_point from) {
+        if (lat.size() < lat.capacity()) lat.push_back(std::chrono::duration<float, std::milli>(Clock::now() - from).count());
+      };
       if (d == 1) {
-        for (int64_t i = t; i < steps && !failed.load(std::memory_order_relaxed); i += n_threads)
+        for (int64_t i = t; i < steps && !failed.load(std::memory_order_relaxed); i += n_threads) {
+          const auto t0 = Clock::now();
           if (!handles[i % n_handles]->Forward()) fail();
+          record(t0);
+        }
       } else {
+        Clock::time_point began[64];  // launch times of the passes in flight (depth <= 64)
         int64_t launched = t, waited = t;  // next step to launch / to wait for
         while (waited < steps) {
           while (launched < steps && (launched - waited) / n_threads < d && !failed.load(std::memory_order_relaxed)) {
+            began[(launched / n_threads) % 64] = Clock::now();
             if (!handles[launched % n_handles]->ForwardLaunch()) fail();
             launched += n_threads;
           }
           if (waited >= launched) break;  // a failure stopped the launches
           if (!handles[waited % n_handles]->ForwardWait()) fail();
+          record(began[(waited / n_threads) % 64]);
           waited += n_threads;
         }
       }
@@ -329,6 +346,20 @@ int Blaze_ServePoolSetDepth(ServePoolHandle handle, int depth) {
   if (pool == nullptr || depth < 1 || depth > 64) return Fail("ServePoolSetDepth: bad arguments");
   std::lock_guard<std::mutex> lock(pool->mu);
   pool->depth = depth;
+  return 0;
+}
+int Blaze_ServePoolLatencies(ServePoolHandle handle, float* out_ms, int64_t capacity, int64_t* count) {
+  auto* pool = reinterpret_cast<ServePool*>(handle);
+  if (pool == nullptr || count == nullptr || capacity < 0 || (capacity > 0 && out_ms == nullptr))
+    return Fail("ServePoolLatencies: bad arguments");
+  std::lock_guard<std::mutex> lock(pool->mu);  // (no job is running: Run returns only when its threads are done)
+  int64_t n = 0;
+  for (const auto& v : pool->latency_ms)
+    for (float x : v) {
+      if (n < capacity) out_ms[n] = x;
+      ++n;
+    }
+  *count = n;
   return 0;
 }
 int Blaze_PredictorForwardLaunch(PredictorHandle handle) {

@@ -28,7 +28,7 @@ EXPORTS = [
     "Blaze_ConvertBlaze", "Blaze_OptimizeBlaze", "Blaze_QuickEmbeddingBuildFp32", "Blaze_QuickEmbeddingBuildFp16",
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
-    "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_PredictorForwardLaunch",
+    "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_ServePoolLatencies", "Blaze_PredictorForwardLaunch",
     "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount"
 ]
 
@@ -85,6 +85,7 @@ def lib():
         l.Blaze_ServePoolRun.argtypes = [vp, C.POINTER(vp), i, C.c_int64]
         l.Blaze_ServePoolDelete.argtypes = [vp]
         l.Blaze_ServePoolSetDepth.argtypes = [vp, i]
+        l.Blaze_ServePoolLatencies.argtypes = [vp, C.POINTER(C.c_float), C.c_int64, C.POINTER(C.c_int64)]
         l.Blaze_PredictorForwardLaunch.argtypes = [vp]
         l.Blaze_PredictorForwardWait.argtypes = [vp]
         l.Blaze_PredictorFeedMany.argtypes = [vp, i, C.POINTER(C.c_char_p), C.POINTER(vp), C.POINTER(C.c_size_t)]
@@ -252,6 +253,17 @@ class ServePool(object):
     def run(self, predictors, steps):
         arr = (C.c_void_p * len(predictors))(*[getattr(p.handle, "value", p.handle) for p in predictors])
         check_call(lib().Blaze_ServePoolRun(self.handle, arr, len(predictors), steps))
+
+    def set_depth(self, depth):
+        check_call(lib().Blaze_ServePoolSetDepth(self.handle, depth))
+
+    def latencies_ms(self):
+        """per-pass latency (launch to the return of the wait) of the last run, all threads, as a float32 array"""
+        n = C.c_int64(0)
+        check_call(lib().Blaze_ServePoolLatencies(self.handle, None, 0, C.byref(n)))
+        out = np.empty(n.value, np.float32)
+        check_call(lib().Blaze_ServePoolLatencies(self.handle, out.ctypes.data_as(C.POINTER(C.c_float)), n.value, C.byref(n)))
+        return out
 
 
 class PredictorManager(object):
