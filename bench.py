@@ -138,7 +138,7 @@ def calibration_copy(torch, bz):
 def bench_predictor_model(np, torch, pb, predictors, batch, threads, steps, lat_steps):
     """samples/s over `threads` serving threads + single-request latency of a list of fed predictors."""
     T = threads
-    pool = pb.ServePool(T)
+    pool = pb.ServePool(T, 1)  # a plain synchronous Forward per request on every thread
     pool.run(predictors, 2 * len(predictors))
     torch.cuda.synchronize()
     t0 = time.perf_counter()

@@ -550,6 +550,15 @@ BZ_API int bz_batch_norm(const bz_bn_desc* desc, bz_stream_t stream);
  */
 BZ_API int bz_softmax_axis(const void* x, void* y, int64_t outer, int64_t c, int64_t inner, int dtype, bz_stream_t stream);
 
+/*
+ * Gather along one axis of a contiguous [outer, axis_size, inner] tensor: y[o, j, :] = data[o, indices[j], :] for j <
+ * n_indices, rows of inner_bytes bytes (blaze/operator/op/gather_op.h:25-87, gather_op.cc:9-21: one memcpy per index).
+ * indices are BZ_I32 or BZ_I64 (ID_TYPE_SWITCH there).  An index outside [0, axis_size), which the reference's memcpy
+ * would read out of bounds, gives a row of zeros.
+ */
+BZ_API int bz_gather_rows(const void* data, const void* indices, int index_dtype, void* y, int64_t outer, int64_t axis_size,
+                          int64_t inner_bytes, int64_t n_indices, bz_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

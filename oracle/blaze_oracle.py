@@ -498,6 +498,47 @@ def split(x, n_out, axis=1, splits=None):
     return [y.reshape(x.shape[:axis] + (s, ) + x.shape[axis + 1:]) for y, s in zip(ys, splits)]
 
 
+def gather(data, indices, axis=0):
+    """Gather op (operator/op/gather_op.h:45-84, gather_op.cc:9-21): output shape = data.shape[:axis] + indices.shape +
+    data.shape[axis+1:]; for every outer index i and every index j a memcpy of inner_size values from
+    data + (i * axis_size + indices[j]) * inner_size to y + i * y_inner_size + j * inner_size."""
+    data = np.ascontiguousarray(data)
+    indices = np.asarray(indices)
+    assert np.issubdtype(indices.dtype, np.integer), "indices->data_type()"
+    axis_size = data.shape[axis]
+    inner = int(np.prod(data.shape[axis + 1:], dtype=np.int64))
+    o_shape = list(data.shape[:axis]) + list(indices.shape) + list(data.shape[axis + 1:])
+    y_inner = int(indices.size) * inner
+    y = np.empty(o_shape, data.dtype)
+    outer = y.size // y_inner if y_inner else 0
+    src, dst, idx = data.reshape(-1), y.reshape(-1), indices.reshape(-1)
+    for i in range(outer):
+        so, do = i * axis_size * inner, i * y_inner
+        for j in range(idx.size):
+            dst[do + j * inner:do + (j + 1) * inner] = src[so + int(idx[j]) * inner:so + (int(idx[j]) + 1) * inner]
+    return y
+
+
+def slice_axis(x, axis=0, start=0, end=1):
+    """Slice op (operator/op/slice_op.h:36-110, slice_op.cc:9-29): one axis, [start, end); outer_size memcpys of
+    (end - start) * inner_size values, source advancing size * inner_size, destination (end - start) * inner_size."""
+    x = np.ascontiguousarray(x)
+    assert start < end and axis < x.ndim and end <= x.shape[axis]
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    size = x.shape[axis]
+    shape = list(x.shape)
+    shape[axis] = end - start
+    y = np.empty(shape, x.dtype)
+    src, dst = x.reshape(-1), y.reshape(-1)
+    x_off, y_off, n = start * inner, 0, (end - start) * inner
+    for _ in range(outer):
+        dst[y_off:y_off + n] = src[x_off:x_off + n]
+        x_off += size * inner
+        y_off += n
+    return y
+
+
 def reduce_sum(x, axis=0, keepdims=1):
     """ReduceSum op (operator/op/reduce_sum_op.h:17-58)."""
     x = _f32(x)

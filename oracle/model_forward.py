@@ -82,3 +82,74 @@ def din_forward(oracle, cfg, tables_np, weights, batch, rnd):
     logit = rnd(x)
     return dict(q=q, his=his, att_in=None, score=score, att=att, hsum=hsum, main_in=main_in, logit=logit,
                 prob=oracle.softmax(logit, 1))
+
+
+def _arg(op, name, default=None):
+    for a in op.arg:
+        if a.name == name:
+            if a.HasField("i"):
+                return a.i
+            if a.HasField("f"):
+                return a.f
+            if a.HasField("s"):
+                return a.s
+            if len(a.ints):
+                return list(a.ints)
+            if len(a.floats):
+                return list(a.floats)
+    return default
+
+
+def run_netdef(oracle, net, feeds, tables):
+    """An operator-by-operator forward of a parsed NetDef (a protobuf message with .op[].type/.input/.output/.arg) on
+    the oracle's functions, in the order the reference's SimpleNet runs it (blaze/graph/simple_net.cc:35-46).  feeds:
+    {external input name: numpy array}; tables: {table name: oracle.Table}.  Covers the operator set of the reference's
+    shipped example model (blaze/example/tdm_data/model_blaze_optimized): Embedding with one pooled item per operator,
+    Gather, Concat, Reshape, Slice, ReduceSum, Div, Gemm, BatchNormalization, PRelu, Softmax, ConstantFill.  Arguments are
+    read as the reference's operators read them -- in particular Slice knows `start` / `end`, `starts` / `ends`, `axis` /
+    `axes` (slice_op.h:36-62) and ignores any other name.  -> {tensor name: numpy array}."""
+    import re
+    t = dict(feeds)
+    np_dtype = {1: np.float32, 2: np.int32, 10: np.int64}
+    for op in net.op:
+        ins = [t[name] for name in op.input]
+        ty = op.type
+        if ty == "ConstantFill":
+            dt = np_dtype[_arg(op, "dtype", 1)]
+            y = np.array(_arg(op, "value"), dt).reshape(_arg(op, "shape"))
+        elif ty == "Embedding":
+            cfg = _arg(op, "embedding_config").decode()
+            table, dim = re.search(r'table_name: "([^"]+)"', cfg).group(1), int(re.search(r"dim: (\d+)", cfg).group(1))
+            udf = int(re.search(r"udf_type: (\d+)", cfg).group(1))
+            assert len(re.findall("embedding_block_config_item", cfg)) == 1 and udf in (0, 1)
+            ids, values, segments = ins
+            y = np.zeros((segments.size, dim), np.float32)
+            oracle.embed_get(tables.get(table), ids, values, segments, [(udf, 0, 0, y, 0)])
+        elif ty == "Gather":
+            y = oracle.gather(ins[0], ins[1], _arg(op, "axis", 0))
+        elif ty == "Concat":
+            y = oracle.concat(ins, _arg(op, "axis", 1))
+        elif ty == "Reshape":
+            y = oracle.reshape(ins[0], [int(v) for v in ins[1].reshape(-1)])
+        elif ty == "Slice":
+            axes, starts, ends = _arg(op, "axes"), _arg(op, "starts"), _arg(op, "ends")
+            axis = axes[0] if axes is not None else _arg(op, "axis", 0)
+            start, end = (starts[0], ends[0]) if starts is not None else (_arg(op, "start", 0), _arg(op, "end", 1))
+            y = oracle.slice_axis(ins[0], axis, start, end)
+        elif ty == "ReduceSum":
+            y = oracle.reduce_sum(ins[0], _arg(op, "axis", 0), _arg(op, "keepdims", 1))
+        elif ty in ("Add", "Sub", "Mul", "Div"):
+            y = oracle.elementwise(ty, ins[0], ins[1])
+        elif ty == "Gemm":
+            y = oracle.gemm_op(ins[0], ins[1], ins[2] if len(ins) > 2 else None, bool(_arg(op, "transA", 0)),
+                               bool(_arg(op, "transB", 0)), _arg(op, "alpha", 1.0), _arg(op, "beta", 1.0))
+        elif ty == "BatchNormalization":
+            y = oracle.batch_norm(ins[0], ins[1], ins[2], ins[3], ins[4], _arg(op, "eps", 0.001), bool(_arg(op, "nosqrt", 0)))
+        elif ty == "PRelu":
+            y = oracle.prelu(ins[0], ins[1])
+        elif ty == "Softmax":
+            y = oracle.softmax(ins[0], _arg(op, "axis", 1))
+        else:
+            raise KeyError("run_netdef: no oracle for operator " + ty)
+        t[op.output[0]] = y
+    return t

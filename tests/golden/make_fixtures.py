@@ -66,6 +66,9 @@ CASES = [
     "op/elementwise/elementwise_where_net_v1_cpu.conf",
     "op/split/split_net_v1_cpu.conf",
     "op/split/split_net_v2_cpu.conf",
+    "op/gather/gather_net_v1_cpu.conf",
+    "op/gather/gather_net_v2_cpu.conf",
+    "op/slice/slice_net_v1_cpu.conf",
 ]
 
 _TOK = re.compile(r'\s*(?:(#[^\n]*)|("(?:\\.|[^"\\])*")|([{}:])|([^\s{}:"#]+))')

@@ -59,6 +59,10 @@ def _run_op(oracle, case):
         return oracle.fuse(ins[0], ins[1], a.get("comm_index", 0))
     if ty == "Reshape":
         return oracle.reshape(ins[0], [int(v) for v in ins[1].reshape(-1)])
+    if ty == "Gather":
+        return oracle.gather(ins[0], ins[1], a.get("axis", 0))
+    if ty == "Slice":
+        return oracle.slice_axis(ins[0], a.get("axis", 0), a.get("start", 0), a.get("end", 1))
     if ty == "BatchNormalization":
         return oracle.batch_norm(ins[0], ins[1], ins[2], ins[3], ins[4], a.get("eps", 0.001), bool(a.get("nosqrt", 0)))
     raise KeyError(ty)
@@ -69,7 +73,8 @@ SHAPE_CASES = [
     "reshape_net_v1_cpu", "batch_normalization_net_v1_cpu", "elementwise_add_net_v1_cpu", "elementwise_add_net_v2_cpu",
     "elementwise_sub_net_v1_cpu", "elementwise_sub_net_v2_cpu", "elementwise_mul_net_v1_cpu", "elementwise_mul_net_v2_cpu",
     "elementwise_div_net_v1_cpu", "elementwise_div_net_v2_cpu", "elementwise_broadcast_to_net_v1_cpu",
-    "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu"
+    "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu", "gather_net_v1_cpu", "gather_net_v2_cpu",
+    "slice_net_v1_cpu"
 ]
 
 DENSE_CASES = SHAPE_CASES + [
@@ -88,6 +93,23 @@ def test_reference_dense_kat(oracle, kats, name):
     want = np.array(exp["values"], np.float32).reshape(exp["shape"])
     assert list(got.shape) == exp["shape"]
     np.testing.assert_allclose(got, want, rtol=0, atol=ATOL_KAT)
+
+
+def test_gather_and_slice_closed_forms(oracle):
+    """oracle.gather / oracle.slice_axis (restated memcpy loops) against numpy's take and basic slicing on every axis,
+    indices of both integer types and of rank 2, repeated indices."""
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((3, 5, 4, 2)).astype(np.float32)
+    for axis in range(4):
+        for idt in (np.int32, np.int64):
+            idx = rng.integers(0, x.shape[axis], (2, 3)).astype(idt)
+            assert np.array_equal(oracle.gather(x, idx, axis), np.take(x, idx, axis=axis))
+        idx = np.array([x.shape[axis] - 1, 0, 0], np.int32)
+        assert np.array_equal(oracle.gather(x, idx, axis), np.take(x, idx, axis=axis))
+        for start, end in ((0, 1), (0, x.shape[axis]), (1, 2), (x.shape[axis] - 1, x.shape[axis])):
+            sl = [slice(None)] * 4
+            sl[axis] = slice(start, end)
+            assert np.array_equal(oracle.slice_axis(x, axis, start, end), x[tuple(sl)])
 
 
 @pytest.mark.parametrize("name", ["split_net_v1_cpu", "split_net_v2_cpu"])

@@ -55,7 +55,8 @@ DENSE = ["gemm_net_v1_cpu", "prelu_net_v1_cpu", "dice_net_v1_cpu", "leaky_relu_n
          "reshape_net_v1_cpu", "batch_normalization_net_v1_cpu", "elementwise_add_net_v1_cpu", "elementwise_add_net_v2_cpu",
          "elementwise_sub_net_v1_cpu", "elementwise_sub_net_v2_cpu", "elementwise_mul_net_v1_cpu", "elementwise_mul_net_v2_cpu",
          "elementwise_div_net_v1_cpu", "elementwise_div_net_v2_cpu", "elementwise_broadcast_to_net_v1_cpu",
-         "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu", "split_net_v1_cpu", "split_net_v2_cpu"]
+         "elementwise_broadcast_to_net_v2_cpu", "elementwise_where_net_v1_cpu", "split_net_v1_cpu", "split_net_v2_cpu",
+         "gather_net_v1_cpu", "gather_net_v2_cpu", "slice_net_v1_cpu"]
 
 
 @pytest.mark.parametrize("name", DENSE)

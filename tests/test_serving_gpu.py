@@ -267,3 +267,59 @@ def test_requests_of_changing_size_allocate_nothing_in_steady_state(pb, oracle):
     p.reshape_input(fgs[0][0] + ".ids", (100000, ))
     with pytest.raises(pb.BlazeError, match="reshaped"):
         p.forward()
+
+
+def test_the_reference_shipped_model_file_end_to_end(pb, oracle):
+    """blaze/example/tdm_data/model_blaze_optimized, the one binary model the reference ships (committed byte for byte as
+    tests/golden/model_blaze_optimized.bin: 70 Embedding, 69 Gather, 10 Slice, ReduceSum, Div, Concat, Reshape, Gemm,
+    BatchNormalization, PRelu, Softmax; exported for the CPU, run_mode hybrid), loaded unmodified through
+    Blaze_PredcitorManagerLoadModel, fed synthetic inputs (69 user-level feature groups over 9 users, expanded to 70 ads by
+    indicator.0; one ad-level group) and a synthetic `item_emb` table, against the oracle's operator-by-operator forward
+    of the same file.  fp32: pooled and gathered blocks bit-exact, probabilities to 1e-5.  The reference ships no
+    expected output for this model: parity rests on the operators' own known answers."""
+    from blaze_proto import NetDef
+    import model_forward
+    path = os.path.join(ROOT, "tests", "golden", "model_blaze_optimized.bin")
+    net = NetDef()
+    net.ParseFromString(open(path, "rb").read())
+    rng = np.random.default_rng(2024)
+    rows, dim, users, ads = 4000, 24, 9, 70
+    table = (rng.standard_normal((rows, dim)) * 0.1).astype(np.float32)
+    keys = np.unique(rng.integers(1, 2**40, rows * 2, dtype=np.int64))[:rows]
+    feeds = {"indicator.0": rng.integers(0, users, ads).astype(np.int32)}
+    groups = sorted({v.name.rsplit(".", 1)[0] for v in net.external_input if v.name != "indicator.0"})
+    assert len(groups) == 70 and len(net.external_input) == 211
+    for fg in groups:
+        batch = ads if fg == "unit_id_expand" else users
+        seg = rng.integers(0, 5, batch).astype(np.int32)
+        seg[rng.integers(0, batch)] = 0
+        nnz = int(seg.sum())
+        ids = rng.choice(np.concatenate([keys, np.array([-5, 2**41], np.int64)]), nnz).astype(np.int64)  # two keys the table lacks
+        feeds[fg + ".ids"], feeds[fg + ".values"], feeds[fg + ".segments"] = ids, rng.uniform(0.5, 1.5, nnz).astype(np.float32), seg
+    want = model_forward.run_netdef(oracle, net, feeds, {"item_emb": oracle.Table(table, keys=keys)})
+    assert want["softmaxoutput0"].shape == (ads, 2) and want["concat10"].shape == (ads, 264)
+
+    pm = pb.PredictorManager()
+    pm.add_table("item_emb", table, keys=keys)
+    pm.load_model(path)
+    p = pm.create_predictor(1, 0)
+    assert sorted(p.list_input_names()) == sorted(feeds)
+    for name, arr in feeds.items():
+        p.feed(name, arr)
+    p.forward()
+    got = p.output_asnumpy("softmaxoutput0")
+    assert got.shape == (ads, 2)
+    np.testing.assert_allclose(got, want["softmaxoutput0"], rtol=1e-5, atol=1e-6)
+    assert np.abs(got.sum(1) - 1).max() < 1e-5 and got.std() > 1e-3
+    # a second request of another size through the same predictor
+    feeds2 = dict(feeds)
+    feeds2["indicator.0"] = feeds["indicator.0"][:33]
+    seg = feeds["unit_id_expand.segments"][:33]
+    n = int(seg.sum())
+    feeds2["unit_id_expand.segments"], feeds2["unit_id_expand.ids"], feeds2["unit_id_expand.values"] = \
+        seg, feeds["unit_id_expand.ids"][:n], feeds["unit_id_expand.values"][:n]
+    want2 = model_forward.run_netdef(oracle, net, feeds2, {"item_emb": oracle.Table(table, keys=keys)})
+    for name in ("indicator.0", "unit_id_expand.segments", "unit_id_expand.ids", "unit_id_expand.values"):
+        p.feed(name, feeds2[name])
+    p.forward()
+    np.testing.assert_allclose(p.output_asnumpy("softmaxoutput0"), want2["softmaxoutput0"], rtol=1e-5, atol=1e-6)

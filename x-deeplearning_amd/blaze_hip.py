@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_args", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew"
+    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew", "bz_gather_rows"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5  # bz_status

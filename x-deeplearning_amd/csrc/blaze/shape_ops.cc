@@ -321,6 +321,116 @@ class ReduceSumOp final : public Operator<Context> {
 REGISTER_HIP_OPERATOR(ReduceSum, ReduceSumOp<HIPContext>);
 OPERATOR_SCHEMA(ReduceSum).NumInputs(1).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("sum over one axis");
 
+// ------------------------------------------------------------------------------------------ Gather
+// blaze/operator/op/gather_op.h:25-87, gather_op.cc:9-45: output shape = data.shape[:axis] + indices.shape +
+// data.shape[axis+1:], y[.., j, ..] = data[.., indices[j], ..]; integer indices (int32 | int64).
+template <class Context>
+class GatherOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  GatherOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    axis_ = OperatorBase::GetSingleArgument<size_t>("axis", 0);
+  }
+  bool RunOnDevice() override {
+    Blob* data = this->Input(0);
+    Blob* indices = this->Input(1);
+    Blob* y = this->Output(0);
+    BLAZE_CONDITION_THROW(indices->data_type() == kInt32 || indices->data_type() == kInt64, "indices->data_type()=",
+                          indices->data_type());
+    const std::vector<TIndex> shape = data->shape();
+    BLAZE_CONDITION_THROW(axis_ < shape.size(), "axis_=", axis_, " shape.size()=", shape.size(), " ", this->def_.name());
+    BLAZE_CONDITION_THROW(y != data && y != indices, "Gather does not run in place");
+    std::vector<TIndex> o_shape;
+    TIndex outer = 1, inner = 1, n_idx = 1;
+    for (size_t i = 0; i < axis_; ++i) {
+      o_shape.push_back(shape[i]);
+      outer *= shape[i];
+    }
+    for (TIndex d : indices->shape()) {
+      o_shape.push_back(d);
+      n_idx *= d;
+    }
+    for (size_t i = axis_ + 1; i < shape.size(); ++i) {
+      o_shape.push_back(shape[i]);
+      inner *= shape[i];
+    }
+    if (y->data_type() != data->data_type()) y->set_data_type((DataType)data->data_type());
+    y->Reshape(o_shape);
+    BZ_CHECK(bz_gather_rows(data->data(), indices->data(), indices->data_type() == kInt32 ? BZ_I32 : BZ_I64, y->data(), (int64_t)outer,
+                            (int64_t)shape[axis_], (int64_t)(inner * DataTypeSize(data->data_type())), (int64_t)n_idx,
+                            context_.hip_stream()));
+    return true;
+  }
+
+ private:
+  size_t axis_;
+};
+REGISTER_HIP_OPERATOR(Gather, GatherOp<HIPContext>);
+OPERATOR_SCHEMA(Gather).NumInputs(2).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("Gather a tensor base on indices.");
+
+// ------------------------------------------------------------------------------------------ Slice
+// blaze/operator/op/slice_op.h:30-153, slice_op.cc:9-46: one axis, [start, end) given as axis | axes[1] and start, end |
+// starts[1], ends[1] (defaults 0, 0, 1); any other argument name is ignored, as there.  A strided copy: outer rows of
+// (end - start) * inner elements.
+template <class Context>
+class SliceOp final : public Operator<Context> {
+ public:
+  USE_OPERATOR_FUNCTIONS(Context);
+  SliceOp(const OperatorDef& def, Workspace* ws) : Operator<Context>(def, ws) {
+    if (OperatorBase::HasArgument("axes")) {
+      const std::vector<size_t> axes = OperatorBase::GetRepeatedArgument<size_t>("axes");
+      BLAZE_CONDITION_THROW(axes.size() == 1, "axes.size()=", axes.size());
+      axis_ = axes[0];
+    } else {
+      axis_ = OperatorBase::GetSingleArgument<size_t>("axis", 0);
+    }
+    if (OperatorBase::HasArgument("starts")) {
+      const std::vector<size_t> starts = OperatorBase::GetRepeatedArgument<size_t>("starts");
+      const std::vector<size_t> ends = OperatorBase::GetRepeatedArgument<size_t>("ends");
+      BLAZE_CONDITION_THROW(starts.size() == 1 && ends.size() == 1, "starts.size()=", starts.size(), " ends.size()=", ends.size());
+      start_ = starts[0];
+      end_ = ends[0];
+    } else {
+      start_ = OperatorBase::GetSingleArgument<size_t>("start", 0);
+      end_ = OperatorBase::GetSingleArgument<size_t>("end", 1);
+    }
+    BLAZE_CONDITION_THROW(start_ < end_, "Slice start=", start_, " end=", end_);
+  }
+  bool RunOnDevice() override {
+    Blob* x = this->Input(0);
+    Blob* y = this->Output(0);
+    const std::vector<TIndex> shape = x->shape();
+    BLAZE_CONDITION_THROW(axis_ < shape.size(), "axis_=", axis_, " shape.size()=", shape.size(), " ", this->def_.name());
+    BLAZE_CONDITION_THROW(end_ <= (size_t)shape[axis_], "axis=", axis_, " shape.size()=", shape.size(), " end_=", end_,
+                          " shape[exes_]=", shape[axis_]);
+    BLAZE_CONDITION_THROW(y != x, "Slice does not run in place");
+    TIndex outer = 1, inner = 1;
+    for (size_t i = 0; i < axis_; ++i) outer *= shape[i];
+    for (size_t i = axis_ + 1; i < shape.size(); ++i) inner *= shape[i];
+    std::vector<TIndex> y_shape = shape;
+    y_shape[axis_] = (TIndex)(end_ - start_);
+    if (y->data_type() != x->data_type()) y->set_data_type((DataType)x->data_type());
+    y->Reshape(y_shape);
+    const int64_t es = (int64_t)DataTypeSize(x->data_type());
+    bz_concat_desc d;
+    memset(&d, 0, sizeof(d));
+    d.src[0] = (const char*)x->data() + (int64_t)start_ * inner * es;
+    d.width[0] = (int64_t)(end_ - start_) * inner * es;
+    d.src_pitch[0] = (int64_t)shape[axis_] * inner * es;
+    d.dst = y->data();
+    d.dst_pitch = d.width[0];
+    d.rows = (int64_t)outer;
+    d.n = 1;
+    BZ_CHECK(bz_concat_cols(&d, context_.hip_stream()));
+    return true;
+  }
+
+ private:
+  size_t axis_, start_, end_;
+};
+REGISTER_HIP_OPERATOR(Slice, SliceOp<HIPContext>);
+OPERATOR_SCHEMA(Slice).NumInputs(1).NumOutputs(1).IdenticalTypeOfInput(0).SetDoc("Procuce a slice of the input tensor along one axis");
+
 // ------------------------------------------------------------------------------------------ Split
 // blaze/operator/op/split_op.h:33-132, split_op.cc:11-44.  Equal parts along axis 0 are views of the input (the
 // reference's RefReshape: the optimizer's FusedParallelGemm + Split pair costs no copy); any other split copies each

@@ -283,6 +283,25 @@ int launch_bcast_t(const bz_bcast_desc& d, const BcastP& p, int vec, hipStream_t
   return launch_bcast<T, int32_t>(d, p, vec, s);
 }
 
+
+// Gather along one axis: y[o, j, :] = data[o, idx[j], :] for `inner` contiguous units of W bytes (gather_op.cc:9-21, a
+// memcpy per index there).  An index outside [0, axis_size) -- undefined behaviour in the reference, whose memcpy reads
+// whatever lies there -- gives a row of zeros here.
+template <typename Unit, typename Index>
+__global__ __launch_bounds__(256) void bz_gather_kernel(const Unit* __restrict__ data, const Index* __restrict__ idx,
+                                                        Unit* __restrict__ y, int64_t outer, int64_t axis_size, int64_t inner,
+                                                        int64_t n_idx) {
+  const int64_t total = outer * n_idx * inner;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = i / inner, e = i - row * inner;
+    const int64_t o = row / n_idx, j = row - o * n_idx;
+    const int64_t src = (int64_t)idx[j];
+    Unit v = {};
+    if (src >= 0 && src < axis_size) v = data[(o * axis_size + src) * inner + e];
+    y[i] = v;
+  }
+}
+
 }  // namespace
 
 extern "C" int bz_broadcast_op(const bz_bcast_desc* desc, bz_stream_t stream) {
@@ -416,5 +435,39 @@ extern "C" int bz_softmax_axis(const void* x, void* y, int64_t outer, int64_t c,
   else
     hipLaunchKernelGGL(bz_softmax_axis_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)x, (__half*)y, outer, c, inner);
   BZ_LAUNCH_OK("bz_softmax_axis_kernel");
+  return BZ_OK;
+}
+
+extern "C" int bz_gather_rows(const void* data, const void* indices, int index_dtype, void* y, int64_t outer, int64_t axis_size,
+                              int64_t inner_bytes, int64_t n_indices, bz_stream_t stream) {
+  BZ_REQUIRE(outer >= 0 && axis_size >= 0 && inner_bytes > 0 && n_indices >= 0, "bz_gather_rows: outer=%lld axis_size=%lld inner_bytes=%lld n=%lld",
+             (long long)outer, (long long)axis_size, (long long)inner_bytes, (long long)n_indices);
+  BZ_REQUIRE(index_dtype == BZ_I32 || index_dtype == BZ_I64, "bz_gather_rows: indices->data_type()=%d", index_dtype);
+  if (outer * n_indices == 0) return BZ_OK;
+  BZ_REQUIRE(data != nullptr && indices != nullptr && y != nullptr, "bz_gather_rows: null operand");
+  hipStream_t s = bz::as_stream(stream);
+  // the widest unit that both tensors' rows are made of and aligned to
+  const uintptr_t bits = (uintptr_t)data | (uintptr_t)y | (uintptr_t)inner_bytes;
+#define BZ_GATHER(Unit)                                                                                                      \
+  do {                                                                                                                       \
+    const int64_t inner = inner_bytes / (int64_t)sizeof(Unit);                                                               \
+    const int grid = grid_for(outer * n_indices * inner);                                                                    \
+    if (index_dtype == BZ_I32)                                                                                               \
+      hipLaunchKernelGGL((bz_gather_kernel<Unit, int32_t>), dim3(grid), dim3(256), 0, s, (const Unit*)data, (const int32_t*)indices, \
+                         (Unit*)y, outer, axis_size, inner, n_indices);                                                      \
+    else                                                                                                                     \
+      hipLaunchKernelGGL((bz_gather_kernel<Unit, int64_t>), dim3(grid), dim3(256), 0, s, (const Unit*)data, (const int64_t*)indices, \
+                         (Unit*)y, outer, axis_size, inner, n_indices);                                                      \
+  } while (0)
+  if (bits % 16 == 0)
+    BZ_GATHER(uint4);
+  else if (bits % 4 == 0)
+    BZ_GATHER(uint32_t);
+  else if (bits % 2 == 0)
+    BZ_GATHER(uint16_t);
+  else
+    BZ_GATHER(uint8_t);
+#undef BZ_GATHER
+  BZ_LAUNCH_OK("bz_gather_kernel");
   return BZ_OK;
 }
