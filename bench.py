@@ -452,7 +452,7 @@ def main():
     mlp = cfg.mlp()
     sparse, dense = cfg.batches(args.pool)
     # kernel-layer harness: per-kernel timing below, and the whole step in --kernel-api mode
-    fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16", fused_mlp=bool(int(os.environ.get("BZ_FUSED_MLP", "0"))))
+    fwd = CtrForward(cfg, tables, mlp, sparse, dense, dtype="f16")
     torch.cuda.synchronize()
     K, W = args.steps, args.warmup
     S = max(2000, args.steady_steps)

@@ -321,55 +321,6 @@ BZ_API int bz_fc_fused(const bz_fc_desc* desc, bz_stream_t stream);
 BZ_API int bz_fc_pack_weight(const void* src_dev, int src_dtype, int trans_b, int k, int n, void* dst_dev, int dst_dtype,
                              int64_t ldw, bz_stream_t stream);
 
-/*
- * A whole FC stack in one launch: y = L_{n-1}( ... L_1( L_0(x) ) ), L_i(a) = act_i(alpha_i * a * W_i + beta_i * bias_i),
- * i.e. the chain Gemm -> activation -> Gemm -> ... the reference executes op by op
- * (blaze/graph/simple_net.cc:35-46 over blaze/operator/op/gemm_op.h:33-107 and the activation ops).  A workgroup
- * keeps 64 rows of the batch on chip for the whole stack; hidden activations are rounded to `dtype` where the
- * op-by-op path would store them.  Shapes it takes: fp16 or bf16; every layer but possibly the last is "wide"
- * (n a multiple of 128, at most BZ_MLP_MAX_WIDTH) with its weight in the fragment-major pack of bz_mlp_pack_weight;
- * the last layer may instead be a "head" of at most BZ_MLP_MAX_HEAD outputs (softmax / sigmoid / ... over them,
- * output fp32 or `dtype`) with its weight in the [n, ldw] pack of bz_fc_pack_weight.  Anything else: call
- * bz_fc_fused per layer.
- */
-#define BZ_MLP_MAX_LAYERS 4
-#define BZ_MLP_MAX_WIDTH 512
-#define BZ_MLP_MAX_HEAD 8
-typedef struct bz_mlp_layer {
-  const void* w;      /* packed weight (see above) */
-  const float* bias;  /* [n] or NULL */
-  const float* p0;    /* PRELU: slope [act_size]; DICE: gamma [n] */
-  const float* p1;    /* DICE: mean [n] */
-  const float* p2;    /* DICE: var [n] */
-  int32_t n, k;
-  int32_t ldw;        /* head layer only: elements between weight rows */
-  int32_t act;        /* bz_act */
-  int32_t act_size;
-  int32_t dice_nosqrt;
-  float alpha, beta;
-  float act_alpha;
-  int32_t reserved_;
-} bz_mlp_layer;
-
-typedef struct bz_mlp_desc {
-  const void* x;      /* device [m, ldx], 16-byte aligned, ldx % 8 == 0 */
-  void* y;            /* device [m, ldy] */
-  int64_t ldx, ldy;   /* elements */
-  int32_t m;
-  int32_t n_layers;
-  int32_t dtype;      /* BZ_F16 | BZ_BF16: x, weights, hidden activations */
-  int32_t out_dtype;  /* dtype, or BZ_F32 for a head */
-  bz_mlp_layer layer[BZ_MLP_MAX_LAYERS];
-} bz_mlp_desc;
-
-BZ_API int bz_mlp_fused(const bz_mlp_desc* desc, bz_stream_t stream);
-
-/* number of elements of the fragment-major pack of a [k, n] weight (k is padded to a multiple of 256); 0 if n is not
- * a multiple of 128 */
-BZ_API int64_t bz_mlp_packed_elems(int k, int n);
-
-/* [n, ldw] K-contiguous weight (the pack of bz_fc_pack_weight, fp16 or bf16) -> fragment-major pack for bz_mlp_fused */
-BZ_API int bz_mlp_pack_weight(const void* w_nk, int dtype, int k, int n, int64_t ldw, void* dst, bz_stream_t stream);
 
 /*
  * Strided-batched C[i] = alpha*op(A[i])*op(B[i]) + beta*C[i], row major, element

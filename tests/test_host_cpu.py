@@ -37,15 +37,15 @@ def test_struct_layouts_match_header():
     import blaze_hip
     src = ('#include "blaze_hip.h"\n#include <stdio.h>\nint main(){printf("%zu %zu %zu %zu %zu ", sizeof(bz_embed_slot), '
            'sizeof(bz_embed_launch), sizeof(bz_fc_desc), sizeof(bz_bgemm_desc), sizeof(bz_act_desc));'
-           'printf("%zu %zu %zu ", sizeof(bz_concat_desc), sizeof(bz_bcast_desc), sizeof(bz_bn_desc));printf("%zu %zu %zu %zu\\n", sizeof(bz_mlp_layer), sizeof(bz_mlp_desc), sizeof(bz_concat_ew_desc), sizeof(bz_weighted_pool_desc));printf("%zu\\n", sizeof(bz_fc_next));return 0;}\n')
+           'printf("%zu %zu %zu ", sizeof(bz_concat_desc), sizeof(bz_bcast_desc), sizeof(bz_bn_desc));printf("%zu %zu\\n", sizeof(bz_concat_ew_desc), sizeof(bz_weighted_pool_desc));printf("%zu\\n", sizeof(bz_fc_next));return 0;}\n')
     with tempfile.TemporaryDirectory() as d:
         open(os.path.join(d, "s.c"), "w").write(src)
         subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), os.path.join(d, "s.c"), "-o", os.path.join(d, "s")])
         sizes = [int(x) for x in subprocess.check_output([os.path.join(d, "s")]).split()]
     assert sizes == [C.sizeof(blaze_hip.EmbedSlot), C.sizeof(blaze_hip.EmbedLaunch), C.sizeof(blaze_hip.FcDesc),
                      C.sizeof(blaze_hip.BgemmDesc), C.sizeof(blaze_hip.ActDesc), C.sizeof(blaze_hip.ConcatDesc),
-                     C.sizeof(blaze_hip.BcastDesc), C.sizeof(blaze_hip.BnDesc), C.sizeof(blaze_hip.MlpLayer),
-                     C.sizeof(blaze_hip.MlpDesc), C.sizeof(blaze_hip.ConcatEwDesc), C.sizeof(blaze_hip.WeightedPoolDesc), C.sizeof(blaze_hip.FcNext)]
+                     C.sizeof(blaze_hip.BcastDesc), C.sizeof(blaze_hip.BnDesc),
+                     C.sizeof(blaze_hip.ConcatEwDesc), C.sizeof(blaze_hip.WeightedPoolDesc), C.sizeof(blaze_hip.FcNext)]
 
 
 def _sample_net():

@@ -306,30 +306,6 @@ def test_embedding_operator_errors(pb):
     assert not p.output_asnumpy("block").any()
 
 
-def test_fc_stack_as_one_launch_matches_layer_by_layer(pb, oracle):
-    """Net argument fuse_fc_stack: the three FC layers of the config-2 model run in the first Gemm's launch
-    (bz_mlp_fused); the other two never run.  Same probabilities as layer by layer, 2e-3."""
-    import torch
-    from ctr_model import build_manager, make_predictor
-    from synth import Config2
-    cfg = Config2(batch=300, rows=4000, slots=26)
-    tables, mlp = cfg.tables(), cfg.mlp()
-    sparse, dense = cfg.batches(1)
-    probs = {}
-    for stack in (False, True):
-        pm, fgs = build_manager(cfg, tables, mlp, np.float16, fc_stack=stack)
-        p = make_predictor(pm, fgs, sparse[0], dense[0], np.float16)
-        p.register_observers(["profile"])
-        p.forward()
-        probs[stack] = p.output_asnumpy("prob").astype(np.float32)
-        ran = [e["name"].split(":")[0] for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
-        assert ran.count("Gemm") == (1 if stack else 2), ran  # (layer by layer, the 256->2 head rides in the 512->256 launch)
-    torch.cuda.synchronize()
-    assert probs[True].shape == (300, 2)
-    np.testing.assert_allclose(probs[True], probs[False], rtol=2e-3, atol=2e-3)
-    np.testing.assert_allclose(probs[True].sum(1), 1.0, rtol=2e-3)
-
-
 def test_concat_inputs_written_in_place_give_identical_results(pb):
     """Concat(dense, block) whose inputs are an external input and an Embedding block read by nothing else: both
     live inside the Concat's output (the Feed copies rows at that tensor's pitch, the pooling kernel writes at it)

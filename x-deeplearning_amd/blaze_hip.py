@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_args", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_mlp_fused", "bz_mlp_packed_elems", "bz_mlp_pack_weight", "bz_concat_ew", "bz_gather_rows"
+    "bz_concat_ew", "bz_gather_rows"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5  # bz_status
@@ -103,18 +103,6 @@ class BnDesc(C.Structure):
                 ("eps", C.c_float), ("reserved_", C.c_int32)]
 
 
-class MlpLayer(C.Structure):
-    _fields_ = [("w", C.c_void_p), ("bias", C.c_void_p), ("p0", C.c_void_p), ("p1", C.c_void_p), ("p2", C.c_void_p),
-                ("n", C.c_int32), ("k", C.c_int32), ("ldw", C.c_int32), ("act", C.c_int32), ("act_size", C.c_int32),
-                ("dice_nosqrt", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float), ("act_alpha", C.c_float),
-                ("reserved_", C.c_int32)]
-
-
-class MlpDesc(C.Structure):
-    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("ldx", C.c_int64), ("ldy", C.c_int64), ("m", C.c_int32),
-                ("n_layers", C.c_int32), ("dtype", C.c_int32), ("out_dtype", C.c_int32), ("layer", MlpLayer * 4)]
-
-
 class BlazeHipError(RuntimeError):
     pass
 
@@ -156,10 +144,6 @@ def lib():
         l.bz_reduce_sum.argtypes = [vp, vp, i64, i64, i64, C.c_int, vp]
         l.bz_batch_norm.argtypes = [C.POINTER(BnDesc), vp]
         l.bz_softmax_axis.argtypes = [vp, vp, i64, i64, i64, C.c_int, vp]
-        l.bz_mlp_fused.argtypes = [C.POINTER(MlpDesc), vp]
-        l.bz_mlp_packed_elems.argtypes = [C.c_int, C.c_int]
-        l.bz_mlp_packed_elems.restype = i64
-        l.bz_mlp_pack_weight.argtypes = [vp, C.c_int, C.c_int, C.c_int, i64, vp, vp]
         _lib = l
     return _lib
 
@@ -618,61 +602,3 @@ def softmax_axis(x, axis, stream=None):
     y = torch.empty_like(x)
     check(lib().bz_softmax_axis(x.data_ptr(), y.data_ptr(), outer, x.shape[axis], inner, bz_dtype(x.dtype), _stream_ptr(stream)))
     return y
-
-
-class FusedMlp:
-    """A stack of FC layers prepared for bz_mlp_fused.
-
-    layers: list of dicts {w: torch [K,N] fp32 master, bias: torch [N] fp32 | None, act: ACT_*, params: tuple of fp32
-    tensors (PReLU: (slope,), Dice: (gamma, mean, var)), act_alpha, dice_nosqrt, alpha, beta}.
-    dtype: F16 | BF16.  The last layer may be a head with N <= 8.
-    """
-
-    def __init__(self, layers, dtype=F16):
-        import torch
-        self.dtype = dtype
-        self.layers = layers
-        self.keep = []
-        d = MlpDesc()
-        d.n_layers = len(layers)
-        d.dtype = dtype
-        for i, l in enumerate(layers):
-            k, n = l["w"].shape
-            wp = pack_weight(l["w"], False, dtype)  # [n, ldw]
-            L = d.layer[i]
-            if n <= 8 and i == len(layers) - 1:
-                L.w, L.ldw = wp.data_ptr(), wp.stride(0)
-                self.keep.append(wp)
-            else:
-                elems = lib().bz_mlp_packed_elems(k, n)
-                assert elems > 0, "layer %d: n=%d is not a multiple of 128" % (i, n)
-                fp = torch.empty(elems, dtype=wp.dtype, device=wp.device)
-                check(lib().bz_mlp_pack_weight(wp.data_ptr(), dtype, k, n, wp.stride(0), fp.data_ptr(), _stream_ptr()))
-                L.w = fp.data_ptr()
-                self.keep.append(fp)
-            L.n, L.k = n, k
-            if l.get("bias") is not None:
-                b = l["bias"].float().contiguous()
-                self.keep.append(b)
-                L.bias = b.data_ptr()
-            L.act = l.get("act", ACT_NONE)
-            ps = [p.float().contiguous() for p in l.get("params", ())]
-            self.keep += ps
-            for name, p in zip(("p0", "p1", "p2"), ps):
-                setattr(L, name, p.data_ptr())
-            L.act_size = ps[0].numel() if ps else 0
-            L.dice_nosqrt = int(l.get("dice_nosqrt", False))
-            L.alpha, L.beta, L.act_alpha = l.get("alpha", 1.0), l.get("beta", 1.0), l.get("act_alpha", 0.0)
-        self.desc = d
-        self.n_out = layers[-1]["w"].shape[1]
-        torch.cuda.synchronize()
-
-    def __call__(self, x, out=None, out_dtype=None, stream=None):
-        import torch
-        d = self.desc
-        if out is None:
-            out = torch.empty((x.shape[0], self.n_out), dtype=torch_dtype(out_dtype or self.dtype), device=x.device)
-        d.x, d.y, d.ldx, d.ldy, d.m = x.data_ptr(), out.data_ptr(), x.stride(0), out.stride(0), x.shape[0]
-        d.out_dtype = bz_dtype(out.dtype)
-        check(lib().bz_mlp_fused(C.byref(d), _stream_ptr(stream)))
-        return out

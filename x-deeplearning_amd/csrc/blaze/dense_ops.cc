@@ -242,31 +242,13 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
     return true;
   }
 
-  // ---- StackableFc: a chain of FC layers as one launch
-  bool StackEligible(int* k_in, int* n_out) override {
-    Blob* b = this->Input(1);
-    if (!b_constant_ || transa_ || b->shape().size() != 2 || b->data_type() != kFloat16) return false;
-    const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
-    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
-    if (this->InputSize() > 2) {
-      Blob* c = this->Input(2);
-      if (!c_constant_ || (int)c->size() != N) return false;  // a per-column bias only
-    }
-    if (fused_ && fused_act_ == BZ_ACT_SOFTMAX && N > BZ_MLP_MAX_HEAD) return false;
-    *k_in = K;
-    *n_out = N;
-    return true;
-  }
+  // ---- StackableFc: the operator whose output is this layer's result (its folded activation, or itself)
   OperatorBase* StackOutputOp() override { return fused_ ? fused_ : this; }
-  void AbsorbStack(const std::vector<StackableFc*>& followers) override {
-    stack_.clear();
-    for (StackableFc* f : followers) stack_.push_back(static_cast<GemmOp*>(f));
-  }
 
   // ---- a following layer of at most 8 outputs in this operator's launch
   bool CanHostHead(int* n_out) override {
     Blob* b = this->Input(1);
-    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr) return false;
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || head_ != nullptr) return false;
     const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
     if (N > 256 || N <= 8 || N % 8 != 0) return false;
     if (this->InputSize() > 2 && (!c_constant_ || (int)this->Input(2)->size() != N)) return false;
@@ -276,7 +258,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   }
   bool CanBeHead(int k_in) override {
     Blob* b = this->Input(1);
-    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr) return false;
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || head_ != nullptr) return false;
     const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
     const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
     if (K != k_in || N > 8 || alpha_ != 1.f || beta_ != 1.f) return false;
@@ -289,7 +271,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   // ---- sibling layers (same input, same shape of constant weight, same arguments) in one launch
   std::string SiblingKey() override {
     Blob* b = this->Input(1);
-    if (!b_constant_ || transa_ || b->shape().size() != 2 || !stack_.empty() || head_ != nullptr || !siblings_.empty()) return "";
+    if (!b_constant_ || transa_ || b->shape().size() != 2 || head_ != nullptr || !siblings_.empty()) return "";
     const TIndex N = transb_ ? b->shape()[0] : b->shape()[1];
     // (the stacked parameter vectors take N floats from every sibling: a bias of another length is no sibling's)
     if (this->InputSize() > 2 && (!c_constant_ || this->Input(2)->shape().size() != 1 || (TIndex)this->Input(2)->size() != N)) return "";
@@ -323,11 +305,11 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   bool HasAdoptedConcat() const override { return concat_ != nullptr; }
   bool CanChainNext(OperatorBase* next_op) override {
     auto* g = dynamic_cast<GemmOp*>(next_op);
-    if (g == nullptr || concat_ == nullptr || head_ != nullptr || !stack_.empty() || !siblings_.empty() || next_ != nullptr) return false;
+    if (g == nullptr || concat_ == nullptr || head_ != nullptr || !siblings_.empty() || next_ != nullptr) return false;
     Blob* b0 = this->Input(1);
     Blob* b = g->Input(1);
     if (!g->b_constant_ || g->transa_ || b->shape().size() != 2 || b->data_type() != b0->data_type()) return false;
-    if (!g->stack_.empty() || !g->siblings_.empty() || g->concat_ != nullptr) return false;
+    if (!g->siblings_.empty() || g->concat_ != nullptr) return false;
     const TIndex N1 = transb_ ? b0->shape()[0] : b0->shape()[1];
     const TIndex K2 = g->transb_ ? b->shape()[1] : b->shape()[0], N2 = g->transb_ ? b->shape()[0] : b->shape()[1];
     if (K2 != N1 || N2 <= 8 || N2 > 64) return false;
@@ -343,7 +325,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   bool RunOnDevice() override {
     launches_ = 1;
     if (concat_ != nullptr) {
-      if (siblings_.empty() && head_ == nullptr && stack_.empty()) {
+      if (siblings_.empty() && head_ == nullptr) {
         bz_concat_ew_desc pieces;
         auto* c = dynamic_cast<ConcatForFc*>(concat_);
         if (c != nullptr && c->DescribeAsPieces(&pieces)) {
@@ -386,89 +368,7 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
       // an input the one-launch form does not take (unaligned rows, mixed types): one launch per layer
       return RunSelf(false) && head_->RunSelf(false);
     }
-    if (!stack_.empty()) {
-      if (RunStack()) return true;
-      // an input the fused kernel does not take (3-D, unaligned, another type): layer by layer
-      if (!RunSelf(false)) return false;
-      for (GemmOp* f : stack_)
-        if (!f->RunSelf(false)) return false;
-      return true;
-    }
     return RunSelf(false);
-  }
-
-  // this layer's entry of the fused stack: packed weight, bias and epilogue parameters
-  void FillStackLayer(bz_mlp_layer* L, bool head, hipStream_t st) {
-    Blob* b = this->Input(1);
-    const int K = (int)(transb_ ? b->shape()[1] : b->shape()[0]);
-    const int N = (int)(transb_ ? b->shape()[0] : b->shape()[1]);
-    const int64_t ldw = (K + 7) / 8 * 8;
-    if (packed_b_.Stale(b) || packed_b_.bytes < (size_t)N * ldw * 2) {
-      packed_b_.Resize((size_t)N * ldw * 2);
-      BZ_CHECK(bz_fc_pack_weight(b->data(), BZ_F16, transb_ ? 1 : 0, K, N, packed_b_.ptr, BZ_F16, ldw, st));
-      packed_b_.Mark(b);
-      stack_pack_.src = nullptr;
-    }
-    memset(L, 0, sizeof(*L));
-    if (head) {
-      L->w = packed_b_.ptr;
-      L->ldw = (int)ldw;
-    } else {
-      if (stack_pack_.Stale(b)) {
-        stack_pack_.Resize((size_t)bz_mlp_packed_elems(K, N) * 2);
-        BZ_CHECK(bz_mlp_pack_weight(packed_b_.ptr, BZ_F16, K, N, ldw, stack_pack_.ptr, st));
-        stack_pack_.Mark(b);
-      }
-      L->w = stack_pack_.ptr;
-    }
-    L->n = N;
-    L->k = K;
-    if (this->InputSize() > 2) L->bias = AsFloatParam(this->Input(2), &bias_f32_, true, st);
-    L->alpha = alpha_;
-    L->beta = beta_;
-    L->act = fused_ ? fused_act_ : BZ_ACT_NONE;
-    L->dice_nosqrt = fused_nosqrt_ ? 1 : 0;
-    L->act_alpha = fused_alpha_;
-    if (fused_ && fused_act_ == BZ_ACT_PRELU) {
-      L->p0 = AsFloatParam(fused_->Input(1), &p_f32_[0], true, st);
-      L->act_size = (int)fused_->Input(1)->size();
-    } else if (fused_ && fused_act_ == BZ_ACT_DICE) {
-      L->p0 = AsFloatParam(fused_->Input(1), &p_f32_[0], true, st);
-      L->p1 = AsFloatParam(fused_->Input(2), &p_f32_[1], true, st);
-      L->p2 = AsFloatParam(fused_->Input(3), &p_f32_[2], true, st);
-      L->act_size = N;
-    }
-  }
-
-  bool RunStack() {
-    Blob* a = this->Input(0);
-    if (a->shape().size() != 2 || a->data_type() != kFloat16) return false;
-    const TIndex M = a->shape()[0], K = a->shape()[1];
-    if (K % 8 != 0 || (uintptr_t)a->data() % 16 != 0) return false;
-    GemmOp* last = stack_.back();
-    Blob* y = last->StackOutputOp()->Output(0);
-    Blob* lb = last->Input(1);
-    const TIndex n_last = last->transb_ ? lb->shape()[0] : lb->shape()[1];
-    const bool head = n_last <= BZ_MLP_MAX_HEAD;
-    if (!(y->data_type() == kFloat16 || (head && y->data_type() == kFloat))) return false;
-    if (!head && n_last % 8 != 0) return false;
-    CheckValid();
-    y->Reshape({M, n_last});
-    hipStream_t st = context_.hip_stream();
-    bz_mlp_desc d;
-    memset(&d, 0, sizeof(d));
-    d.x = a->data();
-    d.ldx = (int64_t)K;
-    d.y = y->data();
-    d.ldy = (int64_t)n_last;
-    d.m = (int)M;
-    d.n_layers = 1 + (int)stack_.size();
-    d.dtype = BZ_F16;
-    d.out_dtype = BzType(y->data_type());
-    FillStackLayer(&d.layer[0], false, st);
-    for (size_t i = 0; i < stack_.size(); ++i) stack_[i]->FillStackLayer(&d.layer[1 + i], head && i + 1 == stack_.size(), st);
-    BZ_CHECK(bz_mlp_fused(&d, st));
-    return true;
   }
 
   // this layer and its absorbed siblings as one launch over the stacked weights; every layer's output blob becomes a
@@ -773,8 +673,6 @@ class GemmOp : public Operator<Context>, public FusableProducer, public Stackabl
   bool transa_, transb_;
   bool b_constant_ = false, c_constant_ = false;
   Derived packed_b_, packed_a_, bias_f32_, p_f32_[3];
-  Derived stack_pack_;           // this layer's weight in the fragment-major pack of bz_mlp_fused
-  std::vector<GemmOp*> stack_;   // the FC layers after this one that run in this operator's launch
   GemmOp* head_ = nullptr;       // the layer of at most 8 outputs computed in this operator's launch
   OperatorBase* concat_ = nullptr;  // the Concat that makes Input(0), computed by this operator's kernel
   GemmOp* next_ = nullptr;          // the narrow layer after this one, computed in this operator's launch

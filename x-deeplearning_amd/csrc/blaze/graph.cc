@@ -211,7 +211,6 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
       if (other_reader || is_output) continue;
       if (producer->TryFuse(operators_[i + 1].get())) skipped_[i + 1] = true;
     }
-    StackFcLayers();
     FuseFcHeads();
     PackSiblingFcs();
     AliasConcatInputs();
@@ -608,76 +607,6 @@ void SimpleNet::AliasConcatInputs() {
       widths.push_back(w);
     }
     if (ok) Blob::LinkColumnSlices(operators_[c]->Output(0), children, widths);
-  }
-}
-
-// Chains of FC layers -> one launch.  Layer widths the fused kernel takes: every layer but possibly the last a
-// multiple of 128 up to BZ_MLP_MAX_WIDTH, the last one alternatively a head of at most BZ_MLP_MAX_HEAD outputs; at
-// most BZ_MLP_MAX_LAYERS layers; all activation buffers within the CU's 160 KB of LDS.
-void SimpleNet::StackFcLayers() {
-  // Opt in (net argument fuse_fc_stack: 1, or BLAZE_FC_STACK=1).  Measured on config 2: the stack kernel keeps the
-  // batch on 32 CUs for 24 us where the three per-layer launches take 23 us on all CUs; under concurrent serving
-  // threads that frees the rest of the chip (+4 % throughput), but a lone request sees a longer forward pass.
-  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_fc_stack");
-  const char* env = getenv("BLAZE_FC_STACK");
-  const bool on = (arg && arg->has_i && arg->i != 0) || (env && atoi(env) != 0);
-  if (!on) return;
-  auto is_external_output = [&](const std::string& name) {
-    for (const auto& eo : external_output_)
-      if (eo == name) return true;
-    return false;
-  };
-  auto wide = [](int n) { return n % 128 == 0 && n >= 128 && n <= BZ_MLP_MAX_WIDTH; };
-  size_t i = 0;
-  while (i < operators_.size()) {
-    auto* head = skipped_[i] ? nullptr : dynamic_cast<StackableFc*>(operators_[i].get());
-    int k_in = 0, n_out = 0;
-    if (!head || !head->StackEligible(&k_in, &n_out) || !wide(n_out)) {
-      ++i;
-      continue;
-    }
-    std::vector<StackableFc*> chain = {head};
-    std::vector<size_t> chain_idx = {i};
-    std::vector<int> widths = {n_out};
-    int lds[2] = {64 * (n_out * 2 + 16), 0};
-    int head_bytes = 0;
-    size_t last = i;
-    while ((int)chain.size() < BZ_MLP_MAX_LAYERS) {
-      // the next operator that runs after the chain's last layer (its folded activation is skipped already)
-      size_t j = last + 1;
-      while (j < operators_.size() && skipped_[j]) ++j;
-      if (j >= operators_.size()) break;
-      auto* next = dynamic_cast<StackableFc*>(operators_[j].get());
-      int k2 = 0, n2 = 0;
-      if (!next || !next->StackEligible(&k2, &n2)) break;
-      const std::string& mid = chain.back()->StackOutputOp()->operator_def().output(0);
-      if (operators_[j]->operator_def().input(0) != mid || k2 != widths.back()) break;
-      OperatorBase* out_op = chain.back()->StackOutputOp();
-      if (ReadersOf(mid, out_op != operators_[last].get() ? out_op : nullptr) != 1 || is_external_output(mid)) break;
-      const bool is_head = n2 <= BZ_MLP_MAX_HEAD;
-      if (!is_head && !wide(n2)) break;
-      int need[2] = {lds[0], lds[1]};
-      int hb = 0;
-      if (is_head)
-        hb = n2 * k2 * 2 + 128;
-      else
-        need[chain.size() & 1] = std::max(need[chain.size() & 1], 64 * (n2 * 2 + 16));
-      if (2 * 64 * (64 * 2 + 16) + need[0] + need[1] + hb > 160 * 1024) break;
-      lds[0] = need[0];
-      lds[1] = need[1];
-      head_bytes = hb;
-      chain.push_back(next);
-      chain_idx.push_back(j);
-      widths.push_back(n2);
-      last = j;
-      if (is_head) break;
-    }
-    (void)head_bytes;
-    if (chain.size() >= 2) {
-      head->AbsorbStack(std::vector<StackableFc*>(chain.begin() + 1, chain.end()));
-      for (size_t c = 1; c < chain_idx.size(); ++c) skipped_[chain_idx[c]] = true;
-    }
-    i = last + 1;
   }
 }
 

@@ -96,7 +96,6 @@ class SimpleNet : public Net {
 
  protected:
   bool RunImpl() override;
-  void StackFcLayers();
   void AliasConcatInputs();
   void FuseConcatPieces();
   void FuseFcHeads();
@@ -106,7 +105,7 @@ class SimpleNet : public Net {
   void ChainNarrowFcs();
   int ReadersOf(const std::string& name, const OperatorBase* folded) const;
   void InterleaveAssignBlocks();
-  std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the head of their FC stack
+  std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the operator that took them over
 };
 
 typedef Registry<std::shared_ptr<Net>, const std::shared_ptr<const NetDef>&, Workspace*> NetRegistryType;
@@ -131,19 +130,12 @@ class FusableProducer {
   virtual bool TryFuse(OperatorBase* consumer) = 0;
 };
 
-// An FC operator (Gemm, with or without a folded activation) that can hand its work to the FC before it, so that a
-// chain of FC layers runs as one launch (bz_mlp_fused: the batch rows stay on chip from the first layer to the
-// last).  SimpleNet links consecutive eligible operators whose only connection is producer -> consumer; the head
-// of the chain then runs all of them and the followers are skipped.  Same results as layer-by-layer execution:
-// hidden activations are rounded to the tensor type where the separate operators would have stored them.
+// An FC operator (Gemm, with or without a folded activation) that can run a following skinny layer in its own launch.
 class StackableFc {
  public:
   virtual ~StackableFc() {}
-  // static eligibility (constant fp16 weight and bias, no transposed A, ...); reports the layer's widths
-  virtual bool StackEligible(int* k_in, int* n_out) = 0;
   // the operator whose Output(0) receives this layer's result (the folded activation, else the operator itself)
   virtual OperatorBase* StackOutputOp() = 0;
-  virtual void AbsorbStack(const std::vector<StackableFc*>& followers) = 0;
   // A layer of at most 256 outputs followed by a layer of at most 8 (the logit / score of a tower): the second is
   // computed in the first one's launch from the output tile still on chip (bz_fc_desc.head_*), and what the first
   // layer would have stored for it is not stored at all.

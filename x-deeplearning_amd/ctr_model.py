@@ -10,10 +10,9 @@ import numpy as np
 import pyblaze_hip as pb
 
 
-def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False, fc_stack=False, net_args=None):
+def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False, net_args=None):
     """tables: list of torch cuda tensors [rows, dim]; mlp: [(W [K,N], b, slope)] torch tensors.
     expose_block: also declare the pooled Embedding block an output of the net (for parity checks).
-    fc_stack: ask the net to run the chain of FC layers as one launch (net argument fuse_fc_stack).
     net_args: further integer net arguments, e.g. {"alias_concat_inputs": 0}."""
     code = pb.K_FLOAT16 if dtype == np.float16 else pb.K_FLOAT
     pm = pb.PredictorManager()
@@ -31,8 +30,6 @@ def build_manager(cfg, tables, mlp, dtype=np.float16, expose_block=False, fc_sta
         inputs += [fg + ".ids", fg + ".values", fg + ".segments"]
     nb.external_input("dense", code)
     nb.external_output("prob", pb.K_FLOAT)
-    if fc_stack:
-        nb.arg("fuse_fc_stack", 1)
     for k, v in (net_args or {}).items():
         nb.arg(k, int(v))
     if expose_block:

@@ -14,16 +14,13 @@ import blaze_hip as bz
 
 
 class CtrForward:
-    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True, fused_mlp=False,
-                 fused_head=True):
-        """fused_mlp: run the FC stack as one bz_mlp_fused launch instead of one bz_fc_fused launch per layer.
-        fused_head: the last (skinny) layer rides in the launch of the layer before it, as SimpleNet runs the model."""
+    def __init__(self, cfg, tables, mlp, sparse_batches, dense_batches, dtype="f16", fused_scan=True, fused_head=True):
+        """fused_head: the last (skinny) layer rides in the launch of the layer before it, as SimpleNet runs the model."""
         import torch
         self.cfg = cfg
         self.fused_scan = fused_scan
         self.fused_head = fused_head and len(mlp) >= 2
         self._launches = None
-        self.fused_mlp = None
         self.lib = bz.lib()
         tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
         bdt = {"f16": bz.F16, "bf16": bz.BF16, "f32": bz.F32}[dtype]
@@ -32,10 +29,6 @@ class CtrForward:
         for (w, b, slope) in mlp:
             self.weights.append((bz.pack_weight(w, False, bdt), b.float().contiguous(), slope.float().contiguous(),
                                  w.shape[0]))
-        if fused_mlp:
-            n = len(mlp)
-            self.fused_mlp = bz.FusedMlp([dict(w=w, bias=b, act=bz.ACT_SOFTMAX if li == n - 1 else bz.ACT_PRELU,
-                                               params=() if li == n - 1 else (slope, )) for li, (w, b, slope) in enumerate(mlp)], bdt)
         self.n_batches = len(sparse_batches)
         self.steps = []
         self.nnz = []
@@ -118,19 +111,10 @@ class CtrForward:
 
     def _make_launches(self):
         n = len(self.weights)
-        if self.fused_mlp is not None:
-            return [("bz_mlp_fused", self.mlp)]
         if self.fused_head:
             return [("bz_fc[%d]" % li, (lambda i, st=None, li=li: self.fc(i, li, st))) for li in range(n - 2)] + \
                    [("bz_fc[%d+%d]" % (n - 2, n - 1), self.fc_with_head)]
         return [("bz_fc[%d]" % li, (lambda i, st=None, li=li: self.fc(i, li, st))) for li in range(n)]
-
-    def mlp(self, i, st=None):
-        s = self.steps[i % self.n_batches]
-        d = self.fused_mlp.desc
-        x, y = s["x"], s["acts"][-1]
-        d.x, d.y, d.ldx, d.ldy, d.m, d.out_dtype = x.data_ptr(), y.data_ptr(), x.stride(0), y.stride(0), x.shape[0], bz.bz_dtype(y.dtype)
-        bz.check(self.lib.bz_mlp_fused(C.byref(d), st or self._stream()))
 
     def step(self, i, st=None):
         st = st or self._stream()
