@@ -278,20 +278,26 @@ def bench_config4(np, torch, bz):
     return res
 
 
-def bench_config5(np, torch, bz):
+def bench_config5(np, torch, bz, tables=True):
+    """tables=False: the FC tower alone on random activations (no 102 GB of tables), for counter runs of its kernels"""
     from synth import Config5, embedding_bytes
     cfg = Config5()
-    free, _ = torch.cuda.mem_get_info()
-    need = cfg.slots * cfg.rows * cfg.dim * 2
-    if free < need * 1.3:
-        return {"workload": cfg.name, "skipped": "needs %.0f GB of free HBM, %.0f GB free" % (need * 1.3 / 1e9, free / 1e9)}
-    tables = cfg.tables()
-    dts = [bz.DeviceTable(t) for t in tables]
     mlp = cfg.mlp()
     B, D = cfg.batch, cfg.dim
     n = 2
     plans, keep, nnz, xs = [], [], [], []
+    dts = None
+    if tables:
+        free, _ = torch.cuda.mem_get_info()
+        need = cfg.slots * cfg.rows * cfg.dim * 2
+        if free < need * 1.3:
+            return {"workload": cfg.name, "skipped": "needs %.0f GB of free HBM, %.0f GB free" % (need * 1.3 / 1e9, free / 1e9)}
+        dts = [bz.DeviceTable(t) for t in cfg.tables()]
     for b in range(n):
+        if not tables:
+            g = torch.Generator(device="cuda").manual_seed(5 + b)
+            xs.append((torch.randn((B, cfg.slots * D), generator=g, device="cuda") * 0.5).to(torch.bfloat16))
+            continue
         x = torch.zeros((B, cfg.slots * D), dtype=torch.bfloat16, device="cuda")
         xs.append(x)
         items = []
@@ -302,8 +308,10 @@ def bench_config5(np, torch, bz):
             items.append(dict(table=dts[s], ids=t[0], values=t[1], segments=t[2], out=x, col=s * D, udf=bz.SUM))
         plans.append(bz.EmbeddingPlan(items))
         nnz.append(sum(ids.size for ids, _, _ in sp))
-    pool_us = graph_timed(torch, lambda i: plans[i % n].run(), n, 4 * n, warm_ms=50.0)
-    alg = float(np.mean([embedding_bytes(z, B, cfg.slots, D * 2, 0, cfg.slots * D, 2) for z in nnz]))
+    pool_us = alg = None
+    if tables:
+        pool_us = graph_timed(torch, lambda i: plans[i % n].run(), n, 4 * n, warm_ms=50.0)
+        alg = float(np.mean([embedding_bytes(z, B, cfg.slots, D * 2, 0, cfg.slots * D, 2) for z in nnz]))
     # the tower: bias + ReLU per layer, sigmoid head riding in the launch of the layer before it
     packed = [bz.pack_weight(w, False, bz.BF16) for w, _ in mlp]
     ys = [torch.empty((B, w.shape[1]), dtype=torch.bfloat16, device="cuda") for w, _ in mlp[:-1]]
@@ -325,21 +333,21 @@ def bench_config5(np, torch, bz):
     w0 = packed[0][:, :L[0]]
     lib_us = graph_timed(torch, lambda i: torch.nn.functional.linear(xs[i % n], w0), n, 4 * n, warm_ms=100.0)
     flops = [2.0 * B * L[i] * L[i + 1] for i in range(len(L) - 1)]
-    step_us = pool_us + sum(fc_us)
-    kern = {"pool": round(pool_us, 2)}
+    kern = {"pool": round(pool_us, 2)} if tables else {}
     for i, u in enumerate(fc_us[:-1]):
         kern["fc[%d]" % i] = round(u, 2)
     kern["fc[%d+%d]" % (len(mlp) - 2, len(mlp) - 1)] = round(fc_us[-1], 2)
-    res = {"workload": cfg.name, "dtype": "f16 tables -> bf16 block; bf16 MFMA, f32 accumulate", "ids_per_launch": int(np.mean(nnz)),
-           "pool_launches_per_step": 1 if plans[0].fused_scan else 2, "kernel_us": kern,
-           "samples/s_kernels_back_to_back": round(B / step_us * 1e6, 1),
-           "roofline": hbm_roofline("bz_embed_pool_kernel", alg, pool_us),
+    res = {"workload": cfg.name, "dtype": "f16 tables -> bf16 block; bf16 MFMA, f32 accumulate", "kernel_us": kern,
            "roofline_fc": dict(mfma_roofline("bz_fc_stream_kernel (layer 0: %dx%dx%d)" % (B, L[0], L[1]), flops[0], fc_us[0]),
                                library_gemm_us=round(lib_us, 2)),
            "fc_stack": {"TFLOP/s": round(sum(flops) / sum(fc_us) / 1e6, 2),
                         "frac_of_mfma_peak": round(sum(flops) / sum(fc_us) / 1e6 / MFMA_PEAK_TFLOPS, 5),
                         "flops": int(sum(flops)), "us": round(sum(fc_us), 2)}}
-    del plans, keep, dts, tables, xs
+    if tables:
+        res.update({"ids_per_launch": int(np.mean(nnz)), "pool_launches_per_step": 1 if plans[0].fused_scan else 2,
+                    "samples/s_kernels_back_to_back": round(B / (pool_us + sum(fc_us)) * 1e6, 1),
+                    "roofline": hbm_roofline("bz_embed_pool_kernel", alg, pool_us)})
+    del plans, keep, dts, xs
     torch.cuda.empty_cache()
     return res
 
