@@ -39,6 +39,7 @@ def _items(bz, torch, rng, tables, batch, max_len, out, mixed):
 @pytest.mark.parametrize("mixed", [False, True])
 def test_static_scratch_entry_point_matches_the_two_call_form(bz, mixed):
     import torch
+    import pyblaze_hip
     rng = np.random.default_rng(17 + int(mixed))
     tables = [bz.DeviceTable(torch.from_numpy((rng.standard_normal((3000, 32)) * 0.1).astype(np.float16)).cuda()) for _ in range(6)]
     width = sum(t.dim * (3 if (mixed and s % 3 == 2) else 1) for s, t in enumerate(tables))
@@ -56,8 +57,16 @@ def test_static_scratch_entry_point_matches_the_two_call_form(bz, mixed):
         assert all(s.offsets is None for s in plan.host) and plan.launch.max_batch == batch
         assert (plan.launch.variant == 0) == mixed
         print("static scratch call %d: mixed=%s batch=%d variant=%#x" % (call, mixed, batch, plan.launch.variant), flush=True)
+        torch.cuda.synchronize()
+        before = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), pyblaze_hip.allocation_count())
         plan.run_static_scratch()
         torch.cuda.synchronize()
+        after = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), pyblaze_hip.allocation_count())
+        # no allocation by the library or through torch, and from the second call on (the first one on a device loads
+        # the kernels' code and looks the buffer's address up) none by the driver either: the device's free memory stands
+        assert after[1:] == before[1:]
+        if call > 0:
+            assert after[0] == before[0], "free device memory changed across a call that must not allocate"
         a, b = got.cpu().numpy(), want.cpu().numpy()
         assert not np.isnan(b).any()
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
