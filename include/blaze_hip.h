@@ -199,6 +199,8 @@ BZ_API int bz_embed_pool_args(const bz_embed_slot* slots_host, const bz_embed_la
  * Limit: n_slots * (launch->max_batch + 1) * 8 bytes must fit the buffer, else BZ_EINVAL (config 5, 200 slots x batch
  * 8192, takes 13.1 MB).  All calls on one GPU share the one buffer: calls whose launches may overlap on the device
  * (different streams, no ordering between them) race on it; calls on one stream, or ordered by events, do not.
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress, which may load the library's code on
+ * that device): make one call per device outside any stream capture before relying on it there.
  */
 #define BZ_EMBED_STATIC_SCRATCH_BYTES (16u << 20)
 BZ_API int bz_embed_pool_static_scratch(const bz_embed_slot* slots_dev, const bz_embed_launch* launch, bz_stream_t stream);
