@@ -660,7 +660,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
-        "data": "synthetic (seeded; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
+        "data": "synthetic (Philox4x32-10 keyed by seed, stream, index; Zipf(1.1) ids, Poisson(8) lengths, N(0,0.01) tables, random-init MLP)",
         "config": {"workload": cfg.name, "batch": cfg.batch, "slots": cfg.slots, "table_rows": cfg.rows, "dim": cfg.dim,
                    "batch_pool": NB,
                    "path": "kernel-layer C ABI (bz_*)" if predictors is None else "Predictor.Forward via Blaze_* C ABI",

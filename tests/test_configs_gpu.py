@@ -22,13 +22,23 @@ def bz():
     return blaze_hip
 
 
-def _touched_table(oracle, dev_rows, ids, dev_scale=None):
-    """Oracle table holding only the rows `ids` name, keyed by id (the device indexes the full table by row)."""
+def _touched_table(oracle, dev_rows, ids, dev_scale=None, regen=None):
+    """Oracle table holding only the rows `ids` name, keyed by id (the device indexes the full table by row).
+    regen(unique rows) -> rows [, scale]: the generator's own values for those rows, computed on the host; the oracle is
+    then fed these, and the device's copy of the same rows must hold the same bits (the fill kernel against numpy)."""
     import torch
     uniq = np.unique(ids)
     idx = torch.from_numpy(uniq).cuda()
     rows = dev_rows[idx].cpu().numpy()
     scale = None if dev_scale is None else dev_scale[idx].cpu().numpy()
+    if regen is not None:
+        host = regen(uniq)
+        host_rows, host_scale = host if isinstance(host, tuple) else (host, None)
+        assert host_rows.dtype == rows.dtype and np.array_equal(host_rows.view(np.uint8), rows.view(np.uint8)), "table rows differ from the generator's"
+        assert (scale is None) == (host_scale is None)
+        if scale is not None:
+            assert np.array_equal(host_scale.view(np.uint32), scale.view(np.uint32)), "row scales differ from the generator's"
+        rows, scale = host_rows, host_scale
     return oracle.Table(rows, scale=scale, keys=uniq.astype(np.uint64))
 
 
@@ -105,7 +115,7 @@ def test_config4_int8_kavg_full_size(bz, oracle):
     got16 = run(1.0, torch.float16)
     want = np.zeros((B, cfg.slots * D), np.float32)
     for s, (ids, vals, seg) in enumerate(sparse):
-        tab = _touched_table(oracle, tables[s][0], ids, tables[s][1])
+        tab = _touched_table(oracle, tables[s][0], ids, tables[s][1], regen=lambda u, s=s: cfg.table_rows(s, u))
         oracle.embed_get(tab, ids, vals, seg, [(1, 0, 0, want, s * D)])
     # fp32 block: the int8 extension is defined as w = scale*(float)q, then the reference's kavg: bit-exact
     assert np.array_equal(got32.view(np.uint32), want.view(np.uint32))
@@ -161,11 +171,11 @@ def test_config5_fp16_tables_bf16_tower_full_size(bz, oracle):
         off = np.concatenate([[0], np.cumsum(seg)])
         if s % 25 == 0:
             full = np.zeros((B, D), np.float32)
-            oracle.embed_get(_touched_table(oracle, tables[s], ids), ids, vals, seg, [(0, 0, 0, full, 0)])
+            oracle.embed_get(_touched_table(oracle, tables[s], ids, regen=lambda u, s=s: cfg.table_rows(s, u)), ids, vals, seg, [(0, 0, 0, full, 0)])
             assert np.array_equal(got32[:, s * D:(s + 1) * D].view(np.uint32), full.view(np.uint32))
         sel = np.concatenate([np.arange(off[r], off[r + 1]) for r in rows])
         sub = np.zeros((64, D), np.float32)
-        oracle.embed_get(_touched_table(oracle, tables[s], ids[sel]), ids[sel], vals[sel], seg[rows], [(0, 0, 0, sub, 0)])
+        oracle.embed_get(_touched_table(oracle, tables[s], ids[sel], regen=lambda u, s=s: cfg.table_rows(s, u)), ids[sel], vals[sel], seg[rows], [(0, 0, 0, sub, 0)])
         want_rows[:, s * D:(s + 1) * D] = sub
     assert np.array_equal(got32[rows].view(np.uint32), want_rows.view(np.uint32))  # fp32 block: bit-exact
     x0 = _bf16_round(want_rows)
@@ -229,9 +239,9 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     assert kinds == ["Concat"] + ["Embedding"] * 2 + ["Gemm"] * 3 + ["MatMul"], kinds
     assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
-    for k, t in zip(din_model.KINDS, tables):
+    for ki, (k, t) in enumerate(zip(din_model.KINDS, tables)):
         ids = np.concatenate([batch[k + ".ids"], batch[k + "_his.ids"]])
-        tabs[k] = _touched_table(oracle, t, ids)
+        tabs[k] = _touched_table(oracle, t, ids, regen=lambda u, ki=ki: cfg.table_rows(ki, u))
     rnd = lambda a: np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
     want = model_forward.din_forward(oracle, cfg, tabs, weights, batch, rnd)
     B, T, D3 = cfg.batch, cfg.T, 3 * cfg.dim

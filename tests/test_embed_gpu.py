@@ -469,3 +469,25 @@ def test_pooling_unaligned_counts_and_trailing_empty_segments(bz, oracle):
         want = np.full((batch, dim), np.nan, np.float32)
         oracle.embed_get(oracle.Table(data), ids, vals, seg, [(0, 0, 0, want, 0)])
         assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_device_fill_matches_the_host_generator_bit_for_bit(bz):
+    """csrc/synth/philox_fill.hip (tables too large to come from the host) against philox.py on the same (seed, stream,
+    index): normal fp32 / fp16, int8, uniform fp32; ranges that start and end inside a call's four words."""
+    import torch
+    import philox
+    st = philox.Stream(12, seed=philox.SEED + 99)
+    for kind, dt, a, b in ((philox.KIND_NORMAL_F32, torch.float32, 0.01, 0.0), (philox.KIND_NORMAL_F16, torch.float16, 0.1, 0.0),
+                           (philox.KIND_INT8, torch.int8, 1.0, 0.0), (philox.KIND_UNIFORM_F32, torch.float32, 1e-3, 1e-2)):
+        for first, n in ((0, 4096), (1, 1), (3, 7), (5, 100003), ((1 << 34) + 2, 513)):
+            print("device fill kind %d first %d n %d" % (kind, first, n), flush=True)
+            t = torch.empty(n + 2, dtype=dt, device="cuda")
+            t.fill_(77)
+            philox.fill(t[1:n + 1], kind, st, first, a, b)
+            torch.cuda.synchronize()
+            got = t.cpu().numpy()
+            want = philox.host(kind, st, n, first, a, b)
+            assert got[0] == 77 and got[-1] == 77  # nothing outside the range is written
+            assert got.dtype == want.dtype and np.array_equal(got[1:-1].view(np.uint8), want.view(np.uint8))
+    m = philox.tensor((1000, 18), philox.KIND_NORMAL_F16, st, "cuda", 0.1)
+    assert np.array_equal(m.cpu().numpy()[[999, 0]], philox.host_rows(philox.KIND_NORMAL_F16, st, [999, 0], 18, 0.1))

@@ -505,3 +505,63 @@ def test_qed_builder_on_the_reference_text_tables(tmp_path, oracle):
             assert bytes(ref.hash_dump()) == himg, "differs from the reference's HashTable::Dump"
     if oracle.have_ref():
         assert bytes(oracle.RefTrie(["a_01", "a_02"], [0, 1]).dump()) == trie
+
+
+# ---------------------------------------------------------------- the synthetic workloads' generator
+def test_philox4x32_10_known_answers_and_element_independence():
+    """philox.py against the published known-answer vectors of Philox4x32-10 (Random123's kat_vectors: zero, all-ones
+    and the digits-of-pi counter / key), and its streams' contract: an element is a function of (seed, stream, index)
+    only, whatever range it is asked for in."""
+    import philox
+    kat = (((0, 0, 0, 0), (0, 0), "6627e8d5 e169c58d bc57ac4c 9b00dbd8"),
+           ((0xffffffff, ) * 4, (0xffffffff, ) * 2, "408f276d 41c83b0e a20bc7c6 6d5451fd"),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0), "d16cfe09 94fdcceb 5001e420 24126ea1"))
+    for ctr, key, want in kat:
+        assert " ".join("%08x" % int(x) for x in philox.philox4x32_10(*ctr, *key)) == want
+    # vectorised over counters = one call at a time
+    st = philox.Stream(7, seed=(0x299f31d0 << 32) | 0xa4093822)
+    i = 0x85a308d3243f6a88
+    assert [int(x) for x in st.calls(i, 3)[0]] == [int(x) for x in philox.philox4x32_10(i & 0xffffffff, i >> 32, 7, 0, 0xa4093822, 0x299f31d0)]
+    # any sub-range, any alignment to the four words of a call, rows of a matrix: the same elements
+    whole = st.words(0, 1000)
+    for first, n in ((0, 1), (1, 6), (3, 1), (4, 4), (997, 3), (123, 500)):
+        assert np.array_equal(st.words(first, n), whole[first:first + n])
+    for dim in (16, 18):
+        full = philox.host(philox.KIND_NORMAL_F16, st, 40 * dim, 0, 0.1).reshape(40, dim)
+        assert np.array_equal(philox.host_rows(philox.KIND_NORMAL_F16, st, [0, 39, 7, 7], dim, 0.1), full[[0, 39, 7, 7]])
+    assert np.array_equal(philox.host_rows(philox.KIND_INT8, st, [5], 64), philox.host(philox.KIND_INT8, st, 64, 5 * 64).reshape(1, 64))
+    a = philox.Stream(1).words(0, 64)
+    assert not np.array_equal(a, philox.Stream(2).words(0, 64)) and not np.array_equal(a, philox.Stream(1, seed=1).words(0, 64))
+    # the draws are what they claim to be
+    x = philox.Stream(3).normal(0, 1 << 20)
+    assert abs(float(x.mean())) < 4e-3 and abs(float(x.std()) - 1.0) < 4e-3 and abs(float((x**4).mean()) - 3.0) < 0.05
+    q = philox.Stream(4).int8(0, 1 << 20)
+    assert q.min() == -127 and q.max() == 127 and abs(float(q.astype(np.float64).mean())) < 0.3
+    u = philox.Stream(5).uniform32(0, 1 << 20, 1e-3, 1e-2)
+    assert u.dtype == np.float32 and u.min() >= np.float32(1e-3) and u.max() <= np.float32(1e-2) and abs(float(u.mean()) - 5.5e-3) < 2e-5
+    u = philox.Stream(6).uniform(0, 1 << 18)
+    assert 0.0 < u.min() and u.max() < 1.0 and abs(u.mean() - 0.5) < 3e-3
+    k = philox.Stream(7).integers(0, 1 << 18, 1, 11)
+    assert k.min() == 1 and k.max() == 10 and abs(k.mean() - 5.5) < 0.03
+    cdf = philox.poisson_cdf(8.0)
+    lens = np.searchsorted(cdf, philox.Stream(8).uniform(0, 1 << 18), side="left")
+    assert abs(lens.mean() - 8.0) < 0.03 and abs(lens.var() - 8.0) < 0.1
+
+
+def test_synthetic_configs_come_from_the_generator_streams():
+    """Batches and tables of a configuration are the generator's streams: batch b of a longer run equals batch b asked
+    for alone, and a table's rows recomputed one by one equal the table."""
+    from synth import Config2, Config4
+    cfg = Config2(batch=64, rows=3000, slots=3)
+    sparse, dense = cfg.batches(3)
+    one_s, one_d = cfg.batches(1, seed_offset=2)
+    assert np.array_equal(dense[2], one_d[0]) and not np.array_equal(dense[1], one_d[0])
+    for (a_ids, _, a_seg), (b_ids, _, b_seg) in zip(sparse[2], one_s[0]):
+        assert np.array_equal(a_ids, b_ids) and np.array_equal(a_seg, b_seg)
+    assert all(1 <= seg.min() and seg.max() <= 64 for _, _, seg in sparse[0])
+    tables = cfg.tables(device="cpu")
+    assert np.array_equal(cfg.table_rows(2, [0, 2999, 17]), tables[2][[0, 2999, 17]].numpy())
+    c4 = Config4(batch=32, rows=2000, slots=2)
+    q, sc = c4.tables(device="cpu")[1]
+    rq, rsc = c4.table_rows(1, [1999, 3])
+    assert np.array_equal(rq, q[[1999, 3]].numpy()) and np.array_equal(rsc, sc[[1999, 3]].numpy())

@@ -15,7 +15,9 @@ blaze/model_importer/ulf_importer.cc; structure after tools/example_model/din/mo
 import numpy as np
 
 import pyblaze_hip as pb
-from synth import SEED, BoundedZipf, lengths
+import philox
+from philox import Stream
+from synth import BoundedZipf, config_seed, lengths
 
 KINDS = ("item", "cate", "shop")
 
@@ -33,41 +35,49 @@ class Config3:
         self.att_layers = (4 * d3, ) + tuple(self.att_layers[1:])
         self.main_layers = (3 * d3, ) + tuple(self.main_layers[1:])
 
+    seed = config_seed(3)
+
     def tables(self, device="cuda"):
-        import torch
-        g = torch.Generator(device=device).manual_seed(SEED + 3)
-        return [(torch.randn((self.rows, self.dim), generator=g, device=device) * 0.1).to(torch.float16) for _ in KINDS]
+        """[rows, dim] fp16 N(0, 0.1) per kind (generator stream = the kind's index)"""
+        return [philox.tensor((self.rows, self.dim), philox.KIND_NORMAL_F16, Stream(s, self.seed), device, 0.1) for s in range(len(KINDS))]
+
+    def table_rows(self, kind_index, rows):
+        """rows (int array) of that kind's table recomputed on the host -> fp16 [len(rows), dim]"""
+        return philox.host_rows(philox.KIND_NORMAL_F16, Stream(kind_index, self.seed), rows, self.dim, 0.1)
 
     def weights(self):
-        """fp32 masters: per layer (W [K,N], b [N], gamma, mean, var)."""
-        rng = np.random.default_rng(SEED + 3003)
+        """fp32 masters: per layer (W [K,N], b [N], gamma, mean, var); generator stream 3000 + layer (attention layers
+        first), elements in that order."""
         out = {}
+        layer = 0
         for tag, layers in (("att", self.att_layers), ("main", self.main_layers)):
             ls = []
             for li in range(len(layers) - 1):
                 k, n = layers[li], layers[li + 1]
-                ls.append(dict(w=(rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32),
-                               b=(rng.standard_normal(n) * 0.01).astype(np.float32),
-                               gamma=(rng.standard_normal(n) * 0.1).astype(np.float32),
-                               mean=(rng.standard_normal(n) * 0.1).astype(np.float32),
-                               var=rng.uniform(0.5, 1.5, n).astype(np.float32)))
+                st = Stream(3000 + layer, self.seed)
+                layer += 1
+                ls.append(dict(w=st.normal(0, k * n, np.float32(1.0 / np.sqrt(k))).reshape(k, n),
+                               b=st.normal(k * n, n, 0.01),
+                               gamma=st.normal(k * n + n, n, 0.1),
+                               mean=st.normal(k * n + 2 * n, n, 0.1),
+                               var=st.uniform32(k * n + 3 * n, n, 0.5, 1.5)))
             out[tag] = ls
         return out
 
     def batch_inputs(self, seed_offset=0):
         """-> dict name -> array: <kind>.ids/.values/.segments (one id per sample), <kind>_his.* (U{1..T} ids per
         sample, the same length for the three kinds), mask [B, T, 1] float32."""
-        rng = np.random.default_rng(SEED + 1003 + seed_offset)
         zipf = BoundedZipf(self.rows, self.zipf_s)
         B, T = self.batch, self.T
-        seg = np.minimum(lengths(rng, "u1_50", B), T).astype(np.int32)
+        first = int(seed_offset) << 32  # (generator streams: 2000 lengths, 1000 + kind target ids, 1100 + kind history ids)
+        seg = np.minimum(lengths(Stream(2000, self.seed), first, "u1_50", B), T).astype(np.int32)
         nnz = int(seg.sum())
         feed = {}
-        for k in KINDS:
-            feed[k + ".ids"] = zipf.sample(rng, B)
+        for ki, k in enumerate(KINDS):
+            feed[k + ".ids"] = zipf.sample(Stream(1000 + ki, self.seed).uniform(first, B))
             feed[k + ".values"] = np.ones(B, np.float32)
             feed[k + ".segments"] = np.ones(B, np.int32)
-            feed[k + "_his.ids"] = zipf.sample(rng, nnz)
+            feed[k + "_his.ids"] = zipf.sample(Stream(1100 + ki, self.seed).uniform(first, nnz))
             feed[k + "_his.values"] = np.ones(nnz, np.float32)
             feed[k + "_his.segments"] = seg.copy()
         feed["mask"] = (np.arange(T)[None, :] < seg[:, None]).astype(np.float32).reshape(B, T, 1)

@@ -3,10 +3,21 @@
 Host-side harness code for bench.py, the smoke check and the full-size parity tests: it builds
 device-resident tables, batches of sparse inputs (<fg>.ids / .values / .segments triples, the
 reference's input layout: blaze/operator/common_helper.h:96-98) and MLP weights.
+
+Every number comes from the counter-based generator of philox.py, keyed by (seed, stream id, index): seed = SEED +
+1000003 * configuration number; stream id = slot for tables (5000 + slot for an int8 table's scales), 1000 + slot for
+ids, 2000 + slot for lengths, 3000 + layer for weights, 4000 for dense features; index = position, with the batch
+number in its upper 32 bits for per-batch data.  Tables are filled on the device and can be recomputed row by row on
+the host with the same bits.
 """
 import numpy as np
 
-SEED = 20240613
+import philox
+from philox import SEED, Stream
+
+
+def config_seed(number):
+    return SEED + 1000003 * number
 
 
 class BoundedZipf:
@@ -19,33 +30,56 @@ class BoundedZipf:
         self.cdf /= self.cdf[-1]
         self.n = n
 
-    def sample(self, rng, size):
-        ranks = np.searchsorted(self.cdf, rng.random(size), side="left").astype(np.int64)
+    def sample(self, u):
+        """u: uniform draws in (0, 1) -> rows"""
+        ranks = np.minimum(np.searchsorted(self.cdf, u, side="left"), self.n - 1).astype(np.int64)
         return (ranks * 2654435761) % self.n
 
 
-def lengths(rng, kind, batch):
-    if kind == "poisson8":  # config 2
-        return np.clip(rng.poisson(8, batch), 1, 64).astype(np.int32)
-    if kind == "poisson20":  # config 4 (0 allowed)
-        return rng.poisson(20, batch).astype(np.int32)
-    if kind == "u1_10":  # config 1
-        return rng.integers(1, 11, batch).astype(np.int32)
-    if kind == "u1_4":  # config 5
-        return rng.integers(1, 5, batch).astype(np.int32)
-    if kind == "u1_50":  # config 3
-        return rng.integers(1, 51, batch).astype(np.int32)
-    raise ValueError(kind)
+class UniformIds:
+    """ids uniform over the table's rows (config 5)"""
+
+    def __init__(self, n):
+        self.n = n
+
+    def sample(self, u):
+        return np.minimum((u * self.n).astype(np.int64), self.n - 1)
 
 
-def sparse_batch(rng, zipf, slots, batch, length_kind):
-    """One batch: list over slots of (ids int64 [nnz], values float32 [nnz] == 1, segments int32 [batch])."""
+_POISSON = {}
+
+
+def lengths(stream, first, kind, batch):
+    """per-sample id counts of one slot: elements first .. first + batch - 1 of the slot's length stream"""
+    if kind in ("poisson8", "poisson20"):  # config 2 (clipped to 1..64) / config 4 (0 allowed): inverse CDF
+        lam = 8 if kind == "poisson8" else 20
+        if lam not in _POISSON:
+            _POISSON[lam] = philox.poisson_cdf(float(lam))
+        k = np.searchsorted(_POISSON[lam], stream.uniform(first, batch), side="left")
+        return (np.clip(k, 1, 64) if kind == "poisson8" else k).astype(np.int32)
+    hi = {"u1_10": 11, "u1_4": 5, "u1_50": 51}[kind]  # configs 1, 5, 3
+    return stream.integers(first, batch, 1, hi).astype(np.int32)
+
+
+def sparse_batch(seed, batch_index, ids_of, slots, batch, length_kind):
+    """Batch number batch_index: list over slots of (ids int64 [nnz], values float32 [nnz] == 1, segments int32 [batch]).
+    ids_of: BoundedZipf or UniformIds."""
     out = []
-    for _ in range(slots):
-        seg = lengths(rng, length_kind, batch)
+    first = int(batch_index) << 32
+    for s in range(slots):
+        seg = lengths(Stream(2000 + s, seed), first, length_kind, batch)
         nnz = int(seg.sum())
-        out.append((zipf.sample(rng, nnz), np.ones(nnz, np.float32), seg))
+        out.append((ids_of.sample(Stream(1000 + s, seed).uniform(first, nnz)), np.ones(nnz, np.float32), seg))
     return out
+
+
+def normal_weights(seed, layer, k, n, device):
+    """fp32 master weight [k, n] N(0, 1/sqrt(k)) and bias [n] N(0, 0.01) of a layer, as torch tensors"""
+    import torch
+    st = Stream(3000 + layer, seed)
+    w = st.normal(0, k * n, np.float32(1.0 / np.sqrt(k))).reshape(k, n)
+    b = st.normal(k * n, n, 0.01)
+    return torch.from_numpy(w).to(device), torch.from_numpy(b).to(device)
 
 
 def embedding_bytes(batches_nnz, batch, slots, row_bytes, scale_bytes, out_cols, out_elem):
@@ -70,31 +104,37 @@ class Config2:
         self.layers = (self.in_dim, ) + tuple(self.layers[1:])
 
     table_dtype = "float16"
+    number = 2
+
+    @property
+    def seed(self):
+        return config_seed(self.number)
 
     def tables(self, device="cuda"):
-        import torch
-        g = torch.Generator(device=device).manual_seed(SEED)
-        return [(torch.randn((self.rows, self.dim), generator=g, device=device) * 0.01).to(getattr(torch, self.table_dtype))
-                for _ in range(self.slots)]
+        """[rows, dim] N(0, 0.01) per slot, rounded to the table type"""
+        kind = philox.KIND_NORMAL_F16 if self.table_dtype == "float16" else philox.KIND_NORMAL_F32
+        return [philox.tensor((self.rows, self.dim), kind, Stream(s, self.seed), device, 0.01) for s in range(self.slots)]
+
+    def table_rows(self, slot, rows):
+        """rows (int array) of slot's table recomputed on the host -> [len(rows), dim] of the table type"""
+        kind = philox.KIND_NORMAL_F16 if self.table_dtype == "float16" else philox.KIND_NORMAL_F32
+        return philox.host_rows(kind, Stream(slot, self.seed), rows, self.dim, 0.01)
 
     def mlp(self, device="cuda"):
         """fp32 master weights [K,N] N(0, 1/sqrt(fan_in)), bias N(0, 0.01), PReLU slope 0.25 per channel."""
         import torch
-        g = torch.Generator(device="cpu").manual_seed(SEED + 3000)
         out = []
         for li in range(len(self.layers) - 1):
-            k, n = self.layers[li], self.layers[li + 1]
-            w = torch.randn((k, n), generator=g) / np.sqrt(k)
-            b = torch.randn(n, generator=g) * 0.01
-            slope = torch.full((n, ), 0.25)
-            out.append((w.to(device), b.to(device), slope.to(device)))
+            w, b = normal_weights(self.seed, li, self.layers[li], self.layers[li + 1], device)
+            out.append((w, b, torch.full((self.layers[li + 1], ), 0.25).to(device)))
         return out
 
     def batches(self, n, seed_offset=0):
-        rng = np.random.default_rng(SEED + 1000 + seed_offset)
+        """batches seed_offset .. seed_offset + n - 1 of the configuration's input stream"""
         zipf = BoundedZipf(self.rows, self.zipf_s)
-        sparse = [sparse_batch(rng, zipf, self.slots, self.batch, self.length_kind) for _ in range(n)]
-        dense = [rng.standard_normal((self.batch, self.dense)).astype(np.float32) for _ in range(n)]
+        sparse = [sparse_batch(self.seed, seed_offset + b, zipf, self.slots, self.batch, self.length_kind) for b in range(n)]
+        dense = [Stream(4000, self.seed).normal((seed_offset + b) << 32, self.batch * self.dense).reshape(self.batch, self.dense)
+                 for b in range(n)]
         return sparse, dense
 
 
@@ -106,6 +146,7 @@ class Config1(Config2):
     layers = (192, 200, 80, 2)
     zipf_s, length_kind = 1.1, "u1_10"
     table_dtype = "float32"
+    number = 1
 
 
 class Config4:
@@ -118,20 +159,21 @@ class Config4:
     def __init__(self, batch=None, rows=None, slots=None):
         self.batch, self.rows, self.slots = batch or self.batch, rows or self.rows, slots or self.slots
 
+    seed = config_seed(4)
+
     def tables(self, device="cuda"):
-        """-> list of (int8 [rows, dim], fp32 scale [rows]) torch tensors."""
-        import torch
-        g = torch.Generator(device=device).manual_seed(SEED + 4)
-        out = []
-        for _ in range(self.slots):
-            q = torch.randint(-127, 128, (self.rows, self.dim), dtype=torch.int8, device=device, generator=g)
-            sc = torch.rand(self.rows, device=device, generator=g) * 9e-3 + 1e-3
-            out.append((q, sc))
-        return out
+        """-> list of (int8 [rows, dim] uniform over -127 .. 127, fp32 scale [rows] uniform over [1e-3, 1e-2)) torch tensors."""
+        return [(philox.tensor((self.rows, self.dim), philox.KIND_INT8, Stream(s, self.seed), device),
+                 philox.tensor((self.rows, ), philox.KIND_UNIFORM_F32, Stream(5000 + s, self.seed), device, 1e-3, 1e-2))
+                for s in range(self.slots)]
+
+    def table_rows(self, slot, rows):
+        """rows (int array) of slot's table recomputed on the host -> (int8 [len(rows), dim], fp32 scale [len(rows)])"""
+        return (philox.host_rows(philox.KIND_INT8, Stream(slot, self.seed), rows, self.dim),
+                philox.host_rows(philox.KIND_UNIFORM_F32, Stream(5000 + slot, self.seed), rows, 1, 1e-3, 1e-2).reshape(-1))
 
     def batch_inputs(self, seed_offset=0):
-        rng = np.random.default_rng(SEED + 1004 + seed_offset)
-        return sparse_batch(rng, BoundedZipf(self.rows, self.zipf_s), self.slots, self.batch, self.length_kind)
+        return sparse_batch(self.seed, seed_offset, BoundedZipf(self.rows, self.zipf_s), self.slots, self.batch, self.length_kind)
 
 
 class Config5:
@@ -147,27 +189,19 @@ class Config5:
         self.batch, self.rows, self.slots = batch or self.batch, rows or self.rows, slots or self.slots
         self.layers = (self.slots * self.dim, ) + tuple(self.layers[1:])
 
+    seed = config_seed(5)
+
     def tables(self, device="cuda"):
-        import torch
-        g = torch.Generator(device=device).manual_seed(SEED + 5)
-        return [(torch.randn((self.rows, self.dim), generator=g, device=device) * 0.01).to(torch.float16)
-                for _ in range(self.slots)]
+        return [philox.tensor((self.rows, self.dim), philox.KIND_NORMAL_F16, Stream(s, self.seed), device, 0.01)
+                for s in range(self.slots)]
+
+    def table_rows(self, slot, rows):
+        """rows (int array) of slot's table recomputed on the host -> fp16 [len(rows), dim]"""
+        return philox.host_rows(philox.KIND_NORMAL_F16, Stream(slot, self.seed), rows, self.dim, 0.01)
 
     def batch_inputs(self, seed_offset=0):
-        rng = np.random.default_rng(SEED + 1005 + seed_offset)
-        out = []
-        for _ in range(self.slots):
-            seg = lengths(rng, self.length_kind, self.batch)
-            nnz = int(seg.sum())
-            out.append((rng.integers(0, self.rows, nnz).astype(np.int64), np.ones(nnz, np.float32), seg))
-        return out
+        return sparse_batch(self.seed, seed_offset, UniformIds(self.rows), self.slots, self.batch, self.length_kind)
 
     def mlp(self, device="cuda"):
         """fp32 master weights [K,N] N(0, 1/sqrt(fan_in)), bias N(0, 0.01)."""
-        import torch
-        g = torch.Generator(device="cpu").manual_seed(SEED + 3005)
-        out = []
-        for li in range(len(self.layers) - 1):
-            k, n = self.layers[li], self.layers[li + 1]
-            out.append(((torch.randn((k, n), generator=g) / np.sqrt(k)).to(device), (torch.randn(n, generator=g) * 0.01).to(device)))
-        return out
+        return [normal_weights(self.seed, li, self.layers[li], self.layers[li + 1], device) for li in range(len(self.layers) - 1)]
