@@ -357,6 +357,10 @@ BZ_API int bz_gemm_strided_batched(const bz_bgemm_desc* desc, bz_stream_t stream
  * before it is used, as the Mul operator's output would be, and both sums add in
  * ascending t, so the outputs equal the three operators' bit for bit.
  * mask null: w is used as it is.  att null or sum null: that output is not computed.
+ * Extension for the Concat that usually follows (DIN joins [target, sum, att] for its main MLP, concat_op.cu:33): att
+ * and sum may be rows of a wider matrix (ld_att / ld_sum elements between rows; 0 = c), and one more piece of copy_c
+ * elements per item is copied alongside, copy_dst[b, 0..copy_c) = copy_src[b, 0..copy_c), so that the three column
+ * ranges of the Concat's output are written by this launch and the Concat has nothing left to do.
  */
 typedef struct bz_weighted_pool_desc {
   const void* w;     /* [batch, t] */
@@ -366,8 +370,12 @@ typedef struct bz_weighted_pool_desc {
   void* sum;         /* [batch, c] or null */
   int64_t batch;
   int32_t t, c;
-  int32_t dtype;     /* BZ_F32 | BZ_F16 for all five */
-  int32_t reserved_;
+  int32_t dtype;     /* BZ_F32 | BZ_F16 for all of them */
+  int32_t copy_c;    /* elements per item of the copied piece; 0 = none */
+  int64_t ld_att, ld_sum;           /* elements between the rows of att / sum; 0 = c */
+  const void* copy_src;             /* [batch, copy_c] at ld_copy_src, or null */
+  void* copy_dst;                   /* [batch, copy_c] at ld_copy_dst */
+  int64_t ld_copy_src, ld_copy_dst; /* elements between rows; 0 = copy_c */
 } bz_weighted_pool_desc;
 
 BZ_API int bz_weighted_pool(const bz_weighted_pool_desc* desc, bz_stream_t stream);

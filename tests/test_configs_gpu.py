@@ -451,3 +451,51 @@ def test_history_blocks_written_into_their_concat_equal_the_copy():
     assert "Concat:concat_his" in ran, ran
     np.testing.assert_array_equal(p.output_asnumpy("his"), outs[1][0]["his"])
     np.testing.assert_array_equal(p.output_asnumpy(mid), outs[1][0]["his"][:, :, :cfg.dim])
+
+
+def test_main_input_concat_written_by_the_attention_tail():
+    """Mul -> MatMul(transA) -> Reshape, ReduceSum, Concat(axis 1)[q, hsum, att]: the attention tail's one launch also
+    writes the Concat's output - its own two results at their columns, the target block copied alongside
+    (fuse_concat_into_weighted_pool, on by default) - and neither the Reshape nor the Concat runs; with the switch off the
+    Concat copies.  Same bits either way, also when the batch changes between forwards; a tail result that is an output
+    of the net keeps its own memory and the Concat runs."""
+    import json
+    import din_model
+    cfg = din_model.Config3(batch=64, rows=3000, T=12)
+    small = din_model.Config3(batch=9, rows=3000, T=12)
+    big = din_model.Config3(batch=130, rows=3000, T=12)
+    tables, weights = cfg.tables(), cfg.weights()
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=1), big.batch_inputs(seed_offset=2), cfg.batch_inputs(seed_offset=3)]
+    outs = {}
+    for fuse in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("main_in", "q"),
+                                             net_args={"fuse_concat_into_weighted_pool": fuse})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for b in batches:
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            got.append({k: p.output_asnumpy(k).copy() for k in ("main_in", "q", "prob")})
+        ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+        ran = [e["name"].split(":")[0] for e in ev]
+        assert ("Concat" in ran) == (fuse == 0), ran
+        assert [e["args"]["launches"] for e in ev if e["name"].split(":")[0] == "MatMul"] == [1]
+        outs[fuse] = got
+    D3 = 3 * cfg.dim
+    for g1, g0, b in zip(outs[1], outs[0], (64, 9, 130, 64)):
+        assert g1["main_in"].shape == (b, 3 * D3) and g1["main_in"][:, D3:].any()
+        np.testing.assert_array_equal(g1["main_in"][:, :D3], g1["q"])
+        for k in g1:
+            np.testing.assert_array_equal(g1[k], g0[k], err_msg=k)
+    # the tail's results as outputs of the net: the rewrite does not apply, everything is stored
+    pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("main_in", "hsum", "att"))
+    p = pm.create_predictor(1, 0)
+    p.register_observers(["profile"])
+    din_model.feed(p, inputs, batches[0], np.float16)
+    p.forward()
+    ran = [e["name"].split(":")[0] for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
+    assert "Concat" in ran, ran
+    np.testing.assert_array_equal(p.output_asnumpy("main_in"), outs[1][0]["main_in"])
+    np.testing.assert_array_equal(p.output_asnumpy("hsum"), outs[1][0]["main_in"][:, D3:2 * D3])
+    np.testing.assert_array_equal(p.output_asnumpy("att"), outs[1][0]["main_in"][:, 2 * D3:])

@@ -478,6 +478,7 @@ def test_fc_split_argument_errors(bz):
 def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T, Cn):
     """bz_weighted_pool against the three launches it replaces (Mul, strided-batched GEMM with transA, ReduceSum), bit
     for bit, and against the oracle's fp32 sums of the rounded operands."""
+    import ctypes as C
     import torch
     print("weighted pool %s B=%d T=%d C=%d" % (dtype_name, B, T, Cn), flush=True)
     tdt = _tdtype(dtype_name)
@@ -501,6 +502,24 @@ def test_weighted_pool_equals_mul_matmul_reducesum(bz, oracle, dtype_name, B, T,
     none2, tot2 = bz.weighted_pool(dx)
     torch.cuda.synchronize()
     assert none is None and none2 is None and torch.equal(att2, c.reshape(B, Cn)) and torch.equal(tot2, s)
+    # both outputs as column ranges of a wider matrix, with a third piece copied alongside from a pitched source: the
+    # Concat that follows the attention tail, written by the same launch; nothing else of the matrix is touched
+    n_copy = 7
+    wide = torch.full((B, 2 * Cn + n_copy + 5), 3.0, dtype=tdt, device="cuda")
+    src = (torch.arange(B * (n_copy + 3), device="cuda").reshape(B, n_copy + 3) % 251).to(tdt)
+    bz.weighted_pool(dx, dw, dm, att_out=wide[:, n_copy + Cn + 2:n_copy + 2 * Cn + 2], sum_out=wide[:, n_copy:n_copy + Cn],
+                     copy=(src[:, 1:1 + n_copy], wide[:, :n_copy]))
+    torch.cuda.synchronize()
+    assert torch.equal(wide[:, :n_copy], src[:, 1:1 + n_copy]) and torch.equal(wide[:, n_copy:n_copy + Cn], tot)
+    assert torch.equal(wide[:, n_copy + Cn + 2:n_copy + 2 * Cn + 2], att)
+    assert bool((wide[:, n_copy + Cn:n_copy + Cn + 2] == 3.0).all()) and bool((wide[:, n_copy + 2 * Cn + 2:] == 3.0).all())
+    bad = bz.WeightedPoolDesc()
+    bad.x, bad.w, bad.att = dx.data_ptr(), dw.data_ptr(), wide.data_ptr()
+    bad.batch, bad.t, bad.c, bad.dtype, bad.ld_att = B, T, Cn, bz.bz_dtype(tdt), Cn - 1
+    if Cn > 1:  # (0 means "c")
+        assert bz.lib().bz_weighted_pool(C.byref(bad), None) == -22 and b"ld_att" in bz.lib().bz_last_error()
+    bad.ld_att, bad.copy_c = 0, 4  # a piece to copy without its pointers
+    assert bz.lib().bz_weighted_pool(C.byref(bad), None) == -22 and b"copied piece" in bz.lib().bz_last_error()
     # oracle: fp32 sums in ascending t of the rounded operands
     wm = _round_to(w * mask, dtype_name)
     want_att = np.zeros((B, Cn), np.float32)

@@ -71,7 +71,9 @@ class BgemmDesc(C.Structure):
 
 class WeightedPoolDesc(C.Structure):
     _fields_ = [("w", C.c_void_p), ("mask", C.c_void_p), ("x", C.c_void_p), ("att", C.c_void_p), ("sum", C.c_void_p),
-                ("batch", C.c_int64), ("t", C.c_int32), ("c", C.c_int32), ("dtype", C.c_int32), ("reserved_", C.c_int32)]
+                ("batch", C.c_int64), ("t", C.c_int32), ("c", C.c_int32), ("dtype", C.c_int32), ("copy_c", C.c_int32),
+                ("ld_att", C.c_int64), ("ld_sum", C.c_int64), ("copy_src", C.c_void_p), ("copy_dst", C.c_void_p),
+                ("ld_copy_src", C.c_int64), ("ld_copy_dst", C.c_int64)]
 
 
 class ActDesc(C.Structure):
@@ -426,18 +428,29 @@ def gemm_strided_batched(a, b, c, m, n, k, batch, stride_a, stride_b, stride_c, 
     return c
 
 
-def weighted_pool(x, w=None, mask=None, want_sum=True, stream=None):
-    """x [B, T, C]; w, mask [B, T] (or [B, T, 1]) -> (att [B, C] or None, sum [B, C] or None), see bz_weighted_pool."""
+def weighted_pool(x, w=None, mask=None, want_sum=True, stream=None, att_out=None, sum_out=None, copy=None):
+    """x [B, T, C]; w, mask [B, T] (or [B, T, 1]) -> (att [B, C] or None, sum [B, C] or None), see bz_weighted_pool.
+    att_out / sum_out: [B, C] views (row stride >= C, unit column stride) to write instead of new tensors;
+    copy = (src [B, n] view, dst [B, n] view): the piece copied alongside."""
     import torch
     B, T, Cn = x.shape
     d = WeightedPoolDesc()
-    att = torch.empty((B, Cn), dtype=x.dtype, device=x.device) if w is not None else None
-    tot = torch.empty((B, Cn), dtype=x.dtype, device=x.device) if want_sum else None
+    att = (att_out if att_out is not None else torch.empty((B, Cn), dtype=x.dtype, device=x.device)) if w is not None else None
+    tot = (sum_out if sum_out is not None else torch.empty((B, Cn), dtype=x.dtype, device=x.device)) if want_sum else None
+    for t in (att, tot):
+        assert t is None or (tuple(t.shape) == (B, Cn) and t.stride(1) == 1 and t.dtype == x.dtype)
     d.x = x.data_ptr()
     d.w = w.data_ptr() if w is not None else None
     d.mask = mask.data_ptr() if mask is not None else None
     d.att = att.data_ptr() if att is not None else None
     d.sum = tot.data_ptr() if tot is not None else None
+    d.ld_att = att.stride(0) if att is not None else 0
+    d.ld_sum = tot.stride(0) if tot is not None else 0
+    if copy is not None:
+        src, dst = copy
+        assert src.shape == dst.shape and src.shape[0] == B and src.stride(1) == 1 and dst.stride(1) == 1 and src.dtype == dst.dtype == x.dtype
+        d.copy_src, d.copy_dst, d.copy_c = src.data_ptr(), dst.data_ptr(), src.shape[1]
+        d.ld_copy_src, d.ld_copy_dst = src.stride(0), dst.stride(0)
     d.batch, d.t, d.c, d.dtype = B, T, Cn, bz_dtype(x.dtype)
     check(lib().bz_weighted_pool(C.byref(d), _stream_ptr(stream)))
     return att, tot

@@ -104,10 +104,14 @@ constexpr int kPoolUnroll = 64;
 template <typename T>
 __global__ __launch_bounds__(256) void bz_weighted_pool_kernel(const T* __restrict__ w, const T* __restrict__ mask,
                                                                const T* __restrict__ x, T* __restrict__ att, T* __restrict__ sum,
-                                                               int64_t batch, int t_len, int c_len) {
+                                                               int64_t batch, int t_len, int c_len, int64_t ld_att, int64_t ld_sum,
+                                                               const T* __restrict__ copy_src, T* __restrict__ copy_dst, int copy_c,
+                                                               int64_t ld_copy_src, int64_t ld_copy_dst) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t item = (int64_t)blockIdx.x * 4 + wave;
   if (item >= batch) return;
+  // the piece copied alongside (asked for first: its loads travel with the history's)
+  for (int c = lane; c < copy_c; c += 64) copy_dst[item * ld_copy_dst + c] = copy_src[item * ld_copy_src + c];
   const T* wp = w + item * t_len;
   const T* mp = mask ? mask + item * t_len : nullptr;
   const T* xp = x + item * (int64_t)t_len * c_len;
@@ -144,8 +148,8 @@ __global__ __launch_bounds__(256) void bz_weighted_pool_kernel(const T* __restri
           acc_s = __fadd_rn(acc_s, xv[u]);
         }
     }
-    if (live && att) st<T>(att + item * c_len + c, acc_w);
-    if (live && sum) st<T>(sum + item * c_len + c, acc_s);
+    if (live && att) st<T>(att + item * ld_att + c, acc_w);
+    if (live && sum) st<T>(sum + item * ld_sum + c, acc_s);
   }
 }
 
@@ -157,6 +161,11 @@ extern "C" int bz_weighted_pool(const bz_weighted_pool_desc* desc, bz_stream_t s
   BZ_REQUIRE(d.x != nullptr && (d.att != nullptr || d.sum != nullptr), "bz_weighted_pool: null x, or neither output asked for");
   BZ_REQUIRE(d.att == nullptr || d.w != nullptr, "bz_weighted_pool: the weighted sum needs w");
   BZ_REQUIRE(d.batch >= 0 && d.t > 0 && d.c > 0, "bz_weighted_pool: bad shape batch=%lld t=%d c=%d", (long long)d.batch, d.t, d.c);
+  const int64_t ld_att = d.ld_att ? d.ld_att : d.c, ld_sum = d.ld_sum ? d.ld_sum : d.c;
+  const int64_t ld_cs = d.ld_copy_src ? d.ld_copy_src : d.copy_c, ld_cd = d.ld_copy_dst ? d.ld_copy_dst : d.copy_c;
+  BZ_REQUIRE(ld_att >= d.c && ld_sum >= d.c, "bz_weighted_pool: ld_att=%lld / ld_sum=%lld below c=%d", (long long)ld_att, (long long)ld_sum, d.c);
+  BZ_REQUIRE(d.copy_c >= 0 && (d.copy_c == 0 || (d.copy_src != nullptr && d.copy_dst != nullptr && ld_cs >= d.copy_c && ld_cd >= d.copy_c)),
+             "bz_weighted_pool: copied piece of %d elements with a null pointer or a leading dimension below it", d.copy_c);
   if (d.batch == 0) return BZ_OK;
   BZ_REQUIRE((d.batch + 3) / 4 < (1ll << 31), "bz_weighted_pool: batch %lld too large", (long long)d.batch);
   const int grid = (int)((d.batch + 3) / 4);
@@ -164,10 +173,12 @@ extern "C" int bz_weighted_pool(const bz_weighted_pool_desc* desc, bz_stream_t s
   const void* w = d.att ? d.w : d.x;  // no weighted sum: any readable address of t elements per item will do
   if (d.dtype == BZ_F32)
     hipLaunchKernelGGL(bz_weighted_pool_kernel<float>, dim3(grid), dim3(256), 0, s, (const float*)w, (const float*)(d.att ? d.mask : nullptr),
-                       (const float*)d.x, (float*)d.att, (float*)d.sum, d.batch, d.t, d.c);
+                       (const float*)d.x, (float*)d.att, (float*)d.sum, d.batch, d.t, d.c, ld_att, ld_sum, (const float*)d.copy_src,
+                       (float*)d.copy_dst, d.copy_c, ld_cs, ld_cd);
   else if (d.dtype == BZ_F16)
     hipLaunchKernelGGL(bz_weighted_pool_kernel<__half>, dim3(grid), dim3(256), 0, s, (const __half*)w,
-                       (const __half*)(d.att ? d.mask : nullptr), (const __half*)d.x, (__half*)d.att, (__half*)d.sum, d.batch, d.t, d.c);
+                       (const __half*)(d.att ? d.mask : nullptr), (const __half*)d.x, (__half*)d.att, (__half*)d.sum, d.batch, d.t, d.c,
+                       ld_att, ld_sum, (const __half*)d.copy_src, (__half*)d.copy_dst, d.copy_c, ld_cs, ld_cd);
   else
     return bz::fail(BZ_ENOTSUP, "bz_weighted_pool: unsupported dtype %d", d.dtype);
   BZ_LAUNCH_OK("bz_weighted_pool_kernel");

@@ -745,6 +745,14 @@ class MatMulOp : public Operator<Context>, public WeightedPoolHost {
     pool_mul_ = mul;
     pool_sum_ = reduce_sum;
   }
+  OperatorBase* AdoptedReduceSum() const override { return pool_sum_; }
+  void AdoptTailConcat(OperatorBase* concat, OperatorBase* reshape, int att_pos, int sum_pos, int copy_pos) override {
+    concat_ = concat;
+    concat_reshape_ = reshape;
+    att_pos_ = att_pos;
+    sum_pos_ = sum_pos;
+    copy_pos_ = copy_pos;
+  }
   int LaunchesOfLastRun() const override { return launches_; }
 
   MatMulOp(const OperatorDef& def, Workspace* workspace) : Operator<Context>(def, workspace) {
@@ -755,13 +763,25 @@ class MatMulOp : public Operator<Context>, public WeightedPoolHost {
 
   bool RunOnDevice() override {
     launches_ = 1;
-    if (pool_mul_ || pool_sum_) {
+    if (pool_mul_ || pool_sum_ || concat_) {
       if (RunWeightedPool()) return true;
       // shapes the one-launch form does not take: the adopted operators run after all
       if (pool_mul_ && !pool_mul_->Run(context_.stream_id())) return false;
       if (pool_sum_ && !pool_sum_->Run(context_.stream_id())) return false;
       launches_ += (pool_mul_ != nullptr) + (pool_sum_ != nullptr);
     }
+    if (!RunPlain()) return false;
+    return RunTailConcat();
+  }
+
+ protected:
+  // the Reshape and the Concat behind this MatMul, when its own launch has not written the Concat's output
+  bool RunTailConcat() {
+    if (!concat_) return true;
+    ++launches_;
+    return concat_reshape_->Run(context_.stream_id()) && concat_->Run(context_.stream_id());
+  }
+  bool RunPlain() {
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
     Blob* c = this->Output(0);
@@ -781,8 +801,6 @@ class MatMulOp : public Operator<Context>, public WeightedPoolHost {
                    a->data_type(), context_.hip_stream());
     return true;
   }
-
- protected:
   void Setup() {
     Blob* a = this->Input(0);
     Blob* b = this->Input(1);
@@ -824,30 +842,72 @@ class MatMulOp : public Operator<Context>, public WeightedPoolHost {
     if (xs[1] <= 0 || xs[2] <= 0 || xs[1] >= (1ll << 31) || xs[2] >= (1ll << 31)) return false;
     Blob* c = this->Output(0);
     c->set_data_type((DataType)x->data_type());
-    c->Reshape({xs[0], 1, xs[2]});
-    Blob* s = nullptr;
-    if (pool_sum_) {
-      s = pool_sum_->Output(0);
-      s->set_data_type((DataType)x->data_type());
-      s->Reshape({xs[0], xs[2]});
-    }
+    Blob* s = pool_sum_ ? pool_sum_->Output(0) : nullptr;
+    if (s) s->set_data_type((DataType)x->data_type());
     bz_weighted_pool_desc d;
     memset(&d, 0, sizeof(d));
+    // the Concat behind it, when its other input (if any) has the rows of this batch: everything lands in its output
+    Blob* other = concat_ && copy_pos_ >= 0 ? concat_->Input(copy_pos_) : nullptr;
+    const bool tail = concat_ && (!other || (other->shape().size() == 2 && other->shape()[0] == xs[0] && other->shape()[1] > 0 &&
+                                             other->shape()[1] < (1ll << 31) && other->data_type() == x->data_type()));
+    if (tail) {
+      Blob* out = concat_->Output(0);
+      const int n_in = concat_->InputSize();
+      TIndex total = 0, col_att = 0, col_sum = 0, col_copy = 0;
+      for (int i = 0; i < n_in; ++i) {
+        if (i == att_pos_) col_att = total;
+        if (i == sum_pos_) col_sum = total;
+        if (i == copy_pos_) col_copy = total;
+        total += i == copy_pos_ ? other->shape()[1] : xs[2];
+      }
+      out->set_data_type((DataType)x->data_type());
+      out->Reshape({xs[0], total});
+      // (the results nobody reads any more keep their shapes and hold no data)
+      c->SetShapeOnly({xs[0], 1, xs[2]});
+      concat_reshape_->Output(0)->set_data_type((DataType)x->data_type());
+      concat_reshape_->Output(0)->SetShapeOnly({xs[0], xs[2]});
+      const size_t es = DataTypeSize(x->data_type());
+      d.att = (char*)out->data() + col_att * es;
+      d.ld_att = total;
+      if (s && sum_pos_ >= 0) {
+        s->SetShapeOnly({xs[0], xs[2]});
+        d.sum = (char*)out->data() + col_sum * es;
+        d.ld_sum = total;
+      } else if (s) {
+        s->Reshape({xs[0], xs[2]});
+        d.sum = s->data();
+      }
+      if (other) {
+        d.copy_src = other->data();
+        d.ld_copy_src = other->pitch() ? other->pitch() : other->shape()[1];
+        d.copy_dst = (char*)out->data() + col_copy * es;
+        d.ld_copy_dst = total;
+        d.copy_c = (int32_t)other->shape()[1];
+      }
+    } else {
+      c->Reshape({xs[0], 1, xs[2]});
+      d.att = c->data();
+      if (s) {
+        s->Reshape({xs[0], xs[2]});
+        d.sum = s->data();
+      }
+    }
     d.w = w->data();
     d.mask = mask ? mask->data() : nullptr;
     d.x = x->data();
-    d.att = c->data();
-    d.sum = s ? s->data() : nullptr;
     d.batch = (int64_t)xs[0];
     d.t = (int32_t)xs[1];
     d.c = (int32_t)xs[2];
     d.dtype = BzType(x->data_type());
     BZ_CHECK(bz_weighted_pool(&d, context_.hip_stream()));
-    return true;
+    return tail ? true : RunTailConcat();
   }
   bool transa_, transb_, from_deepnet_;
   OperatorBase* pool_mul_ = nullptr;
   OperatorBase* pool_sum_ = nullptr;
+  OperatorBase* concat_ = nullptr;          // the Concat behind the weighted pool (AdoptTailConcat) and the Reshape before it
+  OperatorBase* concat_reshape_ = nullptr;
+  int att_pos_ = -1, sum_pos_ = -1, copy_pos_ = -1;
   int launches_ = 1;
 };
 

@@ -219,6 +219,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     FuseWeightedPools();
     FuseConcatsIntoFcs();
     ChainNarrowFcs();
+    FuseConcatsIntoWeightedPools();
   }
 }
 
@@ -313,6 +314,70 @@ void SimpleNet::FuseWeightedPools() {
     host->AdoptWeightedPool(mul >= 0 ? operators_[mul].get() : nullptr, red >= 0 ? operators_[red].get() : nullptr);
     if (mul >= 0) skipped_[mul] = true;
     if (red >= 0) skipped_[red] = true;
+  }
+}
+
+// MatMul that runs as a weighted pool -> Reshape of its [B, 1, C] result to [B, C] -> Concat (axis 1) of that with the
+// adopted ReduceSum's result and at most one more tensor: the MatMul's launch writes the Concat's output (graph.h,
+// WeightedPoolHost::AdoptTailConcat).  The Reshape's and the ReduceSum's results must be read by the Concat alone, the
+// other tensor must be final before the MatMul, and nothing between the MatMul and the Concat may touch the Concat's
+// output.  Switch: fuse_concat_into_weighted_pool: 0.
+void SimpleNet::FuseConcatsIntoWeightedPools() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "fuse_concat_into_weighted_pool");
+  if (arg && arg->has_i && arg->i == 0) return;
+  auto readers_of = [&](const std::string& name) {
+    int readers = 0;
+    for (size_t j = 0; j < operators_.size(); ++j)
+      for (const auto& in : operators_[j]->operator_def().input()) readers += (in == name);
+    for (const auto& eo : external_output_) readers += (eo == name);
+    return readers;
+  };
+  for (size_t m = 0; m < operators_.size(); ++m) {
+    auto* host = skipped_[m] ? nullptr : dynamic_cast<WeightedPoolHost*>(operators_[m].get());
+    if (!host || !host->WeightedPoolEligible()) continue;
+    const OperatorDef& md = operators_[m]->operator_def();
+    if (md.output_size() != 1 || readers_of(md.output(0)) != 1) continue;
+    int r = -1;
+    for (size_t j = m + 1; j < operators_.size() && r < 0; ++j)
+      if (!skipped_[j] && operators_[j]->type() == "Reshape" && operators_[j]->operator_def().input_size() == 2 &&
+          operators_[j]->operator_def().input(0) == md.output(0) && operators_[j]->operator_def().output_size() == 1)
+        r = (int)j;
+    if (r < 0) continue;
+    const std::string& att = operators_[r]->operator_def().output(0);
+    if (att == md.output(0) || readers_of(att) != 1) continue;
+    int c = -1;
+    for (size_t j = r + 1; j < operators_.size() && c < 0; ++j)
+      for (const auto& in : operators_[j]->operator_def().input())
+        if (in == att) c = (int)j;
+    if (c < 0 || skipped_[c] || operators_[c]->type() != "Concat") continue;
+    const OperatorDef& cd = operators_[c]->operator_def();
+    if (ArgumentHelper::GetSingle<int>(cd.arg(), "axis", 1) != 1 || cd.output_size() != 1) continue;
+    OperatorBase* red = host->AdoptedReduceSum();
+    int att_pos = -1, sum_pos = -1, copy_pos = -1;
+    bool ok = true;
+    for (int i = 0; i < cd.input_size() && ok; ++i) {
+      const std::string& name = cd.input(i);
+      if (name == att) {
+        ok = att_pos < 0;
+        att_pos = i;
+      } else if (red && name == red->operator_def().output(0)) {
+        ok = sum_pos < 0 && readers_of(name) == 1;
+        sum_pos = i;
+      } else {
+        ok = copy_pos < 0 && name != cd.output(0);
+        copy_pos = i;
+      }
+    }
+    if (!ok || att_pos < 0) continue;
+    // the copied tensor is final when the MatMul runs; the Concat's output is untouched between the two
+    for (size_t k = m; k < (size_t)c && ok; ++k) {
+      const OperatorDef& kd = operators_[k]->operator_def();
+      for (const auto& out : kd.output()) ok &= (out != cd.output(0)) && (copy_pos < 0 || out != cd.input(copy_pos));
+      for (const auto& in : kd.input()) ok &= (in != cd.output(0));
+    }
+    if (!ok) continue;
+    host->AdoptTailConcat(operators_[c].get(), operators_[r].get(), att_pos, sum_pos, copy_pos);
+    skipped_[r] = skipped_[c] = true;
   }
 }
 

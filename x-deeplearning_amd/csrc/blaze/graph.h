@@ -101,6 +101,7 @@ class SimpleNet : public Net {
   void FuseFcHeads();
   void PackSiblingFcs();
   void FuseWeightedPools();
+  void FuseConcatsIntoWeightedPools();
   void FuseConcatsIntoFcs();
   void ChainNarrowFcs();
   int ReadersOf(const std::string& name, const OperatorBase* folded) const;
@@ -230,6 +231,13 @@ class WeightedPoolHost {  // implemented by MatMul
   virtual bool WeightedPoolEligible() const = 0;  // static part: transA, no transB
   // mul: producer of Input(0) (may be null); reduce_sum: a ReduceSum(axis 1, keepdims 0) of Input(1) (may be null)
   virtual void AdoptWeightedPool(OperatorBase* mul, OperatorBase* reduce_sum) = 0;
+  virtual OperatorBase* AdoptedReduceSum() const = 0;
+  // The Concat (last axis of 2-D tensors) that joins this MatMul's result - flattened from [B, 1, C] to [B, C] by
+  // `reshape`, which nothing else reads - with the adopted ReduceSum's result and at most one other tensor that is
+  // final before the MatMul runs (DIN: [target, sum, att] in front of the main MLP): the launch writes its outputs
+  // into the Concat's output and copies the other tensor there; the Reshape and the Concat do not run.  Positions are
+  // indices among the Concat's inputs, -1 = the Concat has no such input.
+  virtual void AdoptTailConcat(OperatorBase* concat, OperatorBase* reshape, int att_pos, int sum_pos, int copy_pos) = 0;
 };
 
 }  // namespace blaze
