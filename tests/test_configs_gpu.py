@@ -236,7 +236,8 @@ def test_config3_din_attention_end_to_end_through_predictor(oracle):
     ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0]
     launching = [e for e in ev if e["name"].split(":")[0] not in ("ConstantFill", "Reshape")]
     kinds = sorted(e["name"].split(":")[0] for e in launching)
-    assert kinds == ["Concat"] + ["Embedding"] * 2 + ["Gemm"] * 3 + ["MatMul"], kinds
+    assert kinds == ["Concat"] + ["Embedding"] + ["Gemm"] * 3 + ["MatMul"], kinds
+    assert [e["args"]["launches"] for e in launching if e["name"].split(":")[0] == "Embedding"] == [1]
     assert all(e["args"]["launches"] == 1 for e in launching if e["name"].split(":")[0] in ("Gemm", "MatMul")), launching
     tabs = {}
     for ki, (k, t) in enumerate(zip(din_model.KINDS, tables)):
@@ -499,3 +500,40 @@ def test_main_input_concat_written_by_the_attention_tail():
     np.testing.assert_array_equal(p.output_asnumpy("main_in"), outs[1][0]["main_in"])
     np.testing.assert_array_equal(p.output_asnumpy("hsum"), outs[1][0]["main_in"][:, D3:2 * D3])
     np.testing.assert_array_equal(p.output_asnumpy("att"), outs[1][0]["main_in"][:, 2 * D3:])
+
+
+def test_sibling_embedding_operators_share_one_launch():
+    """DIN's two Embedding operators (target item: ksum of one id a sample; history: kAssign) read only inputs of the net:
+    the first runs the second (merge_sibling_embeddings, on by default) and both are looked up in one pooling launch,
+    because the target's lookups are light; with three ids a sample in the target's groups they are not, and the two
+    launch one after the other.  Same bits as two separate operators in every case, also when the batch changes."""
+    import json
+    import din_model
+    cfg = din_model.Config3(batch=64, rows=3000, T=12)
+    small = din_model.Config3(batch=9, rows=3000, T=12)
+    batches = [cfg.batch_inputs(), small.batch_inputs(seed_offset=1), cfg.batch_inputs(seed_offset=2)]
+    heavy = dict(batches[2])
+    for k in din_model.KINDS:  # three ids a sample for the target item: more than "light"
+        heavy[k + ".ids"] = np.concatenate([batches[2][k + ".ids"], batches[0][k + ".ids"], batches[2][k + ".ids"][::-1]]).reshape(3, -1).T.reshape(-1).copy()
+        heavy[k + ".values"] = np.ones(3 * cfg.batch, np.float32)
+        heavy[k + ".segments"] = np.full(cfg.batch, 3, np.int32)
+    batches.append(heavy)
+    tables, weights = cfg.tables(), cfg.weights()
+    outs = {}
+    for merge in (1, 0):
+        pm, inputs = din_model.build_manager(cfg, tables, weights, np.float16, expose=("q", "his"), net_args={"merge_sibling_embeddings": merge})
+        p = pm.create_predictor(1, 0)
+        p.register_observers(["profile"])
+        got = []
+        for i, b in enumerate(batches):
+            din_model.feed(p, inputs, b, np.float16)
+            p.forward()
+            ev = [e for e in json.loads(p.dump_observers()["profile"])["traceEvents"] if e["dur"] > 0 and e["name"].split(":")[0] == "Embedding"]
+            launches = [e["args"]["launches"] for e in ev]
+            assert launches == ([1, 1] if merge == 0 else ([2] if i == 3 else [1])), (merge, i, launches)
+            got.append({k: p.output_asnumpy(k).copy() for k in ("q", "his", "prob")})
+        outs[merge] = got
+    for g1, g0 in zip(outs[1], outs[0]):
+        assert g1["q"].any() and g1["his"].any()
+        for k in g1:
+            np.testing.assert_array_equal(g1[k], g0[k], err_msg=k)

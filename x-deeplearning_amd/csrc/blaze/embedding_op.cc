@@ -15,9 +15,16 @@ namespace blaze {
 using store::SparsePuller;
 
 template <class Context>
-class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
+class EmbeddingOp final : public Operator<Context>, public AssignInterleaver, public EmbeddingSibling {
  public:
   USE_OPERATOR_FUNCTIONS(Context);
+
+  void AdoptSibling(OperatorBase* other) override {
+    auto* e = dynamic_cast<EmbeddingOp*>(other);
+    BLAZE_CONDITION_THROW(e != nullptr && e != this, "AdoptSibling: not another Embedding operator of this device");
+    siblings_.push_back(e);
+  }
+  int LaunchesOfLastRun() const override { return launches_; }
 
   bool AssignBlock(int idx, int* trunc_num, int* dim) const override {
     if (idx < 0 || (size_t)idx >= config_.block_config.size()) return false;
@@ -78,19 +85,39 @@ class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
   }
 
   bool RunOnDevice() override {
-    CheckValid();
-    Blob* id = this->Input(0);
-    Blob* value = this->Input(1);
-    Blob* id_num = this->Input(2);
-    // ID_TYPE_SWITCH / TYPE_SWITCH of embedding_op.cc:70-82; the QED store then insists on int64 / float / int32
-    BLAZE_CONDITION_THROW(id->data_type() == kInt64 || id->data_type() == kInt32, "Unsupported type:", id->data_type());
-    BLAZE_CONDITION_THROW(value->data_type() == kFloat, "Unsupported type:", value->data_type());
-    BLAZE_CONDITION_THROW(id_num->data_type() == kInt64 || id_num->data_type() == kInt32, "Unsupported type:", id_num->data_type());
-    BLAZE_CONDITION_THROW(sparse_puller_ != nullptr, "no sparse puller: call LoadSparseModelWeight before creating predictors");
-    BLAZE_CONDITION_THROW(sparse_puller_->on_device(), "the Embedding operator of this build needs a device sparse puller "
-                          "(qed_hip_sparse_puller); there is no host fallback");
-    Setup();
-    RunEmbedding(id->data_type(), value->data_type(), id_num->data_type());
+    hipStream_t st = context_.hip_stream();
+    Prepare(st);
+    launches_ = 1;
+    if (siblings_.empty()) {
+      Pull(puller_in_, puller_out_, st, &cache_);
+      return true;
+    }
+    // the operators this one runs (graph.h, EmbeddingSibling): everything in one launch when none of them loses by it
+    bool together = RidesFree();
+    for (EmbeddingOp* e : siblings_) {
+      e->Prepare(st);
+      together &= e->RidesFree() && e->sparse_puller_ == sparse_puller_;
+    }
+    if (!together) {
+      Pull(puller_in_, puller_out_, st, &cache_);
+      for (EmbeddingOp* e : siblings_) e->Pull(e->puller_in_, e->puller_out_, st, &e->cache_);
+      launches_ += (int)siblings_.size();
+      return true;
+    }
+    size_t n = puller_in_.size();
+    for (EmbeddingOp* e : siblings_) n += e->puller_in_.size();
+    merged_in_.resize(n);  // (element-wise assignment below: the strings and item lists keep their storage run to run)
+    merged_out_.resize(n);
+    size_t at = 0;
+    auto append = [&](const EmbeddingOp* e) {
+      for (size_t i = 0; i < e->puller_in_.size(); ++i, ++at) {
+        merged_in_[at] = e->puller_in_[i];
+        merged_out_[at] = e->puller_out_[i];
+      }
+    };
+    append(this);
+    for (EmbeddingOp* e : siblings_) append(e);
+    Pull(merged_in_, merged_out_, st, &merged_cache_);
     return true;
   }
 
@@ -202,7 +229,41 @@ class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
     return idx >= 0 && (size_t)idx < config_.block_config.size() ? (TIndex)config_.block_config[idx].stride : 0;
   }
 
-  void RunEmbedding(int key_type, int value_type, int num_type) {
+  // everything of a run but the lookup itself: checks, output shapes, the puller structs, zero fills (on `st`)
+  void Prepare(hipStream_t st) {
+    CheckValid();
+    Blob* id = this->Input(0);
+    Blob* value = this->Input(1);
+    Blob* id_num = this->Input(2);
+    // ID_TYPE_SWITCH / TYPE_SWITCH of embedding_op.cc:70-82; the QED store then insists on int64 / float / int32
+    BLAZE_CONDITION_THROW(id->data_type() == kInt64 || id->data_type() == kInt32, "Unsupported type:", id->data_type());
+    BLAZE_CONDITION_THROW(value->data_type() == kFloat, "Unsupported type:", value->data_type());
+    BLAZE_CONDITION_THROW(id_num->data_type() == kInt64 || id_num->data_type() == kInt32, "Unsupported type:", id_num->data_type());
+    BLAZE_CONDITION_THROW(sparse_puller_ != nullptr, "no sparse puller: call LoadSparseModelWeight before creating predictors");
+    BLAZE_CONDITION_THROW(sparse_puller_->on_device(), "the Embedding operator of this build needs a device sparse puller "
+                          "(qed_hip_sparse_puller); there is no host fallback");
+    Setup();
+    RunEmbedding(id->data_type(), value->data_type(), id_num->data_type(), st);
+  }
+  void Pull(const std::vector<store::SparsePullerInput>& in, std::vector<store::SparsePullerOutput>& out, hipStream_t st,
+            std::unique_ptr<SparsePuller::DeviceCache>* cache) {
+    auto status = sparse_puller_->GetOnStream(in, out, st, cache);
+    BLAZE_CONDITION_THROW(status == store::kOK, "pull data failed, status=", status);
+  }
+  // whether a launch shared with other operators costs this one's lookups nothing: every fed feature group either has
+  // only kAssign items (the generic kernel's work in any launch) or at most two ids a sample on average
+  bool RidesFree() const {
+    for (size_t i = 0; i < puller_in_.size(); ++i) {
+      const auto& in = puller_in_[i];
+      if (fg_input_[i] < 0 || in.in_item.empty()) continue;
+      bool all_assign = true;
+      for (const auto& item : in.in_item) all_assign &= item.udf_type == store::kAssign;
+      if (!all_assign && in.key_size > 2 * in.key_num_size) return false;
+    }
+    return true;
+  }
+
+  void RunEmbedding(int key_type, int value_type, int num_type, hipStream_t st) {
     const size_t n_fg = config_.feature_group_config.size();
     // the puller structs live in the operator: their names, item lists and input positions are the same every run,
     // only pointers and sizes change (a request-sized forward pass should not pay 2 allocations per feature group)
@@ -264,7 +325,6 @@ class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
         out.out_item[j].assign_pitch = 0;
       }
     }
-    hipStream_t st = context_.hip_stream();
     for (size_t b = 0; b < needs_zero_.size(); ++b)
       if (needs_zero_[b]) {
         Blob* block = this->Output((int)b);
@@ -280,8 +340,6 @@ class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
         else
           HIP_CHECK(hipMemsetAsync(block->data(), 0, block->size() * es, st));
       }
-    auto status = sparse_puller_->GetOnStream(inputs, outputs, st, &cache_);
-    BLAZE_CONDITION_THROW(status == store::kOK, "pull data failed, status=", status);
   }
 
   std::shared_ptr<SparsePuller> sparse_puller_;
@@ -295,6 +353,12 @@ class EmbeddingOp final : public Operator<Context>, public AssignInterleaver {
   std::vector<store::SparsePullerOutput> puller_out_;
   std::vector<int> fg_input_;  // feature group -> position of its triple among the inputs, -1 = not fed
   std::unique_ptr<SparsePuller::DeviceCache> cache_;
+  // the Embedding operators this one runs, the joined structs of a shared launch and that launch's own slot cache
+  std::vector<EmbeddingOp*> siblings_;
+  std::vector<store::SparsePullerInput> merged_in_;
+  std::vector<store::SparsePullerOutput> merged_out_;
+  std::unique_ptr<SparsePuller::DeviceCache> merged_cache_;
+  int launches_ = 1;
   int out_dtype_ = 0;
 };
 

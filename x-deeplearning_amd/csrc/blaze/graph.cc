@@ -220,6 +220,7 @@ SimpleNet::SimpleNet(const std::shared_ptr<const NetDef>& net_def, Workspace* ws
     FuseConcatsIntoFcs();
     ChainNarrowFcs();
     FuseConcatsIntoWeightedPools();
+    MergeSiblingEmbeddings();
   }
 }
 
@@ -628,6 +629,44 @@ void SimpleNet::InterleaveAssignBlocks() {
     dynamic_cast<AssignInterleaver*>(operators_[emb].get())->InterleaveInto(blocks, operators_[c]->Output(0));
     for (int r : reshapes) skipped_[r] = true;
     skipped_[c] = true;
+  }
+}
+
+// Embedding operators whose inputs no operator of the net produces: the later ones are run by the first (graph.h,
+// EmbeddingSibling), which may then look everything up in one launch.  Moved up to the first one's position, a later
+// operator's outputs must not be named by anything in between.  Switch: merge_sibling_embeddings: 0.
+void SimpleNet::MergeSiblingEmbeddings() {
+  const Argument* arg = ArgumentHelper::Find(net_def_->arg_, "merge_sibling_embeddings");
+  if (arg && arg->has_i && arg->i == 0) return;
+  auto produced = [&](const std::string& name) {
+    for (const auto& op : operators_)
+      for (const auto& out : op->operator_def().output())
+        if (out == name) return true;
+    return false;
+  };
+  auto from_outside = [&](size_t i) {
+    for (const auto& in : operators_[i]->operator_def().input())
+      if (produced(in)) return false;
+    return true;
+  };
+  int host = -1;
+  for (size_t i = 0; i < operators_.size(); ++i) {
+    if (skipped_[i] || dynamic_cast<EmbeddingSibling*>(operators_[i].get()) == nullptr || !from_outside(i)) continue;
+    if (host < 0) {
+      host = (int)i;
+      continue;
+    }
+    bool ok = true;
+    for (size_t k = host; k < i && ok; ++k) {
+      const OperatorDef& kd = operators_[k]->operator_def();
+      for (const auto& out : operators_[i]->operator_def().output()) {
+        for (const auto& name : kd.input()) ok &= (name != out);
+        for (const auto& name : kd.output()) ok &= (name != out);
+      }
+    }
+    if (!ok) continue;
+    dynamic_cast<EmbeddingSibling*>(operators_[host].get())->AdoptSibling(operators_[i].get());
+    skipped_[i] = true;
   }
 }
 

@@ -106,6 +106,7 @@ class SimpleNet : public Net {
   void ChainNarrowFcs();
   int ReadersOf(const std::string& name, const OperatorBase* folded) const;
   void InterleaveAssignBlocks();
+  void MergeSiblingEmbeddings();
   std::vector<bool> skipped_;  // ops folded into their producer's epilogue, or run by the operator that took them over
 };
 
@@ -238,6 +239,17 @@ class WeightedPoolHost {  // implemented by MatMul
   // into the Concat's output and copies the other tensor there; the Reshape and the Concat do not run.  Positions are
   // indices among the Concat's inputs, -1 = the Concat has no such input.
   virtual void AdoptTailConcat(OperatorBase* concat, OperatorBase* reshape, int att_pos, int sum_pos, int copy_pos) = 0;
+};
+
+// Embedding operators of one net that read only tensors from outside the net: the first one (in order) takes the later
+// ones over and looks everything up in ONE pooling launch when that costs the taken-over lookups nothing - every
+// operator of the group is either all kAssign (the generic kernel's work anyway) or light (at most two ids a sample on
+// average in each of its feature groups, where the specialised kernel's deeper walk buys nothing); decided per run,
+// otherwise each operator launches as before.  DIN: the target item's lookup rides in the history's launch.
+class EmbeddingSibling {  // implemented by Embedding
+ public:
+  virtual ~EmbeddingSibling() {}
+  virtual void AdoptSibling(OperatorBase* other) = 0;
 };
 
 }  // namespace blaze
