@@ -227,7 +227,9 @@ __device__ __forceinline__ void accum_chunk(float (&acc)[RowTraits<DT>::kElems],
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float w = __half2float(__ushort_as_half((unsigned short)((r[i / 2] >> (16 * (i & 1))) & 0xffffu)));
-      acc[i] = UNIT ? __builtin_fmaf(w, 1.0f, acc[i]) : __fadd_rn(acc[i], __builtin_fmaf(w, value, 0.0f));
+      // (UNIT: `value` is a 1.0 the compiler cannot see through, so that the widening and the add stay one
+      // v_fma_mix_f32; with a literal 1 it splits them into a convert and an add)
+      acc[i] = UNIT ? __builtin_fmaf(w, value, acc[i]) : __fadd_rn(acc[i], __builtin_fmaf(w, value, 0.0f));
     }
   } else {
 #pragma unroll
@@ -547,13 +549,18 @@ __device__ __forceinline__ void own_segment(const bz_embed_slot& s, int64_t b0, 
   // this group's own count first (all its lanes ask for the same word), then the counts before b0, 8 loads in flight a
   // thread: everything is requested before anything is used
   const int32_t own = b < s.batch ? s.segments[b] : 0;
+  // (b0 is below 2^31: batch is an int32.  A workgroup near the head of its slot has few counts before it: the rounds
+  // of 8 loads stop, for the whole workgroup, where b0 ends)
+  const uint32_t nb = (uint32_t)b0;
   uint64_t part = 0;
-  for (int64_t i0 = 0; i0 < b0; i0 += 8 * kThreads) {
+  for (uint32_t i0 = 0; i0 < nb; i0 += 8 * kThreads) {
     int32_t c[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int64_t i = i0 + k * kThreads + tid;
-      c[k] = i < b0 ? s.segments[i] : 0;
+      const uint32_t i = i0 + k * kThreads + tid;
+      c[k] = 0;
+      if (i0 + k * kThreads < nb) c[k] = s.segments[i < nb ? i : nb - 1];  // (uniform test; a lane past b0 reads the last count, masked below)
+      if (i >= nb) c[k] = 0;
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) part += (uint32_t)max(c[k], 0);
@@ -568,12 +575,15 @@ __device__ __forceinline__ void own_segment(const bz_embed_slot& s, int64_t b0, 
     s_tot[WAVES + wave] = scan;
   }
   __syncthreads();
-  uint32_t before = 0;
-#pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
-    before = sat_add(before, s_tot[w], cap);
-    if (w < wave) before = sat_add(before, s_tot[WAVES + w], cap);
-  }
+  // what lies before this wave: all the waves' sums of earlier counts and the totals of the waves before it -- entry
+  // WAVES - 1 + wave of the inclusive (saturating) scan over the 2 * WAVES values, done in one row of 16 lanes
+  static_assert(2 * WAVES <= 16, "the waves' totals are scanned within one row of lanes");
+  uint32_t t = (lane & 15) < 2 * WAVES ? s_tot[lane & 15] : 0u;
+  t = sat_add(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x111, 0xf, 0xf, false), cap);  // row_shr:1
+  t = sat_add(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x112, 0xf, 0xf, false), cap);  // row_shr:2
+  t = sat_add(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x114, 0xf, 0xf, false), cap);  // row_shr:4
+  t = sat_add(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x118, 0xf, 0xf, false), cap);  // row_shr:8
+  const uint32_t before = (uint32_t)__builtin_amdgcn_readlane((int)t, WAVES - 1 + wave);
   const uint32_t x = sat_add(before, scan, cap);
   if constexpr (LPR == 1) {
     uint32_t excl = (uint32_t)__shfl_up((int)scan, 1, bz::kWave);
@@ -604,6 +614,9 @@ struct SlotPack {
 };
 static_assert(sizeof(SlotPack) + 64 <= 4096, "the records and the other arguments fit the 4 KB kernel-argument segment");
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr uint32_t kBeyondTable = 0xF0000000u;  // a byte offset no table read through a buffer resource reaches
+
 template <int DT, int LPR>
 __device__ __forceinline__ void pool_samples(const bz_embed_slot& s, int64_t b0, const int64_t* __restrict__ offsets) {
   constexpr int CE = RowTraits<DT>::kElems;
@@ -631,6 +644,16 @@ __device__ __forceinline__ void pool_samples(const bz_embed_slot& s, int64_t b0,
   float acc[CE];
 #pragma unroll
   for (int i = 0; i < CE; ++i) acc[i] = 0.f;
+  float one = 1.f;  // (opaque: see accum_chunk)
+  asm volatile("" : "+v"(one));
+  // fp32 / fp16 tables of up to 2^24 rows and 3.75 GB are read through a buffer resource: the hardware checks every
+  // access against the table's size and returns zeros beyond it, which is what a missing row contributes.  (Measured:
+  // config 2's launch 11.9 -> 11.7 us.  Not for int8 tables: with the rows and their scales through buffer resources
+  // config 4's launch took 97-110 us against 90-92 with plain loads under a branch.)
+  const bool by_buffer = DT != BZ_I8 && s.rows <= (1ll << 24) && (uint64_t)s.rows * (uint64_t)s.pitch <= (uint64_t)kBeyondTable &&
+                         s.pitch < (1 << 24);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)s.table, 0, by_buffer ? (int)(uint32_t)(s.rows * (int64_t)s.pitch) : 0, 0x00020000);
   // each fetching lane takes ids j + k*SRC + l: one coalesced read per k for the whole group.  The
   // next step's ids are requested before this step's rows, so the two round trips overlap.
   int64_t id_next[KPL];  // raw ids: resolved to rows only when consumed, so the wait lands after the row loads
@@ -661,31 +684,46 @@ __device__ __forceinline__ void pool_samples(const bz_embed_slot& s, int64_t b0,
       val_own[k] = row_own[k] >= 0 ? val_next[k] : 1.f;
     }
     if (j + kBlockIds < end) fetch_ids(j + kBlockIds);
+    // ids that carry no weight (value 1, the usual case) take the one-rounding form, when that holds for every lane of
+    // the wave: decided on the lanes' own values, before anything is handed round, so that the values need not be
+    bool unit_own = true;
+#pragma unroll
+    for (int k = 0; k < KPL; ++k) unit_own &= val_own[k] == 1.f;
+    const bool unit = __all(unit_own);
     int row[kBlockIds];
     float val[kBlockIds];
     uint4 raw[kBlockIds];
     float sc[kBlockIds];
 #pragma unroll
-    for (int u = 0; u < kBlockIds; ++u) {
-      row[u] = __shfl(row_own[u / SRC], gbase + (u % SRC), bz::kWave);
-      val[u] = __shfl(val_own[u / SRC], gbase + (u % SRC), bz::kWave);
-    }
+    for (int u = 0; u < kBlockIds; ++u) row[u] = __shfl(row_own[u / SRC], gbase + (u % SRC), bz::kWave);
+    if (!unit) {
 #pragma unroll
-    for (int u = 0; u < kBlockIds; ++u) {
-      raw[u] = make_uint4(0, 0, 0, 0);
-      sc[u] = 1.f;
-      if (has_chunk && row[u] >= 0) {  // row[u] is -1 beyond cnt
-        raw[u] = *(const uint4*)(table + (int64_t)row[u] * s.pitch);
-        if (DT == BZ_I8) sc[u] = load_scale(s, row[u]);
+      for (int u = 0; u < kBlockIds; ++u) val[u] = __shfl(val_own[u / SRC], gbase + (u % SRC), bz::kWave);
+    }
+    if (by_buffer) {
+      // no branch round a load, no zero fill, one multiply-add per address: a row that is not there (row[u] is -1 beyond
+      // cnt and for ids without a row) is asked for beyond the table's end and comes back as zeros
+#pragma unroll
+      for (int u = 0; u < kBlockIds; ++u) {
+        const uint32_t off = (has_chunk && row[u] >= 0) ? __umul24((uint32_t)row[u], (uint32_t)s.pitch) + (uint32_t)l * 16u : kBeyondTable;
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0);
+        raw[u] = make_uint4(v.x, v.y, v.z, v.w);
+        sc[u] = 1.f;
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kBlockIds; ++u) {
+        raw[u] = make_uint4(0, 0, 0, 0);
+        sc[u] = 1.f;
+        if (has_chunk && row[u] >= 0) {
+          raw[u] = *(const uint4*)(table + (int64_t)row[u] * s.pitch);
+          if (DT == BZ_I8) sc[u] = load_scale(s, row[u]);
+        }
       }
     }
-    // ids that carry no weight (value 1, the usual case) take the one-rounding form, when that holds for every lane of the wave
-    bool unit = true;
+    if (unit) {
 #pragma unroll
-    for (int u = 0; u < kBlockIds; ++u) unit &= val[u] == 1.f;
-    if (__all(unit)) {
-#pragma unroll
-      for (int u = 0; u < kBlockIds; ++u) accum_chunk<DT, true>(acc, raw[u], sc[u], 1.f);
+      for (int u = 0; u < kBlockIds; ++u) accum_chunk<DT, true>(acc, raw[u], sc[u], one);
     } else {
 #pragma unroll
       for (int u = 0; u < kBlockIds; ++u) accum_chunk<DT, false>(acc, raw[u], sc[u], val[u]);
