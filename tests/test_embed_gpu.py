@@ -491,3 +491,29 @@ def test_device_fill_matches_the_host_generator_bit_for_bit(bz):
             assert got.dtype == want.dtype and np.array_equal(got[1:-1].view(np.uint8), want.view(np.uint8))
     m = philox.tensor((1000, 18), philox.KIND_NORMAL_F16, st, "cuda", 0.1)
     assert np.array_equal(m.cpu().numpy()[[999, 0]], philox.host_rows(philox.KIND_NORMAL_F16, st, [999, 0], 18, 0.1))
+
+
+def test_table_of_more_than_2_to_24_rows_takes_the_plain_load_path(bz, oracle):
+    """The specialised kernel reads fp32 / fp16 tables of up to 2^24 rows through a buffer resource and larger ones with
+    plain loads under a branch: a table of 17 M rows (ids on both sides of 2^24, some outside the table) against the
+    oracle, bit for bit, next to a small table in the same launch."""
+    rng = np.random.default_rng(2024)
+    rows, dim, batch = 17_000_000, 4, 300
+    big = {"data": (rng.standard_normal((rows, dim)) * 0.1).astype(np.float32)}
+    small = {"data": (rng.standard_normal((1000, dim)) * 0.1).astype(np.float32)}
+    specs, inputs, cols = [], [], []
+    col = 0
+    for ti, udf, n_rows in ((0, 0, rows), (1, 1, 1000), (0, 1, rows)):
+        seg = rng.integers(0, 9, batch).astype(np.int32)
+        nnz = int(seg.sum())
+        ids = rng.integers(-2, n_rows + 2, nnz)
+        ids[::5] = rng.integers(max(0, n_rows - 2000), n_rows, ids[::5].size)  # the table's last rows (beyond 2^24 for the big one)
+        specs.append((ti, udf, 0, 0, dim))
+        inputs.append((ids.astype(np.int64), rng.standard_normal(nnz).astype(np.float32), seg))
+        cols.append(col)
+        col += dim
+    print("table of %d rows" % rows, flush=True)
+    got, _, variant = _run_gpu(bz, [big, small], specs, inputs, batch, np.float32, (col, cols))
+    assert variant != 0  # one row shape, ksum / kavg: the specialised kernel
+    want = _run_oracle(oracle, [big, small], specs, inputs, batch, (col, cols))
+    assert np.array_equal(_bits(got), _bits(want))
