@@ -105,6 +105,20 @@ BLAZE_API int Blaze_QuickEmbeddingBuildFp16(const char* path, const char* meta, 
 BLAZE_API int Blaze_HipStoreAddTable(PredictorManagerHandle handle, const char* table_name, int value_type, int64_t rows, int dim,
                                      const void* rows_ptr, int on_device, const int64_t* keys, const float* scale);
 
+/*
+ * One feature group looked up through the store's host-memory SparsePuller::Get, the form the reference's interface
+ * declares (blaze/store/sparse_puller.h:77-83) and its host Embedding operator calls (embedding_op.cc:87): keys [sum of
+ * key_num] int64, key_num [batch] int32, values [sum of key_num] fp32 and every out[k] are HOST memory.  Item k pools
+ * with udf_type[k] (0 sum, 1 avg, 2 assign) / trunc_direction[k] / trunc_num[k] and writes dim (assign: trunc_num * dim)
+ * elements of out_type (1 fp32, 12 fp16) per sample at out[k] + sample * stride[k]; other columns of the block, and
+ * every column when the table name is unknown, keep what the caller put there.  The tables live on the device: the
+ * call copies the inputs over, runs the pooling kernel, copies the columns back and waits.
+ */
+BLAZE_API int Blaze_HipStoreGet(PredictorManagerHandle handle, const char* table_name, const int64_t* keys, const int32_t* key_num,
+                                size_t batch, const float* values, int dim, int n_items, const int* udf_type,
+                                const int* trunc_direction, const int* trunc_num, void* const* out, const size_t* stride,
+                                int out_type);
+
 /* load a model from memory: a NetDef in protobuf text format (is_text) or proto2 wire format */
 BLAZE_API int Blaze_PredictorManagerLoadModelFromString(PredictorManagerHandle handle, const char* data, size_t len, int is_text);
 

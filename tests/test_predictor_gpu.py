@@ -727,3 +727,77 @@ def test_folded_gemm_chain_gives_the_same_outputs(pb, oracle, tmp_path):
             got.append(p.output_asnumpy("output").copy())
         assert got[0].shape == (2, 3) and got[0].any()
         np.testing.assert_allclose(got[1], got[0], rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("out_dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("with_keys", [False, True])
+def test_store_get_with_host_pointers(pb, oracle, out_dtype, with_keys):
+    """SparsePuller::Get in the reference's own form (blaze/store/sparse_puller.h:77-83: every pointer host memory), as
+    its host Embedding operator calls it (embedding_op.cc:87): bit-identical to the oracle's QuickEmbeddingDict::Get on
+    the same block; columns of no item and the columns of an unknown table keep the caller's contents; two calls in a
+    row on one thread (the second smaller) reuse the staging state; calls from other threads are served too."""
+    import threading
+    rng = np.random.default_rng(77)
+    rows, dim = 500, 12
+    data = rng.standard_normal((rows, dim)).astype(np.float32)
+    keys = rng.choice(1 << 40, rows, replace=False).astype(np.int64) if with_keys else None
+    pm = pb.PredictorManager()
+    pm.add_table("t", data, keys=keys)
+    table = oracle.Table(data, keys=None if keys is None else keys.astype(np.uint64))
+
+    def case(batch, seed):
+        r = np.random.default_rng(seed)
+        seg = r.integers(0, 7, batch).astype(np.int32)
+        seg[r.integers(0, batch)] = 0
+        nnz = int(seg.sum())
+        pick = r.integers(0, rows, nnz)
+        ids = (keys[pick] if with_keys else pick).astype(np.int64)
+        ids[r.random(nnz) < 0.1] = (1 << 41) + 5  # unknown keys are skipped
+        vals = r.standard_normal(nnz).astype(np.float32)
+        return ids, seg, vals
+
+    def run(batch, seed):
+        ids, seg, vals = case(batch, seed)
+        stride = 3 + dim + dim + 4 * dim + 2
+        layout = [(oracle.SUM, oracle.REVERSE, 0, 3), (oracle.AVG, oracle.ORDER, 3, 3 + dim),
+                  (oracle.ASSIGN, oracle.REVERSE, 4, 3 + 2 * dim)]
+        sentinel = r0 = np.random.default_rng(seed + 1).standard_normal((batch, stride)).astype(np.float32)
+        want = sentinel.copy()
+        oracle.embed_get(table, ids, vals, seg, [(u, d, n, want, c) for u, d, n, c in layout])
+        got = sentinel.astype(out_dtype)
+        pm.store_get("t", ids, seg, vals, dim, [(u, d, n, got, c) for u, d, n, c in layout])
+        if out_dtype == np.float32:
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        else:
+            # item columns: the fp32 result narrowed once (round to nearest even); the rest: the caller's halves
+            item = np.zeros(stride, bool)
+            item[3:3 + 6 * dim] = True
+            expect = np.where(item[None, :], want, r0.astype(np.float16).astype(np.float32)).astype(np.float16)
+            assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
+        # unknown table: nothing is written
+        keep = sentinel.astype(out_dtype)
+        before = keep.copy()
+        pm.store_get("no_such_table", ids, seg, vals, dim, [(u, d, n, keep, c) for u, d, n, c in layout])
+        assert np.array_equal(keep.view(np.uint8), before.view(np.uint8))
+
+    run(300, 1)
+    run(37, 2)
+    run(1, 3)
+    errors = []
+
+    def worker(seed):
+        try:
+            run(120, seed)
+        except BaseException as e:  # noqa: BLE001 -- reported by the main thread
+            errors.append(e)
+
+    ts = [threading.Thread(target=worker, args=(10 + i,)) for i in range(3)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errors, errors
+    # the counts must add up to the ids handed over
+    ids, seg, vals = case(20, 5)
+    with pytest.raises(pb.BlazeError):
+        pm.store_get("t", ids, seg, vals, dim, [(oracle.SUM, 0, 0, np.zeros((20, 4), np.float32), 0)])  # stride < dim

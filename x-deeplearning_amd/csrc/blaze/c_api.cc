@@ -565,6 +565,47 @@ int Blaze_HipStoreAddTable(PredictorManagerHandle handle, const char* table_name
   return 0;
 }
 
+int Blaze_HipStoreGet(PredictorManagerHandle handle, const char* table_name, const int64_t* keys, const int32_t* key_num,
+                      size_t batch, const float* values, int dim, int n_items, const int* udf_type, const int* trunc_direction,
+                      const int* trunc_num, void* const* out, const size_t* stride, int out_type) {
+  auto* pm = reinterpret_cast<PredictorManager*>(handle);
+  if (pm == nullptr || table_name == nullptr) return Fail("The predict manager is nullptr");
+  if (n_items < 0 || (n_items > 0 && (udf_type == nullptr || trunc_direction == nullptr || trunc_num == nullptr || out == nullptr ||
+                                      stride == nullptr)))
+    return Fail("null argument");
+  try {
+    auto& puller = pm->EnsureSparsePuller("qed_hip_sparse_puller");
+    std::vector<blaze::store::SparsePullerInput> in(1);
+    std::vector<blaze::store::SparsePullerOutput> o(1);
+    in[0].name = table_name;
+    in[0].key = const_cast<int64_t*>(keys);
+    in[0].key_num = const_cast<int32_t*>(key_num);
+    in[0].key_num_size = batch;
+    in[0].value = const_cast<float*>(values);
+    in[0].key_type = blaze::kInt64;
+    in[0].value_type = blaze::kFloat;
+    in[0].num_type = blaze::kInt32;
+    in[0].dim = dim;
+    o[0].out_type = out_type;
+    for (int k = 0; k < n_items; ++k) {
+      blaze::store::SparsePullerInput::Param p;
+      p.udf_type = (blaze::store::UDFType)udf_type[k];
+      p.trunc_direction = (blaze::store::TruncDirection)trunc_direction[k];
+      p.trunc_num = trunc_num[k];
+      in[0].in_item.push_back(p);
+      blaze::store::SparsePullerOutput::OutItem item;
+      item.out = out[k];
+      item.stride = stride[k];
+      o[0].out_item.push_back(item);
+    }
+    if (puller->Get(in, o) != blaze::store::kOK) return Fail("Get failed");
+  } catch (std::exception& e) {
+    blaze::last_error_for_thread() = e.what();
+    return Fail("Get failed");
+  }
+  return 0;
+}
+
 int Blaze_ConvertNetDef(const char* in, size_t len, int in_is_text, int out_is_text, char* out, size_t cap, size_t* out_len) {
   if (in == nullptr || out_len == nullptr) return Fail("null argument");
   try {

@@ -331,9 +331,138 @@ std::shared_ptr<const DeviceTable> QedHipSparsePuller::table(uint16_t gid) const
   return it == tables_.end() ? nullptr : it->second;
 }
 
-Status QedHipSparsePuller::Get(const std::vector<SparsePullerInput>&, std::vector<SparsePullerOutput>&) {
-  LOG_ERROR("qed_hip_sparse_puller serves device memory only: call GetOnStream (there is no host fallback)");
-  return kFail;
+namespace {
+
+// What one thread needs to serve host-memory Get calls: a stream, one growing device arena for the staged inputs and
+// output columns, and the launch cache GetOnStream keeps.  Lives until the thread ends.
+struct HostStage {
+  int device = -1;
+  hipStream_t stream = nullptr;
+  char* arena = nullptr;
+  size_t cap = 0;
+  std::unique_ptr<SparsePuller::DeviceCache> cache;
+  ~HostStage() {
+    if (arena) (void)hipFree(arena);
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+};
+
+size_t Align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+}  // namespace
+
+// SparsePuller::Get as the reference declares it (blaze/store/sparse_puller.h:77-83) and as its host Embedding operator
+// calls it (embedding_op.cc:87): every pointer is HOST memory.  The tables live on the device, so the ids, counts and
+// values are copied there, the pooling kernel runs, and each item's columns are copied back into the caller's block:
+// two PCIe crossings and a wait per call.  The lookup itself is the same kernel GetOnStream launches; nothing is
+// computed on the host.  Columns of the block that belong to no item, and the columns of an unknown table's items,
+// are left as the caller had them (quick_embedding_dict.cc:95).  Re-entrant: the staging state is per thread.
+Status QedHipSparsePuller::Get(const std::vector<SparsePullerInput>& input, std::vector<SparsePullerOutput>& output) {
+  if (input.size() != output.size()) return kFail;
+  thread_local HostStage hs;
+  int device = 0;
+  HIP_CHECK(hipGetDevice(&device));
+  if (hs.device != device) {
+    BLAZE_CONDITION_THROW(hs.device < 0, "a thread's host-memory Get calls must stay on one device");
+    HIP_CHECK(hipStreamCreateWithFlags(&hs.stream, hipStreamNonBlocking));
+    hs.device = device;
+  }
+  struct ItemPlan {
+    size_t at = 0, span = 0;  // arena offset; elements per sample on the device copy
+    bool copy_back = false;
+  };
+  struct GroupPlan {
+    size_t key_at = 0, num_at = 0, value_at = 0, nkeys = 0;
+    int esz = 4;
+    std::vector<ItemPlan> items;
+  };
+  std::vector<GroupPlan> plan(input.size());
+  size_t need = 0;
+  for (size_t i = 0; i < input.size(); ++i) {
+    const SparsePullerInput& in = input[i];
+    const SparsePullerOutput& out = output[i];
+    if (in.in_item.size() != out.out_item.size()) return kFail;
+    if (in.in_item.empty()) continue;
+    BLAZE_CONDITION_THROW(in.key_type == kInt64, "Unsupported key type:", in.key_type);
+    BLAZE_CONDITION_THROW(in.value_type == kFloat, "Unsupported value type:", in.value_type);
+    BLAZE_CONDITION_THROW(in.num_type == kInt32, "Unsupported num type:", in.num_type);
+    const int out_type = out.out_type ? out.out_type : in.value_type;
+    BLAZE_CONDITION_THROW(out_type == kFloat || out_type == kFloat16, "Unsupported block type:", out_type);
+    BLAZE_CONDITION_THROW(in.dim > 0, "dim ", in.dim);
+    GroupPlan& g = plan[i];
+    g.esz = out_type == kFloat ? 4 : 2;
+    // the reference's structure carries no id count: it is the sum of the per-sample counts
+    const int32_t* counts = (const int32_t*)in.key_num;
+    BLAZE_CONDITION_THROW(in.key_num_size == 0 || counts != nullptr, "key_num is null");
+    size_t nkeys = 0;
+    for (size_t b = 0; b < in.key_num_size; ++b) nkeys += counts[b] > 0 ? (size_t)counts[b] : 0;
+    BLAZE_CONDITION_THROW(in.key_size == 0 || in.key_size == nkeys, "key_size ", in.key_size, " but the counts add up to ", nkeys);
+    BLAZE_CONDITION_THROW(nkeys == 0 || in.key != nullptr, "key is null");
+    g.nkeys = nkeys;
+    g.key_at = need;
+    need += Align256(nkeys * 8);
+    g.num_at = need;
+    need += Align256(in.key_num_size * 4);
+    g.value_at = need;
+    if (in.value != nullptr) need += Align256(nkeys * 4);
+    uint16_t gid = 0;
+    std::shared_ptr<const DeviceTable> t;
+    if (LookupGid(in.name, &gid)) t = table(gid);
+    const bool known = t != nullptr && t->rows > 0;
+    g.items.resize(in.in_item.size());
+    for (size_t k = 0; k < in.in_item.size(); ++k) {
+      ItemPlan& it = g.items[k];
+      const size_t pitch = out.out_item[k].assign_pitch ? out.out_item[k].assign_pitch : (size_t)in.dim;
+      const size_t positions = in.in_item[k].udf_type == kAssign ? (size_t)std::max(1, in.in_item[k].trunc_num) : 1;
+      it.span = (positions - 1) * pitch + (size_t)in.dim;
+      BLAZE_CONDITION_THROW(out.out_item[k].out != nullptr && out.out_item[k].stride >= it.span, "item ", k, " of ", in.name,
+                            ": ", it.span, " elements a sample do not fit a stride of ", out.out_item[k].stride);
+      it.copy_back = known && in.key_num_size > 0;
+      it.at = need;
+      need += Align256(in.key_num_size * it.span * g.esz);
+    }
+  }
+  if (need == 0) return kOK;
+  if (hs.cap < need) {
+    if (hs.arena) HIP_CHECK(hipFree(hs.arena));  // (the previous call waited for its stream before it returned)
+    hs.arena = nullptr;
+    hs.cap = 0;
+    ++AllocationCount();
+    HIP_CHECK(hipMalloc((void**)&hs.arena, need + need / 2));
+    hs.cap = need + need / 2;
+  }
+  std::vector<SparsePullerInput> dev_in(input);
+  std::vector<SparsePullerOutput> dev_out(output);
+  for (size_t i = 0; i < input.size(); ++i) {
+    const SparsePullerInput& in = input[i];
+    if (in.in_item.empty()) continue;
+    const GroupPlan& g = plan[i];
+    if (g.nkeys) HIP_CHECK(hipMemcpyAsync(hs.arena + g.key_at, in.key, g.nkeys * 8, hipMemcpyHostToDevice, hs.stream));
+    if (in.key_num_size) HIP_CHECK(hipMemcpyAsync(hs.arena + g.num_at, in.key_num, in.key_num_size * 4, hipMemcpyHostToDevice, hs.stream));
+    if (in.value != nullptr && g.nkeys) HIP_CHECK(hipMemcpyAsync(hs.arena + g.value_at, in.value, g.nkeys * 4, hipMemcpyHostToDevice, hs.stream));
+    dev_in[i].key = hs.arena + g.key_at;
+    dev_in[i].key_num = hs.arena + g.num_at;
+    dev_in[i].value = in.value != nullptr ? hs.arena + g.value_at : nullptr;
+    dev_in[i].key_size = g.nkeys;
+    for (size_t k = 0; k < g.items.size(); ++k) {
+      dev_out[i].out_item[k].out = hs.arena + g.items[k].at;
+      dev_out[i].out_item[k].stride = g.items[k].span;
+    }
+  }
+  Status st = GetOnStream(dev_in, dev_out, hs.stream, &hs.cache);
+  if (st == kOK) {
+    for (size_t i = 0; i < input.size(); ++i) {
+      const GroupPlan& g = plan[i];
+      for (size_t k = 0; k < g.items.size(); ++k) {
+        if (!g.items[k].copy_back) continue;
+        const size_t row_bytes = g.items[k].span * g.esz;
+        HIP_CHECK(hipMemcpy2DAsync(output[i].out_item[k].out, output[i].out_item[k].stride * g.esz, hs.arena + g.items[k].at,
+                                   row_bytes, row_bytes, input[i].key_num_size, hipMemcpyDeviceToHost, hs.stream));
+      }
+    }
+  }
+  HIP_CHECK(hipStreamSynchronize(hs.stream));
+  return st;
 }
 
 Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& input, std::vector<SparsePullerOutput>& output,

@@ -45,7 +45,8 @@ class QedHipSparsePuller : public SparsePuller {
   QedHipSparsePuller() {}
   ~QedHipSparsePuller() override {}
   Status Load(const std::string& url) override;
-  // host pointers are not served: this store reads device memory.  Fails loudly instead of falling back.
+  // host pointers, as the reference's interface passes them: staged through the device (copy in, the same pooling
+  // kernel, copy back, wait); nothing is computed on the host
   Status Get(const std::vector<SparsePullerInput>& input, std::vector<SparsePullerOutput>& output) override;
   Status GetOnStream(const std::vector<SparsePullerInput>& input, std::vector<SparsePullerOutput>& output, void* stream,
                      std::unique_ptr<DeviceCache>* cache) override;

@@ -3,8 +3,8 @@
 // Same ABI as the reference's blaze/store/sparse_puller.h:40-105 and store.h:15-35: a store is created by name
 // through REGISTER_SPARSE_PULLER_CREATION, loaded once per PredictorManager, shared by every predictor (so Get
 // must be re-entrant and read-only), and receives one SparsePullerInput / SparsePullerOutput per feature group.
-// In this build the pointers inside are DEVICE pointers and Get enqueues work on the calling thread's stream
-// (`stream`, an extension field the reference does not have: its store runs on the host).
+// Get takes HOST pointers, as in the reference; GetOnStream (an extension: the reference's store runs on the host) takes
+// the same structs with DEVICE pointers and enqueues its work on the caller's stream.
 #pragma once
 
 #include <functional>

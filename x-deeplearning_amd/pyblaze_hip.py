@@ -29,7 +29,7 @@ EXPORTS = [
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
     "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_ServePoolLatencies", "Blaze_PredictorForwardLaunch",
-    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount"
+    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount", "Blaze_HipStoreGet"
 ]
 
 
@@ -77,6 +77,7 @@ def lib():
         l.Blaze_QuickEmbeddingBuildFp32.argtypes = [cp, cp, cp, i]
         l.Blaze_QuickEmbeddingBuildFp16.argtypes = [cp, cp, cp, i]
         l.Blaze_HipStoreAddTable.argtypes = [vp, cp, i, C.c_int64, i, vp, i, vp, vp]
+        l.Blaze_HipStoreGet.argtypes = [vp, cp, vp, vp, sz, vp, i, i, vp, vp, vp, vp, vp, i]
         l.Blaze_ConvertNetDef.argtypes = [cp, sz, i, i, vp, sz, C.POINTER(sz)]
         l.Blaze_OptimizeBlaze.argtypes = [cp, cp, i]
         l.Blaze_PredictorInputDevicePtr.argtypes = [vp, cp, C.POINTER(vp)]
@@ -318,6 +319,25 @@ class PredictorManager(object):
             keys = np.ascontiguousarray(keys).astype(np.int64)
             kp = keys.ctypes.data
         check_call(lib().Blaze_HipStoreAddTable(self.handle, name.encode(), vt, n, dim, rp, int(on_device), kp, sp))
+
+    def store_get(self, table, ids, key_num, values, dim, items):
+        """The store's host-memory Get for one feature group.  ids int64 [sum(key_num)], key_num int32 [batch], values
+        float32 like ids: numpy arrays.  items: list of (udf, trunc_direction, trunc_num, block, column): block is a
+        C-contiguous numpy [batch, stride] float32 or float16 array written in place from column `column` on."""
+        ids = np.ascontiguousarray(ids, dtype=np.int64)
+        key_num = np.ascontiguousarray(key_num, dtype=np.int32)
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        n = len(items)
+        dt = items[0][3].dtype if n else np.dtype(np.float32)
+        udf, tdir, tnum = ((C.c_int * n)(*[it[k] for it in items]) for k in range(3))
+        outs, strides = (C.c_void_p * n)(), (C.c_size_t * n)()
+        for k, (_, _, _, block, col) in enumerate(items):
+            assert block.flags.c_contiguous and block.ndim == 2 and block.dtype == dt and block.shape[0] == key_num.size
+            outs[k] = block.ctypes.data + col * block.itemsize
+            strides[k] = block.shape[1]
+        check_call(lib().Blaze_HipStoreGet(self.handle, table.encode(), ids.ctypes.data, key_num.ctypes.data, key_num.size,
+                                           values.ctypes.data, dim, n, udf, tdir, tnum, outs, strides,
+                                           K_FLOAT if dt == np.float32 else K_FLOAT16))
 
     def create_predictor(self, device_type=1, device_id=0):
         h = C.c_void_p()
