@@ -174,6 +174,15 @@ BLAZE_API int Blaze_ServePoolSetDepth(ServePoolHandle handle, int depth);
  * after thread, and the number there are to *count.
  */
 BLAZE_API int Blaze_ServePoolLatencies(ServePoolHandle handle, float* out_ms, int64_t capacity, int64_t* count);
+/*
+ * The pool creates its threads' streams itself, at its first job, and spreads them evenly over the device's hardware
+ * queues (the runtime serves few of them, 4 by default, and would otherwise hand a new stream the queue that the fewest
+ * streams of the whole process use, idle ones included: eight threads can end up 3-3-1-1 and run at the pace of the
+ * threads that share).  Which streams share a queue is measured: a kernel queued behind a busy stream of the same queue
+ * cannot finish before it.  This call reports the result: queue_of_thread[t] = the queue (numbered in order of
+ * discovery) of thread t's stream; *count = the number of threads, 0 before the first job.
+ */
+BLAZE_API int Blaze_ServePoolStreamQueues(ServePoolHandle handle, int* queue_of_thread, int capacity, int* count);
 BLAZE_API int Blaze_ServePoolDelete(ServePoolHandle handle);
 
 #ifdef __cplusplus

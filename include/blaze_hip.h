@@ -59,6 +59,13 @@ BZ_API const char* bz_last_error(void);
  * current device, returns BZ_ENOTSUP when it is not gfx950 */
 BZ_API int bz_device_check(char* name, size_t cap);
 
+/*
+ * One wave that keeps `stream` busy for about `microseconds` (0 .. 10000; 0 = an empty kernel).  No counterpart in the
+ * reference: the serving pool uses it to find out which of its streams share a hardware queue (a kernel queued on a
+ * stream that shares the busy one's queue cannot finish before it).
+ */
+BZ_API int bz_spin(int64_t microseconds, bz_stream_t stream);
+
 /* ------------------------------------------------------------------------- */
 /* Embedding                                                                  */
 /* ------------------------------------------------------------------------- */

@@ -392,6 +392,50 @@ def test_forward_in_two_halves_and_serve_pool_match_plain_forward(pb):
     torch.cuda.synchronize()
 
 
+def test_serve_pool_spreads_its_streams_evenly_over_the_hardware_queues(pb):
+    """The pool creates its threads' streams and measures which of them share a hardware queue: every queue it saw
+    serves as many threads as any other, give or take one, whatever streams the process holds besides (some idle ones
+    are created first), and neighbouring threads sit on different queues.  Results are the plain Forward's."""
+    import collections
+    import torch
+    from ctr_model import build_manager, make_predictor
+    from synth import Config2
+    cfg = Config2(batch=64, rows=500, slots=26)
+    tables, mlp = cfg.tables(), cfg.mlp()
+    sparse, dense = cfg.batches(8)
+    pm, fgs = build_manager(cfg, tables, mlp, np.float16)
+    preds = [make_predictor(pm, fgs, sparse[b], dense[b], np.float16) for b in range(8)]
+    want = []
+    for p in preds:
+        p.forward()
+        want.append(p.output_asnumpy("prob").copy())
+    idle = [torch.cuda.Stream() for _ in range(3)]  # streams of the process that serve nothing
+    for st in idle:
+        with torch.cuda.stream(st):
+            torch.zeros(1, device="cuda")
+    torch.cuda.synchronize()
+    for threads in (8, 4, 2, 1):
+        pool = pb.ServePool(threads, 1)
+        assert pool.stream_queues() == []
+        pool.run(preds, 16)
+        q = pool.stream_queues()
+        print("threads", threads, "queues", q, flush=True)
+        assert len(q) == threads
+        per_queue = collections.Counter(q)
+        assert max(per_queue.values()) - min(per_queue.values()) <= 1, q
+        if threads == 8:
+            n_queues = len(per_queue)
+            assert n_queues >= 2, q  # the runtime's default is 4
+        assert len(per_queue) == min(threads, n_queues), q
+        if threads > 1 and len(per_queue) > 1:
+            assert all(q[t] != q[t + 1] for t in range(threads - 1)), q
+        pool.run(preds, 8)
+        assert pool.stream_queues() == q  # measured once
+        for b in range(8):
+            np.testing.assert_array_equal(preds[b].output_asnumpy("prob"), want[b])
+        del pool
+
+
 def test_skinny_last_layer_rides_in_the_launch_before_it(pb, oracle):
     """Gemm+PRelu (512 -> 256) followed by Gemm+Softmax (256 -> 2): by default the second runs inside the first one's
     launch (bz_fc_desc.head_*) and the 256-wide tensor between them is never stored; fuse_fc_head: 0 runs them one by

@@ -22,7 +22,7 @@ EXPORTS = [
     "bz_last_error", "bz_device_check", "bz_table_pitch", "bz_embed_plan", "bz_segments_to_offsets", "bz_segments_to_offsets_slots",
     "bz_embed_pool", "bz_embed_pool_args", "bz_embed_pool_static_scratch", "bz_embed_pool_kernel_name", "bz_fc_fused", "bz_fc_pack_weight", "bz_gemm_strided_batched", "bz_weighted_pool",
     "bz_activation", "bz_concat_cols", "bz_broadcast_op", "bz_reduce_sum", "bz_batch_norm", "bz_softmax_axis",
-    "bz_concat_ew", "bz_gather_rows"
+    "bz_concat_ew", "bz_gather_rows", "bz_spin"
 ]
 EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ASSIGN, EW_WHERE = 0, 1, 2, 3, 4, 5
 OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5  # bz_status
@@ -129,6 +129,7 @@ def lib():
         l.bz_table_pitch.argtypes = [i64, C.c_int]
         l.bz_table_pitch.restype = i32
         l.bz_embed_plan.argtypes = [C.POINTER(EmbedSlot), C.c_int, C.POINTER(EmbedLaunch)]
+        l.bz_spin.argtypes = [i64, vp]
         l.bz_segments_to_offsets.argtypes = [vp, vp, i64, vp]
         l.bz_segments_to_offsets_slots.argtypes = [vp, C.c_int, vp]
         l.bz_embed_pool.argtypes = [vp, C.POINTER(EmbedLaunch), vp]

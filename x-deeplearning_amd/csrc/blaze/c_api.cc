@@ -7,6 +7,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -17,6 +18,7 @@
 #include "blaze/predictor.h"
 #include "blaze/qed_builder.h"
 #include "blaze/qed_store.h"
+#include "blaze_hip.h"
 
 using blaze::Predictor;
 using blaze::PredictorManager;
@@ -226,8 +228,17 @@ struct ServePool {
   // request sees under the load of that job, as the reference's example times each Forward inside its serving loop
   // (example/cpp/predictor_example.cc:129-140)
   std::vector<std::vector<float>> latency_ms;
+  // The threads' streams, spread evenly over the hardware queues.  The runtime serves a handful of hardware queues (4 by
+  // default) and gives a new stream the least used one, counting every stream of the process, idle ones included: eight
+  // threads that each create a stream can end up 3-3-1-1 on the queues, and the threads that share a queue with two
+  // others then set the pace of the whole pool.  So the pool creates the streams itself at its first job, finds out by
+  // measurement which of them share a queue (ShareQueue), keeps an even selection and hands one to each thread.
+  int streams_device = -1;
+  std::vector<hipStream_t> assigned;  // stream of thread t (owned by the thread once it has adopted it)
+  std::vector<int> queue_of;          // the queue group of thread t's stream, numbered in order of discovery
+  std::vector<char> adopted;
 
-  explicit ServePool(int n) : latency_ms(n) {
+  explicit ServePool(int n) : latency_ms(n), adopted(n, 0) {
     for (int t = 0; t < n; ++t) threads.emplace_back([this, t] { Loop(t); });
   }
   ~ServePool() {
@@ -237,6 +248,91 @@ struct ServePool {
     }
     cv_work.notify_all();
     for (auto& th : threads) th.join();
+    for (size_t t = 0; t < assigned.size(); ++t)
+      if (!adopted[t] && assigned[t]) (void)hipStreamDestroy(assigned[t]);
+  }
+
+  // Do two streams share a hardware queue?  A kernel queued on b while a is kept busy finishes at once when they do not,
+  // and only after a's kernel when they do.  "At once" cannot be wrong; "late" can be the host's doing, so it is asked twice.
+  static bool ShareQueue(hipStream_t a, hipStream_t b) {
+    constexpr int kBusyUs = 300;
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      BZ_CHECK(bz_spin(kBusyUs, a));
+      const auto t0 = std::chrono::steady_clock::now();
+      BZ_CHECK(bz_spin(0, b));
+      HIP_CHECK(hipStreamSynchronize(b));
+      const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+      HIP_CHECK(hipStreamSynchronize(a));
+      if (us < kBusyUs / 2) return false;
+    }
+    return true;
+  }
+
+  void AssignStreams(int device) {
+    const int n = (int)threads.size();
+    int cur = 0;
+    HIP_CHECK(hipGetDevice(&cur));
+    if (cur != device) HIP_CHECK(hipSetDevice(device));
+    std::vector<hipStream_t> cand;
+    std::vector<int> group;               // of each candidate
+    std::vector<hipStream_t> first_of;    // a member of each group
+    std::vector<int> picked;              // candidates kept, in thread order
+    const int per_round = std::max(n, 8);  // a few more than a small pool needs, so that every queue shows up
+    for (int round = 0; round < 4 && (int)picked.size() < n; ++round) {
+      for (int i = 0; i < per_round; ++i) {
+        hipStream_t s = nullptr;
+        HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+        BZ_CHECK(bz_spin(0, s));  // the runtime binds a stream to its queue at the first launch
+        HIP_CHECK(hipStreamSynchronize(s));
+        int g = -1;
+        for (size_t k = 0; k < first_of.size() && g < 0; ++k)
+          if (ShareQueue(first_of[k], s)) g = (int)k;
+        if (g < 0) {
+          g = (int)first_of.size();
+          first_of.push_back(s);
+        }
+        cand.push_back(s);
+        group.push_back(g);
+      }
+      // as even a share of the n threads for every queue seen as there can be, the fuller shares to the queues that
+      // have the most candidates
+      const int G = (int)first_of.size();
+      std::vector<int> have(G, 0), order(G), cap(G, 0);
+      for (int g : group) ++have[g];
+      for (int g = 0; g < G; ++g) order[g] = g;
+      std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return have[a] > have[b]; });
+      for (int k = 0; k < G; ++k) cap[order[k]] = n / G + (k < n % G ? 1 : 0);
+      picked.clear();
+      std::vector<int> taken(G, 0);
+      for (size_t c = 0; c < cand.size() && (int)picked.size() < n; ++c)
+        if (taken[group[c]] < cap[group[c]]) {
+          ++taken[group[c]];
+          picked.push_back((int)c);
+        }
+    }
+    // (queues that never offered enough candidates: fill up with what there is)
+    std::vector<char> used(cand.size(), 0);
+    for (int c : picked) used[c] = 1;
+    for (size_t c = 0; c < cand.size() && (int)picked.size() < n; ++c)
+      if (!used[c]) {
+        used[c] = 1;
+        picked.push_back((int)c);
+      }
+    // threads that follow each other take different queues
+    std::vector<std::vector<int>> by_group(first_of.size());
+    for (int c : picked) by_group[group[c]].push_back(c);
+    assigned.clear();
+    queue_of.clear();
+    for (size_t k = 0; (int)assigned.size() < n; ++k)
+      for (auto& members : by_group)
+        if (k < members.size()) {
+          assigned.push_back(cand[members[k]]);
+          queue_of.push_back(group[members[k]]);
+        }
+    for (size_t c = 0; c < cand.size(); ++c)
+      if (!used[c]) HIP_CHECK(hipStreamDestroy(cand[c]));
+    streams_device = device;
+    if (cur != device) HIP_CHECK(hipSetDevice(cur));
   }
   void Loop(int t) {
     uint64_t seen = 0;
@@ -253,6 +349,18 @@ struct ServePool {
         if (stop) return;
         seen = generation;
         n_threads = (int)threads.size();
+      }
+      if (!adopted[t] && t < (int)assigned.size()) {
+        try {
+          blaze::HIPContext::AdoptThreadStream(streams_device, 0, assigned[t]);
+          adopted[t] = 1;
+        } catch (std::exception& e) {
+          blaze::last_error_for_thread() = e.what();
+          if (!failed.exchange(1)) {
+            std::lock_guard<std::mutex> lock(mu);
+            error = e.what();
+          }
+        }
       }
       // step i of the job runs predictor i % n_handles; thread t takes the steps i == t (mod n_threads), so a
       // predictor is only ever used by one thread when n_handles is a multiple of n_threads.  With at least `depth`
@@ -302,6 +410,14 @@ struct ServePool {
     }
   }
   bool Run(Predictor** h, int n, int64_t k) {
+    if (streams_device < 0 && n > 0 && h[0] != nullptr && h[0]->device_id() >= 0) {
+      try {
+        AssignStreams(h[0]->device_id());
+      } catch (std::exception& e) {
+        error = e.what();
+        return false;
+      }
+    }
     std::unique_lock<std::mutex> lock(mu);
     handles = h;
     n_handles = n;
@@ -374,6 +490,14 @@ int Blaze_PredictorForwardWait(PredictorHandle handle) {
   if (!p->ForwardWait()) return Fail("ForwardWait failed");
   return 0;
 }
+int Blaze_ServePoolStreamQueues(ServePoolHandle handle, int* queue_of_thread, int capacity, int* count) {
+  auto* pool = reinterpret_cast<ServePool*>(handle);
+  if (pool == nullptr || count == nullptr || (capacity > 0 && queue_of_thread == nullptr)) return Fail("ServePoolStreamQueues: bad arguments");
+  *count = (int)pool->queue_of.size();
+  for (int t = 0; t < *count && t < capacity; ++t) queue_of_thread[t] = pool->queue_of[t];
+  return 0;
+}
+
 int Blaze_ServePoolDelete(ServePoolHandle handle) {
   delete reinterpret_cast<ServePool*>(handle);
   (void)hipGetLastError();

@@ -207,6 +207,13 @@ int Predictor::InputDataType(const char* name) const {
   return idx < 0 ? (int)kPDT_Invalid : external_input_blob_[idx]->data_type();
 }
 
+int Predictor::device_id() const {
+  for (const auto* list : {&external_output_blob_, &external_input_blob_})
+    for (Blob* b : *list)
+      if (b->device_type() == kHIP) return b->device_option().device_id();
+  return -1;
+}
+
 bool Predictor::ForwardLaunch() {
   try {
     for (size_t i = 0; i < external_input_blob_.size(); ++i)

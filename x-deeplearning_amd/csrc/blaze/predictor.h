@@ -72,6 +72,8 @@ class Predictor {
   void RegisterObservers(const std::vector<std::string>& observer_names);
   void DumpObservers(std::unordered_map<std::string, std::string>* dump_map);
 
+  // extension: the device this predictor's blobs live on (-1: none of them is on a device)
+  int device_id() const;
   // extension: device address of an input / output blob, for callers that fill inputs on the device
   void* InputDevicePtr(const char* name);
   void* OutputDevicePtr(const char* name);

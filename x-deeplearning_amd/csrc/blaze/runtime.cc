@@ -71,28 +71,47 @@ void HIPContext::Activate() const {
   }
 }
 
+namespace {
+struct ThreadStreams {
+  std::vector<std::vector<hipStream_t>> per_device;
+  ~ThreadStreams() {
+    for (auto& v : per_device)
+      for (auto s : v)
+        if (s) (void)hipStreamDestroy(s);
+  }
+  hipStream_t& at(int device_id, int stream_id) {
+    BLAZE_CONDITION_THROW(device_id >= 0 && stream_id >= 0 && stream_id < kMaxStreamNum, "device_id=", device_id, " stream_id=", stream_id);
+    if ((int)per_device.size() <= device_id) per_device.resize(device_id + 1);
+    auto& v = per_device[device_id];
+    if (v.empty()) v.resize(kMaxStreamNum, nullptr);
+    return v[stream_id];
+  }
+};
+ThreadStreams& StreamsOfThisThread() {
+  static thread_local ThreadStreams tls;
+  return tls;
+}
+}  // namespace
+
 hipStream_t HIPContext::hip_stream(int device_id, int stream_id) {
-  struct Streams {
-    std::vector<std::vector<hipStream_t>> per_device;
-    ~Streams() {
-      for (auto& v : per_device)
-        for (auto s : v)
-          if (s) (void)hipStreamDestroy(s);
-    }
-  };
-  static thread_local Streams tls;
-  BLAZE_CONDITION_THROW(stream_id >= 0 && stream_id < kMaxStreamNum, "stream_id=", stream_id);
-  if ((int)tls.per_device.size() <= device_id) tls.per_device.resize(device_id + 1);
-  auto& v = tls.per_device[device_id];
-  if (v.empty()) v.resize(kMaxStreamNum, nullptr);
-  if (v[stream_id] == nullptr) {
+  hipStream_t& s = StreamsOfThisThread().at(device_id, stream_id);
+  if (s == nullptr) {
     int cur = 0;
     HIP_CHECK(hipGetDevice(&cur));
     if (cur != device_id) HIP_CHECK(hipSetDevice(device_id));
-    HIP_CHECK(hipStreamCreateWithFlags(&v[stream_id], hipStreamNonBlocking));  // default priority
+    HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
     if (cur != device_id) HIP_CHECK(hipSetDevice(cur));
   }
-  return v[stream_id];
+  return s;
+}
+
+void HIPContext::AdoptThreadStream(int device_id, int stream_id, hipStream_t stream) {
+  hipStream_t& s = StreamsOfThisThread().at(device_id, stream_id);
+  if (s != nullptr && s != stream) {
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipStreamDestroy(s));
+  }
+  s = stream;
 }
 
 void CopyBytes(void* dst, int dst_device_type, const void* src, int src_device_type, size_t bytes, hipStream_t stream) {

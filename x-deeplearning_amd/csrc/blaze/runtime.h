@@ -239,6 +239,10 @@ class HIPContext {
   hipStream_t hip_stream() const { return hip_stream(device_id_, stream_id_); }
   void* device_stream() const { return (void*)hip_stream(); }
   static hipStream_t hip_stream(int device_id, int stream_id);  // thread-local, created on first use
+  // makes `stream` (created on device_id, default priority) the calling thread's stream from now on; the thread owns it:
+  // it is destroyed when the thread ends, like one created on first use.  A stream the thread already had is
+  // waited for and destroyed.
+  static void AdoptThreadStream(int device_id, int stream_id, hipStream_t stream);
   void FinishDeviceComputation() {
     Activate();
     HIP_CHECK(hipStreamSynchronize(hip_stream()));

@@ -29,7 +29,7 @@ EXPORTS = [
     "Blaze_HipStoreAddTable", "Blaze_PredictorManagerLoadModelFromString", "Blaze_PredictorInputDevicePtr",
     "Blaze_PredictorOutputDevicePtr", "Blaze_PredictorForwardN", "Blaze_ConvertNetDef", "Blaze_ServePoolCreate",
     "Blaze_ServePoolRun", "Blaze_ServePoolDelete", "Blaze_ServePoolSetDepth", "Blaze_ServePoolLatencies", "Blaze_PredictorForwardLaunch",
-    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount", "Blaze_HipStoreGet"
+    "Blaze_PredictorForwardWait", "Blaze_PredictorFeedMany", "Blaze_AllocationCount", "Blaze_HipStoreGet", "Blaze_ServePoolStreamQueues"
 ]
 
 
@@ -257,6 +257,14 @@ class ServePool(object):
 
     def set_depth(self, depth):
         check_call(lib().Blaze_ServePoolSetDepth(self.handle, depth))
+
+    def stream_queues(self):
+        """the hardware-queue group of each thread's stream, as the pool measured it at its first job ([] before)"""
+        n = C.c_int(0)
+        check_call(lib().Blaze_ServePoolStreamQueues(self.handle, None, 0, C.byref(n)))
+        out = (C.c_int * max(n.value, 1))()
+        check_call(lib().Blaze_ServePoolStreamQueues(self.handle, out, n.value, C.byref(n)))
+        return list(out[:n.value])
 
     def latencies_ms(self):
         """per-pass latency (launch to the return of the wait) of the last run, all threads, as a float32 array"""
