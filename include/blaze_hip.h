@@ -187,12 +187,13 @@ BZ_API int bz_embed_pool(const bz_embed_slot* slots_dev, const bz_embed_launch* 
 /*
  * The same launch with the slot records handed over as kernel arguments instead of read from device memory (one trip
  * to memory fewer at the head of every workgroup, and no device copy of the records to keep).  slots_host: the records
- * bz_embed_plan saw, in host memory; they are copied into the launch.  Takes plans of one row shape (ksum / kavg, one
- * table dtype and dim: launch->variant != 0) with the scan fused in and at most BZ_EMBED_ARG_SLOTS slots; otherwise
- * BZ_ENOTSUP and nothing is launched -- call bz_embed_pool with a device copy then.  Same results bit for bit.
+ * bz_embed_plan saw, in host memory; they are copied into the launch.  Takes plans with the scan fused in
+ * (launch->fused_scan, no slot bringing offsets) and at most BZ_EMBED_ARG_SLOTS slots of one row shape
+ * (launch->variant != 0) or at most 16 mixed ones (kassign items, several dims or dtypes); otherwise BZ_ENOTSUP and nothing is launched -- call bz_embed_pool with a
+ * device copy then.  Same results bit for bit.
  * Reference: as bz_embed_pool.
  */
-#define BZ_EMBED_ARG_SLOTS 26 /* 26 records of 144 bytes + the other arguments fit the 4 KB kernel-argument segment */
+#define BZ_EMBED_ARG_SLOTS 26 /* 26 records of 152 bytes + the other arguments fit the 4 KB kernel-argument segment */
 BZ_API int bz_embed_pool_args(const bz_embed_slot* slots_host, const bz_embed_launch* launch, bz_stream_t stream);
 
 /*

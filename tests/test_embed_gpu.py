@@ -63,6 +63,15 @@ def _run_gpu(bz, tables_np, specs, inputs, batch, out_np_dtype, strides_cols, fu
     plan.run()
     torch.cuda.synchronize()
     offs = [o.cpu().numpy() for o in plan.offsets]
+    if plan.args_eligible():
+        # the same launch with the slot records handed over as kernel arguments: the same bits (NaN fill included:
+        # the columns of no item stay as they were)
+        out2 = torch.full_like(out, float("nan"))
+        for it in items:
+            it["out"] = out2
+        bz.EmbeddingPlan(items, fused_scan=fused_scan).pool_args()
+        torch.cuda.synchronize()
+        assert np.array_equal(out2.cpu().numpy().view(np.uint8), out.cpu().numpy().view(np.uint8)), "kernel-argument form differs"
     return out.cpu().numpy(), offs, plan.launch.variant
 
 

@@ -334,8 +334,8 @@ class EmbeddingPlan:
         check(lib().bz_embed_pool(self.slots_dev.data_ptr(), C.byref(self.launch), _stream_ptr(stream)))
 
     def args_eligible(self):
-        """what bz_embed_pool_args takes: one row shape, scan fused in, few slots"""
-        return bool(self.launch.variant != 0 and self.launch.fused_scan and not self.launch.scan_first and self.n <= 26)
+        """what bz_embed_pool_args takes: scan fused in, few slots"""
+        return bool(self.launch.fused_scan and not self.launch.scan_first and self.n <= 26)
 
     def pool_args(self, stream=None):
         """the same launch with the slot records handed over as kernel arguments"""

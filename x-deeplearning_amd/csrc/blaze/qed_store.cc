@@ -546,8 +546,8 @@ Status QedHipSparsePuller::GetOnStream(const std::vector<SparsePullerInput>& inp
     }
     BZ_CHECK(bz_embed_plan(slots.data(), (int)slots.size(), &sc->launch));
   }
-  // a ksum / kavg operator of one row shape and few slots: the records travel as kernel arguments, nothing to upload
-  if (sc->launch.variant != 0 && sc->launch.fused_scan && !sc->launch.scan_first && slots.size() <= (size_t)BZ_EMBED_ARG_SLOTS) {
+  // an operator of few slots: the records travel as kernel arguments, nothing to upload
+  if (sc->launch.fused_scan && !sc->launch.scan_first && slots.size() <= (size_t)(sc->launch.variant != 0 ? BZ_EMBED_ARG_SLOTS : 16)) {
     BZ_CHECK(bz_embed_pool_args(slots.data(), &sc->launch, st));
     return kOK;
   }

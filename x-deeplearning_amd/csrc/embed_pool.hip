@@ -42,6 +42,8 @@
 
 #include "bz_common.h"
 
+#include <limits.h>
+
 namespace {
 
 constexpr int kThreads = 512;  // measured at 128 / 256 / 512 / 1024 on config 2: 14.7 / 13.5 / 13.3 / 13.4 us per launch,
@@ -612,7 +614,7 @@ constexpr int64_t kScanFirstBytes = 128ll << 20;
 struct SlotPack {
   bz_embed_slot s[BZ_EMBED_ARG_SLOTS];
 };
-static_assert(sizeof(SlotPack) + 64 <= 4096, "the records and the other arguments fit the 4 KB kernel-argument segment");
+static_assert(sizeof(SlotPack) + 4 * 16 + 32 <= 4096, "the records and the other arguments fit the 4 KB kernel-argument segment");
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t kBeyondTable = 0xF0000000u;  // a byte offset no table read through a buffer resource reaches
@@ -771,6 +773,61 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_args_kernel(const Slot
 
 __device__ __forceinline__ int chunk_elems(int dt) { return dt == BZ_F32 ? 4 : (dt == BZ_F16 ? 8 : 16); }
 
+// one workgroup of the generic path: workgroup v of the launch, owned by slot s
+__device__ __forceinline__ void pool_generic(const bz_embed_slot& s, int v, const int64_t* __restrict__ offsets, int64_t* s_off,
+                                             int64_t* s_part) {
+  const int ce = chunk_elems(s.table_dtype);
+  const int nchunks = (s.dim + ce - 1) / ce;
+  // lpr, a power of two: shifts, not divisions (a 64-bit division is some 150 instructions, and this kernel's threads
+  // each do little else than one or four row gathers)
+  int lpr_log = 0;
+  while ((1 << lpr_log) < nchunks && (1 << lpr_log) < bz::kWave) ++lpr_log;
+  const int lpr = 1 << lpr_log;
+  const int groups = kThreads >> lpr_log;
+  const int tid = threadIdx.x;
+  const int g = tid >> lpr_log;
+  const int l = tid - (g << lpr_log);
+  // a lane group owns one item: a sample (ksum / kavg) or kAssignRun output positions of a sample (kassign)
+  const int64_t per = items_per_sample(s);
+  const int64_t n_items = (int64_t)s.batch * per;
+  const int64_t i0 = (int64_t)(v - s.wg_begin) * groups;
+  int64_t i_last = i0 + groups - 1;
+  if (i_last >= n_items) i_last = n_items - 1;
+  // item -> sample: no division for pooled slots (per == 1), a 32-bit one while the item count allows it
+  auto sample_of = [&](int64_t item) -> int64_t {
+    if (per == 1) return item;
+    if (n_items < (1ll << 31)) return (int64_t)((uint32_t)item / (uint32_t)per);
+    return item / per;
+  };
+  const int64_t b_first = sample_of(i0);
+  const int n_samples = (int)(sample_of(i_last) - b_first) + 1;  // <= groups
+  stage_offsets(s, offsets, b_first, n_samples, s_off, s_part);
+  const int64_t item = i0 + g;
+  if (item >= n_items) return;
+  const int64_t b = sample_of(item);
+  const int p = (int)(item - b * per) * (s.udf == BZ_ASSIGN ? kAssignRun : 1);
+  if (s.table == nullptr) {
+    pool_zero(s, b, p, l, lpr);
+    return;
+  }
+  const int64_t start = s_off[b - b_first], end = s_off[b - b_first + 1];
+  for (int c = l; c < nchunks; c += lpr) {
+    if (s.udf == BZ_ASSIGN) {
+      switch (s.table_dtype) {
+        case BZ_F32: pool_assign<BZ_F32>(s, start, end, c, b, p); break;
+        case BZ_F16: pool_assign<BZ_F16>(s, start, end, c, b, p); break;
+        default: pool_assign<BZ_I8>(s, start, end, c, b, p); break;
+      }
+    } else {
+      switch (s.table_dtype) {
+        case BZ_F32: pool_sum<BZ_F32>(s, start, end, c, b); break;
+        case BZ_F16: pool_sum<BZ_F16>(s, start, end, c, b); break;
+        default: pool_sum<BZ_I8>(s, start, end, c, b); break;
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const bz_embed_slot* __restrict__ slots,
                                                                          int n_slots, int total_wg, int wg_per_xcd,
                                                                          int wg_per_slot, const int64_t* __restrict__ ext_off,
@@ -799,56 +856,30 @@ __global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_kernel(const b
   }
   // slots with wg_count == 0 sharing this begin come before the one that owns the workgroup
   const bz_embed_slot s = slots[lo];
-  const int ce = chunk_elems(s.table_dtype);
-  const int nchunks = (s.dim + ce - 1) / ce;
-  // lpr, a power of two: shifts, not divisions (a 64-bit division is some 150 instructions, and this kernel's threads
-  // each do little else than one or four row gathers)
-  int lpr_log = 0;
-  while ((1 << lpr_log) < nchunks && (1 << lpr_log) < bz::kWave) ++lpr_log;
-  const int lpr = 1 << lpr_log;
-  const int groups = kThreads >> lpr_log;
-  const int tid = threadIdx.x;
-  const int g = tid >> lpr_log;
-  const int l = tid - (g << lpr_log);
-  // a lane group owns one item: a sample (ksum / kavg) or kAssignRun output positions of a sample (kassign)
-  const int64_t per = items_per_sample(s);
-  const int64_t n_items = (int64_t)s.batch * per;
-  const int64_t i0 = (int64_t)(v - s.wg_begin) * groups;
-  int64_t i_last = i0 + groups - 1;
-  if (i_last >= n_items) i_last = n_items - 1;
-  // item -> sample: no division for pooled slots (per == 1), a 32-bit one while the item count allows it
-  auto sample_of = [&](int64_t item) -> int64_t {
-    if (per == 1) return item;
-    if (n_items < (1ll << 31)) return (int64_t)((uint32_t)item / (uint32_t)per);
-    return item / per;
-  };
-  const int64_t b_first = sample_of(i0);
-  const int n_samples = (int)(sample_of(i_last) - b_first) + 1;  // <= groups
-  stage_offsets(s, ext_off != nullptr ? ext_off + (int64_t)lo * ext_stride : s.offsets, b_first, n_samples, s_off, s_part);
-  const int64_t item = i0 + g;
-  if (item >= n_items) return;
-  const int64_t b = sample_of(item);
-  const int p = (int)(item - b * per) * (s.udf == BZ_ASSIGN ? kAssignRun : 1);
-  if (s.table == nullptr) {
-    pool_zero(s, b, p, l, lpr);
-    return;
+  pool_generic(s, v, ext_off != nullptr ? ext_off + (int64_t)lo * ext_stride : s.offsets, s_off, s_part);
+}
+
+// the same with the slot records as kernel arguments: no trip for the begins, none for the record
+struct SlotBegins {
+  int b[16];  // wg_begin of every slot, INT_MAX behind the last: read with one wide scalar load
+};
+
+__global__ __launch_bounds__(kThreads) void bz_embed_pool_generic_args_kernel(const SlotPack pack, const SlotBegins begins,
+                                                                              int total_wg, int wg_per_xcd, int wg_per_slot) {
+  __shared__ int64_t s_off[kThreads + 1];
+  __shared__ int64_t s_part[2 * kThreads / bz::kWave];
+  const int v = (int)(blockIdx.x % bz::kNumXcd) * wg_per_xcd + (int)(blockIdx.x / bz::kNumXcd);
+  if (v >= total_wg) return;
+  int lo;
+  if (wg_per_slot > 0) {
+    lo = v / wg_per_slot;
+  } else {
+    lo = -1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) lo += begins.b[i] <= v ? 1 : 0;  // uniform: scalar compares
   }
-  const int64_t start = s_off[b - b_first], end = s_off[b - b_first + 1];
-  for (int c = l; c < nchunks; c += lpr) {
-    if (s.udf == BZ_ASSIGN) {
-      switch (s.table_dtype) {
-        case BZ_F32: pool_assign<BZ_F32>(s, start, end, c, b, p); break;
-        case BZ_F16: pool_assign<BZ_F16>(s, start, end, c, b, p); break;
-        default: pool_assign<BZ_I8>(s, start, end, c, b, p); break;
-      }
-    } else {
-      switch (s.table_dtype) {
-        case BZ_F32: pool_sum<BZ_F32>(s, start, end, c, b); break;
-        case BZ_F16: pool_sum<BZ_F16>(s, start, end, c, b); break;
-        default: pool_sum<BZ_I8>(s, start, end, c, b); break;
-      }
-    }
-  }
+  const bz_embed_slot s = pack.s[lo];
+  pool_generic(s, v, s.offsets, s_off, s_part);
 }
 
 int groups_per_wg(const bz_embed_slot& s) {
@@ -1039,10 +1070,9 @@ int bz_embed_pool_args(const bz_embed_slot* slots_host, const bz_embed_launch* l
   const bz_embed_launch& L = *launch;
   BZ_REQUIRE(L.n_slots > 0 && L.total_wg >= 0 && L.wg_per_slot >= 0, "bz_embed_pool_args: bad launch record (n_slots=%d total_wg=%d)",
              L.n_slots, L.total_wg);
-  if (L.variant == 0 || L.n_slots > BZ_EMBED_ARG_SLOTS || !L.fused_scan || L.scan_first)
-    return bz::fail(BZ_ENOTSUP, "bz_embed_pool_args: takes ksum / kavg plans of one row shape with at most %d slots and the scan fused in",
-                    BZ_EMBED_ARG_SLOTS);
-  BZ_REQUIRE(L.wg_per_slot > 0 && (int64_t)L.wg_per_slot * L.n_slots == L.total_wg,
+  if (L.n_slots > BZ_EMBED_ARG_SLOTS || !L.fused_scan || L.scan_first)
+    return bz::fail(BZ_ENOTSUP, "bz_embed_pool_args: takes plans with at most %d slots and the scan fused in", BZ_EMBED_ARG_SLOTS);
+  BZ_REQUIRE(L.variant == 0 || (L.wg_per_slot > 0 && (int64_t)L.wg_per_slot * L.n_slots == L.total_wg),
              "bz_embed_pool_args: variant %#x needs equal work per slot", L.variant);
   if (L.total_wg == 0) return BZ_OK;
   SlotPack pack;
@@ -1051,6 +1081,17 @@ int bz_embed_pool_args(const bz_embed_slot* slots_host, const bz_embed_launch* l
   const int per_xcd = (L.total_wg + bz::kNumXcd - 1) / bz::kNumXcd;
   const dim3 grid(per_xcd * bz::kNumXcd), block(kThreads);
   hipStream_t st = bz::as_stream(stream);
+  if (L.variant == 0) {
+    if (L.n_slots > 16) return bz::fail(BZ_ENOTSUP, "bz_embed_pool_args: a plan of mixed row shapes takes at most 16 slots");
+    for (int i = 0; i < L.n_slots; ++i)
+      BZ_REQUIRE(pack.s[i].offsets == nullptr, "bz_embed_pool_args: slot %d brings offsets, but the plan says the scan is fused in", i);
+    SlotBegins begins;
+    for (int i = 0; i < 16; ++i) begins.b[i] = i < L.n_slots ? pack.s[i].wg_begin : INT_MAX;
+    hipLaunchKernelGGL(bz_embed_pool_generic_args_kernel, grid, block, 0, st, pack, begins, L.total_wg, per_xcd,
+                       ((int64_t)L.wg_per_slot * L.n_slots == L.total_wg) ? L.wg_per_slot : 0);
+    BZ_LAUNCH_OK("bz_embed_pool_generic_args_kernel");
+    return BZ_OK;
+  }
   const int dt = L.variant >> 8, lpr = L.variant & 0xff;
 #define BZ_POOL(DT, LPR) \
   hipLaunchKernelGGL((bz_embed_pool_args_kernel<DT, LPR>), grid, block, 0, st, pack, L.total_wg, per_xcd, L.wg_per_slot)
