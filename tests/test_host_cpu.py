@@ -565,3 +565,41 @@ def test_synthetic_configs_come_from_the_generator_streams():
     q, sc = c4.tables(device="cpu")[1]
     rq, rsc = c4.table_rows(1, [1999, 3])
     assert np.array_equal(rq, q[[1999, 3]].numpy()) and np.array_equal(rsc, sc[[1999, 3]].numpy())
+
+
+@pytest.mark.timeout(600)
+def test_file_parsers_under_address_and_undefined_behaviour_sanitizers(tmp_path, kats):
+    """The host code that reads files from outside (NetDef text and wire format, the optimizer passes, the Embedding
+    config text, the QED builder's text tables) is compiled with -fsanitize=address,undefined and fed seeded mutations
+    of the golden inputs (tests/sanitize_host_parsers.cc): rejecting an input is fine, a sanitizer finding aborts."""
+    import shutil
+    import subprocess
+    if shutil.which("g++") is None:
+        pytest.skip("no g++")
+    csrc = os.path.join(ROOT, "x-deeplearning_amd", "csrc")
+    exe = str(tmp_path / "sanitize_host_parsers")
+    cmd = ["g++", "-std=c++17", "-O1", "-g", "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
+           "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"), "-I" + csrc,
+           os.path.join(ROOT, "tests", "sanitize_host_parsers.cc")] + [os.path.join(csrc, "blaze", f) for f in
+                                                                       ("proto.cc", "optimizer.cc", "common.cc", "qed_builder.cc")] + ["-o", exe]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=300)
+    # an embedding config of the reference's own operator tests as the seed for that parser
+    ec = None
+    for case in kats.values():
+        for op in case.get("ops", []):
+            if "embedding_config" in op.get("args", {}):
+                ec = op["args"]["embedding_config"]
+                break
+        if ec:
+            break
+    assert ec, "no embedding_config among the reference operator fixtures"
+    ec_file = tmp_path / "embedding_config.txt"
+    ec_file.write_text(ec)
+    golden = os.path.join(ROOT, "tests", "golden")
+    nets = [os.path.join(golden, "model_blaze_optimized.bin")] + [os.path.join(golden, "pattern", f) for f in
+                                                                  ("parallel_gemm_fusion.blaze", "in_order_gemm_gemm_fusion.blaze",
+                                                                   "in_order_gemm_gemm_fusion4.blaze")]
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=1")
+    r = subprocess.run([exe, "1500", "7", str(tmp_path / "scratch"), os.path.join(golden, "quick_embedding"), str(ec_file)] + nets,
+                       capture_output=True, text=True, errors="replace", timeout=500, env=env)
+    assert r.returncode == 0 and "sanitize_host_parsers: done" in r.stdout, (r.returncode, r.stderr[-3000:])
