@@ -632,6 +632,13 @@ __device__ __forceinline__ void pool_samples(const bz_embed_slot& s, int64_t b0,
   int64_t start, end;
   if (offsets == nullptr && s.nnz < (1ll << 31)) {
     own_segment<LPR>(s, b0, (uint32_t*)s_part, &start, &end);
+  } else if (offsets != nullptr) {
+    // every lane of a group asks for its sample's two offsets itself (one address a group): nothing goes through LDS
+    // and no wave waits for another's.  Caller-made offsets get the same bounds as the scan's.
+    const int64_t bb = b0 + g < s.batch ? b0 + g : s.batch - 1;  // (lanes past the batch return below)
+    const int64_t o0 = offsets[bb], o1 = offsets[bb + 1];
+    start = o0 < 0 ? 0 : (o0 < s.nnz ? o0 : s.nnz);
+    end = o1 < 0 ? 0 : (o1 < s.nnz ? o1 : s.nnz);
   } else {
     stage_offsets(s, offsets, b0, GROUPS, s_off, s_part);
     start = s_off[g];
