@@ -306,12 +306,12 @@ def test_baseline_forward_with_library_sgemm_agrees_with_the_pinned_sums(oracle)
 
 # ---------------------------------------------------------------- documents and reference-held data files
 def test_integration_c_snippet_compiles_against_the_header():
-    """The C example of INTEGRATION.md names only entry points include/blaze_c_api.h declares (gcc -fsyntax-only)."""
+    """The C example of the integration guide names only entry points include/blaze_c_api.h declares (gcc -fsyntax-only)."""
     import subprocess
     import tempfile
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     blocks = re.findall(r"```c\n(.*?)```", text, flags=re.S)
-    assert blocks, "no ```c block in INTEGRATION.md"
+    assert blocks, "no ```c block in the integration guide"
     body = blocks[0].replace("...", "")
     m = re.match(r"(\s*#include[^\n]*\n)(.*)", body, flags=re.S)
     src = (m.group(1) + "#include <stdint.h>\nvoid example(const int* shape, void* ids, int nnz, void* out, size_t out_bytes) {\n" +
